@@ -1,0 +1,95 @@
+"""Tiny configurations (config.json dictionaries) used by the tests.
+
+TINY_LLAMA and TINY_MISTRAL differ in every size and option: head counts and
+groups, head size, width and hidden width that are no powers of two, number of
+layers, vocabulary, eps, theta, window, tied / untied head."""
+import copy
+
+TINY_LLAMA = {
+    "architectures": ["LlamaForCausalLM"],
+    "hidden_size": 64,
+    "intermediate_size": 176,
+    "num_hidden_layers": 2,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 2,
+    "head_dim": 16,
+    "vocab_size": 256,
+    "max_position_embeddings": 128,
+    "rope_theta": 10000.0,
+    "rms_norm_eps": 1e-5,
+    "hidden_act": "silu",
+    "tie_word_embeddings": True,
+    "bos_token_id": 1,
+    "eos_token_id": 2,
+}
+
+TINY_MISTRAL = {
+    "architectures": ["MistralForCausalLM"],
+    "hidden_size": 96,
+    "intermediate_size": 256,
+    "num_hidden_layers": 3,
+    "num_attention_heads": 3,
+    "num_key_value_heads": 1,
+    "head_dim": 32,
+    "vocab_size": 320,
+    "max_position_embeddings": 64,
+    "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-6,
+    "hidden_act": "silu",
+    "sliding_window": 16,
+    "tie_word_embeddings": False,
+    "bos_token_id": 1,
+    "eos_token_id": 2,
+}
+
+# llama3 rope scaling with a small original length, so that all three frequency
+# regimes occur inside 128 positions; vocabulary that is no multiple of 16.
+TINY_LLAMA3 = copy.deepcopy(TINY_LLAMA)
+TINY_LLAMA3.update({
+    "vocab_size": 250,
+    "head_dim": 32,
+    "num_attention_heads": 2,
+    "num_key_value_heads": 2,
+    "rope_theta": 500.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 32},
+    "max_position_embeddings": 256,
+})
+
+# heads * head_dim != hidden_size (the reference silently assumes equality,
+# model.cpp:289); a longer context with a window in the middle of it.
+TINY_WIDE_HEADS = copy.deepcopy(TINY_MISTRAL)
+TINY_WIDE_HEADS.update({
+    "hidden_size": 80,
+    "intermediate_size": 208,
+    "num_attention_heads": 6,
+    "num_key_value_heads": 3,
+    "head_dim": 48,
+    "vocab_size": 311,
+    "num_hidden_layers": 2,
+    "sliding_window": 100,
+    "max_position_embeddings": 512,
+    "rms_norm_eps": 3e-6,
+})
+
+# a long context without a window: many pages of the cache, far keys
+TINY_LONG = copy.deepcopy(TINY_LLAMA)
+TINY_LONG.update({
+    "max_position_embeddings": 1024,
+    "num_hidden_layers": 2,
+    "head_dim": 64,
+    "hidden_size": 128,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 1,
+    "intermediate_size": 144,
+    "vocab_size": 200,
+    "tie_word_embeddings": False,
+})
+
+ALL = {
+    "tiny_llama": TINY_LLAMA,
+    "tiny_mistral": TINY_MISTRAL,
+    "tiny_llama3": TINY_LLAMA3,
+    "tiny_wide_heads": TINY_WIDE_HEADS,
+    "tiny_long": TINY_LONG,
+}
