@@ -1,0 +1,389 @@
+"""Each HIP kernel alone against its plain reference (the functions of
+tests/plain/reference_model.py, or float64 library routines), at sizes other
+than the engine's tiny models use: widths and vocabularies that are no powers
+of two, head sizes in steps of 16, odd head counts and groups."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from plain import reference_model as R
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def K():
+    from yalm_amd.ops import kernels
+    return kernels
+
+
+def rnd(shape, seed, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g, dtype=torch.float64) * scale).to(dtype)
+
+
+def tol(dtype):
+    return 2e-5 if dtype == torch.float32 else 1.2e-2
+
+
+def close(got, want, dtype, what, factor=1.0):
+    got = got.detach().to("cpu", torch.float64)
+    want = want.to(torch.float64)
+    assert torch.isfinite(got).all(), what
+    err = (got - want).abs().max().item()
+    lim = factor * tol(dtype) * max(1.0, want.abs().max().item())
+    assert err <= lim, "%s: max error %.3e, allowed %.3e" % (what, err, lim)
+
+
+def i32(x):
+    return torch.tensor(x, dtype=torch.int32, device=DEV)
+
+
+# ------------------------------------------------------------------ embedding, norm
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(dtype):
+    V, D = 37, 50
+    table = rnd((V, D), 1, dtype)
+    tokens = [0, 36, 5, 5, -1, 12]
+    out = torch.full((len(tokens), D), 7.0, device=DEV)
+    K().embed(table.to(DEV), i32(tokens), out)
+    want = R.embedding(table, torch.tensor([t if t >= 0 else 0 for t in tokens]))
+    want[4] = 0
+    assert torch.equal(out.cpu().double(), want)
+
+
+@pytest.mark.parametrize("out_dtype", DTYPES)
+@pytest.mark.parametrize("w_dtype", DTYPES)
+@pytest.mark.parametrize("D", [50, 1000, 4100])
+def test_rmsnorm(D, w_dtype, out_dtype):
+    x = rnd((7, D), 2, scale=3.0)
+    w = (1 + 0.1 * rnd((D,), 3)).to(w_dtype)
+    out = torch.empty((7, D), dtype=out_dtype, device=DEV)
+    K().rmsnorm(x.to(DEV), w.to(DEV), out, 1e-3)
+    close(out, R.rmsnorm(x, w, 1e-3), out_dtype, "rmsnorm")
+    # gathered rows, one of them padding
+    idx = [6, 0, -1, 3]
+    out = torch.empty((4, D), dtype=out_dtype, device=DEV)
+    K().rmsnorm(x.to(DEV), w.to(DEV), out, 1e-3, i32(idx))
+    want = R.rmsnorm(x[[6, 0, 0, 3]], w, 1e-3)
+    want[2] = 0
+    close(out, want, out_dtype, "rmsnorm rows")
+    # eps inside the root, added to the mean: ones with eps 3 -> 1/2
+    one = torch.ones((1, D), device=DEV)
+    out = torch.empty((1, D), dtype=torch.float32, device=DEV)
+    K().rmsnorm(one, torch.ones(D, device=DEV), out, 3.0)
+    assert torch.allclose(out.cpu(), torch.full((1, D), 0.5))
+
+
+# ------------------------------------------------------------------ GEMM
+
+GEMM_SHAPES = [(1, 16, 256), (3, 70, 96), (64, 130, 264), (65, 64, 80), (200, 333, 1000), (8, 4096 + 16, 136),
+               (130, 100, 50)]
+
+
+@pytest.mark.parametrize("simple", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,Kd", GEMM_SHAPES)
+def test_gemm_store_and_add(M, N, Kd, dtype, simple):
+    k = K()
+    a = rnd((M, Kd), 4, dtype)
+    w = rnd((N, Kd), 5, dtype, scale=1 / math.sqrt(Kd))
+    want = a.double() @ w.double().T
+    k.FORCE_SIMPLE = simple
+    try:
+        out = torch.empty((M, N), dtype=torch.float32, device=DEV)
+        k.gemm(a.to(DEV), w.to(DEV), out, k.EPI_STORE_F32)
+        close(out, want, torch.float32, "gemm f32 out", factor=4 if dtype == torch.float32 else 1)
+        out2 = torch.empty((M, N), dtype=dtype, device=DEV)
+        k.gemm(a.to(DEV), w.to(DEV), out2, k.EPI_STORE)
+        close(out2, want, dtype, "gemm store")
+        res = rnd((M, N), 6)
+        acc = res.to(DEV).clone()
+        k.gemm(a.to(DEV), w.to(DEV), acc, k.EPI_ADD_F32)
+        close(acc, want + res.double(), torch.float32, "gemm add", factor=4 if dtype == torch.float32 else 1)
+    finally:
+        k.FORCE_SIMPLE = False
+
+
+@pytest.mark.parametrize("simple", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,H,D", [(1, 16, 64), (5, 176, 64), (70, 100, 96), (64, 1000, 264), (3, 14336, 128)])
+def test_gemm_gated(M, H, D, dtype, simple):
+    from yalm_amd.parts.swiglu import interleave_gate_up
+    k = K()
+    x = rnd((M, D), 7, dtype)
+    wg = rnd((H, D), 8, dtype, scale=1 / math.sqrt(D))
+    wu = rnd((H, D), 9, dtype, scale=1 / math.sqrt(D))
+    g = x.double() @ wg.double().T
+    u = x.double() @ wu.double().T
+    want = R.silu(g) * u
+    k.FORCE_SIMPLE = simple
+    try:
+        out = torch.empty((M, H), dtype=dtype, device=DEV)
+        k.gemm(x.to(DEV), interleave_gate_up(wg, wu).to(DEV), out, k.EPI_GATED, hidden=H)
+        close(out, want, dtype, "gated gemm")
+    finally:
+        k.FORCE_SIMPLE = False
+
+
+def test_gemm_vector_of_the_reference():
+    """src/test.cpp:157-168: n = 256 inputs, d = 16 outputs, N(0,1), absolute 1e-4."""
+    k = K()
+    for seed in (0, 1):
+        w = rnd((16, 256), seed)
+        x = rnd((1, 256), seed + 10)
+        out = torch.empty((1, 16), device=DEV)
+        k.gemm(x.to(DEV), w.to(DEV), out, k.EPI_STORE_F32)
+        assert (out.cpu().double() - x.double() @ w.double().T).abs().max() < 1e-4
+
+
+# ------------------------------------------------------------------ rotation + cache write
+
+def make_table(n_pos, hd, rd, theta):
+    f = R.rope_inv_freq(hd, rd, theta)[: rd // 2]
+    ang = torch.arange(n_pos, dtype=torch.float64)[:, None] * f[None, :]
+    return torch.stack([torch.cos(ang), torch.sin(ang)], -1).float().contiguous()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,rd", [(4, 2, 16, 16), (3, 1, 48, 48), (6, 3, 32, 16), (2, 2, 128, 128)])
+def test_rope_kv_write(n_heads, n_kv, hd, rd, dtype):
+    k = K()
+    PAGE = k.PAGE
+    n_pages, n_slots, ring = 9, 4, 3
+    # two sequences: slot 2 with positions 60..69 (crosses a page), slot 0 with positions 0..4
+    pos = list(range(60, 70)) + list(range(5))
+    seq = [0] * 10 + [1] * 5
+    T = len(pos)
+    Q, KV = n_heads * hd, n_kv * hd
+    qkv = rnd((T, Q + 2 * KV), 11)
+    table = make_table(80, hd, rd, 10000.0)
+    bt = torch.full((n_slots, ring), -1, dtype=torch.int32)
+    bt[2, 0], bt[2, 1], bt[0, 0] = 5, 7, 1
+    kp = torch.zeros((n_pages, n_kv, PAGE, hd), dtype=dtype, device=DEV)
+    vp = torch.zeros((n_pages, n_kv, hd, PAGE), dtype=dtype, device=DEV)
+    q_out = torch.empty((T, Q), dtype=dtype, device=DEV)
+    k_out = torch.empty((T, KV), dtype=dtype, device=DEV)
+    v_out = torch.empty((T, KV), dtype=dtype, device=DEV)
+    k.rope_kv_write(qkv.to(DEV), q_out, k_out, v_out, kp, vp, bt.to(DEV), ring, i32(seq), i32(pos), i32([2, 0]),
+                    i32([70, 5]), table.to(DEV), n_heads, n_kv, hd, rd)
+    f = R.rope_inv_freq(hd, rd, 10000.0)
+    p = torch.tensor(pos)
+    q_want = R.rope_interleaved(qkv[:, :Q].reshape(T, n_heads, hd), p, f).reshape(T, Q)
+    k_want = R.rope_interleaved(qkv[:, Q:Q + KV].reshape(T, n_kv, hd), p, f).reshape(T, KV)
+    v_want = qkv[:, Q + KV:].double()
+    close(q_out, q_want, dtype, "q")
+    close(k_out, k_want, dtype, "k")
+    close(v_out, v_want, dtype, "v")
+    kp, vp = kp.cpu(), vp.cpu()
+    for t in range(T):
+        page = {0: {0: 5, 1: 7}, 1: {0: 1}}[seq[t]][pos[t] // PAGE]
+        r = pos[t] % PAGE
+        assert torch.equal(kp[page, :, r, :].reshape(-1), k_out[t].cpu())
+        assert torch.equal(vp[page, :, :, r].reshape(-1), v_out[t].cpu())
+    # nothing else was touched
+    touched = torch.zeros((n_pages, PAGE), dtype=torch.bool)
+    for t in range(T):
+        touched[{0: {0: 5, 1: 7}, 1: {0: 1}}[seq[t]][pos[t] // PAGE], pos[t] % PAGE] = True
+    assert (kp.float().abs().sum(dim=(1, 3)) > 0).equal(touched)
+
+
+def test_rope_kv_write_ring_keeps_the_last_pages_only():
+    k = K()
+    PAGE = k.PAGE
+    n_kv, hd, ring = 1, 16, 2
+    L = 3 * PAGE + 5                         # pages 0..3 exist, the ring keeps pages 2 and 3
+    qkv = rnd((L, 2 * hd + hd), 12)          # one query head
+    bt = torch.tensor([[4, 6]], dtype=torch.int32)
+    kp = torch.zeros((8, n_kv, PAGE, hd), device=DEV)
+    vp = torch.zeros((8, n_kv, hd, PAGE), device=DEV)
+    q_out = torch.empty((L, hd), device=DEV)
+    k.rope_kv_write(qkv.to(DEV), q_out, None, None, kp, vp, bt.to(DEV), ring, i32([0] * L), i32(list(range(L))),
+                    i32([0]), i32([L]), None, 1, n_kv, hd, 0)
+    kp = kp.cpu()
+    # absolute page 2 -> column 0 (page 4), page 3 -> column 1 (page 6)
+    assert torch.equal(kp[4, 0], qkv[2 * PAGE:3 * PAGE, hd:2 * hd])
+    assert torch.equal(kp[6, 0, :5], qkv[3 * PAGE:, hd:2 * hd])
+    assert kp[6, 0, 5:].abs().sum() == 0
+    assert torch.equal(q_out.cpu(), qkv[:, :hd])           # no table: no rotation
+
+
+# ------------------------------------------------------------------ attention
+
+def packed_attention_reference(q, k, v, lens, n_heads, n_kv, hd, window):
+    outs, o = [], 0
+    for n in lens:
+        outs.append(R.attention(q[o:o + n].reshape(n, n_heads, hd), k[o:o + n].reshape(n, n_kv, hd),
+                                v[o:o + n].reshape(n, n_kv, hd), window).reshape(n, n_heads * hd))
+        o += n
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("simple", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,window,lens", [
+    (4, 2, 16, 0, [5, 17, 1]), (3, 1, 32, 16, [2, 30, 70]), (6, 3, 48, 100, [130, 64]), (8, 2, 128, 0, [200]),
+    (2, 2, 80, 7, [65, 3]), (5, 5, 64, 0, [129])])
+def test_attn_prefill(n_heads, n_kv, hd, window, lens, dtype, simple):
+    k = K()
+    T = sum(lens)
+    q = rnd((T, n_heads * hd), 13, dtype)
+    kk = rnd((T, n_kv * hd), 14, dtype)
+    v = rnd((T, n_kv * hd), 15, dtype)
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    seq = np.repeat(np.arange(len(lens)), lens)
+    pos = np.concatenate([np.arange(n) for n in lens])
+    out = torch.empty((T, n_heads * hd), dtype=dtype, device=DEV)
+    k.FORCE_SIMPLE = simple
+    try:
+        k.attn_prefill(q.to(DEV), kk.to(DEV), v.to(DEV), out, i32(cu), i32(seq), i32(pos), n_heads, n_kv, hd, window)
+    finally:
+        k.FORCE_SIMPLE = False
+    close(out, packed_attention_reference(q, kk, v, lens, n_heads, n_kv, hd, window), dtype, "prefill attention")
+
+
+def paged_case(lens, n_kv, hd, window, dtype, seed, poison=True):
+    """Random keys/values of sequences of the given lengths laid out in pages the way
+    the cache does (ring for a window), the rest of the pool poisoned with NaN."""
+    k = K()
+    PAGE = k.PAGE
+    B = len(lens)
+    full = max((n + PAGE - 1) // PAGE for n in lens)
+    ring = min(full, (window + PAGE - 1) // PAGE + 1) if window else full
+    n_pages = B * ring + 3
+    kp = torch.full((n_pages, n_kv, PAGE, hd), float("nan") if poison else 0.0, dtype=dtype)
+    vp = torch.full((n_pages, n_kv, hd, PAGE), float("nan") if poison else 0.0, dtype=dtype)
+    order = np.random.default_rng(seed).permutation(n_pages)
+    bt = torch.full((B + 2, ring), -1, dtype=torch.int32)
+    slots = list(np.random.default_rng(seed + 1).permutation(B + 2)[:B])
+    keys, vals = [], []
+    nxt = 0
+    for b, n in enumerate(lens):
+        kb = rnd((n, n_kv, hd), seed + 10 * b, dtype)
+        vb = rnd((n, n_kv, hd), seed + 10 * b + 1, dtype)
+        keys.append(kb)
+        vals.append(vb)
+        last_ap = (n - 1) // PAGE
+        for ap in range(max(0, last_ap - ring + 1), last_ap + 1):
+            page = int(order[nxt])
+            nxt += 1
+            bt[slots[b], ap % ring] = page
+            rows = range(ap * PAGE, min(n, (ap + 1) * PAGE))
+            for p in rows:
+                kp[page, :, p % PAGE, :] = kb[p]
+                vp[page, :, :, p % PAGE] = vb[p]
+    return kp, vp, bt, [int(s) for s in slots], ring, keys, vals
+
+
+def one_query_reference(q, keys, vals, window):
+    """The last position's attention (src/infer.cpp:218-250 per head over the visible rows)."""
+    n_heads, hd = q.shape
+    n, n_kv = keys.shape[0], keys.shape[1]
+    lo = max(0, n - window) if window else 0
+    out = torch.zeros((n_heads, hd), dtype=torch.float64)
+    for h in range(n_heads):
+        g = h // (n_heads // n_kv)
+        p = R.attention_probs_one_query(q[h], keys[lo:n, g], hd)
+        out[h] = p @ vals[lo:n, g].double()
+    return out
+
+
+@pytest.mark.parametrize("simple", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,window,lens,splits", [
+    (4, 2, 16, 0, [5, 64, 65, 1], 1), (3, 1, 32, 16, [2, 30, 200], 2), (6, 3, 48, 100, [130, 640, 99], 3),
+    (8, 2, 128, 0, [1000, 3], 7), (2, 2, 80, 0, [129], 4), (32, 8, 128, 0, [300], 2), (5, 5, 64, 70, [700, 64], 16)])
+def test_attn_decode(n_heads, n_kv, hd, window, lens, splits, dtype, simple):
+    k = K()
+    B = len(lens)
+    kp, vp, bt, slots, ring, keys, vals = paged_case(lens, n_kv, hd, window, dtype, 20)
+    q = rnd((B, n_heads * hd), 16, dtype)
+    # one padding row at the end
+    qd = torch.cat([q, torch.zeros((1, n_heads * hd), dtype=dtype)]).to(DEV)
+    out = torch.full((B + 1, n_heads * hd), 5.0, dtype=dtype, device=DEV)
+    partial = torch.empty(k.attn_decode_workspace_floats(B + 1, n_heads, hd, splits), device=DEV)
+    k.FORCE_SIMPLE = simple
+    try:
+        k.attn_decode(qd, kp.to(DEV), vp.to(DEV), bt.to(DEV), ring, i32(slots + [-1]), i32(lens + [0]), out, partial,
+                      n_heads, n_kv, hd, window, splits)
+    finally:
+        k.FORCE_SIMPLE = False
+    for b, n in enumerate(lens):
+        want = one_query_reference(q[b].double().reshape(n_heads, hd), keys[b], vals[b], window).reshape(-1)
+        close(out[b], want, dtype, "decode attention row %d" % b)
+    assert (out[B] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_decode_finds_a_far_key(dtype):
+    """One key among a thousand, in an early page, carries all the weight: the query
+    is scaled along that key, so a kernel that skips or misplaces a page misses it."""
+    k = K()
+    n_heads, n_kv, hd, n = 4, 1, 64, 1000
+    for far in (3, 64 * 7 + 63, 998):
+        kp, vp, bt, slots, ring, keys, vals = paged_case([n], n_kv, hd, 0, dtype, 30)
+        q = (keys[0][far, 0].double() * 40.0).to(dtype).repeat(n_heads)[None]
+        out = torch.empty((1, n_heads * hd), dtype=dtype, device=DEV)
+        partial = torch.empty(k.attn_decode_workspace_floats(1, n_heads, hd, 5), device=DEV)
+        k.attn_decode(q.to(DEV), kp.to(DEV), vp.to(DEV), bt.to(DEV), ring, i32(slots), i32([n]), out, partial, n_heads,
+                      n_kv, hd, 0, 5)
+        got = out.cpu().double().reshape(n_heads, hd)
+        assert (got - vals[0][far, 0].double()).abs().max() < 0.05, far
+
+
+def test_attn_vector_of_the_reference():
+    """src/test.cpp:67-126 through both attention kernels (head size padded from 3 to 16 with zeros)."""
+    k = K()
+    hd = 16
+    q = torch.zeros((4, 2 * hd))
+    q[3, 1], q[3, hd + 2] = 1e4, 1e4
+    kv = torch.zeros((4, hd))
+    kv[0, 0], kv[1, 1], kv[2, 2], kv[3, 0] = 1, 1, 1, -1
+    out = torch.empty((4, 2 * hd), device=DEV)
+    # the reference divides by sqrt(3); here sqrt(16): the scores stay far apart, the result is the same
+    k.attn_prefill(q.to(DEV), kv.to(DEV), kv.to(DEV), out, i32([0, 4]), i32([0] * 4), i32([0, 1, 2, 3]), 2, 1, hd, 0)
+    got = out.cpu()[3].reshape(2, hd)
+    assert torch.allclose(got[0, :3], torch.tensor([0., 1, 0]), atol=1e-4)
+    assert torch.allclose(got[1, :3], torch.tensor([0., 0, 1]), atol=1e-4)
+
+
+# ------------------------------------------------------------------ sampling
+
+def test_argmax_and_sample():
+    k = K()
+    V = 1000
+    g = torch.Generator().manual_seed(40)
+    logits = torch.randn((6, V), generator=g) * 3
+    logits[0, 17] = logits[0, 900] = 50.0                # a tie: the lowest index wins
+    logits[1, V - 1] = 60.0
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    k.argmax(logits.to(DEV), out)
+    assert out.cpu().tolist() == [R.sample_argmax(l) for l in logits]
+    assert out[0] == 17 and out[1] == V - 1
+    for temp in (1.0, 0.8, 2.5):
+        u = torch.tensor([0.0, 0.999999, 0.5, 0.25, 0.9, 0.1])
+        k.sample(logits.to(DEV), u.to(DEV), temp, out)
+        got = out.cpu().tolist()
+        for r in range(6):
+            p = torch.softmax(logits[r].double() / temp, 0)
+            c = torch.cumsum(p, 0)
+            want = R.sample_temperature(logits[r], temp, float(u[r]))
+            # equal up to an edge of the running sum: the picked token's interval contains u within rounding
+            lo = float(c[got[r]] - p[got[r]])
+            assert got[r] == want or (lo - 1e-5 <= float(u[r]) <= float(c[got[r]]) + 1e-5), (temp, r, got[r], want)
+    # the distribution on a toy of 4 logits: frequencies match softmax
+    l4 = torch.tensor([[0.0, 1.0, 2.0, -1.0]]).repeat(4000, 1)
+    u = torch.rand(4000, generator=g)
+    out = torch.empty(4000, dtype=torch.int32, device=DEV)
+    k.sample(l4.to(DEV), u.to(DEV), 1.0, out)
+    freq = torch.bincount(out.cpu().long(), minlength=4).double() / 4000
+    assert (freq - torch.softmax(l4[0].double(), 0)).abs().max() < 0.03
+    prob = torch.empty(6, device=DEV)
+    k.token_prob(logits.to(DEV), i32([0, 1, 2, 3, 4, 999]), prob)
+    want = [R.sample_prob(logits[r], i) for r, i in enumerate([0, 1, 2, 3, 4, 999])]
+    assert torch.allclose(prob.cpu().double(), torch.tensor(want, dtype=torch.float64), rtol=1e-4, atol=1e-9)

@@ -1,0 +1,168 @@
+"""The engine against the plain implementation under every way of cutting the
+requests into steps: each request alone and whole; with the last 32 tokens one
+by one; in batches of unequal lengths whose shorter requests end earlier, one
+batch after another so that slots and pages are used again (the cache is
+poisoned with NaN between batches).  float32 and bfloat16, five tiny
+configurations."""
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import schedules
+import tiny_configs
+
+pytestmark = pytest.mark.gpu
+
+LENGTHS = {
+    "tiny_llama": [5, 17, 1, 40, 100, 128],
+    "tiny_mistral": [2, 30, 9, 23, 64, 50],
+    "tiny_llama3": [3, 70, 200, 33],
+    "tiny_wide_heads": [150, 33, 260, 64, 65],
+    "tiny_long": [700, 64, 129],
+}
+# batches: (request indices, first-step lengths)
+GROUPS = {
+    "tiny_llama": [([0, 1, 2], [5, 17, 1]), ([3, 4, 5], [8, 64, 65]), ([1, 0], [1, 2])],
+    "tiny_mistral": [([0, 1, 2, 3], [2, 30, 9, 23]), ([4, 5], [40, 17]), ([3, 2, 1], [1, 3, 16])],
+    "tiny_llama3": [([0, 1], [1, 33]), ([2, 3], [130, 20]), ([1], [64])],
+    "tiny_wide_heads": [([0, 1, 2], [120, 3, 101]), ([3, 4], [63, 64]), ([1, 0], [32, 100])],
+    "tiny_long": [([0, 1, 2], [500, 1, 100]), ([2, 1], [128, 63])],
+}
+
+_engines = {}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    tmp = tmp_path_factory.mktemp("models")
+    return {name: helpers.make_folder(tmp, name, cfg, seed=3) for name, cfg in tiny_configs.ALL.items()}
+
+
+def engine_for(folders, name, dtype, max_tokens=4096):
+    from yalm_amd.engine import Engine, Model
+    key = (name, dtype)
+    if key not in _engines:
+        model = Model.from_folder(folders[name], dtype=helpers.torch_dtype(dtype), device="cuda:0")
+        _engines[key] = Engine(model, max_tokens=max_tokens)
+    return _engines[key]
+
+
+def poison_when_idle(engine):
+    def before(step):
+        if not engine.cache.slots.held:
+            for g in engine.cache.kv_groups:
+                g.k_pages.fill_(float("nan"))
+                g.v_pages.fill_(float("nan"))
+    return before
+
+
+def compare(folders, name, dtype, steps, requests, engine, what):
+    out = schedules.replay_in_process(engine, steps, before_step=poison_when_idle(engine))
+    got = schedules.per_request(steps, out, requests)
+    for rid, toks in requests.items():
+        want = helpers.plain_logits(folders[name], tuple(toks), dtype)
+        helpers.check_logits(got[rid], want, dtype, "%s %s %s request %s (%d tokens)" % (name, dtype, what, rid, len(toks)))
+    assert not engine.cache.slots.held
+    for g in engine.cache.kv_groups:
+        assert g.pool.n_free == g.n_pages
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(LENGTHS))
+def test_each_request_alone_and_whole(folders, name, dtype):
+    cfg = tiny_configs.ALL[name]
+    requests = helpers.random_requests(cfg, LENGTHS[name], seed=5)
+    compare(folders, name, dtype, schedules.whole(requests), requests, engine_for(folders, name, dtype), "whole")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(LENGTHS))
+def test_last_32_tokens_one_by_one(folders, name, dtype):
+    cfg = tiny_configs.ALL[name]
+    requests = helpers.random_requests(cfg, LENGTHS[name], seed=5)
+    compare(folders, name, dtype, schedules.tail_one_by_one(requests, 32), requests,
+            engine_for(folders, name, dtype), "last 32 one by one")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(LENGTHS))
+def test_unequal_batches_with_reuse(folders, name, dtype):
+    cfg = tiny_configs.ALL[name]
+    base = helpers.random_requests(cfg, LENGTHS[name], seed=5)
+    requests, groups, prompt_lens = {}, [], {}
+    for gi, (idx, firsts) in enumerate(GROUPS[name]):
+        ids = []
+        for i, p in zip(idx, firsts):
+            rid = "g%d_r%d" % (gi, i)
+            requests[rid] = base["r%d" % i]
+            prompt_lens[rid] = min(p, len(requests[rid]))
+            ids.append(rid)
+        groups.append(ids)
+    steps = schedules.batches(requests, groups, prompt_lens)
+    compare(folders, name, dtype, steps, requests, engine_for(folders, name, dtype), "batches")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_eager_equals_graph(folders, dtype):
+    """The same steps with and without HIP graphs give the same bits."""
+    from yalm_amd.engine import Engine, Model
+    name = "tiny_mistral"
+    cfg = tiny_configs.ALL[name]
+    requests = helpers.random_requests(cfg, [20, 45, 7], seed=8)
+    steps = schedules.batches(requests, [list(requests)], {"r0": 3, "r1": 20, "r2": 1})
+    model = Model.from_folder(folders[name], dtype=helpers.torch_dtype(dtype), device="cuda:0")
+    a = schedules.replay_in_process(Engine(model, max_tokens=1024, use_graphs=True), steps)
+    b = schedules.replay_in_process(Engine(model, max_tokens=1024, use_graphs=False), steps)
+    for k in a:
+        assert np.array_equal(a[k], b[k]), "step %s differs between graph and eager decode" % k
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_padding_and_company_change_nothing(folders, dtype):
+    """A request's logits are the same alone, in a batch of 3 (padded to a bucket of 4),
+    and in another slot, up to rounding; in float32 the decode bits are equal."""
+    name = "tiny_llama"
+    cfg = tiny_configs.ALL[name]
+    engine = engine_for(folders, name, dtype)
+    requests = helpers.random_requests(cfg, [30, 12, 50], seed=9)
+    alone = schedules.batches({"r0": requests["r0"]}, [["r0"]], {"r0": 10})
+    a = schedules.per_request(alone, schedules.replay_in_process(engine, alone), {"r0": requests["r0"]})["r0"]
+    # occupy a slot first, so that r0 lands elsewhere, then run it in company
+    dummy = engine.start(1)
+    both = schedules.batches(requests, [["r2", "r0", "r1"]], {"r0": 10, "r1": 12, "r2": 31})
+    b = schedules.per_request(both, schedules.replay_in_process(engine, both), requests)["r0"]
+    engine.release(dummy)
+    want = helpers.plain_logits(folders[name], tuple(requests["r0"]), dtype)
+    helpers.check_logits(a, want, dtype, "alone")
+    helpers.check_logits(b, want, dtype, "in company")
+    tol = 1e-5 if dtype == "float32" else 2e-2
+    assert np.abs(a - b).max() <= tol * max(1.0, np.abs(want).max())
+
+
+def test_trace_run_program(folders, tmp_path):
+    """bin/trace_run itself, as a user runs it: unequal batches in both dtypes."""
+    name = "tiny_mistral"
+    cfg = tiny_configs.ALL[name]
+    requests = helpers.random_requests(cfg, [33, 12, 40], seed=10)
+    steps = schedules.batches(requests, [["r0", "r1"], ["r2"]], {"r0": 7, "r1": 12, "r2": 1})
+    # a step that wants nothing writes no file
+    steps[1]["entries"][0]["want"] = []
+    for dtype in ("float32", "bfloat16"):
+        out = schedules.replay_trace_run(folders[name], dtype, steps, str(tmp_path / dtype),
+                                         schedules.max_tokens_needed(steps))
+        vocab = cfg["vocab_size"]
+        got = {rid: np.full((len(t), vocab), np.nan, np.float32) for rid, t in requests.items()}
+        pos = {rid: 0 for rid in requests}
+        for s in steps:
+            row = 0
+            for e in s["entries"]:
+                for j in e["want"]:
+                    got[e["id"]][pos[e["id"]] + j] = out[s["step"]][row]
+                    row += 1
+                pos[e["id"]] += len(e["tokens"])
+        for rid, toks in requests.items():
+            want = helpers.plain_logits(folders[name], tuple(toks), dtype)
+            keep = ~np.isnan(got[rid]).any(axis=1)
+            assert keep.sum() >= len(toks) - 1
+            helpers.check_logits(got[rid][keep], want[keep], dtype, "trace_run %s %s" % (dtype, rid))

@@ -1,0 +1,246 @@
+// Attention in float32 arithmetic for every storage type: the kernels of the
+// true 32-bit path and the fallback of the bfloat16 path.  One wave per
+// (query, head); keys are taken 64 at a time, a lane per key for the scores
+// and a lane per output element for the mix; softmax state in float32.
+#include <float.h>
+#include "common.h"
+#include "yalm_hip.h"
+
+int yalm_attn_prefill_bf16_mfma(const void* q, const void* k, const void* v, void* out, const int* cu_seqlens,
+                                const int* tok_seq, const int* tok_pos, int T, int B, int n_heads, int n_kv_heads,
+                                int head_dim, int window, hipStream_t stream);
+int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                               int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
+                               float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
+                               int n_splits, int n_pages, hipStream_t stream);
+
+namespace {
+constexpr int MAX_HD = 256;              // head sizes up to 256 (4 output elements per lane)
+constexpr int ACC = MAX_HD / WAVE;
+
+// ---------------------------------------------------------------------------
+// prefill: a step's tokens over the same step's keys
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, T* __restrict__ out,
+    const int* __restrict__ cu_seqlens, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_heads,
+    int n_kv_heads, int hd, int window) {
+  __shared__ float qs[MAX_HD];
+  __shared__ float ps[WAVE];
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int b = tok_seq[t], pos = tok_pos[t];
+  const int g = h / (n_heads / n_kv_heads);
+  const int KV = n_kv_heads * hd;
+  const int start = cu_seqlens[b];
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const float inv = sqrtf((float)hd);
+
+  for (int i = lane; i < hd; i += WAVE) qs[i] = to_f32(q[((size_t)t * n_heads + h) * hd + i]);
+  __syncthreads();
+
+  float m = -FLT_MAX, l = 0.f;
+  float acc[ACC];
+#pragma unroll
+  for (int a = 0; a < ACC; ++a) acc[a] = 0.f;
+
+  for (int j0 = lo; j0 <= pos; j0 += WAVE) {
+    int j = j0 + lane;
+    bool valid = j <= pos;
+    float s = -FLT_MAX;
+    if (valid) {
+      const T* kr = k + (size_t)(start + j) * KV + g * hd;
+      float d = 0.f;
+      for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kr[i]), d);
+      s = d / inv;
+    }
+    float m_new = fmaxf(m, wave_max(s));
+    float p = valid ? expf(s - m_new) : 0.f;
+    float corr = expf(m - m_new);
+    l = l * corr + wave_sum(p);
+    m = m_new;
+    __syncthreads();
+    ps[lane] = p;
+    __syncthreads();
+    int n = min(WAVE, pos - j0 + 1);
+#pragma unroll
+    for (int a = 0; a < ACC; ++a) {
+      int d = lane + a * WAVE;
+      if (d < hd) {
+        float s2 = 0.f;
+        const T* vc = v + (size_t)(start + j0) * KV + g * hd + d;
+        for (int jj = 0; jj < n; ++jj) s2 = fmaf(ps[jj], to_f32(vc[(size_t)jj * KV]), s2);
+        acc[a] = acc[a] * corr + s2;
+      }
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < ACC; ++a) {
+    int d = lane + a * WAVE;
+    if (d < hd) out[((size_t)t * n_heads + h) * hd + d] = from_f32<T>(acc[a] / l);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// decode: one query per sequence over the pages of the cache, split over pages
+// partial layout: [B, n_heads, n_splits, hd + 2] = (acc[hd], m, l)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
+    const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_len, float* __restrict__ partial, int n_heads, int n_kv_heads, int hd, int window,
+    int n_splits, int n_pages) {
+  __shared__ float qs[MAX_HD];
+  __shared__ float ps[WAVE];
+  const int b = blockIdx.x, h = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
+  float* part = partial + (((size_t)b * n_heads + h) * n_splits + split) * (hd + 2);
+  const int slot = seq_slot[b];
+  const int L = slot >= 0 ? seq_len[b] : 0;
+  float m = -FLT_MAX, l = 0.f;
+  float acc[ACC];
+#pragma unroll
+  for (int a = 0; a < ACC; ++a) acc[a] = 0.f;
+
+  if (L > 0) {
+    const int g = h / (n_heads / n_kv_heads);
+    const int lo = window > 0 ? max(0, L - window) : 0;       // first visible position
+    const int first_page = lo / PAGE, last_page = (L - 1) / PAGE;
+    const int total = last_page - first_page + 1;
+    const int per = (total + n_splits - 1) / n_splits;
+    const int p_begin = first_page + split * per;
+    const int p_end = min(last_page + 1, p_begin + per);
+    const float inv = sqrtf((float)hd);
+    for (int i = lane; i < hd; i += WAVE) qs[i] = to_f32(q[((size_t)b * n_heads + h) * hd + i]);
+    __syncthreads();
+    for (int ap = p_begin; ap < p_end; ++ap) {
+      int phys = block_table[(size_t)slot * table_stride + (ap % ring_pages)];
+      if (phys < 0 || phys >= n_pages) continue;               // never the case for a live sequence
+      const T* kp = k_pages + ((size_t)phys * n_kv_heads + g) * PAGE * hd;
+      const T* vp = v_pages + ((size_t)phys * n_kv_heads + g) * PAGE * hd;
+      int pos = ap * PAGE + lane;
+      bool valid = pos >= lo && pos < L;
+      float s = -FLT_MAX;
+      if (valid) {
+        const T* kr = kp + (size_t)lane * hd;
+        float d = 0.f;
+        for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kr[i]), d);
+        s = d / inv;
+      }
+      float m_new = fmaxf(m, wave_max(s));
+      float p = valid ? expf(s - m_new) : 0.f;
+      float corr = expf(m - m_new);
+      l = l * corr + wave_sum(p);
+      m = m_new;
+      __syncthreads();
+      ps[lane] = p;
+      __syncthreads();
+#pragma unroll
+      for (int a = 0; a < ACC; ++a) {
+        int d = lane + a * WAVE;
+        if (d < hd) {
+          const T* vr = vp + (size_t)d * PAGE;
+          float s2 = 0.f;
+          for (int jj = 0; jj < PAGE; ++jj) {
+            float pj = ps[jj];
+            if (pj != 0.f) s2 = fmaf(pj, to_f32(vr[jj]), s2);   // rows outside the mask may hold anything
+          }
+          acc[a] = acc[a] * corr + s2;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int a = 0; a < ACC; ++a) {
+    int d = lane + a * WAVE;
+    if (d < hd) part[d] = acc[a];
+  }
+  if (lane == 0) {
+    part[hd] = m;
+    part[hd + 1] = l;
+  }
+}
+
+template <typename T>
+__global__ void attn_decode_combine_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_heads,
+                                           int hd, int n_splits) {
+  const int b = blockIdx.x, h = blockIdx.y;
+  const float* part = partial + ((size_t)b * n_heads + h) * n_splits * (hd + 2);
+  float m = -FLT_MAX;
+  for (int s = 0; s < n_splits; ++s) m = fmaxf(m, part[(size_t)s * (hd + 2) + hd]);
+  float l = 0.f;
+  for (int s = 0; s < n_splits; ++s) {
+    const float* ps = part + (size_t)s * (hd + 2);
+    l += ps[hd + 1] * expf(ps[hd] - m);
+  }
+  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    float a = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float* ps = part + (size_t)s * (hd + 2);
+      a += ps[d] * expf(ps[hd] - m);
+    }
+    out[((size_t)b * n_heads + h) * hd + d] = from_f32<T>(l > 0.f ? a / l : 0.f);
+  }
+}
+
+bool bad_heads(int n_heads, int n_kv_heads, int hd) {
+  return n_heads <= 0 || n_kv_heads <= 0 || n_heads % n_kv_heads != 0 || hd <= 0 || hd > MAX_HD;
+}
+}  // namespace
+
+extern "C" int yalm_attn_prefill(const void* q, const void* k, const void* v, void* out, const int* cu_seqlens,
+                                 const int* tok_seq, const int* tok_pos, int T, int B, int n_heads, int n_kv_heads,
+                                 int head_dim, int window, int dtype, int force_simple, hipStream_t stream) {
+  if (T <= 0) return YALM_OK;
+  if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0) return YALM_ERR_ARG;
+  dim3 grid(T, n_heads);
+  if (dtype == YALM_F32) {
+    attn_prefill_simple_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)q, (const float*)k, (const float*)v,
+                                                                 (float*)out, cu_seqlens, tok_seq, tok_pos, n_heads,
+                                                                 n_kv_heads, head_dim, window);
+    return launch_status();
+  }
+  if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
+  if (!force_simple) {
+    int rc = yalm_attn_prefill_bf16_mfma(q, k, v, out, cu_seqlens, tok_seq, tok_pos, T, B, n_heads, n_kv_heads,
+                                         head_dim, window, stream);
+    if (rc != YALM_ERR_ARG) return rc;
+  }
+  attn_prefill_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)q, (const bf16*)k, (const bf16*)v,
+                                                              (bf16*)out, cu_seqlens, tok_seq, tok_pos, n_heads,
+                                                              n_kv_heads, head_dim, window);
+  return launch_status();
+}
+
+extern "C" long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits) {
+  return (long)B * n_heads * n_splits * (head_dim + 2) * (long)sizeof(float);
+}
+
+extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
+                                float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
+                                int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream) {
+  if (B <= 0) return YALM_OK;
+  if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0)
+    return YALM_ERR_ARG;
+  dim3 grid(B, n_heads, n_splits), cgrid(B, n_heads);
+  if (dtype == YALM_F32) {
+    attn_decode_simple_kernel<float><<<grid, WAVE, 0, stream>>>(
+        (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
+        seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
+    attn_decode_combine_kernel<float><<<cgrid, WAVE, 0, stream>>>(partial, (float*)out, n_heads, head_dim, n_splits);
+    return launch_status();
+  }
+  if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
+  if (!force_simple) {
+    int rc = yalm_attn_decode_bf16_mfma(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len,
+                                        out, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages,
+                                        stream);
+    if (rc != YALM_ERR_ARG) return rc;
+  }
+  attn_decode_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>(
+      (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
+      seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
+  attn_decode_combine_kernel<bf16><<<cgrid, WAVE, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
+  return launch_status();
+}

@@ -1,0 +1,68 @@
+// Shared device helpers for the gfx950 kernels: storage types, conversions,
+// wave64 reductions and the launch-error convention of the C entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define YALM_OK 0
+#define YALM_ERR_ARG 1001          // an argument the kernel family refuses
+#define YALM_ERR_DTYPE 1002        // unknown dtype code
+
+// dtype codes shared with the Python side
+#define YALM_F32 0
+#define YALM_BF16 1
+
+#define WAVE 64
+#define PAGE 64                    // tokens per cache page; equals the wave width on purpose
+
+typedef __bf16 bf16;
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16 v) { return static_cast<float>(v); }
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16 from_f32<bf16>(float v) { return static_cast<bf16>(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+
+// Sum over a block of NW waves; every thread gets the result.  `red` holds NW floats.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  if (NW == 1) return v;
+  __syncthreads();
+  if ((threadIdx.x & (WAVE - 1)) == 0) red[threadIdx.x / WAVE] = v;
+  __syncthreads();
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) s += red[i];
+  return s;
+}
+template <int NW>
+__device__ __forceinline__ float block_max(float v, float* red) {
+  v = wave_max(v);
+  if (NW == 1) return v;
+  __syncthreads();
+  if ((threadIdx.x & (WAVE - 1)) == 0) red[threadIdx.x / WAVE] = v;
+  __syncthreads();
+  float s = red[0];
+#pragma unroll
+  for (int i = 1; i < NW; ++i) s = fmaxf(s, red[i]);
+  return s;
+}
+
+static inline int launch_status() {
+  hipError_t e = hipGetLastError();
+  return e == hipSuccess ? YALM_OK : (int)e;
+}
+
+static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

@@ -1,0 +1,81 @@
+// C entry points of the gfx950 kernel library.  Every function launches on the
+// given stream and returns 0, a YALM_ERR_* code for refused arguments, or the
+// hipError_t of a failed launch.  Pointers are device pointers unless noted.
+// dtype codes: 0 = float32, 1 = bfloat16.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* yalm_error_string(int code);
+int yalm_abi_version(void);
+
+// x[t, :] = float(table[tokens[t], :]); a negative token gives a row of zeros.
+// reference: copy_embedding_* (src/infer.cu:636-658)
+int yalm_embed(const void* table, int table_dtype, const int* tokens, float* out, int T, int D, int V,
+               hipStream_t stream);
+
+// out[r, :] = x[row(r), :] * rsqrt(mean(x^2) + eps) * w, row(r) = row_index ? row_index[r] : r.
+// x is the float32 residual stream; w may be float32 or bfloat16; out float32 or bfloat16.
+// reference: rmsnorm (src/infer.cu:525-539)
+int yalm_rmsnorm(const float* x, const void* w, int w_dtype, void* out, int out_dtype, const int* row_index, int R,
+                 int D, float eps, hipStream_t stream);
+
+// C = A[M,K] * W[N,K]^T with float32 accumulation.  A and W have dtype `dtype`.
+// epilogue 0: C float32 [M,N] = acc
+//          1: C `dtype`  [M,N] = acc
+//          2: C float32 [M,N] += acc                      (residual add)
+//          3: gated: W holds gate and up rows interleaved in blocks of 16
+//             (16 gate rows, 16 up rows, ...), N = 32 * ceil(H/16);
+//             C `dtype` [M,H] = silu(gate) * up
+// reference: matmul_wide, fused_matmul_add_residuals, fused_qkv_matmul_clip,
+// fused_ffn_w1_w3_glu_act (src/infer.cu:250-337, 610-634)
+int yalm_gemm(const void* A, const void* W, void* C, int M, int N, int K, int dtype, int epilogue, int H,
+              int force_simple, hipStream_t stream);
+
+// Rotates q and k of every token (adjacent pairs, angles from the table), writes q,
+// optionally k and v token-major (for attention over the step's own tokens), and
+// k and v into the pages of the cache.
+//   qkv      float32 [T, (n_heads + 2 n_kv_heads) * head_dim]
+//   cos_sin  float32 [n_positions, rotary_dim/2, 2] or null (no rotation)
+//   k_pages  [n_pages, n_kv_heads, PAGE, head_dim], v_pages [n_pages, n_kv_heads, head_dim, PAGE]
+//   block_table int32 [n_slots, table_stride]; page of position p: table[slot][(p / PAGE) % ring_pages]
+//   a token is written iff its page is among the last ring_pages pages of its sequence
+// reference: fused_rope_and_cache_update (src/infer.cu:660-705)
+int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_out, void* v_out, void* k_pages, void* v_pages,
+                       const int* block_table, int table_stride, int ring_pages, const int* tok_seq,
+                       const int* tok_pos, const int* seq_slot, const int* seq_len, const float* cos_sin,
+                       int n_positions, int T, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
+                       int n_pages, int dtype, hipStream_t stream);
+
+// Causal attention of a step's tokens over the same step's keys (sequences that
+// start at position 0), packed without padding.  window 0 = all keys.
+//   q [T, n_heads, hd], k, v [T, n_kv_heads, hd], out [T, n_heads, hd], all `dtype`
+// reference: attn_dot + attn_softmax + att_mix (src/infer.cu:339-523) for every position
+int yalm_attn_prefill(const void* q, const void* k, const void* v, void* out, const int* cu_seqlens,
+                      const int* tok_seq, const int* tok_pos, int T, int B, int n_heads, int n_kv_heads, int head_dim,
+                      int window, int dtype, int force_simple, hipStream_t stream);
+
+// One query per sequence over the pages of the cache (the new key is already written).
+//   q, out [B, n_heads, hd]; seq_len[b] = keys of sequence b including the new one;
+//   seq_slot[b] < 0 marks a padding row (out = 0).
+//   partial: float32 workspace of yalm_attn_decode_workspace(...) bytes
+int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                     int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
+                     float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits,
+                     int n_pages, int dtype, int force_simple, hipStream_t stream);
+long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits);
+
+// out[r] = index of the maximum of logits[r, :], lowest index on ties (src/sampler.cpp:27-38)
+int yalm_argmax(const float* logits, int* out, int R, int V, hipStream_t stream);
+// out[r] = first index whose running sum of exp((l - max)/T) reaches u[r] * total, else V-1
+// (src/sampler.cpp:40-65 with the uniform numbers given by the caller)
+int yalm_sample(const float* logits, const float* u, float temperature, int* out, int R, int V, hipStream_t stream);
+// prob[r] = softmax(logits[r, :])[index[r]] (src/sampler.cpp:11-25)
+int yalm_token_prob(const float* logits, const int* index, float* prob, int R, int V, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,52 @@
+"""What a step hands to the parts: the step's tokens and their places as device
+tensors, the cache, and a workspace of reusable buffers."""
+import torch
+
+
+class Workspace:
+    """Named device buffers that are reused from step to step and grow on demand.
+    A buffer is a flat allocation; `get` returns a view of the asked shape."""
+
+    def __init__(self, device):
+        self.device = device
+        self._flat = {}
+        self.frozen = False           # set while a graph that uses these buffers exists
+
+    def get(self, name, shape, dtype):
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = (name, dtype)
+        buf = self._flat.get(key)
+        if buf is None or buf.numel() < n:
+            if self.frozen:
+                raise RuntimeError("workspace buffer %r would have to grow inside a captured graph" % (name,))
+            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._flat[key] = buf
+        return buf[:n].view(*shape)
+
+    def bytes(self):
+        return sum(b.numel() * b.element_size() for b in self._flat.values())
+
+
+class StepContext:
+    """mode: 'prefill' (sequences that start at position 0, whole prompts, packed)
+    or 'decode' (one token per sequence).  Device tensors, all int32:
+      tokens[T], tok_seq[T] (row of the batch), tok_pos[T] (position in its sequence),
+      seq_slot[B] (-1: padding row), seq_len[B] (length after this step), cu_seqlens[B+1].
+    max_position: the largest position in the step (host value, for table checks)."""
+
+    def __init__(self, mode, cache, ws, act_dtype, shared_lines=()):
+        self.mode = mode
+        self.cache = cache
+        self.ws = ws
+        self.act_dtype = act_dtype
+        self.shared_lines = set(shared_lines)
+        self.tokens = self.tok_seq = self.tok_pos = self.seq_slot = self.seq_len = self.cu_seqlens = None
+        self.max_position = 0
+        self.host_slots = []
+        self.host_n_tokens = []
+        self.host_start = []
+
+    def line_is_shared(self, line):
+        return line in self.shared_lines

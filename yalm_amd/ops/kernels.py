@@ -1,0 +1,227 @@
+"""Python faces of the HIP kernels.  Each function checks on the host that the
+operands have the shapes, dtypes and layout its kernel and grid assume (a
+mismatch is an error here, never a wrong result or a fault on the device), then
+launches on torch's current stream.  Tensors must live on the GPU; there is no
+CPU path."""
+import torch
+
+from . import library
+
+PAGE = 64                       # tokens per cache page (csrc/common.h)
+MAX_HEAD_DIM = 256
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+# set by tests to run the float32-arithmetic kernels also for bfloat16 storage
+FORCE_SIMPLE = False
+
+
+def dtype_code(dtype):
+    try:
+        return _DT[dtype]
+    except KeyError:
+        raise TypeError("unsupported dtype %s (float32 or bfloat16)" % dtype) from None
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(t, name, dtype=None, shape=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("%s: expected a tensor" % name)
+    if not t.is_cuda:
+        raise RuntimeError("%s: the HIP kernels need GPU tensors (got %s); there is no CPU path" % (name, t.device))
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous" % name)
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError("%s: expected %s, got %s" % (name, dtype, t.dtype))
+    if shape is not None:
+        if t.dim() != len(shape) or any(s is not None and s != d for s, d in zip(shape, t.shape)):
+            raise ValueError("%s: expected shape %s, got %s" % (name, list(shape), list(t.shape)))
+    return t.data_ptr()
+
+
+def _opt(t, name, dtype=None, shape=None):
+    return None if t is None else _need(t, name, dtype, shape)
+
+
+def embed(table, tokens, out):
+    """out[t] = float(table[tokens[t]]); a negative token gives zeros."""
+    V, D = table.shape
+    T = tokens.shape[0]
+    p_table = _need(table, "table")
+    code = dtype_code(table.dtype)
+    p_tok = _need(tokens, "tokens", torch.int32, (T,))
+    p_out = _need(out, "out", torch.float32, (T, D))
+    library.check(library.lib().yalm_embed(p_table, code, p_tok, p_out, T, D, V, _stream()), "embed")
+    return out
+
+
+def rmsnorm(x, weight, out, eps, row_index=None):
+    """out[r] = x[row_index[r] or r] * rsqrt(mean(x^2) + eps) * weight."""
+    D = x.shape[-1]
+    R = out.shape[0]
+    p_x = _need(x, "x", torch.float32, (None, D))
+    p_w = _need(weight, "weight", None, (D,))
+    p_o = _need(out, "out", None, (R, D))
+    p_i = _opt(row_index, "row_index", torch.int32, (R,))
+    if row_index is None and x.shape[0] < R:
+        raise ValueError("rmsnorm: %d rows wanted of %d" % (R, x.shape[0]))
+    library.check(library.lib().yalm_rmsnorm(p_x, p_w, dtype_code(weight.dtype), p_o, dtype_code(out.dtype), p_i, R, D,
+                                             float(eps), _stream()), "rmsnorm")
+    return out
+
+
+EPI_STORE_F32, EPI_STORE, EPI_ADD_F32, EPI_GATED = 0, 1, 2, 3
+
+
+def gemm(a, w, out, epilogue, hidden=0):
+    """out = a[M,K] @ w[N,K]^T with float32 accumulation and one of four epilogues:
+    EPI_STORE_F32 (float32 out), EPI_STORE (out in a's dtype), EPI_ADD_F32
+    (float32 out += product), EPI_GATED (w = gate/up rows interleaved in blocks of
+    16; out[M, hidden] = silu(gate) * up in a's dtype)."""
+    M, K = a.shape
+    N = w.shape[0]
+    dt = a.dtype
+    p_a = _need(a, "a", dt, (M, K))
+    p_w = _need(w, "w", dt, (N, K))
+    if epilogue == EPI_GATED:
+        if hidden <= 0 or N != 32 * ((hidden + 15) // 16):
+            raise ValueError("gated gemm: weight rows %d do not match hidden %d" % (N, hidden))
+        p_o = _need(out, "out", dt, (M, hidden))
+    elif epilogue == EPI_STORE:
+        p_o = _need(out, "out", dt, (M, N))
+    elif epilogue in (EPI_STORE_F32, EPI_ADD_F32):
+        p_o = _need(out, "out", torch.float32, (M, N))
+    else:
+        raise ValueError("unknown epilogue %r" % (epilogue,))
+    library.check(library.lib().yalm_gemm(p_a, p_w, p_o, M, N, K, dtype_code(dt), epilogue, hidden,
+                                          1 if FORCE_SIMPLE else 0, _stream()), "gemm")
+    return out
+
+
+def _check_heads(n_heads, n_kv_heads, head_dim):
+    if n_heads % n_kv_heads != 0:
+        raise ValueError("n_heads %d is no multiple of n_kv_heads %d" % (n_heads, n_kv_heads))
+    if head_dim % 2 != 0 or head_dim <= 0 or head_dim > MAX_HEAD_DIM:
+        raise ValueError("head_dim %d is not supported (even, at most %d)" % (head_dim, MAX_HEAD_DIM))
+
+
+def rope_kv_write(qkv, q_out, k_out, v_out, k_pages, v_pages, block_table, ring_pages, tok_seq, tok_pos, seq_slot,
+                  seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim):
+    """Rotates q and k by the angles of `cos_sin` at each token's position, writes q
+    (and k, v token-major if k_out is given) in q_out's dtype and k, v into the pages."""
+    _check_heads(n_heads, n_kv_heads, head_dim)
+    T = qkv.shape[0]
+    Q, KV = n_heads * head_dim, n_kv_heads * head_dim
+    dt = q_out.dtype
+    p_qkv = _need(qkv, "qkv", torch.float32, (T, Q + 2 * KV))
+    p_q = _need(q_out, "q_out", dt, (T, Q))
+    p_k = _opt(k_out, "k_out", dt, (T, KV))
+    p_v = _opt(v_out, "v_out", dt, (T, KV))
+    if (k_out is None) != (v_out is None):
+        raise ValueError("k_out and v_out go together")
+    n_pages = 0
+    p_kp = p_vp = p_bt = None
+    stride = 0
+    if k_pages is not None:
+        n_pages = k_pages.shape[0]
+        p_kp = _need(k_pages, "k_pages", dt, (n_pages, n_kv_heads, PAGE, head_dim))
+        p_vp = _need(v_pages, "v_pages", dt, (n_pages, n_kv_heads, head_dim, PAGE))
+        p_bt = _need(block_table, "block_table", torch.int32, (None, None))
+        stride = block_table.shape[1]
+        if ring_pages <= 0 or ring_pages > stride:
+            raise ValueError("ring_pages %d does not fit the block table (%d columns)" % (ring_pages, stride))
+    B = seq_slot.shape[0]
+    p_ts = _need(tok_seq, "tok_seq", torch.int32, (T,))
+    p_tp = _need(tok_pos, "tok_pos", torch.int32, (T,))
+    p_ss = _need(seq_slot, "seq_slot", torch.int32, (B,))
+    p_sl = _need(seq_len, "seq_len", torch.int32, (B,))
+    n_pos = 0
+    p_cs = None
+    if cos_sin is not None:
+        if rotary_dim % 2 != 0 or rotary_dim > head_dim or rotary_dim <= 0:
+            raise ValueError("rotary_dim %d does not fit head_dim %d" % (rotary_dim, head_dim))
+        n_pos = cos_sin.shape[0]
+        p_cs = _need(cos_sin, "cos_sin", torch.float32, (n_pos, rotary_dim // 2, 2))
+    else:
+        rotary_dim = 0
+    library.check(library.lib().yalm_rope_kv_write(
+        p_qkv, p_q, p_k, p_v, p_kp, p_vp, p_bt, stride, max(ring_pages, 1), p_ts, p_tp, p_ss, p_sl, p_cs, n_pos, T,
+        n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, dtype_code(dt), _stream()), "rope_kv_write")
+
+
+def attn_prefill(q, k, v, out, cu_seqlens, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim, window):
+    """Causal (and windowed) attention of packed sequences that start at position 0."""
+    _check_heads(n_heads, n_kv_heads, head_dim)
+    T = q.shape[0]
+    dt = q.dtype
+    B = cu_seqlens.shape[0] - 1
+    p_q = _need(q, "q", dt, (T, n_heads * head_dim))
+    p_k = _need(k, "k", dt, (T, n_kv_heads * head_dim))
+    p_v = _need(v, "v", dt, (T, n_kv_heads * head_dim))
+    p_o = _need(out, "out", dt, (T, n_heads * head_dim))
+    p_cu = _need(cu_seqlens, "cu_seqlens", torch.int32, (B + 1,))
+    p_ts = _need(tok_seq, "tok_seq", torch.int32, (T,))
+    p_tp = _need(tok_pos, "tok_pos", torch.int32, (T,))
+    library.check(library.lib().yalm_attn_prefill(p_q, p_k, p_v, p_o, p_cu, p_ts, p_tp, T, B, n_heads, n_kv_heads,
+                                                  head_dim, int(window), dtype_code(dt), 1 if FORCE_SIMPLE else 0,
+                                                  _stream()), "attn_prefill")
+    return out
+
+
+def attn_decode_workspace_floats(B, n_heads, head_dim, n_splits):
+    return library.lib().yalm_attn_decode_workspace(B, n_heads, head_dim, n_splits) // 4
+
+
+def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len, out, partial, n_heads, n_kv_heads,
+                head_dim, window, n_splits):
+    """One query per sequence over the cache pages; seq_len counts the new key."""
+    _check_heads(n_heads, n_kv_heads, head_dim)
+    B = q.shape[0]
+    dt = q.dtype
+    n_pages = k_pages.shape[0]
+    p_q = _need(q, "q", dt, (B, n_heads * head_dim))
+    p_kp = _need(k_pages, "k_pages", dt, (n_pages, n_kv_heads, PAGE, head_dim))
+    p_vp = _need(v_pages, "v_pages", dt, (n_pages, n_kv_heads, head_dim, PAGE))
+    p_bt = _need(block_table, "block_table", torch.int32, (None, None))
+    stride = block_table.shape[1]
+    if ring_pages <= 0 or ring_pages > stride:
+        raise ValueError("ring_pages %d does not fit the block table (%d columns)" % (ring_pages, stride))
+    p_ss = _need(seq_slot, "seq_slot", torch.int32, (B,))
+    p_sl = _need(seq_len, "seq_len", torch.int32, (B,))
+    p_o = _need(out, "out", dt, (B, n_heads * head_dim))
+    need = attn_decode_workspace_floats(B, n_heads, head_dim, n_splits)
+    p_w = _need(partial, "partial", torch.float32)
+    if partial.numel() < need:
+        raise ValueError("attn_decode workspace too small: %d floats, %d needed" % (partial.numel(), need))
+    library.check(library.lib().yalm_attn_decode(
+        p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_w, B, n_heads, n_kv_heads, head_dim,
+        int(window), int(n_splits), n_pages, dtype_code(dt), 1 if FORCE_SIMPLE else 0, _stream()), "attn_decode")
+    return out
+
+
+def argmax(logits, out):
+    R, V = logits.shape
+    library.check(library.lib().yalm_argmax(_need(logits, "logits", torch.float32), _need(out, "out", torch.int32, (R,)),
+                                            R, V, _stream()), "argmax")
+    return out
+
+
+def sample(logits, u, temperature, out):
+    R, V = logits.shape
+    if not temperature > 0:
+        raise ValueError("temperature must be positive here (0 is argmax)")
+    library.check(library.lib().yalm_sample(_need(logits, "logits", torch.float32), _need(u, "u", torch.float32, (R,)),
+                                            float(temperature), _need(out, "out", torch.int32, (R,)), R, V, _stream()),
+                  "sample")
+    return out
+
+
+def token_prob(logits, index, out):
+    R, V = logits.shape
+    library.check(library.lib().yalm_token_prob(_need(logits, "logits", torch.float32),
+                                                _need(index, "index", torch.int32, (R,)),
+                                                _need(out, "out", torch.float32, (R,)), R, V, _stream()), "token_prob")
+    return out

@@ -1,0 +1,110 @@
+"""Grouped-query self-attention over the cache, with a position encoding that
+it owns and an optional window.
+
+Per token (src/infer.cpp:278-338): q, k, v = W h; q and k rotated at the token's
+position; k and v stored in the cache; per query head h with KV head h // group:
+scores q.k / sqrt(head_dim) over the visible keys, softmax in float32, mix of
+the values; the output projection is added to the residual stream.  Key j is
+visible to the query at position i iff j <= i and (window == 0 or i - j <
+window) (the reference's kv_len rows, src/infer.cpp:486-488).
+
+The three projections are one matrix [q; k; v] (the reference fuses them by
+pointer, src/infer.cu:290-337); q/k rows are re-ordered at load if the folder
+keeps them half-split (convert.py:145-158)."""
+import torch
+
+from ..cache.manager import KVRequest
+from ..ops import kernels
+from ..weights.loader import ParamSpec, place
+from .base import Part, build_part, part
+
+# decode attention is split over pages so that about this many workgroups run
+TARGET_WORKGROUPS = 1024
+
+
+@part("mixer", "gqa_attention")
+class GQAttention(Part):
+    def __init__(self, spec, dim, prefix):
+        super().__init__(spec, dim, prefix)
+        p = spec.params
+        self.n_heads = int(p["n_heads"])
+        self.n_kv_heads = int(p["n_kv_heads"])
+        self.head_dim = int(p["head_dim"])
+        self.window = int(p.get("window", 0) or 0)
+        if self.n_heads % self.n_kv_heads:
+            raise ValueError("n_heads %d is no multiple of n_kv_heads %d" % (self.n_heads, self.n_kv_heads))
+        if self.head_dim % 2 or self.head_dim > kernels.MAX_HEAD_DIM:
+            raise ValueError("head_dim %d is not supported (even, at most %d)" % (self.head_dim, kernels.MAX_HEAD_DIM))
+        self.q_dim = self.n_heads * self.head_dim
+        self.kv_dim = self.n_kv_heads * self.head_dim
+        self.position = build_part("position", p["position"], dim, prefix)
+        self.wqkv = None
+        self.wo = None
+
+    def children(self):
+        return [self.position]
+
+    def param_specs(self):
+        D = self.dim
+        return [ParamSpec(self.prefix + "q_proj.weight", (self.q_dim, D), fan_in=D),
+                ParamSpec(self.prefix + "k_proj.weight", (self.kv_dim, D), fan_in=D),
+                ParamSpec(self.prefix + "v_proj.weight", (self.kv_dim, D), fan_in=D),
+                ParamSpec(self.prefix + "o_proj.weight", (D, self.q_dim), fan_in=self.q_dim)]
+
+    def load(self, get, compute_dtype, device):
+        wq = self.position.arrange_projection_rows(get(self.prefix + "q_proj.weight"), self.n_heads)
+        wk = self.position.arrange_projection_rows(get(self.prefix + "k_proj.weight"), self.n_kv_heads)
+        wv = get(self.prefix + "v_proj.weight")
+        self.wqkv = place(torch.cat([wq, wk, wv], dim=0), compute_dtype, device)
+        self.wo = place(get(self.prefix + "o_proj.weight"), compute_dtype, device)
+
+    def weight_bytes(self):
+        return (self.wqkv.numel() + self.wo.numel()) * self.wqkv.element_size()
+
+    def cache_request(self):
+        return KVRequest(self.n_kv_heads, self.head_dim, self.window)
+
+    def decode_splits(self, B, ring_pages):
+        return max(1, min(ring_pages, TARGET_WORKGROUPS // max(1, B * self.n_heads)))
+
+    def forward(self, h, x, ctx, line, writes_cache=True):
+        T = h.shape[0]
+        act = h.dtype
+        ws = ctx.ws
+        pos = self.position
+        if pos.table is not None and ctx.max_position >= pos.n_positions:
+            raise ValueError("position %d is beyond the %d positions the rotation table holds"
+                             % (ctx.max_position, pos.n_positions))
+        qkv = ws.get("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
+        kernels.gemm(h, self.wqkv, qkv, kernels.EPI_STORE_F32)
+        q = ws.get("attn.q", (T, self.q_dim), act)
+        group = ctx.cache.group_of(line)
+        k_pages, v_pages = group.line_pages(line)
+        prefill = ctx.mode == "prefill"
+        if prefill:
+            # a line that later entries read keeps its token-major keys and values for them
+            tag = "attn.kv%d" % line if ctx.line_is_shared(line) else "attn.kv"
+            k = ws.get(tag + ".k", (T, self.kv_dim), act)
+            v = ws.get(tag + ".v", (T, self.kv_dim), act)
+        else:
+            k = v = None
+        if writes_cache:
+            kernels.rope_kv_write(qkv, q, k, v, k_pages, v_pages, group.table, group.ring_pages, ctx.tok_seq,
+                                  ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads,
+                                  self.head_dim, pos.rotary_dim)
+        else:
+            kernels.rope_kv_write(qkv, q, None, None, None, None, None, 0, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot,
+                                  ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads, self.head_dim,
+                                  pos.rotary_dim)
+        o = ws.get("attn.o", (T, self.q_dim), act)
+        if prefill:
+            kernels.attn_prefill(q, k, v, o, ctx.cu_seqlens, ctx.tok_seq, ctx.tok_pos, self.n_heads, self.n_kv_heads,
+                                 self.head_dim, self.window)
+        else:
+            n_splits = self.decode_splits(T, group.ring_pages)
+            partial = ws.get("attn.partial",
+                             (kernels.attn_decode_workspace_floats(T, self.n_heads, self.head_dim, n_splits),),
+                             torch.float32)
+            kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o,
+                                partial, self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits)
+        kernels.gemm(o, self.wo, x, kernels.EPI_ADD_F32)

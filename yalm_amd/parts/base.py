@@ -1,0 +1,77 @@
+"""Interfaces of the parts a model is put together from, and their registries.
+
+A part is built from a PartSpec (its sizes and constants), the width of the
+residual stream and the prefix of its tensor names.  No part knows which model
+it is in.  Kinds of parts and the methods each must have:
+
+  norm           forward(x_f32[R, dim], out[R, dim], ctx, row_index=None)
+  position       prepare(n_positions, device); used by a mixer, which owns it
+  mixer          cache_request() -> KVRequest | StateRequest | None
+                 forward(h[T, dim], x_f32[T, dim], ctx, line, writes_cache): adds its output to x
+  feed_forward   forward(h[T, dim], x_f32[T, dim], ctx): adds its output to x
+  block          forward(x_f32[T, dim], ctx, line, writes_cache): one layer on the residual stream
+  embedding      forward(tokens_i32[T], x_f32[T, dim], ctx)
+  head           forward(h[R, dim], logits_f32[R, vocab], ctx)
+
+All of them: param_specs() -> [ParamSpec], load(get, compute_dtype, device),
+weight_bytes().  `h` is in the compute dtype (bfloat16 or float32); the
+residual stream `x` is always float32."""
+from typing import Callable, Dict, List
+
+from ..config.spec import PartSpec
+from ..weights.loader import ParamSpec
+
+ROLES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")
+_REGISTRY: Dict[str, Dict[str, type]] = {r: {} for r in ROLES}
+
+
+def register_part(role, kind, cls, replace=False):
+    """Registers class `cls` as the part `kind` of role `role`."""
+    if role not in _REGISTRY:
+        raise ValueError("unknown role %r (one of %s)" % (role, ROLES))
+    if kind in _REGISTRY[role] and not replace and _REGISTRY[role][kind] is not cls:
+        raise ValueError("%s part %r is already registered" % (role, kind))
+    _REGISTRY[role][kind] = cls
+    return cls
+
+
+def unregister_part(role, kind):
+    _REGISTRY[role].pop(kind, None)
+
+
+def part(role, kind):
+    """Decorator form of register_part."""
+    def deco(cls):
+        return register_part(role, kind, cls)
+    return deco
+
+
+def build_part(role, spec: PartSpec, dim: int, prefix: str, **extra):
+    try:
+        cls = _REGISTRY[role][spec.kind]
+    except KeyError:
+        raise ValueError("no %s part named %r is registered (known: %s)"
+                         % (role, spec.kind, sorted(_REGISTRY[role]))) from None
+    return cls(spec, dim, prefix + spec.prefix, **extra)
+
+
+class Part:
+    """Common ground of all parts."""
+
+    def __init__(self, spec: PartSpec, dim: int, prefix: str):
+        self.spec = spec
+        self.dim = dim
+        self.prefix = prefix
+
+    def param_specs(self) -> List[ParamSpec]:
+        return []
+
+    def load(self, get: Callable, compute_dtype, device):
+        """Takes its tensors (`get(name)` gives a CPU tensor) and lays them out on the device."""
+
+    def weight_bytes(self) -> int:
+        """Bytes of weights one step reads (every weight once)."""
+        return 0
+
+    def children(self):
+        return []

@@ -1,0 +1,56 @@
+"""SwiGLU feed-forward, dense: x += down( silu(gate h) * (up h) )
+(src/infer.cpp:356-385 with one expert of weight 1; silu(z) = z / (1 + exp(-z))).
+Gate and up rows are interleaved in blocks of 16 at load so that one GEMM
+produces both and its epilogue multiplies them (the reference fuses the two
+products by pointer, src/infer.cu:610-634)."""
+import torch
+
+from ..ops import kernels
+from ..weights.loader import ParamSpec, place
+from .base import Part, part
+
+GATE_BLOCK = 16
+
+
+def interleave_gate_up(gate, up):
+    """[H, D] x 2 -> [32 * ceil(H/16), D]: 16 gate rows, 16 up rows, ...; zero rows pad the last block."""
+    H, D = gate.shape
+    nb = (H + GATE_BLOCK - 1) // GATE_BLOCK
+    out = torch.zeros((nb, 2, GATE_BLOCK, D), dtype=gate.dtype, device=gate.device)
+    pad = nb * GATE_BLOCK
+    g = torch.zeros((pad, D), dtype=gate.dtype, device=gate.device)
+    u = torch.zeros((pad, D), dtype=gate.dtype, device=gate.device)
+    g[:H] = gate
+    u[:H] = up
+    out[:, 0] = g.reshape(nb, GATE_BLOCK, D)
+    out[:, 1] = u.reshape(nb, GATE_BLOCK, D)
+    return out.reshape(nb * 2 * GATE_BLOCK, D)
+
+
+@part("feed_forward", "swiglu")
+class SwiGLU(Part):
+    def __init__(self, spec, dim, prefix):
+        super().__init__(spec, dim, prefix)
+        self.hidden = int(spec.params["hidden"])
+        self.w_gate_up = None
+        self.w_down = None
+
+    def param_specs(self):
+        D, H = self.dim, self.hidden
+        return [ParamSpec(self.prefix + "gate_proj.weight", (H, D), fan_in=D),
+                ParamSpec(self.prefix + "up_proj.weight", (H, D), fan_in=D),
+                ParamSpec(self.prefix + "down_proj.weight", (D, H), fan_in=H)]
+
+    def load(self, get, compute_dtype, device):
+        gu = interleave_gate_up(get(self.prefix + "gate_proj.weight"), get(self.prefix + "up_proj.weight"))
+        self.w_gate_up = place(gu, compute_dtype, device)
+        self.w_down = place(get(self.prefix + "down_proj.weight"), compute_dtype, device)
+
+    def weight_bytes(self):
+        return 3 * self.hidden * self.dim * self.w_down.element_size()
+
+    def forward(self, h, x, ctx):
+        T = h.shape[0]
+        mid = ctx.ws.get("ffn.hidden", (T, self.hidden), h.dtype)
+        kernels.gemm(h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
+        kernels.gemm(mid, self.w_down, x, kernels.EPI_ADD_F32)
