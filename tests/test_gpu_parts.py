@@ -1,0 +1,320 @@
+"""Each part of a layer alone against the plain implementation's function for it,
+and the proof that parts are exchangeable: a toy mixer with state of its own
+and a toy architecture, both defined here, are registered, built and stepped
+without a change to the package's files."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import helpers
+import schedules
+from plain import reference_model as R
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def make_ctx(cache, lens, dtype, mode="prefill", starts=None):
+    """A StepContext as Engine.step builds it, for parts driven by hand."""
+    from yalm_amd.engine.context import StepContext, Workspace
+    B = len(lens)
+    if mode == "prefill":
+        slots = cache.acquire(B)
+        starts = [0] * B
+    else:
+        slots = starts[0]
+        starts = starts[1]
+    new_lens = cache.extend(slots, lens)
+    ctx = StepContext(mode, cache, Workspace(DEV), dtype)
+    i32 = lambda x: torch.tensor(np.asarray(x), dtype=torch.int32, device=DEV)
+    ctx.tok_seq = i32(np.repeat(np.arange(B), lens))
+    ctx.tok_pos = i32(np.concatenate([np.arange(s, s + n) for s, n in zip(starts, lens)]))
+    ctx.seq_slot = i32(slots)
+    ctx.seq_len = i32(new_lens)
+    ctx.cu_seqlens = i32(np.concatenate([[0], np.cumsum(lens)]))
+    ctx.max_position = max(new_lens) - 1
+    ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), list(lens), list(starts)
+    return ctx, slots
+
+
+def rnd(shape, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(shape, generator=g, dtype=torch.float64).float() * scale
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from yalm_amd.config import PartSpec
+    from yalm_amd.parts import build_part
+    D = 72
+    p = build_part("norm", PartSpec("rmsnorm", {"eps": 2e-4}, prefix="n."), D, "layer.")
+    assert [s.name for s in p.param_specs()] == ["layer.n.weight"] and p.param_specs()[0].shape == (D,)
+    w = 1 + 0.1 * rnd((D,), 1)
+    p.load({"layer.n.weight": w}.__getitem__, dtype, DEV)
+    assert p.weight.dtype == torch.float32            # a vector stored in 32-bit stays so
+    x = rnd((5, D), 2, 4.0)
+    out = torch.empty((5, D), dtype=dtype, device=DEV)
+    p.forward(x.to(DEV), out, None)
+    want = R.rmsnorm(x, w, 2e-4)
+    lim = 1e-5 if dtype == torch.float32 else 1e-2
+    assert (out.cpu().double() - want).abs().max() <= lim * want.abs().max()
+
+
+def test_rope_part_table_and_row_order():
+    from yalm_amd.config import PartSpec
+    from yalm_amd.parts import build_part
+    from yalm_amd.parts.rope import interleave_rows, inverse_frequencies
+    scaling = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+               "original_max_position_embeddings": 32}
+    for hd, rd, theta, sc in [(16, 16, 1e4, None), (32, 32, 500.0, scaling), (48, 24, 1e6, None)]:
+        p = build_part("position", PartSpec("rope", {"head_dim": hd, "rotary_dim": rd, "theta": theta, "scaling": sc,
+                                                      "weight_rows": "half_split"}), 64, "")
+        p.prepare(100, DEV)
+        f = R.rope_inv_freq(hd, rd, theta)[: rd // 2]
+        if sc:
+            f = R.llama3_scaled_inv_freq(f, 8.0, 1.0, 4.0, 32)
+        assert torch.allclose(inverse_frequencies(hd, rd, theta, sc), f, rtol=1e-14, atol=0)
+        ang = torch.arange(100, dtype=torch.float64)[:, None] * f[None]
+        assert p.table.shape == (100, rd // 2, 2)
+        assert torch.allclose(p.table[..., 0].cpu().double(), torch.cos(ang), atol=1e-7)
+        assert torch.allclose(p.table[..., 1].cpu().double(), torch.sin(ang), atol=1e-7)
+        w = rnd((3 * hd, 10), 3)
+        assert torch.equal(p.arrange_projection_rows(w, 3), R.hf_rows_to_interleaved(w, 3, rd))
+        assert torch.equal(interleave_rows(w, 3, hd, rd), R.hf_rows_to_interleaved(w, 3, rd))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_heads,n_kv,hd,window,D", [(4, 2, 16, 0, 64), (3, 1, 32, 16, 80), (6, 6, 48, 0, 72)])
+def test_attention_part_prefill_then_decode(n_heads, n_kv, hd, window, D, dtype):
+    """The mixer alone: whole prompts of unequal lengths, then one more token each,
+    against the plain rope + attention + projections."""
+    from yalm_amd.cache import CacheManager
+    from yalm_amd.config import PartSpec
+    from yalm_amd.parts import build_part
+    pos_spec = PartSpec("rope", {"head_dim": hd, "rotary_dim": hd, "theta": 1e4, "scaling": None,
+                                 "weight_rows": "half_split"})
+    spec = PartSpec("gqa_attention", {"n_heads": n_heads, "n_kv_heads": n_kv, "head_dim": hd, "window": window,
+                                      "position": pos_spec}, prefix="attn.")
+    part = build_part("mixer", spec, D, "l.")
+    Q, KV = n_heads * hd, n_kv * hd
+    names = {s.name: s.shape for s in part.param_specs()}
+    assert names == {"l.attn.q_proj.weight": (Q, D), "l.attn.k_proj.weight": (KV, D),
+                     "l.attn.v_proj.weight": (KV, D), "l.attn.o_proj.weight": (D, Q)}
+    w = {n: rnd(s, 10 + i, 1 / math.sqrt(s[1])) for i, (n, s) in enumerate(sorted(names.items()))}
+    if dtype == torch.bfloat16:
+        w = {n: t.bfloat16().float() for n, t in w.items()}
+    part.load(w.__getitem__, dtype, DEV)
+    part.position.prepare(256, DEV)
+    cache = CacheManager({0: part.cache_request()}, 64 * 16, 256, dtype, DEV, n_slots=4)
+    lens = [70, 5, 33]
+    T = sum(lens)
+    h_all = [rnd((n + 1, D), 20 + i).to(dtype).float() for i, n in enumerate(lens)]     # one more token for decode
+
+    def plain(h):
+        n = h.shape[0]
+        f = R.rope_inv_freq(hd, hd, 1e4)
+        pos = torch.arange(n)
+        q = (h.double() @ R.hf_rows_to_interleaved(w["l.attn.q_proj.weight"].double(), n_heads, hd).T)
+        k = (h.double() @ R.hf_rows_to_interleaved(w["l.attn.k_proj.weight"].double(), n_kv, hd).T)
+        v = h.double() @ w["l.attn.v_proj.weight"].double().T
+        a = R.attention(R.rope_interleaved(q.reshape(n, n_heads, hd), pos, f),
+                        R.rope_interleaved(k.reshape(n, n_kv, hd), pos, f), v.reshape(n, n_kv, hd), window)
+        return a.reshape(n, Q) @ w["l.attn.o_proj.weight"].double().T
+
+    want = [plain(h) for h in h_all]
+    ctx, slots = make_ctx(cache, lens, dtype)
+    h = torch.cat([x[:-1] for x in h_all]).to(DEV, dtype)
+    x = torch.zeros((T, D), device=DEV)
+    part.forward(h, x, ctx, 0, True)
+    lim = 2e-5 if dtype == torch.float32 else 3e-2
+    got = x.cpu().double()
+    o = 0
+    for i, n in enumerate(lens):
+        assert (got[o:o + n] - want[i][:n]).abs().max() <= lim * max(1, want[i].abs().max()), ("prefill", i)
+        o += n
+    ctx, _ = make_ctx(cache, [1, 1, 1], dtype, "decode", (slots, lens))
+    h = torch.stack([x[-1] for x in h_all]).to(DEV, dtype)
+    x = torch.ones((3, D), device=DEV)                               # the mixer adds to the residual stream
+    part.forward(h, x, ctx, 0, True)
+    got = x.cpu().double() - 1
+    for i in range(3):
+        assert (got[i] - want[i][-1]).abs().max() <= lim * max(1, want[i].abs().max()), ("decode", i)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    from yalm_amd.config import PartSpec
+    from yalm_amd.engine.context import StepContext, Workspace
+    from yalm_amd.parts import build_part
+    D, H = 72, 200
+    part = build_part("feed_forward", PartSpec("swiglu", {"hidden": H}, prefix="mlp."), D, "l.")
+    w = {"l.mlp.gate_proj.weight": rnd((H, D), 1, D ** -0.5), "l.mlp.up_proj.weight": rnd((H, D), 2, D ** -0.5),
+         "l.mlp.down_proj.weight": rnd((D, H), 3, H ** -0.5)}
+    if dtype == torch.bfloat16:
+        w = {n: t.bfloat16().float() for n, t in w.items()}
+    assert {s.name: s.shape for s in part.param_specs()} == {n: tuple(t.shape) for n, t in w.items()}
+    part.load(w.__getitem__, dtype, DEV)
+    h = rnd((9, D), 4).to(dtype)
+    x0 = rnd((9, D), 5)
+    x = x0.to(DEV).clone()
+    part.forward(h.to(DEV), x, StepContext("prefill", None, Workspace(DEV), dtype))
+    want = x0.double() + R.swiglu_ffn(h.float(), w["l.mlp.gate_proj.weight"], w["l.mlp.down_proj.weight"],
+                                      w["l.mlp.up_proj.weight"])
+    lim = 2e-5 if dtype == torch.float32 else 2e-2
+    assert (x.cpu().double() - want).abs().max() <= lim * want.abs().max()
+
+
+def test_embedding_and_tied_head():
+    from yalm_amd.config import PartSpec
+    from yalm_amd.parts import build_part
+    V, D = 50, 24
+    emb = build_part("embedding", PartSpec("token_embedding", {"vocab_size": V}, prefix="emb."), D, "")
+    head = build_part("head", PartSpec("lm_head", {"vocab_size": V, "tied": True}, prefix="head."), D, "",
+                      embedding=emb)
+    assert head.param_specs() == []
+    table = rnd((V, D), 1)
+    emb.load({"emb.weight": table}.__getitem__, torch.float32, DEV)
+    head.load(None, torch.float32, DEV)
+    assert head.weight.data_ptr() == emb.table.data_ptr()            # one copy on the device
+    x = torch.empty((3, D), device=DEV)
+    emb.forward(torch.tensor([4, 0, 49], dtype=torch.int32, device=DEV), x, None)
+    assert torch.equal(x.cpu(), table[[4, 0, 49]])
+    logits = torch.empty((3, V), device=DEV)
+    head.forward(x, logits, None)
+    assert torch.allclose(logits.cpu().double(), table[[4, 0, 49]].double() @ table.double().T, atol=1e-4)
+
+
+# ---------------------------------------------------------------------------
+# a toy mixer with state of its own, and a toy architecture that uses it
+# ---------------------------------------------------------------------------
+
+def toy_mixer_plain(h, w):
+    """out[t] = W mean(h[0..t]) for one whole sequence, float64."""
+    h = h.double()
+    mean = torch.cumsum(h, 0) / torch.arange(1, h.shape[0] + 1, dtype=torch.float64)[:, None]
+    return mean @ w.double().T
+
+
+def define_toy_parts():
+    from yalm_amd.cache import StateRequest
+    from yalm_amd.parts import Part, register_part
+    from yalm_amd.weights import ParamSpec
+
+    class RunningMeanMixer(Part):
+        """x += W * (mean of all inputs of the sequence so far).  Its state is the
+        running sum, one vector per sequence, kept in the cache's state store."""
+        graph_safe = False                    # its launches depend on host values
+
+        def param_specs(self):
+            return [ParamSpec(self.prefix + "w.weight", (self.dim, self.dim), fan_in=self.dim)]
+
+        def load(self, get, compute_dtype, device):
+            self.w = get(self.prefix + "w.weight").to(device, torch.float32)
+
+        def cache_request(self):
+            return StateRequest((self.dim,), torch.float32)
+
+        def forward(self, h, x, ctx, line, writes_cache=True):
+            state = ctx.cache.group_of(line).line_state(line)          # [n_slots, dim]
+            o = 0
+            for slot, n, start in zip(ctx.host_slots, ctx.host_n_tokens, ctx.host_start):
+                hs = h[o:o + n].float()
+                sums = state[slot][None, :] + torch.cumsum(hs, 0)
+                counts = torch.arange(start + 1, start + n + 1, device=h.device, dtype=torch.float32)[:, None]
+                x[o:o + n] += (sums / counts) @ self.w.T
+                state[slot] = sums[-1]
+                o += n
+
+    register_part("mixer", "toy_running_mean", RunningMeanMixer, replace=True)
+    return RunningMeanMixer
+
+
+class ToyConfig:
+    """A toy architecture: layer 0 mixes with the running mean, layer 1 with
+    attention; the schedule runs layer 1 twice (two cache lines)."""
+
+    def __init__(self, d):
+        self.d = d
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d)
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def to_spec(self):
+        from yalm_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+        d = self.d
+        D = d["width"]
+        norm = {"eps": d["eps"]}
+        pos = PartSpec("rope", {"head_dim": 16, "rotary_dim": 16, "theta": 100.0, "scaling": None,
+                                "weight_rows": "interleaved"})
+        mixers = [PartSpec("toy_running_mean", {}, prefix="mean."),
+                  PartSpec("gqa_attention", {"n_heads": 2, "n_kv_heads": 1, "head_dim": 16, "window": 0,
+                                             "position": pos}, prefix="attn.")]
+        layers = [LayerSpec("prenorm_residual", m, PartSpec("swiglu", {"hidden": d["hidden"]}, prefix="ff."),
+                            PartSpec("rmsnorm", norm, prefix="n1."), PartSpec("rmsnorm", norm, prefix="n2."),
+                            "toy.%d." % i) for i, m in enumerate(mixers)]
+        return ModelSpec("ToyForCausalLM", D, d["vocab"], d["positions"],
+                         PartSpec("token_embedding", {"vocab_size": d["vocab"]}, prefix="toy.emb."), layers,
+                         PartSpec("rmsnorm", norm, prefix="toy.norm."),
+                         PartSpec("lm_head", {"vocab_size": d["vocab"], "tied": True}),
+                         schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1), ScheduleEntry(1, 2)])
+
+
+def toy_plain_forward(w, d, tokens):
+    """The toy model written out with the plain implementation's functions."""
+    T = len(tokens)
+    x = R.embedding(w["toy.emb.weight"], torch.tensor(tokens))
+    f = R.rope_inv_freq(16, 16, 100.0)
+    pos = torch.arange(T)
+
+    def ffn(x, p):
+        return R.swiglu_ffn(R.rmsnorm(x, w[p + "n2.weight"], d["eps"]), w[p + "ff.gate_proj.weight"],
+                            w[p + "ff.down_proj.weight"], w[p + "ff.up_proj.weight"])
+
+    x = x + toy_mixer_plain(R.rmsnorm(x, w["toy.0.n1.weight"], d["eps"]), w["toy.0.mean.w.weight"])
+    x = x + ffn(x, "toy.0.")
+    for _ in range(2):
+        h = R.rmsnorm(x, w["toy.1.n1.weight"], d["eps"])
+        q = (h @ w["toy.1.attn.q_proj.weight"].double().T).reshape(T, 2, 16)
+        k = (h @ w["toy.1.attn.k_proj.weight"].double().T).reshape(T, 1, 16)
+        v = (h @ w["toy.1.attn.v_proj.weight"].double().T).reshape(T, 1, 16)
+        a = R.attention(R.rope_interleaved(q, pos, f), R.rope_interleaved(k, pos, f), v)
+        x = x + a.reshape(T, 32) @ w["toy.1.attn.o_proj.weight"].double().T
+        x = x + ffn(x, "toy.1.")
+    return R.rmsnorm(x, w["toy.norm.weight"], d["eps"]) @ w["toy.emb.weight"].double().T
+
+
+def test_toy_mixer_and_architecture_from_outside(tmp_path):
+    from yalm_amd import Engine, Model, register_architecture, write_random_model
+    from yalm_amd.cache import StateGroup
+    from yalm_amd.config import unregister_architecture
+    from yalm_amd.parts import unregister_part
+    define_toy_parts()
+    register_architecture("ToyForCausalLM", ToyConfig, replace=True)
+    try:
+        d = {"architectures": ["ToyForCausalLM"], "width": 40, "hidden": 48, "vocab": 61, "positions": 200,
+             "eps": 1e-5}
+        folder = write_random_model(str(tmp_path / "toy"), d, seed=2)
+        model = Model.from_folder(folder, dtype=torch.float32, device=DEV)
+        assert not model.graph_safe()
+        engine = Engine(model, max_tokens=1024)
+        assert len(engine.cache.state_groups) == 1 and isinstance(engine.cache.group_of(0), StateGroup)
+        assert engine.cache.group_of(1) is engine.cache.group_of(2)          # the layer that runs twice: two lines
+        cfg, w = R.read_folder(folder)
+        requests = {"a": [5, 9, 60, 3, 3, 17, 44, 8, 0, 31], "b": [7, 7, 2], "c": list(range(40, 61)) + list(range(30)),
+                    "d": [60, 0, 1, 59, 2, 58]}
+        for steps in (schedules.whole(requests), schedules.tail_one_by_one(requests, 4),
+                      schedules.batches(requests, [["a", "b"], ["c", "d"]], {"a": 4, "b": 1, "c": 33, "d": 2})):
+            out = schedules.replay_in_process(engine, steps)
+            got = schedules.per_request(steps, out, requests)
+            for rid, toks in requests.items():
+                want = toy_plain_forward(w, d, toks).float().numpy()
+                helpers.check_logits(got[rid], want, "float32", "toy %s" % rid)
+    finally:
+        unregister_architecture("ToyForCausalLM")
+        unregister_part("mixer", "toy_running_mean")
