@@ -1,0 +1,164 @@
+#!/usr/bin/env python3
+"""Measures the library on one MI355X: decode tokens/s at batch 8 (the value),
+at batch 1 and 64 (points), and the prefill of a 2,048-token prompt, for a
+Mistral-7B-shaped model with random weights and random token ids.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--dtype bf16|fp32]
+
+A step is one decode step as generation does it: the step function for a batch
+of sequences (one token each, from the cache), greedy sampling on the device
+and the read-back of the tokens.  One JSON line is printed.  Peaks are MI355X's
+published ones: HBM 8 TB/s; dense MFMA bf16/fp16 2.5 PFLOP/s, fp32 157.3 TFLOP/s."""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# BASELINE.json configs[2]: Mistral-7B-v0.2 shape
+MISTRAL_7B = {
+    "architectures": ["MistralForCausalLM"], "hidden_size": 4096, "intermediate_size": 14336,
+    "num_hidden_layers": 32, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+    "vocab_size": 32000, "max_position_embeddings": 32768, "rope_theta": 1000000.0, "rms_norm_eps": 1e-5,
+    "hidden_act": "silu", "tie_word_embeddings": False, "bos_token_id": 1, "eos_token_id": 2,
+}
+CONTEXT = 4096
+PROMPT = 2048
+HBM_PEAK = 8.0e12
+FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+BASELINE_TOK_S = 63.8            # the reference's published batch-1 figure (RTX 4090), README.md:14
+
+
+def prefill_flops(cfg, n_layers, T):
+    """GEMM flops of a prompt of T tokens + causal attention + the head on one row."""
+    D, H, V = cfg["hidden_size"], cfg["intermediate_size"], cfg["vocab_size"]
+    Q = cfg["num_attention_heads"] * cfg["head_dim"]
+    KV = cfg["num_key_value_heads"] * cfg["head_dim"]
+    per_layer = 2 * T * D * (Q + 2 * KV) + 2 * T * Q * D + 3 * 2 * T * D * H
+    attn = 4 * cfg["num_attention_heads"] * cfg["head_dim"] * (T * (T + 1) // 2)
+    return n_layers * (per_layer + attn) + 2 * D * V
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=0, help="build only the first N layers (0 = all)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--points", default="1,64", help="further batch sizes to measure")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this library runs on one GPU; --gpus %d is not measured" % args.gpus, flush=True)
+        return 2
+
+    import torch
+    from yalm_amd import Engine, Model, Sampler
+    from yalm_amd.cache import PAGE
+
+    dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
+    n_layers = args.layers or MISTRAL_7B["num_hidden_layers"]
+    dev = "cuda:0"
+    t0 = time.time()
+    model = Model.random(MISTRAL_7B, seed=0, dtype=dtype, device=dev, n_layers=n_layers)
+    torch.cuda.synchronize()
+    sys.stderr.write("[bench] %d layers of random weights in %.1f s\n" % (n_layers, time.time() - t0))
+    batches = sorted({args.batch} | {int(b) for b in args.points.split(",") if b})
+    engine = Engine(model, max_tokens=max(batches) * CONTEXT, max_batch=max(batches))
+    sampler = Sampler(0)
+    V = MISTRAL_7B["vocab_size"]
+    gen = torch.Generator().manual_seed(1)
+
+    def sync():
+        torch.cuda.synchronize()
+
+    # ---------------------------------------------------------------- prefill of one 2,048-token prompt
+    prefill = None
+    if not args.no_prefill:
+        prompt = torch.randint(0, V, (PROMPT,), generator=gen).tolist()
+        times = []
+        for i in range(3):
+            slots = engine.start(1)
+            sync()
+            t = time.perf_counter()
+            logits = engine.step(slots, [prompt])
+            sampler.sample(logits, 0.0, [0], [0])
+            sync()
+            times.append(time.perf_counter() - t)
+            engine.release(slots)
+        sec = min(times[1:])
+        fl = prefill_flops(MISTRAL_7B, n_layers, PROMPT)
+        prefill = {"value": round(PROMPT / sec, 1), "tokens": PROMPT, "ms": round(sec * 1e3, 3),
+                   "frac": round(fl / sec / FLOP_PEAK[args.dtype], 4)}
+        sys.stderr.write("[bench] prefill %s\n" % prefill)
+
+    # ---------------------------------------------------------------- decode
+    def decode(B, steps, warmup):
+        prompts = [torch.randint(0, V, (PROMPT,), generator=gen).tolist() for _ in range(B)]
+        slots = engine.start(B)
+        ids = list(range(B))
+        # prompts in chunks of sequences, so that the prefill workspace stays small
+        tokens = []
+        for i in range(0, B, 8):
+            logits = engine.step(slots[i:i + 8], prompts[i:i + 8])
+            tokens += sampler.sample(logits, 0.0, ids[i:i + 8], [0] * len(slots[i:i + 8]))
+        for _ in range(warmup):
+            logits = engine.step(slots, [[t] for t in tokens])
+            tokens = sampler.sample(logits, 0.0, ids, [0] * B)
+        sync()
+        start_len = engine.length(slots[0])
+        t = time.perf_counter()
+        for _ in range(steps):
+            logits = engine.step(slots, [[t_] for t_ in tokens])
+            tokens = sampler.sample(logits, 0.0, ids, [0] * B)
+        sync()
+        sec = time.perf_counter() - t
+        end_len = engine.length(slots[0])
+        engine.release(slots)
+        mean_ctx = (start_len + 1 + end_len) / 2.0
+        kv_bytes = sum(g.bytes_per_token() for g in engine.cache.kv_groups) * mean_ctx * B
+        step_bytes = model.weight_bytes() + (B - 1) * model.embedding.weight_bytes() + kv_bytes
+        return {"tok_s": B * steps / sec, "ms": sec / steps * 1e3, "bytes": step_bytes, "ctx": mean_ctx}
+
+    results = {}
+    for B in batches:
+        results[B] = decode(B, args.steps, args.warmup)
+        sys.stderr.write("[bench] decode B=%d: %.1f tok/s, %.3f ms/step, %.1f GB/step -> %.0f GB/s\n" % (
+            B, results[B]["tok_s"], results[B]["ms"], results[B]["bytes"] / 1e9,
+            results[B]["bytes"] / results[B]["ms"] / 1e6))
+
+    main_r = results[args.batch]
+    achieved = main_r["bytes"] / (main_r["ms"] * 1e-3) / 1e9
+    line = {
+        "metric": "decode tok/s @ batch %d, Mistral-7B shape, context %d" % (args.batch, CONTEXT),
+        "value": round(main_r["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(main_r["ms"], 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": round(results[1]["tok_s"] / BASELINE_TOK_S, 2) if 1 in results else None,
+        "dtype": args.dtype, "data": "synthetic: seeded random weights and token ids",
+        "config": {
+            "model": "Mistral-7B-v0.2 shape", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
+            "layers": n_layers, "layers_of_config": MISTRAL_7B["num_hidden_layers"], "dim": 4096, "hidden_dim": 14336,
+            "n_heads": 32, "n_kv_heads": 8, "head_dim": 128, "vocab_size": 32000, "rope_theta": 1e6,
+            "norm_eps": 1e-5, "tied": False, "window": 0, "prompt_len": PROMPT,
+            "decode_mean_context": round(main_r["ctx"], 1), "kv_dtype": args.dtype, "page_tokens": PAGE,
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4)},
+        "points": {"decode_b%d" % B: round(r["tok_s"], 1) for B, r in results.items() if B != args.batch},
+        "points_roofline_frac": {"decode_b%d" % B: round(r["bytes"] / (r["ms"] * 1e-3) / HBM_PEAK, 4)
+                                 for B, r in results.items()},
+        "vs_baseline_note": "batch-1 decode tok/s over the reference's published 63.8 tok/s (RTX 4090, fp16)",
+    }
+    if prefill is not None:
+        line["prefill"] = prefill
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
