@@ -165,31 +165,32 @@ def test_rope_kv_write(n_heads, n_kv, hd, rd, dtype):
     table = make_table(80, hd, rd, 10000.0)
     bt = torch.full((n_slots, ring), -1, dtype=torch.int32)
     bt[2, 0], bt[2, 1], bt[0, 0] = 5, 7, 1
+    page_of = {0: {0: 5, 1: 7}, 1: {0: 1}}
+    tile_of = {0: {0: 0, 1: 1}, 1: {0: 2}}            # staging: sequence 0 has tiles 0, 1; sequence 1 tile 2
     kp = torch.zeros((n_pages, n_kv, PAGE, hd), dtype=dtype, device=DEV)
     vp = torch.zeros((n_pages, n_kv, hd, PAGE), dtype=dtype, device=DEV)
+    ks = torch.zeros((3, n_kv, PAGE, hd), dtype=dtype, device=DEV)
+    vs = torch.zeros((3, n_kv, hd, PAGE), dtype=dtype, device=DEV)
     q_out = torch.empty((T, Q), dtype=dtype, device=DEV)
-    k_out = torch.empty((T, KV), dtype=dtype, device=DEV)
-    v_out = torch.empty((T, KV), dtype=dtype, device=DEV)
-    k.rope_kv_write(qkv.to(DEV), q_out, k_out, v_out, kp, vp, bt.to(DEV), ring, i32(seq), i32(pos), i32([2, 0]),
-                    i32([70, 5]), table.to(DEV), n_heads, n_kv, hd, rd)
+    k.rope_kv_write(qkv.to(DEV), q_out, ks, vs, i32([0, 2, 3]), kp, vp, bt.to(DEV), ring, i32(seq), i32(pos),
+                    i32([2, 0]), i32([70, 5]), table.to(DEV), n_heads, n_kv, hd, rd)
     f = R.rope_inv_freq(hd, rd, 10000.0)
     p = torch.tensor(pos)
     q_want = R.rope_interleaved(qkv[:, :Q].reshape(T, n_heads, hd), p, f).reshape(T, Q)
-    k_want = R.rope_interleaved(qkv[:, Q:Q + KV].reshape(T, n_kv, hd), p, f).reshape(T, KV)
-    v_want = qkv[:, Q + KV:].double()
+    k_want = R.rope_interleaved(qkv[:, Q:Q + KV].reshape(T, n_kv, hd), p, f)
+    v_want = qkv[:, Q + KV:].double().reshape(T, n_kv, hd)
     close(q_out, q_want, dtype, "q")
-    close(k_out, k_want, dtype, "k")
-    close(v_out, v_want, dtype, "v")
-    kp, vp = kp.cpu(), vp.cpu()
+    kp, vp, ks, vs = kp.cpu(), vp.cpu(), ks.cpu(), vs.cpu()
     for t in range(T):
-        page = {0: {0: 5, 1: 7}, 1: {0: 1}}[seq[t]][pos[t] // PAGE]
-        r = pos[t] % PAGE
-        assert torch.equal(kp[page, :, r, :].reshape(-1), k_out[t].cpu())
-        assert torch.equal(vp[page, :, :, r].reshape(-1), v_out[t].cpu())
+        page, tile, r = page_of[seq[t]][pos[t] // PAGE], tile_of[seq[t]][pos[t] // PAGE], pos[t] % PAGE
+        close(ks[tile, :, r, :], k_want[t], dtype, "staged k")
+        close(vs[tile, :, :, r], v_want[t], dtype, "staged v")
+        assert torch.equal(kp[page, :, r, :], ks[tile, :, r, :])
+        assert torch.equal(vp[page, :, :, r], vs[tile, :, :, r])
     # nothing else was touched
     touched = torch.zeros((n_pages, PAGE), dtype=torch.bool)
     for t in range(T):
-        touched[{0: {0: 5, 1: 7}, 1: {0: 1}}[seq[t]][pos[t] // PAGE], pos[t] % PAGE] = True
+        touched[page_of[seq[t]][pos[t] // PAGE], pos[t] % PAGE] = True
     assert (kp.float().abs().sum(dim=(1, 3)) > 0).equal(touched)
 
 
@@ -203,8 +204,8 @@ def test_rope_kv_write_ring_keeps_the_last_pages_only():
     kp = torch.zeros((8, n_kv, PAGE, hd), device=DEV)
     vp = torch.zeros((8, n_kv, hd, PAGE), device=DEV)
     q_out = torch.empty((L, hd), device=DEV)
-    k.rope_kv_write(qkv.to(DEV), q_out, None, None, kp, vp, bt.to(DEV), ring, i32([0] * L), i32(list(range(L))),
-                    i32([0]), i32([L]), None, 1, n_kv, hd, 0)
+    k.rope_kv_write(qkv.to(DEV), q_out, None, None, None, kp, vp, bt.to(DEV), ring, i32([0] * L),
+                    i32(list(range(L))), i32([0]), i32([L]), None, 1, n_kv, hd, 0)
     kp = kp.cpu()
     # absolute page 2 -> column 0 (page 4), page 3 -> column 1 (page 6)
     assert torch.equal(kp[4, 0], qkv[2 * PAGE:3 * PAGE, hd:2 * hd])
@@ -224,11 +225,27 @@ def packed_attention_reference(q, k, v, lens, n_heads, n_kv, hd, window):
     return torch.cat(outs)
 
 
+def stage(kk, v, lens, n_kv, hd, dtype, poison=True):
+    """Keys and values of packed sequences in the staging format of a prefill step."""
+    PAGE = K().PAGE
+    tile0 = np.concatenate([[0], np.cumsum([(n + PAGE - 1) // PAGE for n in lens])])
+    fill = float("nan") if poison else 0.0
+    ks = torch.full((int(tile0[-1]), n_kv, PAGE, hd), fill, dtype=dtype)
+    vs = torch.full((int(tile0[-1]), n_kv, hd, PAGE), fill, dtype=dtype)
+    o = 0
+    for b, n in enumerate(lens):
+        for p in range(n):
+            ks[tile0[b] + p // PAGE, :, p % PAGE, :] = kk[o + p].reshape(n_kv, hd)
+            vs[tile0[b] + p // PAGE, :, :, p % PAGE] = v[o + p].reshape(n_kv, hd)
+        o += n
+    return ks, vs, tile0
+
+
 @pytest.mark.parametrize("simple", [False, True])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens", [
     (4, 2, 16, 0, [5, 17, 1]), (3, 1, 32, 16, [2, 30, 70]), (6, 3, 48, 100, [130, 64]), (8, 2, 128, 0, [200]),
-    (2, 2, 80, 7, [65, 3]), (5, 5, 64, 0, [129])])
+    (2, 2, 80, 7, [65, 3]), (5, 5, 64, 0, [129]), (4, 1, 64, 70, [300, 64, 1]), (8, 2, 128, 100, [17, 257])])
 def test_attn_prefill(n_heads, n_kv, hd, window, lens, dtype, simple):
     k = K()
     T = sum(lens)
@@ -238,10 +255,12 @@ def test_attn_prefill(n_heads, n_kv, hd, window, lens, dtype, simple):
     cu = np.concatenate([[0], np.cumsum(lens)])
     seq = np.repeat(np.arange(len(lens)), lens)
     pos = np.concatenate([np.arange(n) for n in lens])
+    ks, vs, tile0 = stage(kk, v, lens, n_kv, hd, dtype)
     out = torch.empty((T, n_heads * hd), dtype=dtype, device=DEV)
     k.FORCE_SIMPLE = simple
     try:
-        k.attn_prefill(q.to(DEV), kk.to(DEV), v.to(DEV), out, i32(cu), i32(seq), i32(pos), n_heads, n_kv, hd, window)
+        k.attn_prefill(q.to(DEV), ks.to(DEV), vs.to(DEV), out, i32(cu), i32(tile0), i32(seq), i32(pos), n_heads, n_kv,
+                       hd, window)
     finally:
         k.FORCE_SIMPLE = False
     close(out, packed_attention_reference(q, kk, v, lens, n_heads, n_kv, hd, window), dtype, "prefill attention")
@@ -345,8 +364,10 @@ def test_attn_vector_of_the_reference():
     kv = torch.zeros((4, hd))
     kv[0, 0], kv[1, 1], kv[2, 2], kv[3, 0] = 1, 1, 1, -1
     out = torch.empty((4, 2 * hd), device=DEV)
+    ks, vs, tile0 = stage(kv, kv, [4], 1, hd, torch.float32, poison=False)
     # the reference divides by sqrt(3); here sqrt(16): the scores stay far apart, the result is the same
-    k.attn_prefill(q.to(DEV), kv.to(DEV), kv.to(DEV), out, i32([0, 4]), i32([0] * 4), i32([0, 1, 2, 3]), 2, 1, hd, 0)
+    k.attn_prefill(q.to(DEV), ks.to(DEV), vs.to(DEV), out, i32([0, 4]), i32(tile0), i32([0] * 4), i32([0, 1, 2, 3]), 2,
+                   1, hd, 0)
     got = out.cpu()[3].reshape(2, hd)
     assert torch.allclose(got[0, :3], torch.tensor([0., 1, 0]), atol=1e-4)
     assert torch.allclose(got[1, :3], torch.tensor([0., 0, 1]), atol=1e-4)

@@ -34,6 +34,8 @@ def make_ctx(cache, lens, dtype, mode="prefill", starts=None):
     ctx.seq_slot = i32(slots)
     ctx.seq_len = i32(new_lens)
     ctx.cu_seqlens = i32(np.concatenate([[0], np.cumsum(lens)]))
+    tile0 = np.concatenate([[0], np.cumsum([(n + 63) // 64 for n in lens])])
+    ctx.seq_tile0, ctx.n_tiles = i32(tile0), int(tile0[-1])
     ctx.max_position = max(new_lens) - 1
     ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), list(lens), list(starts)
     return ctx, slots

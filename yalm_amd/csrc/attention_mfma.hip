@@ -1,13 +1,370 @@
-// bfloat16 attention on the matrix cores (placeholder until the MFMA kernels
-// land: it refuses every shape, so the float32-arithmetic kernels run instead).
+// bfloat16 attention on the matrix cores (v_mfma_f32_16x16x32_bf16), softmax state
+// in float32.  Keys are kept [row][element] and values transposed [element][row] in
+// pages of 64 rows, so every operand is a 16-byte load:
+//
+//   scores^T[key, col] = K[key, :] . Q[col, :]     A = 16 key rows x 32 elements, B = queries
+//   out^T[elem, col]  += V^T[elem, key] P^T[key, col]   A = 16 elements x 32 keys, B = P^T
+//
+// The C layout of the first product (a lane holds 4 consecutive rows of one column)
+// feeds the second product's B operand directly: key tile t reads the page rows
+// key_row(t, i), chosen so that a lane ends up with 8 consecutive keys per 32-key
+// step, the same keys its 16-byte load of V^T covers.  No shuffles, no LDS.
+//
+// A column is a query head of the group (decode: up to 16 heads share one pass over
+// the keys of their KV head) or a query position (prefill: 16 positions a wave).
+#include <float.h>
+#include <math.h>
 #include "common.h"
 #include "yalm_hip.h"
 
-int yalm_attn_prefill_bf16_mfma(const void*, const void*, const void*, void*, const int*, const int*, const int*, int,
-                                int, int, int, int, int, hipStream_t) {
-  return YALM_ERR_ARG;
+int yalm_attn_decode_combine_bf16(const float* partial, void* out, int B, int n_heads, int head_dim, int n_splits,
+                                  hipStream_t stream);   // attention_simple.hip
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ bf16x8 zero8() { return (bf16x8){0, 0, 0, 0, 0, 0, 0, 0}; }
+
+// page row that MFMA row i (0..15) of key tile t (0..3) reads
+__device__ __forceinline__ int key_row(int t, int i) { return 32 * (t >> 1) + 8 * (i >> 2) + 4 * (t & 1) + (i & 3); }
+
+// ---------------------------------------------------------------------------
+// decode: grid (split, kv head, sequence); 4 waves take the pages of the split in turn
+// ---------------------------------------------------------------------------
+template <int HD>
+__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
+    const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
+    const int* __restrict__ seq_len, float* __restrict__ partial, int n_heads, int n_kv_heads, int window,
+    int n_splits, int n_pages) {
+  constexpr int KS = HD / 32, DT = HD / 16;
+  __shared__ float sm_m[4][16];
+  __shared__ float sm_l[4][16];
+  __shared__ f32x4 sm_o[4][DT][WAVE];
+  const int split = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, qd = lane / 16, j = lane % 16;
+  const int G = n_heads / n_kv_heads;
+  const int slot = seq_slot[b];
+  const int L = slot >= 0 ? seq_len[b] : 0;
+
+  float m = -FLT_MAX, l = 0.f;
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  if (L > 0) {
+    const int lo = window > 0 ? max(0, L - window) : 0;
+    const int first_page = lo / PAGE, last_page = (L - 1) / PAGE;
+    const int total = last_page - first_page + 1;
+    const int per = (total + n_splits - 1) / n_splits;
+    const int p_begin = first_page + split * per;
+    const int p_end = min(last_page + 1, p_begin + per);
+    const float root = sqrtf((float)HD);
+    const size_t page_elems = (size_t)n_kv_heads * PAGE * HD;
+    const int* table = block_table + (size_t)slot * table_stride;
+
+    bf16x8 qv[KS];
+    {
+      const bool head_ok = j < G;
+      const bf16* qrow = q + ((size_t)b * n_heads + g * G + (head_ok ? j : 0)) * HD;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) qv[ks] = head_ok ? ld8(qrow + ks * 32 + qd * 8) : zero8();
+    }
+
+    bf16x8 kreg[4][KS];
+    int ap = p_begin + wave;
+    if (ap < p_end) {
+      int phys = min(max(table[ap % ring_pages], 0), n_pages - 1);
+      const bf16* kp = k_pages + phys * page_elems + (size_t)g * PAGE * HD;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kreg[t][ks] = ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
+    }
+    for (; ap < p_end; ap += 4) {
+      int phys = min(max(table[ap % ring_pages], 0), n_pages - 1);
+      const bf16* vp = v_pages + phys * page_elems + (size_t)g * PAGE * HD;
+      bf16x8 vreg[DT][2];
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) vreg[dt][s] = ld8(vp + (dt * 16 + j) * PAGE + s * 32 + qd * 8);
+
+      f32x4 sc[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        sc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[t][ks], qv[ks], sc[t], 0, 0, 0);
+      }
+      const int apn = ap + 4;
+      if (apn < p_end) {                         // the keys of the wave's next page, while this one is mixed
+        int physn = min(max(table[apn % ring_pages], 0), n_pages - 1);
+        const bf16* kp = k_pages + physn * page_elems + (size_t)g * PAGE * HD;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) kreg[t][ks] = ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
+      }
+
+      const int base = ap * PAGE;
+      const bool edge = base < lo || base + PAGE > L;
+      float mx = -FLT_MAX;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = sc[t][r] / root;
+          if (edge) {
+            int pos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
+            if (pos < lo || pos >= L) v = -INFINITY;
+          }
+          sc[t][r] = v;
+          mx = fmaxf(mx, v);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+      const float m_new = fmaxf(m, mx);
+      const float corr = expf(m - m_new);
+      float psum = 0.f;
+      bf16x8 pb[2];
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          float p = expf(sc[2 * s + (e >> 2)][e & 3] - m_new);
+          psum += p;
+          pb[s][e] = static_cast<bf16>(p);
+        }
+      l = l * corr + psum;
+      m = m_new;
+      if (base + PAGE > L) {                     // rows behind the length may hold anything: 0 * NaN must not happen
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (base + 32 * s + 8 * qd + e >= L) {
+#pragma unroll
+              for (int dt = 0; dt < DT; ++dt) vreg[dt][s][e] = static_cast<bf16>(0.f);
+            }
+      }
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        o[dt] *= corr;
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+          o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt][s], pb[s], o[dt], 0, 0, 0);
+      }
+    }
+  }
+
+  // the four lanes of a column hold parts of its sum; then the four waves merge
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  if (qd == 0) sm_m[wave][j] = m;
+  __syncthreads();
+  float m_all = fmaxf(fmaxf(sm_m[0][j], sm_m[1][j]), fmaxf(sm_m[2][j], sm_m[3][j]));
+  const float scale = expf(m - m_all);
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) sm_o[wave][dt][lane] = o[dt] * scale;
+  if (qd == 0) sm_l[wave][j] = l * scale;
+  __syncthreads();
+  if (j < G) {
+    float* part = partial + (((size_t)b * n_heads + g * G + j) * n_splits + split) * (HD + 2);
+    for (int dt = wave; dt < DT; dt += 4) {
+      f32x4 v = sm_o[0][dt][lane] + sm_o[1][dt][lane] + sm_o[2][dt][lane] + sm_o[3][dt][lane];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) part[dt * 16 + 4 * qd + r] = v[r];
+    }
+    if (wave == 0 && qd == 0) {
+      part[HD] = m_all;
+      part[HD + 1] = sm_l[0][j] + sm_l[1][j] + sm_l[2][j] + sm_l[3][j];
+    }
+  }
 }
-int yalm_attn_decode_bf16_mfma(const void*, const void*, const void*, const int*, int, int, const int*, const int*,
-                               void*, float*, int, int, int, int, int, int, int, hipStream_t) {
-  return YALM_ERR_ARG;
+
+// ---------------------------------------------------------------------------
+// prefill: grid (tile of 64 query positions, head); a wave takes 16 positions
+// ---------------------------------------------------------------------------
+template <int HD>
+__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
+    const bf16* __restrict__ q, const bf16* __restrict__ k_stage, const bf16* __restrict__ v_stage,
+    bf16* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_tile0, int B, int n_heads,
+    int n_kv_heads, int window) {
+  constexpr int KS = HD / 32, DT = HD / 16;
+  const int gt = blockIdx.x, h = blockIdx.y;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, qd = lane / 16, j = lane % 16;
+  // the sequence of this tile: the last b with seq_tile0[b] <= gt (seq_tile0 has B + 1 entries)
+  int b = 0;
+  {
+    int lo_b = 0, hi_b = B - 1;
+    while (lo_b < hi_b) {
+      int mid = (lo_b + hi_b + 1) >> 1;
+      if (seq_tile0[mid] <= gt) lo_b = mid; else hi_b = mid - 1;
+    }
+    b = lo_b;
+  }
+  const int tile0 = seq_tile0[b];
+  const int tq = gt - tile0;
+  const int start = cu_seqlens[b], len = cu_seqlens[b + 1] - start;
+  const int pos0 = tq * PAGE + wave * 16;
+  if (pos0 >= len) return;                        // no barrier follows: a wave may leave
+  const int g = h / (n_heads / n_kv_heads);
+  const int pos_q = pos0 + j;
+  const bool q_ok = pos_q < len;
+  const float root = sqrtf((float)HD);
+
+  bf16x8 qv[KS];
+  {
+    const bf16* qrow = q + ((size_t)(start + (q_ok ? pos_q : 0)) * n_heads + h) * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qv[ks] = q_ok ? ld8(qrow + ks * 32 + qd * 8) : zero8();
+  }
+  float m = -FLT_MAX, l = 0.f;
+  f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  const int last_q = min(pos0 + 15, len - 1);
+  const int kt_hi = last_q / PAGE;
+  const int kt_lo = window > 0 ? max(0, pos0 - window + 1) / PAGE : 0;
+  const size_t tile_elems = (size_t)n_kv_heads * PAGE * HD;
+
+  bf16x8 kreg[4][KS];
+  {
+    const bf16* kp = k_stage + (tile0 + kt_lo) * tile_elems + (size_t)g * PAGE * HD;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) kreg[t][ks] = ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
+  }
+  for (int kt = kt_lo; kt <= kt_hi; ++kt) {
+    const bf16* vp = v_stage + (tile0 + kt) * tile_elems + (size_t)g * PAGE * HD;
+    bf16x8 vreg[DT][2];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int s = 0; s < 2; ++s) vreg[dt][s] = ld8(vp + (dt * 16 + j) * PAGE + s * 32 + qd * 8);
+
+    f32x4 sc[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      sc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[t][ks], qv[ks], sc[t], 0, 0, 0);
+    }
+    if (kt < kt_hi) {
+      const bf16* kp = k_stage + (tile0 + kt + 1) * tile_elems + (size_t)g * PAGE * HD;
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) kreg[t][ks] = ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
+    }
+
+    const int base = kt * PAGE;
+    const bool edge = base + PAGE - 1 > pos0 || (window > 0 && base < pos0 + 15 - window + 1);
+    float mx = -FLT_MAX;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = sc[t][r] / root;
+        if (edge) {
+          int kpos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
+          bool vis = kpos <= pos_q && (window == 0 || pos_q - kpos < window) && q_ok;
+          if (!vis) v = -INFINITY;
+        }
+        sc[t][r] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(m, mx);
+    const float corr = expf(m - m_new);
+    float psum = 0.f;
+    bf16x8 pb[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float p = expf(sc[2 * s + (e >> 2)][e & 3] - m_new);
+        psum += p;
+        pb[s][e] = static_cast<bf16>(p);
+      }
+    l = l * corr + psum;
+    m = m_new;
+    if (base + PAGE > len) {                      // rows behind the sequence's end may hold anything
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (base + 32 * s + 8 * qd + e >= len) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) vreg[dt][s][e] = static_cast<bf16>(0.f);
+          }
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      o[dt] *= corr;
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt][s], pb[s], o[dt], 0, 0, 0);
+    }
+  }
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  if (q_ok) {
+    bf16* orow = out + ((size_t)(start + pos_q) * n_heads + h) * HD;
+    const float inv_l = 1.0f / l;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) orow[dt * 16 + 4 * qd + r] = static_cast<bf16>(o[dt][r] * inv_l);
+  }
+}
+
+bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
+  return (head_dim == 64 || head_dim == 128) && n_kv_heads > 0 && n_heads % n_kv_heads == 0;
+}
+}  // namespace
+
+int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out,
+                                const int* cu_seqlens, const int* seq_tile0, int T, int B, int n_tiles, int n_heads,
+                                int n_kv_heads, int head_dim, int window, hipStream_t stream) {
+  if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim)) return YALM_ERR_ARG;
+  dim3 grid(n_tiles, n_heads);
+  if (head_dim == 128)
+    attn_prefill_mfma_kernel<128><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,
+                                                            (const bf16*)v_stage, (bf16*)out, cu_seqlens, seq_tile0,
+                                                            B, n_heads, n_kv_heads, window);
+  else
+    attn_prefill_mfma_kernel<64><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,
+                                                           (const bf16*)v_stage, (bf16*)out, cu_seqlens, seq_tile0, B,
+                                                           n_heads, n_kv_heads, window);
+  return launch_status();
+}
+
+int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                               int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
+                               float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
+                               int n_splits, int n_pages, hipStream_t stream) {
+  if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_heads / n_kv_heads > 16) return YALM_ERR_ARG;
+  dim3 grid(n_splits, n_kv_heads, B);
+  if (head_dim == 128)
+    attn_decode_mfma_kernel<128><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages,
+                                                           (const bf16*)v_pages, block_table, table_stride,
+                                                           ring_pages, seq_slot, seq_len, partial, n_heads,
+                                                           n_kv_heads, window, n_splits, n_pages);
+  else
+    attn_decode_mfma_kernel<64><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
+                                                          block_table, table_stride, ring_pages, seq_slot, seq_len,
+                                                          partial, n_heads, n_kv_heads, window, n_splits, n_pages);
+  int rc = launch_status();
+  if (rc != YALM_OK) return rc;
+  return yalm_attn_decode_combine_bf16(partial, out, B, n_heads, head_dim, n_splits, stream);
 }

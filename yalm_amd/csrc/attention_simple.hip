@@ -6,9 +6,9 @@
 #include "common.h"
 #include "yalm_hip.h"
 
-int yalm_attn_prefill_bf16_mfma(const void* q, const void* k, const void* v, void* out, const int* cu_seqlens,
-                                const int* tok_seq, const int* tok_pos, int T, int B, int n_heads, int n_kv_heads,
-                                int head_dim, int window, hipStream_t stream);
+int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out,
+                                const int* cu_seqlens, const int* seq_tile0, int T, int B, int n_tiles, int n_heads,
+                                int n_kv_heads, int head_dim, int window, hipStream_t stream);
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
@@ -23,18 +23,17 @@ constexpr int ACC = MAX_HD / WAVE;
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, T* __restrict__ out,
-    const int* __restrict__ cu_seqlens, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_heads,
+    const T* __restrict__ q, const T* __restrict__ k_stage, const T* __restrict__ v_stage, T* __restrict__ out,
+    const int* __restrict__ seq_tile0, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_heads,
     int n_kv_heads, int hd, int window) {
   __shared__ float qs[MAX_HD];
   __shared__ float ps[WAVE];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int b = tok_seq[t], pos = tok_pos[t];
   const int g = h / (n_heads / n_kv_heads);
-  const int KV = n_kv_heads * hd;
-  const int start = cu_seqlens[b];
   const int lo = window > 0 ? max(0, pos - window + 1) : 0;
   const float inv = sqrtf((float)hd);
+  const size_t tile0 = (size_t)seq_tile0[b];
 
   for (int i = lane; i < hd; i += WAVE) qs[i] = to_f32(q[((size_t)t * n_heads + h) * hd + i]);
   __syncthreads();
@@ -44,12 +43,14 @@ __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
 #pragma unroll
   for (int a = 0; a < ACC; ++a) acc[a] = 0.f;
 
-  for (int j0 = lo; j0 <= pos; j0 += WAVE) {
-    int j = j0 + lane;
-    bool valid = j <= pos;
+  for (int tile = lo / PAGE; tile <= pos / PAGE; ++tile) {
+    const T* kp = k_stage + ((tile0 + tile) * n_kv_heads + g) * PAGE * hd;
+    const T* vp = v_stage + ((tile0 + tile) * n_kv_heads + g) * PAGE * hd;
+    int j = tile * PAGE + lane;
+    bool valid = j >= lo && j <= pos;
     float s = -FLT_MAX;
     if (valid) {
-      const T* kr = k + (size_t)(start + j) * KV + g * hd;
+      const T* kr = kp + (size_t)lane * hd;
       float d = 0.f;
       for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kr[i]), d);
       s = d / inv;
@@ -62,14 +63,16 @@ __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
     __syncthreads();
     ps[lane] = p;
     __syncthreads();
-    int n = min(WAVE, pos - j0 + 1);
 #pragma unroll
     for (int a = 0; a < ACC; ++a) {
       int d = lane + a * WAVE;
       if (d < hd) {
+        const T* vr = vp + (size_t)d * PAGE;
         float s2 = 0.f;
-        const T* vc = v + (size_t)(start + j0) * KV + g * hd + d;
-        for (int jj = 0; jj < n; ++jj) s2 = fmaf(ps[jj], to_f32(vc[(size_t)jj * KV]), s2);
+        for (int jj = 0; jj < PAGE; ++jj) {
+          float pj = ps[jj];
+          if (pj != 0.f) s2 = fmaf(pj, to_f32(vr[jj]), s2);     // rows outside the mask may hold anything
+        }
         acc[a] = acc[a] * corr + s2;
       }
     }
@@ -188,27 +191,37 @@ bool bad_heads(int n_heads, int n_kv_heads, int hd) {
 }
 }  // namespace
 
-extern "C" int yalm_attn_prefill(const void* q, const void* k, const void* v, void* out, const int* cu_seqlens,
-                                 const int* tok_seq, const int* tok_pos, int T, int B, int n_heads, int n_kv_heads,
-                                 int head_dim, int window, int dtype, int force_simple, hipStream_t stream) {
+extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void* v_stage, void* out,
+                                 const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
+                                 int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
+                                 int dtype, int force_simple, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
-  if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0) return YALM_ERR_ARG;
+  if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_tiles <= 0) return YALM_ERR_ARG;
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32) {
-    attn_prefill_simple_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)q, (const float*)k, (const float*)v,
-                                                                 (float*)out, cu_seqlens, tok_seq, tok_pos, n_heads,
-                                                                 n_kv_heads, head_dim, window);
+    attn_prefill_simple_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)q, (const float*)k_stage,
+                                                                 (const float*)v_stage, (float*)out, seq_tile0,
+                                                                 tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
+                                                                 window);
     return launch_status();
   }
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
   if (!force_simple) {
-    int rc = yalm_attn_prefill_bf16_mfma(q, k, v, out, cu_seqlens, tok_seq, tok_pos, T, B, n_heads, n_kv_heads,
-                                         head_dim, window, stream);
+    int rc = yalm_attn_prefill_bf16_mfma(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, T, B, n_tiles, n_heads,
+                                         n_kv_heads, head_dim, window, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
-  attn_prefill_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)q, (const bf16*)k, (const bf16*)v,
-                                                              (bf16*)out, cu_seqlens, tok_seq, tok_pos, n_heads,
-                                                              n_kv_heads, head_dim, window);
+  attn_prefill_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,
+                                                              (const bf16*)v_stage, (bf16*)out, seq_tile0, tok_seq,
+                                                              tok_pos, n_heads, n_kv_heads, head_dim, window);
+  return launch_status();
+}
+
+// merges the partial results of the splits (also used by the MFMA kernel)
+int yalm_attn_decode_combine_bf16(const float* partial, void* out, int B, int n_heads, int head_dim, int n_splits,
+                                  hipStream_t stream) {
+  dim3 cgrid(B, n_heads);
+  attn_decode_combine_kernel<bf16><<<cgrid, WAVE, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
   return launch_status();
 }
 

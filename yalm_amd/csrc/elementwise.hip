@@ -84,8 +84,9 @@ extern "C" int yalm_rmsnorm(const float* x, const void* w, int w_dtype, void* ou
 // grid (T, n_heads + 2 n_kv_heads); one wave per (token, head); a lane per pair
 // ---------------------------------------------------------------------------
 template <typename T>
-__global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_out,
-                                     T* __restrict__ v_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
+__global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_stage,
+                                     T* __restrict__ v_stage, const int* __restrict__ seq_tile0,
+                                     T* __restrict__ k_pages, T* __restrict__ v_pages,
                                      const int* __restrict__ block_table, int table_stride, int ring_pages,
                                      const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                      const int* __restrict__ seq_slot, const int* __restrict__ seq_len,
@@ -138,9 +139,17 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
     }
   }
 
+  // the step's own keys and values, in page format, for attention over the step's tokens
+  T* kst = nullptr;
+  T* vst = nullptr;
+  if (k_stage != nullptr && b >= 0 && pos >= 0) {
+    size_t tile = (size_t)seq_tile0[b] + pos / PAGE;
+    kst = k_stage + (tile * n_kv_heads + g) * PAGE * hd;
+    vst = v_stage + (tile * n_kv_heads + g) * PAGE * hd;
+  }
+
   if (is_k) {
     const float* src = row + Q + g * hd;
-    T* dst = k_out ? k_out + (size_t)t * KV + g * hd : nullptr;
     for (int p = threadIdx.x; p < hd / 2; p += WAVE) {
       float x0 = src[2 * p], x1 = src[2 * p + 1];
       if (rotate && p < half_rot) {
@@ -151,9 +160,9 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
         x1 = y1;
       }
       T a = from_f32<T>(x0), bb = from_f32<T>(x1);
-      if (dst) {
-        dst[2 * p] = a;
-        dst[2 * p + 1] = bb;
+      if (kst) {
+        kst[r * hd + 2 * p] = a;
+        kst[r * hd + 2 * p + 1] = bb;
       }
       if (kpage) {
         kpage[r * hd + 2 * p] = a;
@@ -162,17 +171,16 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
     }
   } else {
     const float* src = row + Q + KV + g * hd;
-    T* dst = v_out ? v_out + (size_t)t * KV + g * hd : nullptr;
     for (int i = threadIdx.x; i < hd; i += WAVE) {
       T a = from_f32<T>(src[i]);
-      if (dst) dst[i] = a;
+      if (vst) vst[(size_t)i * PAGE + r] = a;
       if (vpage) vpage[(size_t)i * PAGE + r] = a;      // values are kept transposed inside a page
     }
   }
 }
 
-extern "C" int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_out, void* v_out, void* k_pages,
-                                  void* v_pages, const int* block_table, int table_stride, int ring_pages,
+extern "C" int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_stage, void* v_stage,
+                                  const int* seq_tile0, void* k_pages, void* v_pages, const int* block_table, int table_stride, int ring_pages,
                                   const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_len,
                                   const float* cos_sin, int n_positions, int T, int n_heads, int n_kv_heads,
                                   int head_dim, int rotary_dim, int n_pages, int dtype, hipStream_t stream) {
@@ -183,12 +191,12 @@ extern "C" int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_out, vo
   dim3 grid(T, n_heads + 2 * n_kv_heads);
   if (dtype == YALM_F32)
     rope_kv_write_kernel<float><<<grid, WAVE, 0, stream>>>(
-        qkv, (float*)q_out, (float*)k_out, (float*)v_out, (float*)k_pages, (float*)v_pages, block_table,
+        qkv, (float*)q_out, (float*)k_stage, (float*)v_stage, seq_tile0, (float*)k_pages, (float*)v_pages, block_table,
         table_stride, ring_pages, tok_seq, tok_pos, seq_slot, seq_len, (const float2*)cos_sin, n_positions, n_heads,
         n_kv_heads, head_dim, rotary_dim, n_pages);
   else if (dtype == YALM_BF16)
     rope_kv_write_kernel<bf16><<<grid, WAVE, 0, stream>>>(
-        qkv, (bf16*)q_out, (bf16*)k_out, (bf16*)v_out, (bf16*)k_pages, (bf16*)v_pages, block_table, table_stride,
+        qkv, (bf16*)q_out, (bf16*)k_stage, (bf16*)v_stage, seq_tile0, (bf16*)k_pages, (bf16*)v_pages, block_table, table_stride,
         ring_pages, tok_seq, tok_pos, seq_slot, seq_len, (const float2*)cos_sin, n_positions, n_heads, n_kv_heads,
         head_dim, rotary_dim, n_pages);
   else

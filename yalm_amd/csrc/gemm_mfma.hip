@@ -1,6 +1,338 @@
-// bfloat16 GEMMs on the matrix cores (placeholder until the MFMA kernels land:
-// it refuses every shape, so the float32-arithmetic kernel runs instead).
+// bfloat16 GEMMs on the matrix cores: C = A[M,K] * W[N,K]^T, float32 accumulation.
+//
+//  * gemm_skinny  (M <= 64, decode): bound by the one pass over the weights.  A
+//    workgroup owns 16 or 32 weight rows and all of K; its waves split K in
+//    chunks of 128, every lane streaming 64 contiguous bytes of a weight row per
+//    chunk; the batch is the other MFMA operand (16 rows a tile, up to 4 tiles);
+//    partial sums of the waves meet in LDS, then the epilogue runs once.
+//  * gemm_tiled   (M > 64, prefill): 128x128x64 tiles through LDS with a register
+//    prefetch of the next tile, 4 waves of 64x64, v_mfma_f32_32x32x16_bf16.
+//
+// Both take any M and N and any K that is a multiple of 8 (rows must be 16-byte
+// aligned); other shapes are refused so that the caller runs the float32-arithmetic kernel.
 #include "common.h"
 #include "yalm_hip.h"
 
-int yalm_gemm_bf16_mfma(const void*, const void*, void*, int, int, int, int, int, hipStream_t) { return YALM_ERR_ARG; }
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+__device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
+  bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+  return ok ? *reinterpret_cast<const bf16x8*>(p) : z;
+}
+
+// ---------------------------------------------------------------------------
+// skinny GEMM
+// ---------------------------------------------------------------------------
+// MFMA 16x16x32: operand A = activations (row i = batch row, 8 k per lane), operand
+// B = weights (column j = weight row, 8 k per lane); C[i][j]: lane (q = lane/16,
+// j = lane%16) holds batch rows 4q..4q+3 of weight row j.  Which k a lane's slot
+// holds is the same for both operands, so any assignment of k to slots is right;
+// here lane group q takes the 32 consecutive k  [kc + 32q, kc + 32q + 32).
+template <int MT, int NT, int NWAVES, int EPI>
+__global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ X,
+                                                                     const bf16* __restrict__ W,
+                                                                     void* __restrict__ Cv, int M, int N, int K,
+                                                                     int H) {
+  constexpr int KC = 128;                        // k per wave iteration
+  __shared__ f32x4 red[NWAVES][MT * NT][WAVE];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int q = lane / 16, j = lane % 16;
+  const int n0 = blockIdx.x * 16 * NT;
+
+  const bf16* wrow[NT];
+  bool wok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    int n = n0 + t * 16 + j;
+    wok[t] = n < N;
+    wrow[t] = W + (size_t)(wok[t] ? n : 0) * K;
+  }
+  const bf16* xrow[MT];
+  bool xok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int m = mt * 16 + j;
+    xok[mt] = m < M;
+    xrow[mt] = X + (size_t)(xok[mt] ? m : 0) * K;
+  }
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[mt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  bf16x8 wv[NT][4], xv[MT][4];
+  int kc = wave * KC;
+  if (kc < K) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      int k = kc + s * 32 + q * 8;
+      bool ok = k < K;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) wv[t][s] = load8(wrow[t] + k, ok && wok[t]);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) xv[mt][s] = load8(xrow[mt] + k, ok && xok[mt]);
+    }
+  }
+  for (; kc < K; kc += NWAVES * KC) {
+    bf16x8 wn[NT][4], xn[MT][4];
+    int kn = kc + NWAVES * KC;
+    if (kn < K) {                                // prefetch the wave's next chunk
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        int k = kn + s * 32 + q * 8;
+        bool ok = k < K;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) wn[t][s] = load8(wrow[t] + k, ok && wok[t]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xn[mt][s] = load8(xrow[mt] + k, ok && xok[mt]);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
+    if (kn < K) {
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) wv[t][s] = wn[t][s];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xv[mt][s] = xn[mt][s];
+      }
+    }
+  }
+
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) red[wave][mt * NT + t][lane] = acc[mt][t];
+  __syncthreads();
+
+  constexpr int NTP = (EPI == 3) ? NT / 2 : NT;  // gated: a gate tile and its up tile finish together
+  for (int idx = wave; idx < MT * NTP; idx += NWAVES) {
+    const int mt = idx / NTP, tp = idx % NTP;
+    if (EPI == 3) {
+      f32x4 g = (f32x4){0.f, 0.f, 0.f, 0.f}, u = g;
+#pragma unroll
+      for (int w = 0; w < NWAVES; ++w) {
+        g += red[w][mt * NT + 2 * tp][lane];
+        u += red[w][mt * NT + 2 * tp + 1][lane];
+      }
+      int hcol = (n0 / 32 + tp) * 16 + j;
+      bf16* C = (bf16*)Cv;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        int m = mt * 16 + 4 * q + r;
+        if (m < M && hcol < H) C[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(g[r]) * u[r]);
+      }
+    } else {
+      f32x4 v = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int w = 0; w < NWAVES; ++w) v += red[w][mt * NT + tp][lane];
+      int n = n0 + tp * 16 + j;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        int m = mt * 16 + 4 * q + r;
+        if (m < M && n < N) {
+          size_t o = (size_t)m * N + n;
+          if (EPI == 0) ((float*)Cv)[o] = v[r];
+          if (EPI == 1) ((bf16*)Cv)[o] = static_cast<bf16>(v[r]);
+          if (EPI == 2) ((float*)Cv)[o] += v[r];
+        }
+      }
+    }
+  }
+}
+
+template <int MT, int EPI>
+int skinny_launch(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
+  // few weight rows: 16 rows and 8 waves a workgroup, so that every CU has work; many: 32 rows, 4 waves
+  bool wide = EPI == 3 || N >= 16384;
+  if (wide)
+    gemm_skinny_kernel<MT, 2, 4, EPI><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H);
+  else
+    gemm_skinny_kernel<MT, 1, 8, (EPI == 3 ? 0 : EPI)><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H);
+  return launch_status();
+}
+
+template <int EPI>
+int skinny_dispatch(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
+  switch ((M + 15) / 16) {
+    case 1: return skinny_launch<1, EPI>(X, W, C, M, N, K, H, stream);
+    case 2: return skinny_launch<2, EPI>(X, W, C, M, N, K, H, stream);
+    case 3: return skinny_launch<3, EPI>(X, W, C, M, N, K, H, stream);
+    case 4: return skinny_launch<4, EPI>(X, W, C, M, N, K, H, stream);
+  }
+  return YALM_ERR_ARG;
+}
+
+// ---------------------------------------------------------------------------
+// tiled GEMM
+// ---------------------------------------------------------------------------
+constexpr int TM = 128, TN = 128, TK = 64;
+constexpr int LDS_ROW = TK + 8;                  // bf16 elements; 16 bytes of padding keep b128 reads off each other's banks
+
+// MFMA 32x32x16: operand rows i/j = lane % 32, 8 k per lane at k offset 8 * (lane / 32);
+// C: lane holds column j = lane % 32 and rows 8 * (r / 4) + 4 * (lane / 32) + r % 4 for r < 16.
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                         void* __restrict__ Cv, int M, int N, int K, int H) {
+  __shared__ __attribute__((aligned(16))) bf16 As[2][TM * LDS_ROW];
+  __shared__ __attribute__((aligned(16))) bf16 Ws[2][TN * LDS_ROW];
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int wm = wave / 2, wn = wave % 2;       // the wave's 64x64 quadrant
+  const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+  const int li = lane % 32, lh = lane / 32;
+
+  // global -> LDS: thread t carries 16 bytes of row (t / 8) + 32 p, p < 4, at k offset 8 * (t % 8)
+  const int lrow = tid / 8, lk = (tid % 8) * 8;
+  const bf16* ap[4];
+  const bf16* wp[4];
+  bool aok[4], wok[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    int m = m0 + lrow + 32 * p, n = n0 + lrow + 32 * p;
+    aok[p] = m < M;
+    wok[p] = n < N;
+    ap[p] = A + (size_t)(aok[p] ? m : 0) * K + lk;
+    wp[p] = W + (size_t)(wok[p] ? n : 0) * K + lk;
+  }
+
+  f32x16 acc[2][2];
+#pragma unroll
+  for (int a = 0; a < 2; ++a)
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  // rows of the W tile that feed the wave's two column tiles: plain, or for the gated
+  // epilogue tile 0 = the gate rows and tile 1 = the up rows of the wave's two blocks
+  int wrow_lds[2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b) {
+    if (EPI == 3)
+      wrow_lds[b] = wn * 64 + (li / 16) * 32 + b * 16 + (li % 16);
+    else
+      wrow_lds[b] = wn * 64 + b * 32 + li;
+  }
+
+  bf16x8 ra[4], rw[4];
+  const int nk = (K + TK - 1) / TK;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    bool kok = lk < K;
+    ra[p] = load8(ap[p], aok[p] && kok);
+    rw[p] = load8(wp[p], wok[p] && kok);
+  }
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    *reinterpret_cast<bf16x8*>(&As[0][(lrow + 32 * p) * LDS_ROW + lk]) = ra[p];
+    *reinterpret_cast<bf16x8*>(&Ws[0][(lrow + 32 * p) * LDS_ROW + lk]) = rw[p];
+  }
+  __syncthreads();
+
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) {
+      int k = (kt + 1) * TK + lk;
+      bool kok = k < K;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        ra[p] = load8(ap[p] + (size_t)(kt + 1) * TK, aok[p] && kok);
+        rw[p] = load8(wp[p] + (size_t)(kt + 1) * TK, wok[p] && kok);
+      }
+    }
+#pragma unroll
+    for (int ks = 0; ks < TK / 16; ++ks) {
+      bf16x8 fa[2], fw[2];
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+        fa[a] = *reinterpret_cast<const bf16x8*>(&As[cur][(wm * 64 + a * 32 + li) * LDS_ROW + ks * 16 + lh * 8]);
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+        fw[b] = *reinterpret_cast<const bf16x8*>(&Ws[cur][wrow_lds[b] * LDS_ROW + ks * 16 + lh * 8]);
+#pragma unroll
+      for (int a = 0; a < 2; ++a)
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fw[b], acc[a][b], 0, 0, 0);
+    }
+    if (kt + 1 < nk) {
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        *reinterpret_cast<bf16x8*>(&As[cur ^ 1][(lrow + 32 * p) * LDS_ROW + lk]) = ra[p];
+        *reinterpret_cast<bf16x8*>(&Ws[cur ^ 1][(lrow + 32 * p) * LDS_ROW + lk]) = rw[p];
+      }
+    }
+    __syncthreads();
+  }
+
+  // epilogue
+#pragma unroll
+  for (int a = 0; a < 2; ++a) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      int m = m0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+      if (m >= M) continue;
+      if (EPI == 3) {
+        int hcol = (n0 + wn * 64) / 2 + li;
+        if (hcol < H)
+          ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(acc[a][0][r]) * acc[a][1][r]);
+      } else {
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          int n = n0 + wn * 64 + b * 32 + li;
+          if (n >= N) continue;
+          size_t o = (size_t)m * N + n;
+          if (EPI == 0) ((float*)Cv)[o] = acc[a][b][r];
+          if (EPI == 1) ((bf16*)Cv)[o] = static_cast<bf16>(acc[a][b][r]);
+          if (EPI == 2) ((float*)Cv)[o] += acc[a][b][r];
+        }
+      }
+    }
+  }
+}
+
+template <int EPI>
+int tiled_launch(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
+  dim3 grid(ceil_div(N, TN), ceil_div(M, TM));
+  gemm_tiled_kernel<EPI><<<grid, 256, 0, stream>>>(A, W, C, M, N, K, H);
+  return launch_status();
+}
+
+}  // namespace
+
+int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, int M, int N, int K, int epilogue, int H,
+                        hipStream_t stream) {
+  if (K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  if (M <= 64) {
+    switch (epilogue) {
+      case 0: return skinny_dispatch<0>(a, w, C, M, N, K, H, stream);
+      case 1: return skinny_dispatch<1>(a, w, C, M, N, K, H, stream);
+      case 2: return skinny_dispatch<2>(a, w, C, M, N, K, H, stream);
+      case 3: return skinny_dispatch<3>(a, w, C, M, N, K, H, stream);
+    }
+    return YALM_ERR_ARG;
+  }
+  switch (epilogue) {
+    case 0: return tiled_launch<0>(a, w, C, M, N, K, H, stream);
+    case 1: return tiled_launch<1>(a, w, C, M, N, K, H, stream);
+    case 2: return tiled_launch<2>(a, w, C, M, N, K, H, stream);
+    case 3: return tiled_launch<3>(a, w, C, M, N, K, H, stream);
+  }
+  return YALM_ERR_ARG;
+}

@@ -36,27 +36,31 @@ int yalm_gemm(const void* A, const void* W, void* C, int M, int N, int K, int dt
               int force_simple, hipStream_t stream);
 
 // Rotates q and k of every token (adjacent pairs, angles from the table), writes q,
-// optionally k and v token-major (for attention over the step's own tokens), and
-// k and v into the pages of the cache.
+// optionally k and v into a staging area in page format (for attention over the step's
+// own tokens: tile seq_tile0[sequence] + position / PAGE), and k and v into the pages
+// of the cache.
+//   k_stage [n_tiles, n_kv_heads, PAGE, head_dim], v_stage [n_tiles, n_kv_heads, head_dim, PAGE] or null
 //   qkv      float32 [T, (n_heads + 2 n_kv_heads) * head_dim]
 //   cos_sin  float32 [n_positions, rotary_dim/2, 2] or null (no rotation)
 //   k_pages  [n_pages, n_kv_heads, PAGE, head_dim], v_pages [n_pages, n_kv_heads, head_dim, PAGE]
 //   block_table int32 [n_slots, table_stride]; page of position p: table[slot][(p / PAGE) % ring_pages]
 //   a token is written iff its page is among the last ring_pages pages of its sequence
 // reference: fused_rope_and_cache_update (src/infer.cu:660-705)
-int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_out, void* v_out, void* k_pages, void* v_pages,
-                       const int* block_table, int table_stride, int ring_pages, const int* tok_seq,
+int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_stage, void* v_stage, const int* seq_tile0,
+                       void* k_pages, void* v_pages, const int* block_table, int table_stride, int ring_pages, const int* tok_seq,
                        const int* tok_pos, const int* seq_slot, const int* seq_len, const float* cos_sin,
                        int n_positions, int T, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
                        int n_pages, int dtype, hipStream_t stream);
 
 // Causal attention of a step's tokens over the same step's keys (sequences that
 // start at position 0), packed without padding.  window 0 = all keys.
-//   q [T, n_heads, hd], k, v [T, n_kv_heads, hd], out [T, n_heads, hd], all `dtype`
+//   q, out [T, n_heads, hd]; k_stage, v_stage: the staging area rope_kv_write filled
+//   (key j of sequence b: tile seq_tile0[b] + j / PAGE, row j % PAGE), all `dtype`
 // reference: attn_dot + attn_softmax + att_mix (src/infer.cu:339-523) for every position
-int yalm_attn_prefill(const void* q, const void* k, const void* v, void* out, const int* cu_seqlens,
-                      const int* tok_seq, const int* tok_pos, int T, int B, int n_heads, int n_kv_heads, int head_dim,
-                      int window, int dtype, int force_simple, hipStream_t stream);
+int yalm_attn_prefill(const void* q, const void* k_stage, const void* v_stage, void* out, const int* cu_seqlens,
+                      const int* seq_tile0, const int* tok_seq, const int* tok_pos, int T, int B, int n_tiles,
+                      int n_heads, int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
+                      hipStream_t stream);
 
 // One query per sequence over the pages of the cache (the new key is already written).
 //   q, out [B, n_heads, hd]; seq_len[b] = keys of sequence b including the new one;

@@ -33,7 +33,8 @@ class StepContext:
     """mode: 'prefill' (sequences that start at position 0, whole prompts, packed)
     or 'decode' (one token per sequence).  Device tensors, all int32:
       tokens[T], tok_seq[T] (row of the batch), tok_pos[T] (position in its sequence),
-      seq_slot[B] (-1: padding row), seq_len[B] (length after this step), cu_seqlens[B+1].
+      seq_slot[B] (-1: padding row), seq_len[B] (length after this step), cu_seqlens[B+1],
+      seq_tile0[B+1] (prefill: first 64-token tile of each sequence in the staging area; n_tiles in all).
     max_position: the largest position in the step (host value, for table checks)."""
 
     def __init__(self, mode, cache, ws, act_dtype, shared_lines=()):
@@ -43,6 +44,8 @@ class StepContext:
         self.act_dtype = act_dtype
         self.shared_lines = set(shared_lines)
         self.tokens = self.tok_seq = self.tok_pos = self.seq_slot = self.seq_len = self.cu_seqlens = None
+        self.seq_tile0 = None
+        self.n_tiles = 0
         self.max_position = 0
         self.host_slots = []
         self.host_n_tokens = []

@@ -108,20 +108,24 @@ def _check_heads(n_heads, n_kv_heads, head_dim):
         raise ValueError("head_dim %d is not supported (even, at most %d)" % (head_dim, MAX_HEAD_DIM))
 
 
-def rope_kv_write(qkv, q_out, k_out, v_out, k_pages, v_pages, block_table, ring_pages, tok_seq, tok_pos, seq_slot,
-                  seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim):
-    """Rotates q and k by the angles of `cos_sin` at each token's position, writes q
-    (and k, v token-major if k_out is given) in q_out's dtype and k, v into the pages."""
+def rope_kv_write(qkv, q_out, k_stage, v_stage, seq_tile0, k_pages, v_pages, block_table, ring_pages, tok_seq, tok_pos,
+                  seq_slot, seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim):
+    """Rotates q and k by the angles of `cos_sin` at each token's position, writes q in
+    q_out's dtype, k and v into the staging area (page format, tile seq_tile0[sequence] +
+    position // PAGE) if one is given, and into the pages of the cache if given."""
     _check_heads(n_heads, n_kv_heads, head_dim)
     T = qkv.shape[0]
     Q, KV = n_heads * head_dim, n_kv_heads * head_dim
     dt = q_out.dtype
     p_qkv = _need(qkv, "qkv", torch.float32, (T, Q + 2 * KV))
     p_q = _need(q_out, "q_out", dt, (T, Q))
-    p_k = _opt(k_out, "k_out", dt, (T, KV))
-    p_v = _opt(v_out, "v_out", dt, (T, KV))
-    if (k_out is None) != (v_out is None):
-        raise ValueError("k_out and v_out go together")
+    B = seq_slot.shape[0]
+    p_ks = p_vs = p_t0 = None
+    if k_stage is not None:
+        n_tiles = k_stage.shape[0]
+        p_ks = _need(k_stage, "k_stage", dt, (n_tiles, n_kv_heads, PAGE, head_dim))
+        p_vs = _need(v_stage, "v_stage", dt, (n_tiles, n_kv_heads, head_dim, PAGE))
+        p_t0 = _need(seq_tile0, "seq_tile0", torch.int32, (B + 1,))
     n_pages = 0
     p_kp = p_vp = p_bt = None
     stride = 0
@@ -133,7 +137,6 @@ def rope_kv_write(qkv, q_out, k_out, v_out, k_pages, v_pages, block_table, ring_
         stride = block_table.shape[1]
         if ring_pages <= 0 or ring_pages > stride:
             raise ValueError("ring_pages %d does not fit the block table (%d columns)" % (ring_pages, stride))
-    B = seq_slot.shape[0]
     p_ts = _need(tok_seq, "tok_seq", torch.int32, (T,))
     p_tp = _need(tok_pos, "tok_pos", torch.int32, (T,))
     p_ss = _need(seq_slot, "seq_slot", torch.int32, (B,))
@@ -148,26 +151,30 @@ def rope_kv_write(qkv, q_out, k_out, v_out, k_pages, v_pages, block_table, ring_
     else:
         rotary_dim = 0
     library.check(library.lib().yalm_rope_kv_write(
-        p_qkv, p_q, p_k, p_v, p_kp, p_vp, p_bt, stride, max(ring_pages, 1), p_ts, p_tp, p_ss, p_sl, p_cs, n_pos, T,
-        n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, dtype_code(dt), _stream()), "rope_kv_write")
+        p_qkv, p_q, p_ks, p_vs, p_t0, p_kp, p_vp, p_bt, stride, max(ring_pages, 1), p_ts, p_tp, p_ss, p_sl, p_cs,
+        n_pos, T, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, dtype_code(dt), _stream()), "rope_kv_write")
 
 
-def attn_prefill(q, k, v, out, cu_seqlens, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim, window):
-    """Causal (and windowed) attention of packed sequences that start at position 0."""
+def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
+                 window):
+    """Causal (and windowed) attention of packed sequences that start at position 0, over
+    the keys and values that rope_kv_write staged for this step."""
     _check_heads(n_heads, n_kv_heads, head_dim)
     T = q.shape[0]
     dt = q.dtype
     B = cu_seqlens.shape[0] - 1
+    n_tiles = k_stage.shape[0]
     p_q = _need(q, "q", dt, (T, n_heads * head_dim))
-    p_k = _need(k, "k", dt, (T, n_kv_heads * head_dim))
-    p_v = _need(v, "v", dt, (T, n_kv_heads * head_dim))
+    p_k = _need(k_stage, "k_stage", dt, (n_tiles, n_kv_heads, PAGE, head_dim))
+    p_v = _need(v_stage, "v_stage", dt, (n_tiles, n_kv_heads, head_dim, PAGE))
     p_o = _need(out, "out", dt, (T, n_heads * head_dim))
     p_cu = _need(cu_seqlens, "cu_seqlens", torch.int32, (B + 1,))
+    p_t0 = _need(seq_tile0, "seq_tile0", torch.int32, (B + 1,))
     p_ts = _need(tok_seq, "tok_seq", torch.int32, (T,))
     p_tp = _need(tok_pos, "tok_pos", torch.int32, (T,))
-    library.check(library.lib().yalm_attn_prefill(p_q, p_k, p_v, p_o, p_cu, p_ts, p_tp, T, B, n_heads, n_kv_heads,
-                                                  head_dim, int(window), dtype_code(dt), 1 if FORCE_SIMPLE else 0,
-                                                  _stream()), "attn_prefill")
+    library.check(library.lib().yalm_attn_prefill(p_q, p_k, p_v, p_o, p_cu, p_t0, p_ts, p_tp, T, B, n_tiles, n_heads,
+                                                  n_kv_heads, head_dim, int(window), dtype_code(dt),
+                                                  1 if FORCE_SIMPLE else 0, _stream()), "attn_prefill")
     return out
 
 

@@ -65,6 +65,10 @@ class GQAttention(Part):
         return KVRequest(self.n_kv_heads, self.head_dim, self.window)
 
     def decode_splits(self, B, ring_pages):
+        mfma = self.head_dim in (64, 128) and self.n_heads // self.n_kv_heads <= 16 and not kernels.FORCE_SIMPLE
+        if mfma:         # a workgroup of 4 waves per (split, KV head, sequence), a page per wave at a time
+            per = max(1, B * self.n_kv_heads)
+            return max(1, min((ring_pages + 3) // 4, TARGET_WORKGROUPS // per))
         return max(1, min(ring_pages, TARGET_WORKGROUPS // max(1, B * self.n_heads)))
 
     def forward(self, h, x, ctx, line, writes_cache=True):
@@ -82,24 +86,25 @@ class GQAttention(Part):
         k_pages, v_pages = group.line_pages(line)
         prefill = ctx.mode == "prefill"
         if prefill:
-            # a line that later entries read keeps its token-major keys and values for them
-            tag = "attn.kv%d" % line if ctx.line_is_shared(line) else "attn.kv"
-            k = ws.get(tag + ".k", (T, self.kv_dim), act)
-            v = ws.get(tag + ".v", (T, self.kv_dim), act)
+            # the step's own keys and values in page format; a line that later entries read
+            # keeps them for those entries
+            tag = "attn.stage%d" % line if ctx.line_is_shared(line) else "attn.stage"
+            kst = ws.get(tag + ".k", (ctx.n_tiles, self.n_kv_heads, kernels.PAGE, self.head_dim), act)
+            vst = ws.get(tag + ".v", (ctx.n_tiles, self.n_kv_heads, self.head_dim, kernels.PAGE), act)
         else:
-            k = v = None
+            kst = vst = None
         if writes_cache:
-            kernels.rope_kv_write(qkv, q, k, v, k_pages, v_pages, group.table, group.ring_pages, ctx.tok_seq,
-                                  ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads,
-                                  self.head_dim, pos.rotary_dim)
+            kernels.rope_kv_write(qkv, q, kst, vst, ctx.seq_tile0, k_pages, v_pages, group.table, group.ring_pages,
+                                  ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads,
+                                  self.n_kv_heads, self.head_dim, pos.rotary_dim)
         else:
-            kernels.rope_kv_write(qkv, q, None, None, None, None, None, 0, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot,
-                                  ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads, self.head_dim,
+            kernels.rope_kv_write(qkv, q, None, None, None, None, None, None, 0, ctx.tok_seq, ctx.tok_pos,
+                                  ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads, self.head_dim,
                                   pos.rotary_dim)
         o = ws.get("attn.o", (T, self.q_dim), act)
         if prefill:
-            kernels.attn_prefill(q, k, v, o, ctx.cu_seqlens, ctx.tok_seq, ctx.tok_pos, self.n_heads, self.n_kv_heads,
-                                 self.head_dim, self.window)
+            kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, ctx.seq_tile0, ctx.tok_seq, ctx.tok_pos,
+                                 self.n_heads, self.n_kv_heads, self.head_dim, self.window)
         else:
             n_splits = self.decode_splits(T, group.ring_pages)
             partial = ws.get("attn.partial",
