@@ -38,8 +38,8 @@ template <int HD>
 __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
-    const int* __restrict__ seq_len, float* __restrict__ partial, int n_heads, int n_kv_heads, int window,
-    int n_splits, int n_pages) {
+    const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out,
+    int n_heads, int n_kv_heads, int window, int n_splits, int n_pages) {
   constexpr int KS = HD / 32, DT = HD / 16;
   __shared__ float sm_m[4][16];
   __shared__ float sm_l[4][16];
@@ -173,6 +173,19 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   for (int dt = 0; dt < DT; ++dt) sm_o[wave][dt][lane] = o[dt] * scale;
   if (qd == 0) sm_l[wave][j] = l * scale;
   __syncthreads();
+  if (n_splits == 1) {                            // nothing to merge with: this is the result
+    if (j < G) {
+      bf16* orow = out + ((size_t)b * n_heads + g * G + j) * HD;
+      const float lt = sm_l[0][j] + sm_l[1][j] + sm_l[2][j] + sm_l[3][j];
+      const float inv_l = lt > 0.f ? 1.0f / lt : 0.f;
+      for (int dt = wave; dt < DT; dt += 4) {
+        f32x4 v = sm_o[0][dt][lane] + sm_o[1][dt][lane] + sm_o[2][dt][lane] + sm_o[3][dt][lane];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) orow[dt * 16 + 4 * qd + r] = static_cast<bf16>(v[r] * inv_l);
+      }
+    }
+    return;
+  }
   if (j < G) {
     float* part = partial + (((size_t)b * n_heads + g * G + j) * n_splits + split) * (HD + 2);
     for (int dt = wave; dt < DT; dt += 4) {
@@ -358,13 +371,15 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
   if (head_dim == 128)
     attn_decode_mfma_kernel<128><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages,
                                                            (const bf16*)v_pages, block_table, table_stride,
-                                                           ring_pages, seq_slot, seq_len, partial, n_heads,
-                                                           n_kv_heads, window, n_splits, n_pages);
+                                                           ring_pages, seq_slot, seq_len, partial,
+                                                           (bf16*)out, n_heads, n_kv_heads, window, n_splits,
+                                                           n_pages);
   else
     attn_decode_mfma_kernel<64><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
                                                           block_table, table_stride, ring_pages, seq_slot, seq_len,
-                                                          partial, n_heads, n_kv_heads, window, n_splits, n_pages);
+                                                          partial, (bf16*)out, n_heads, n_kv_heads, window,
+                                                          n_splits, n_pages);
   int rc = launch_status();
-  if (rc != YALM_OK) return rc;
+  if (rc != YALM_OK || n_splits == 1) return rc;   // one split writes the result itself
   return yalm_attn_decode_combine_bf16(partial, out, B, n_heads, head_dim, n_splits, stream);
 }

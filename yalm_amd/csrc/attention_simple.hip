@@ -176,13 +176,14 @@ __global__ void attn_decode_combine_kernel(const float* __restrict__ partial, T*
     const float* ps = part + (size_t)s * (hd + 2);
     l += ps[hd + 1] * expf(ps[hd] - m);
   }
+  const float inv_l = l > 0.f ? 1.0f / l : 0.f;
   for (int d = threadIdx.x; d < hd; d += blockDim.x) {
     float a = 0.f;
     for (int s = 0; s < n_splits; ++s) {
       const float* ps = part + (size_t)s * (hd + 2);
       a += ps[d] * expf(ps[hd] - m);
     }
-    out[((size_t)b * n_heads + h) * hd + d] = from_f32<T>(l > 0.f ? a / l : 0.f);
+    out[((size_t)b * n_heads + h) * hd + d] = from_f32<T>(a * inv_l);
   }
 }
 
@@ -221,7 +222,8 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
 int yalm_attn_decode_combine_bf16(const float* partial, void* out, int B, int n_heads, int head_dim, int n_splits,
                                   hipStream_t stream) {
   dim3 cgrid(B, n_heads);
-  attn_decode_combine_kernel<bf16><<<cgrid, WAVE, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
+  int threads = head_dim > 64 ? 128 : 64;
+  attn_decode_combine_kernel<bf16><<<cgrid, threads, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
   return launch_status();
 }
 

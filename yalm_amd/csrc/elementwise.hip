@@ -23,7 +23,7 @@ extern "C" int yalm_embed(const void* table, int table_dtype, const int* tokens,
                           hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (D <= 0 || V <= 0) return YALM_ERR_ARG;
-  int threads = D >= 256 ? 256 : 64;
+  int threads = D >= 1024 ? 1024 : (D >= 256 ? 256 : 64);
   if (table_dtype == YALM_F32)
     embed_kernel<float><<<T, threads, 0, stream>>>((const float*)table, tokens, out, D, V);
   else if (table_dtype == YALM_BF16)

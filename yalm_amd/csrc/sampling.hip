@@ -14,13 +14,11 @@ __global__ __launch_bounds__(NT) void argmax_kernel(const float* __restrict__ lo
   __shared__ float bv[NT];
   __shared__ int bi[NT];
   const float* l = logits + (size_t)blockIdx.x * V;
-  int chunk = (V + NT - 1) / NT;
-  int lo = threadIdx.x * chunk, hi = min(V, lo + chunk);
   float best = -FLT_MAX;
   int arg = V;                                   // "none": larger than every index
-  for (int i = lo; i < hi; ++i) {
+  for (int i = threadIdx.x; i < V; i += NT) {    // indices rise within a thread: strict '>' keeps its first maximum
     float v = l[i];
-    if (v > best) {                              // strict: the lowest index wins ties
+    if (v > best) {
       best = v;
       arg = i;
     }
@@ -28,16 +26,20 @@ __global__ __launch_bounds__(NT) void argmax_kernel(const float* __restrict__ lo
   bv[threadIdx.x] = best;
   bi[threadIdx.x] = arg;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    float b = -FLT_MAX;
-    int a = 0;
-    for (int t = 0; t < NT; ++t)
-      if (bi[t] < V && bv[t] > b) {
-        b = bv[t];
-        a = bi[t];
+  for (int stride = NT / 2; stride > 0; stride >>= 1) {
+    if (threadIdx.x < stride) {
+      float ov = bv[threadIdx.x + stride];
+      int oi = bi[threadIdx.x + stride];
+      float mv = bv[threadIdx.x];
+      int mi = bi[threadIdx.x];
+      if (oi < V && (mi >= V || ov > mv || (ov == mv && oi < mi))) {   // the lowest index wins ties
+        bv[threadIdx.x] = ov;
+        bi[threadIdx.x] = oi;
       }
-    out[blockIdx.x] = a;
+    }
+    __syncthreads();
   }
+  if (threadIdx.x == 0) out[blockIdx.x] = bi[0] < V ? bi[0] : 0;
 }
 
 __global__ __launch_bounds__(NT) void sample_kernel(const float* __restrict__ logits, const float* __restrict__ u,

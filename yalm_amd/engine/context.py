@@ -25,6 +25,19 @@ class Workspace:
             self._flat[key] = buf
         return buf[:n].view(*shape)
 
+    def get_zeroed(self, name, shape, dtype):
+        """Like get, but the buffer is zero when it is first made (users keep it so)."""
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = (name, dtype)
+        buf = self._flat.get(key)
+        if buf is None or buf.numel() < n:
+            if self.frozen:
+                raise RuntimeError("workspace buffer %r would have to grow inside a captured graph" % (name,))
+            self._flat[key] = torch.zeros(max(n, 1), dtype=dtype, device=self.device)
+        return self._flat[key][:n].view(*shape)
+
     def bytes(self):
         return sum(b.numel() * b.element_size() for b in self._flat.values())
 
@@ -35,7 +48,9 @@ class StepContext:
       tokens[T], tok_seq[T] (row of the batch), tok_pos[T] (position in its sequence),
       seq_slot[B] (-1: padding row), seq_len[B] (length after this step), cu_seqlens[B+1],
       seq_tile0[B+1] (prefill: first 64-token tile of each sequence in the staging area; n_tiles in all).
-    max_position: the largest position in the step (host value, for table checks)."""
+    max_position: the largest position in the step (host value, for table checks).
+    pages_bucket: decode only; an upper bound (a power of two) of the pages of the step's
+    longest sequence, the only way launch shapes may depend on lengths."""
 
     def __init__(self, mode, cache, ws, act_dtype, shared_lines=()):
         self.mode = mode
@@ -46,6 +61,7 @@ class StepContext:
         self.tokens = self.tok_seq = self.tok_pos = self.seq_slot = self.seq_len = self.cu_seqlens = None
         self.seq_tile0 = None
         self.n_tiles = 0
+        self.pages_bucket = 1 << 30       # decode: no sequence of the step has more pages than this
         self.max_position = 0
         self.host_slots = []
         self.host_n_tokens = []

@@ -180,10 +180,16 @@ class Engine:
         B = len(slots)
         use_graph = self.use_graphs and self.model.graph_safe()
         Bk = self._bucket(B) if use_graph else B
-        g = self._graphs.get(Bk) if use_graph else None
+        # launch shapes may depend on the longest sequence only through this bucket (a power of
+        # two of pages), so that a captured graph stays valid until a sequence outgrows it
+        pages_bucket = 1
+        while pages_bucket * PAGE < max(new_lens):
+            pages_bucket *= 2
+        g = self._graphs.get((Bk, pages_bucket)) if use_graph else None
         if use_graph and g is None:
             g = _DecodeGraph(self, Bk)
-            self._graphs[Bk] = g
+            g.ctx.pages_bucket = pages_bucket
+            self._graphs[(Bk, pages_bucket)] = g
         if g is not None:
             if g.copied is not None:
                 g.copied.synchronize()                   # the last upload has read the pinned buffer
@@ -205,6 +211,7 @@ class Engine:
             meta = self.ws.get("meta", (6 * Bk + 1,), torch.int32)
             meta.copy_(torch.from_numpy(host))
             ctx = self._context("decode", self.ws, meta, Bk, Bk, max(starts))
+            ctx.pages_bucket = pages_bucket
             ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), [1] * B, list(starts)
             logits = self.ws.get("logits", (Bk, self.model.vocab_size), torch.float32)
             self.model.forward(ctx, meta[5 * Bk:6 * Bk], logits)      # cu_seqlens[0:Bk] = 0..Bk-1 = all rows

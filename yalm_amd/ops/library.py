@@ -30,7 +30,7 @@ _SIGNATURES = {
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
 }
 
-ABI_VERSION = 2
+ABI_VERSION = 4
 
 
 class KernelError(RuntimeError):

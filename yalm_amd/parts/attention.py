@@ -64,12 +64,12 @@ class GQAttention(Part):
     def cache_request(self):
         return KVRequest(self.n_kv_heads, self.head_dim, self.window)
 
-    def decode_splits(self, B, ring_pages):
+    def decode_splits(self, B, max_pages):
         mfma = self.head_dim in (64, 128) and self.n_heads // self.n_kv_heads <= 16 and not kernels.FORCE_SIMPLE
         if mfma:         # a workgroup of 4 waves per (split, KV head, sequence), a page per wave at a time
             per = max(1, B * self.n_kv_heads)
-            return max(1, min((ring_pages + 3) // 4, TARGET_WORKGROUPS // per))
-        return max(1, min(ring_pages, TARGET_WORKGROUPS // max(1, B * self.n_heads)))
+            return max(1, min((max_pages + 3) // 4, TARGET_WORKGROUPS // per))
+        return max(1, min(max_pages, TARGET_WORKGROUPS // max(1, B * self.n_heads)))
 
     def forward(self, h, x, ctx, line, writes_cache=True):
         T = h.shape[0]
@@ -106,7 +106,7 @@ class GQAttention(Part):
             kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, ctx.seq_tile0, ctx.tok_seq, ctx.tok_pos,
                                  self.n_heads, self.n_kv_heads, self.head_dim, self.window)
         else:
-            n_splits = self.decode_splits(T, group.ring_pages)
+            n_splits = self.decode_splits(T, min(group.ring_pages, ctx.pages_bucket))
             partial = ws.get("attn.partial",
                              (kernels.attn_decode_workspace_floats(T, self.n_heads, self.head_dim, n_splits),),
                              torch.float32)
