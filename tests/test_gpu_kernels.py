@@ -408,3 +408,74 @@ def test_argmax_and_sample():
     k.token_prob(logits.to(DEV), i32([0, 1, 2, 3, 4, 999]), prob)
     want = [R.sample_prob(logits[r], i) for r, i in enumerate([0, 1, 2, 3, 4, 999])]
     assert torch.allclose(prob.cpu().double(), torch.tensor(want, dtype=torch.float64), rtol=1e-4, atol=1e-9)
+
+
+# ------------------------------------------------------------------ fused decode GEMMs
+
+@pytest.mark.parametrize("M,N,Kd", [(1, 64, 256), (8, 4096 + 32, 136), (7, 100, 96), (3, 17000, 64), (2, 4096, 4096), (8, 48, 4096)])
+def test_gemm_norm(M, N, Kd):
+    """rmsnorm folded into the product: against the plain rmsnorm followed by a float64 product."""
+    k = K()
+    x = rnd((M, Kd), 50, scale=3.0)
+    nw = 1 + 0.1 * rnd((Kd,), 51)
+    w = rnd((N, Kd), 52, torch.bfloat16, scale=1 / math.sqrt(Kd))
+    want = R.rmsnorm(x, nw, 1e-5) @ w.double().T
+    out = torch.empty((M, N), device=DEV)
+    k.gemm_norm(x.to(DEV), nw.to(DEV), 1e-5, w.to(DEV), out, k.EPI_STORE_F32)
+    close(out, want, torch.bfloat16, "gemm_norm")          # the activations are rounded to bfloat16 on the way
+
+
+@pytest.mark.parametrize("M,H,D", [(1, 176, 64), (8, 1000, 264), (5, 14336, 128)])
+def test_gemm_norm_gated(M, H, D):
+    from yalm_amd.parts.swiglu import interleave_gate_up
+    k = K()
+    x = rnd((M, D), 53, scale=2.0)
+    nw = 1 + 0.1 * rnd((D,), 54)
+    wg = rnd((H, D), 55, torch.bfloat16, scale=1 / math.sqrt(D))
+    wu = rnd((H, D), 56, torch.bfloat16, scale=1 / math.sqrt(D))
+    h = R.rmsnorm(x, nw, 1e-6)
+    want = R.silu(h @ wg.double().T) * (h @ wu.double().T)
+    out = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
+    k.gemm_norm(x.to(DEV), nw.to(DEV), 1e-6, interleave_gate_up(wg, wu).to(DEV), out, k.EPI_GATED, hidden=H)
+    close(out, want, torch.bfloat16, "gemm_norm gated", factor=1.5)
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,rd,D", [(4, 2, 16, 16, 64), (3, 1, 48, 48, 80), (6, 3, 32, 16, 96),
+                                                   (32, 8, 128, 128, 256)])
+def test_gemm_norm_qkv_rope(n_heads, n_kv, hd, rd, D):
+    """norm + q/k/v + rotation + cache write in one kernel against the plain parts."""
+    k = K()
+    PAGE = k.PAGE
+    M = 5
+    pos = [0, 63, 64, 130, 7]
+    slots = [3, 0, -1, 2, 1]                       # row 2 is a padding row
+    Q, KV = n_heads * hd, n_kv * hd
+    x = rnd((M, D), 57, scale=2.0)
+    nw = 1 + 0.1 * rnd((D,), 58)
+    w = rnd((Q + 2 * KV, D), 59, torch.bfloat16, scale=1 / math.sqrt(D))
+    table = make_table(200, hd, rd, 10000.0)
+    ring, n_pages = 4, 12
+    bt = torch.arange(4 * ring, dtype=torch.int32).reshape(4, ring) % n_pages
+    kp = torch.zeros((n_pages, n_kv, PAGE, hd), dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros((n_pages, n_kv, hd, PAGE), dtype=torch.bfloat16, device=DEV)
+    q_out = torch.zeros((M, Q), dtype=torch.bfloat16, device=DEV)
+    k.gemm_norm_qkv_rope(x.to(DEV), nw.to(DEV), 1e-5, w.to(DEV), q_out, kp, vp, bt.to(DEV), ring, i32(pos), i32(slots),
+                         table.to(DEV), n_heads, n_kv, hd, rd)
+    qkv = R.rmsnorm(x, nw, 1e-5) @ w.double().T
+    f = R.rope_inv_freq(hd, rd, 10000.0)
+    p = torch.tensor(pos)
+    q_want = R.rope_interleaved(qkv[:, :Q].reshape(M, n_heads, hd), p, f).reshape(M, Q)
+    k_want = R.rope_interleaved(qkv[:, Q:Q + KV].reshape(M, n_kv, hd), p, f)
+    v_want = qkv[:, Q + KV:].reshape(M, n_kv, hd)
+    close(q_out, q_want, torch.bfloat16, "q", factor=1.5)
+    kp, vp = kp.cpu(), vp.cpu()
+    touched = torch.zeros((n_pages, PAGE), dtype=torch.bool)
+    for m in range(M):
+        if slots[m] < 0:
+            continue
+        page, r = int(bt[slots[m], (pos[m] // PAGE) % ring]), pos[m] % PAGE
+        close(kp[page, :, r, :], k_want[m], torch.bfloat16, "k row %d" % m, factor=1.5)
+        close(vp[page, :, :, r], v_want[m], torch.bfloat16, "v row %d" % m, factor=1.5)
+        touched[page, r] = True
+    assert (kp.float().abs().sum(dim=(1, 3)) > 0).equal(touched)
+    assert (vp.float().abs().sum(dim=(1, 2)) > 0).equal(touched)

@@ -35,6 +35,20 @@ int yalm_rmsnorm(const float* x, const void* w, int w_dtype, void* out, int out_
 int yalm_gemm(const void* A, const void* W, void* C, int M, int N, int K, int dtype, int epilogue, int H,
               int force_simple, hipStream_t stream);
 
+// Decode GEMMs from the float32 residual stream, M <= 8 rows (M * (K + 8) * 2 bytes <= 72 KB), bfloat16 weights:
+// C = epilogue(rmsnorm(x, norm_w, eps) * W^T); epilogue 0 (float32 store) or 3 (gated, as yalm_gemm).
+// norm_w is float32 [K].  Refuses (YALM_ERR_ARG) other shapes: use yalm_rmsnorm + yalm_gemm then.
+int yalm_gemm_norm(const float* x, const float* norm_w, float eps, const void* W, void* C, int M, int N, int K,
+                   int epilogue, int H, hipStream_t stream);
+// The same for the fused q/k/v projection of a decode step (row m = sequence m), followed by what
+// yalm_rope_kv_write does: q rotated into q_out (bfloat16 [M, n_heads * head_dim]), k rotated and v
+// into the pages of the cache at each row's position.  head_dim must be a multiple of 16.
+int yalm_gemm_norm_qkv_rope(const float* x, const float* norm_w, float eps, const void* Wqkv, void* q_out,
+                            void* k_pages, void* v_pages, const int* block_table, int table_stride, int ring_pages,
+                            const int* tok_pos, const int* seq_slot, const float* cos_sin, int n_positions, int M,
+                            int K, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, int n_pages,
+                            hipStream_t stream);
+
 // Rotates q and k of every token (adjacent pairs, angles from the table), writes q,
 // optionally k and v into a staging area in page format (for attention over the step's
 // own tokens: tile seq_tile0[sequence] + position / PAGE), and k and v into the pages

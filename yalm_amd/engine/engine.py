@@ -214,7 +214,7 @@ class Engine:
             ctx.pages_bucket = pages_bucket
             ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), [1] * B, list(starts)
             logits = self.ws.get("logits", (Bk, self.model.vocab_size), torch.float32)
-            self.model.forward(ctx, meta[5 * Bk:6 * Bk], logits)      # cu_seqlens[0:Bk] = 0..Bk-1 = all rows
+            self.model.forward(ctx, None, logits)                     # every row
         else:
             g.meta.copy_(g.meta_host, non_blocking=True)
             if g.copied is None:
@@ -234,13 +234,12 @@ class Engine:
     def _capture(self, g):
         """Runs the step once eagerly on the graph's buffers (every buffer gets its
         size), then captures it."""
-        rows = g.meta[5 * g.bucket:6 * g.bucket]
-        self.model.forward(g.ctx, rows, g.logits)
+        self.model.forward(g.ctx, None, g.logits)
         torch.cuda.synchronize(self.device)
         g.ws.frozen = True
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
-            self.model.forward(g.ctx, rows, g.logits)
+            self.model.forward(g.ctx, None, g.logits)
         g.graph = graph
 
     def synchronize(self):

@@ -132,17 +132,21 @@ class Model:
     # ------------------------------------------------------------------ forward
     def forward(self, ctx, want_rows, logits):
         """Runs the step's tokens through the layers (the cache is read and written
-        through ctx) and writes logits for the rows want_rows (int32 device tensor)."""
+        through ctx) and writes logits for the rows want_rows (int32 device tensor;
+        None: every row, in order)."""
         T = ctx.tokens.shape[0]
         x = ctx.ws.get("x", (T, self.dim), torch.float32)
         self.embedding.forward(ctx.tokens, x, ctx)
         for e in self.schedule:
             self.blocks[e.layer].forward(x, ctx, e.cache, e.writes_cache)
-        if want_rows is not None and logits is not None and logits.shape[0] > 0:
+        if logits is not None and logits.shape[0] > 0:
             R = logits.shape[0]
-            h = ctx.ws.get("head.h", (R, self.dim), ctx.act_dtype)
-            self.final_norm.forward(x, h, ctx, row_index=want_rows)
-            self.head.forward(h, logits, ctx)
+            if want_rows is None and R == T and self.head.fuses_norm(self.final_norm, x, ctx):
+                self.head.forward_prenorm(x, self.final_norm, logits, ctx)
+            else:
+                h = ctx.ws.get("head.h", (R, self.dim), ctx.act_dtype)
+                self.final_norm.forward(x, h, ctx, row_index=want_rows)
+                self.head.forward(h, logits, ctx)
         return logits
 
 

@@ -101,6 +101,70 @@ def gemm(a, w, out, epilogue, hidden=0):
     return out
 
 
+FUSED_NORM_MAX_ROWS = 8
+
+
+def can_fuse_norm(M, K, dtype):
+    """Whether gemm_norm / gemm_norm_qkv_rope take this shape (else: rmsnorm, then gemm)."""
+    return dtype == torch.bfloat16 and 1 <= M <= FUSED_NORM_MAX_ROWS and K % 8 == 0 and \
+        M * (K + 8) * 2 <= 72 * 1024 and not FORCE_SIMPLE
+
+
+def gemm_norm(x, norm_w, eps, w, out, epilogue, hidden=0):
+    """out = epilogue(rmsnorm(x, norm_w, eps) @ w^T) for at most 16 rows of the float32
+    residual stream x; w bfloat16 [N, K], norm_w float32 [K]; EPI_STORE_F32 or EPI_GATED.
+    (Shapes: see can_fuse_norm.)"""
+    M, K = x.shape
+    N = w.shape[0]
+    p_x = _need(x, "x", torch.float32, (M, K))
+    p_n = _need(norm_w, "norm_w", torch.float32, (K,))
+    p_w = _need(w, "w", torch.bfloat16, (N, K))
+    if epilogue == EPI_GATED:
+        if hidden <= 0 or N != 32 * ((hidden + 15) // 16):
+            raise ValueError("gated gemm: weight rows %d do not match hidden %d" % (N, hidden))
+        p_o = _need(out, "out", torch.bfloat16, (M, hidden))
+    elif epilogue == EPI_STORE_F32:
+        p_o = _need(out, "out", torch.float32, (M, N))
+    else:
+        raise ValueError("gemm_norm: epilogue %r is not offered" % (epilogue,))
+    library.check(library.lib().yalm_gemm_norm(p_x, p_n, float(eps), p_w, p_o, M, N, K, epilogue, hidden, _stream()),
+                  "gemm_norm")
+    return out
+
+
+def gemm_norm_qkv_rope(x, norm_w, eps, wqkv, q_out, k_pages, v_pages, block_table, ring_pages, tok_pos, seq_slot,
+                       cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim):
+    """A decode step's rmsnorm + q/k/v projection + rotation + cache write in one kernel
+    (row m is sequence m; see rope_kv_write for the operands)."""
+    _check_heads(n_heads, n_kv_heads, head_dim)
+    if head_dim % 16:
+        raise ValueError("gemm_norm_qkv_rope needs a head_dim that is a multiple of 16")
+    M, K = x.shape
+    Q, KV = n_heads * head_dim, n_kv_heads * head_dim
+    p_x = _need(x, "x", torch.float32, (M, K))
+    p_n = _need(norm_w, "norm_w", torch.float32, (K,))
+    p_w = _need(wqkv, "wqkv", torch.bfloat16, (Q + 2 * KV, K))
+    p_q = _need(q_out, "q_out", torch.bfloat16, (M, Q))
+    n_pages = k_pages.shape[0]
+    p_kp = _need(k_pages, "k_pages", torch.bfloat16, (n_pages, n_kv_heads, PAGE, head_dim))
+    p_vp = _need(v_pages, "v_pages", torch.bfloat16, (n_pages, n_kv_heads, head_dim, PAGE))
+    p_bt = _need(block_table, "block_table", torch.int32, (None, None))
+    stride = block_table.shape[1]
+    if ring_pages <= 0 or ring_pages > stride:
+        raise ValueError("ring_pages %d does not fit the block table (%d columns)" % (ring_pages, stride))
+    p_tp = _need(tok_pos, "tok_pos", torch.int32, (M,))
+    p_ss = _need(seq_slot, "seq_slot", torch.int32, (M,))
+    n_pos, p_cs = 0, None
+    if cos_sin is not None:
+        n_pos = cos_sin.shape[0]
+        p_cs = _need(cos_sin, "cos_sin", torch.float32, (n_pos, rotary_dim // 2, 2))
+    else:
+        rotary_dim = 0
+    library.check(library.lib().yalm_gemm_norm_qkv_rope(
+        p_x, p_n, float(eps), p_w, p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_tp, p_ss, p_cs, n_pos, M, K, n_heads,
+        n_kv_heads, head_dim, rotary_dim, n_pages, _stream()), "gemm_norm_qkv_rope")
+
+
 def _check_heads(n_heads, n_kv_heads, head_dim):
     if n_heads % n_kv_heads != 0:
         raise ValueError("n_heads %d is no multiple of n_kv_heads %d" % (n_heads, n_kv_heads))

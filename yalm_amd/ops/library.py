@@ -20,6 +20,9 @@ _SIGNATURES = {
     "yalm_embed": (_I, [_P, _I, _P, _P, _I, _I, _I, _P]),
     "yalm_rmsnorm": (_I, [_P, _P, _I, _P, _I, _P, _I, _I, _F, _P]),
     "yalm_gemm": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_gemm_norm": (_I, [_P, _P, _F, _P, _P, _I, _I, _I, _I, _I, _P]),
+    "yalm_gemm_norm_qkv_rope": (_I, [_P, _P, _F, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
+                                     _I, _P]),
     "yalm_rope_kv_write": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                 _I, _I, _P]),
     "yalm_attn_prefill": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
@@ -30,7 +33,7 @@ _SIGNATURES = {
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
 }
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class KernelError(RuntimeError):

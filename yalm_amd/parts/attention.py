@@ -71,6 +71,42 @@ class GQAttention(Part):
             return max(1, min((max_pages + 3) // 4, TARGET_WORKGROUPS // per))
         return max(1, min(max_pages, TARGET_WORKGROUPS // max(1, B * self.n_heads)))
 
+    def fuses_norm(self, norm, x, ctx):
+        return hasattr(norm, "fused") and ctx.mode == "decode" and self.head_dim % 16 == 0 and \
+            kernels.can_fuse_norm(x.shape[0], self.dim, self.wo.dtype)
+
+    def forward_prenorm(self, x, norm, ctx, line, writes_cache=True):
+        """A decode step from the residual stream: norm, q/k/v, rotation and cache write in
+        one kernel, attention over the cache, output projection added to x."""
+        if not writes_cache:                      # a reader of another entry's line: the plain way
+            h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
+            norm.forward(x, h, ctx)
+            return self.forward(h, x, ctx, line, writes_cache)
+        T = x.shape[0]
+        pos = self.position
+        if pos.table is not None and ctx.max_position >= pos.n_positions:
+            raise ValueError("position %d is beyond the %d positions the rotation table holds"
+                             % (ctx.max_position, pos.n_positions))
+        nw, eps = norm.fused()
+        group = ctx.cache.group_of(line)
+        k_pages, v_pages = group.line_pages(line)
+        q = ctx.ws.get("attn.q", (T, self.q_dim), self.wo.dtype)
+        kernels.gemm_norm_qkv_rope(x, nw, eps, self.wqkv, q, k_pages, v_pages, group.table, group.ring_pages,
+                                   ctx.tok_pos, ctx.seq_slot, pos.table, self.n_heads, self.n_kv_heads,
+                                   self.head_dim, pos.rotary_dim)
+        o = ctx.ws.get("attn.o", (T, self.q_dim), self.wo.dtype)
+        self._decode_attention(q, o, ctx, group, k_pages, v_pages)
+        kernels.gemm(o, self.wo, x, kernels.EPI_ADD_F32)
+
+    def _decode_attention(self, q, o, ctx, group, k_pages, v_pages):
+        T = q.shape[0]
+        n_splits = self.decode_splits(T, min(group.ring_pages, ctx.pages_bucket))
+        partial = ctx.ws.get("attn.partial",
+                             (kernels.attn_decode_workspace_floats(T, self.n_heads, self.head_dim, n_splits),),
+                             torch.float32)
+        kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o, partial,
+                            self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits)
+
     def forward(self, h, x, ctx, line, writes_cache=True):
         T = h.shape[0]
         act = h.dtype
@@ -106,10 +142,5 @@ class GQAttention(Part):
             kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, ctx.seq_tile0, ctx.tok_seq, ctx.tok_pos,
                                  self.n_heads, self.n_kv_heads, self.head_dim, self.window)
         else:
-            n_splits = self.decode_splits(T, min(group.ring_pages, ctx.pages_bucket))
-            partial = ws.get("attn.partial",
-                             (kernels.attn_decode_workspace_floats(T, self.n_heads, self.head_dim, n_splits),),
-                             torch.float32)
-            kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o,
-                                partial, self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits)
+            self._decode_attention(q, o, ctx, group, k_pages, v_pages)
         kernels.gemm(o, self.wo, x, kernels.EPI_ADD_F32)

@@ -13,6 +13,10 @@ it is in.  Kinds of parts and the methods each must have:
   embedding      forward(tokens_i32[T], x_f32[T, dim], ctx)
   head           forward(h[R, dim], logits_f32[R, vocab], ctx)
 
+A mixer, feed-forward or head may fold the norm in front of it into its first
+product: fuses_norm(norm, x, ctx) says so for a step, and forward_prenorm(x, norm,
+...) then replaces norm.forward + forward.
+
 All of them: param_specs() -> [ParamSpec], load(get, compute_dtype, device),
 weight_bytes().  `h` is in the compute dtype (bfloat16 or float32); the
 residual stream `x` is always float32."""
@@ -75,3 +79,8 @@ class Part:
 
     def children(self):
         return []
+
+    def fuses_norm(self, norm, x, ctx):
+        """True if this part can take the float32 residual stream x and do `norm` itself
+        (it then offers forward_prenorm in place of forward)."""
+        return False

@@ -18,8 +18,15 @@ class PreNormResidualBlock(Part):
         return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
 
     def forward(self, x, ctx, line, writes_cache=True):
-        h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
-        self.mixer_norm.forward(x, h, ctx)
-        self.mixer.forward(h, x, ctx, line, writes_cache)
-        self.feed_forward_norm.forward(x, h, ctx)
-        self.feed_forward.forward(h, x, ctx)
+        if self.mixer.fuses_norm(self.mixer_norm, x, ctx):
+            self.mixer.forward_prenorm(x, self.mixer_norm, ctx, line, writes_cache)
+        else:
+            h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
+            self.mixer_norm.forward(x, h, ctx)
+            self.mixer.forward(h, x, ctx, line, writes_cache)
+        if self.feed_forward.fuses_norm(self.feed_forward_norm, x, ctx):
+            self.feed_forward.forward_prenorm(x, self.feed_forward_norm, ctx)
+        else:
+            h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
+            self.feed_forward_norm.forward(x, h, ctx)
+            self.feed_forward.forward(h, x, ctx)

@@ -51,5 +51,14 @@ class LMHead(Part):
     def weight_bytes(self):
         return self.weight.numel() * self.weight.element_size()
 
+    def fuses_norm(self, norm, x, ctx):
+        return hasattr(norm, "fused") and ctx.mode == "decode" and \
+            kernels.can_fuse_norm(x.shape[0], self.dim, self.weight.dtype)
+
+    def forward_prenorm(self, x, norm, logits, ctx):
+        """logits for every row of x (no row selection)."""
+        nw, eps = norm.fused()
+        return kernels.gemm_norm(x, nw, eps, self.weight, logits, kernels.EPI_STORE_F32)
+
     def forward(self, h, logits, ctx):
         return kernels.gemm(h, self.weight, logits, kernels.EPI_STORE_F32)

@@ -49,6 +49,17 @@ class SwiGLU(Part):
     def weight_bytes(self):
         return 3 * self.hidden * self.dim * self.w_down.element_size()
 
+    def fuses_norm(self, norm, x, ctx):
+        return hasattr(norm, "fused") and ctx.mode == "decode" and \
+            kernels.can_fuse_norm(x.shape[0], self.dim, self.w_down.dtype)
+
+    def forward_prenorm(self, x, norm, ctx):
+        nw, eps = norm.fused()
+        T = x.shape[0]
+        mid = ctx.ws.get("ffn.hidden", (T, self.hidden), self.w_down.dtype)
+        kernels.gemm_norm(x, nw, eps, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
+        kernels.gemm(mid, self.w_down, x, kernels.EPI_ADD_F32)
+
     def forward(self, h, x, ctx):
         T = h.shape[0]
         mid = ctx.ws.get("ffn.hidden", (T, self.hidden), h.dtype)
