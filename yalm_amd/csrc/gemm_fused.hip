@@ -17,6 +17,7 @@
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
@@ -81,6 +82,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_norm_kernel(const float* _
     float ss[MAX_ROWS];
 #pragma unroll
     for (int m = 0; m < MAX_ROWS; ++m) ss[m] = 0.f;
+#pragma unroll 2
     for (int k = threadIdx.x * 4; k < K; k += NTHREADS * 4) {
       const float4 w4 = *reinterpret_cast<const float4*>(norm_w + k);
 #pragma unroll
@@ -88,11 +90,12 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_norm_kernel(const float* _
         if (m < M) {
           const float4 a = *reinterpret_cast<const float4*>(X + (size_t)m * K + k);
           ss[m] += a.x * a.x + a.y * a.y + a.z * a.z + a.w * a.w;
-          bf16* d = xs + (size_t)m * xs_row + k;
+          bf16x4 d;
           d[0] = static_cast<bf16>(a.x * w4.x);
           d[1] = static_cast<bf16>(a.y * w4.y);
           d[2] = static_cast<bf16>(a.z * w4.z);
           d[3] = static_cast<bf16>(a.w * w4.w);
+          *reinterpret_cast<bf16x4*>(xs + (size_t)m * xs_row + k) = d;
         }
       }
     }
@@ -229,7 +232,7 @@ int launch(const float* X, const float* norm_w, float eps, const bf16* W, void* 
   bool wide = EPI == EPI_GATED || N >= 16384;
   size_t lds = (size_t)M * (K + 8) * sizeof(bf16);
   if (wide)
-    gemm_norm_kernel<2, 4, EPI><<<ceil_div(N, 32), 4 * WAVE, lds, stream>>>(X, norm_w, eps, W, C, M, N, K, H, ra);
+    gemm_norm_kernel<4, 4, EPI><<<ceil_div(N, 64), 4 * WAVE, lds, stream>>>(X, norm_w, eps, W, C, M, N, K, H, ra);
   else
     gemm_norm_kernel<1, 8, (EPI == EPI_GATED ? EPI_F32 : EPI)><<<ceil_div(N, 16), 8 * WAVE, lds, stream>>>(
         X, norm_w, eps, W, C, M, N, K, H, ra);

@@ -33,13 +33,14 @@ __device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
 // B = weights (column j = weight row, 8 k per lane); C[i][j]: lane (q = lane/16,
 // j = lane%16) holds batch rows 4q..4q+3 of weight row j.  Which k a lane's slot
 // holds is the same for both operands, so any assignment of k to slots is right;
-// here lane group q takes the 32 consecutive k  [kc + 32q, kc + 32q + 32).
-template <int MT, int NT, int NWAVES, int EPI>
+// here step s of a chunk takes k = kc + 32 s + 8 q ... + 8, so that the four lane groups of
+// a weight row read 64 contiguous bytes per load.
+template <int MT, int NT, int NWAVES, int EPI, int KS>
 __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ X,
                                                                      const bf16* __restrict__ W,
                                                                      void* __restrict__ Cv, int M, int N, int K,
                                                                      int H) {
-  constexpr int KC = 128;                        // k per wave iteration
+  constexpr int KC = 32 * KS;                    // k per wave iteration
   __shared__ f32x4 red[NWAVES][MT * NT][WAVE];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int q = lane / 16, j = lane % 16;
@@ -68,11 +69,11 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[mt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  bf16x8 wv[NT][4], xv[MT][4];
+  bf16x8 wv[NT][KS], xv[MT][KS];
   int kc = wave * KC;
   if (kc < K) {
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int s = 0; s < KS; ++s) {
       int k = kc + s * 32 + q * 8;
       bool ok = k < K;
 #pragma unroll
@@ -82,11 +83,11 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
     }
   }
   for (; kc < K; kc += NWAVES * KC) {
-    bf16x8 wn[NT][4], xn[MT][4];
+    bf16x8 wn[NT][KS], xn[MT][KS];
     int kn = kc + NWAVES * KC;
     if (kn < K) {                                // prefetch the wave's next chunk
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
+      for (int s = 0; s < KS; ++s) {
         int k = kn + s * 32 + q * 8;
         bool ok = k < K;
 #pragma unroll
@@ -96,7 +97,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
       }
     }
 #pragma unroll
-    for (int s = 0; s < 4; ++s)
+    for (int s = 0; s < KS; ++s)
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -104,7 +105,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
           acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
     if (kn < K) {
 #pragma unroll
-      for (int s = 0; s < 4; ++s) {
+      for (int s = 0; s < KS; ++s) {
 #pragma unroll
         for (int t = 0; t < NT; ++t) wv[t][s] = wn[t][s];
 #pragma unroll
@@ -157,12 +158,18 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
 
 template <int MT, int EPI>
 int skinny_launch(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
-  // few weight rows: 16 rows and 8 waves a workgroup, so that every CU has work; many: 32 rows, 4 waves
+  // few weight rows: 16 rows and 8 waves a workgroup, so that every CU has work;
+  // many: 64 rows (32 if the batch needs the registers) and 4 waves
   bool wide = EPI == 3 || N >= 16384;
-  if (wide)
-    gemm_skinny_kernel<MT, 2, 4, EPI><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H);
-  else
-    gemm_skinny_kernel<MT, 1, 8, (EPI == 3 ? 0 : EPI)><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H);
+  if (wide) {
+    if (MT <= 2)
+      gemm_skinny_kernel<MT, 4, 4, EPI, 4><<<ceil_div(N, 64), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H);
+    else
+      gemm_skinny_kernel<MT, 2, 4, EPI, 4><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H);
+  } else {
+    constexpr int E = EPI == 3 ? 0 : EPI;
+    gemm_skinny_kernel<MT, 1, 8, E, 4><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H);
+  }
   return launch_status();
 }
 

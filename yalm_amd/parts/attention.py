@@ -19,7 +19,7 @@ from ..weights.loader import ParamSpec, place
 from .base import Part, build_part, part
 
 # decode attention is split over pages so that about this many workgroups run
-TARGET_WORKGROUPS = 1024
+TARGET_WORKGROUPS = 256
 
 
 @part("mixer", "gqa_attention")
