@@ -201,17 +201,28 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// prefill: grid (tile of 64 query positions, head); a wave takes 16 positions
+// prefill: a workgroup takes 128 query positions of one head (4 waves x 32 positions,
+// two 16-position column tiles a wave); key/value tiles of 64 rows go through LDS once
+// per workgroup, double-buffered, rows stored in the order the MFMA operands read them.
+// grid (64-position tile, head): the workgroup of every second tile of a sequence works.
 // ---------------------------------------------------------------------------
+__device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
+
 template <int HD>
-__global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
+__global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_stage, const bf16* __restrict__ v_stage,
     bf16* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_tile0, int B, int n_heads,
     int n_kv_heads, int window) {
   constexpr int KS = HD / 32, DT = HD / 16;
+  constexpr int KROW = HD + 8;                    // LDS row strides (elements): 16 bytes of padding
+  constexpr int VROW = PAGE + 8;
+  constexpr int KTILE = PAGE * KROW, VTILE = HD * VROW;
+  constexpr int NLOAD = HD / 32;                  // 16-byte chunks per thread and tile
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16* smem = reinterpret_cast<bf16*>(smem_raw);   // [2][KTILE + VTILE]
+
   const int gt = blockIdx.x, h = blockIdx.y;
-  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, qd = lane / 16, j = lane % 16;
-  // the sequence of this tile: the last b with seq_tile0[b] <= gt (seq_tile0 has B + 1 entries)
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE, qd = lane / 16, j = lane % 16;
   int b = 0;
   {
     int lo_b = 0, hi_b = B - 1;
@@ -223,121 +234,159 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
   }
   const int tile0 = seq_tile0[b];
   const int tq = gt - tile0;
+  if (tq & 1) return;                             // the workgroup of the even tile covers this one too
   const int start = cu_seqlens[b], len = cu_seqlens[b + 1] - start;
-  const int pos0 = tq * PAGE + wave * 16;
-  if (pos0 >= len) return;                        // no barrier follows: a wave may leave
   const int g = h / (n_heads / n_kv_heads);
-  const int pos_q = pos0 + j;
-  const bool q_ok = pos_q < len;
-  const float root = sqrtf((float)HD);
+  const float inv_root = 1.0f / sqrtf((float)HD);
 
-  bf16x8 qv[KS];
-  {
-    const bf16* qrow = q + ((size_t)(start + (q_ok ? pos_q : 0)) * n_heads + h) * HD;
+  const int blk0 = tq * PAGE;                     // first position of the workgroup
+  const int pos0 = blk0 + wave * 32;              // first position of the wave
+  const bool wave_live = pos0 < len;
+  bf16x8 qv[2][KS];
+  bool q_ok[2];
+  int pos_q[2];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qv[ks] = q_ok ? ld8(qrow + ks * 32 + qd * 8) : zero8();
+  for (int c = 0; c < 2; ++c) {
+    pos_q[c] = pos0 + c * 16 + j;
+    q_ok[c] = pos_q[c] < len;
+    const bf16* qrow = q + ((size_t)(start + (q_ok[c] ? pos_q[c] : 0)) * n_heads + h) * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qv[c][ks] = q_ok[c] ? ld8(qrow + ks * 32 + qd * 8) : zero8();
   }
-  float m = -FLT_MAX, l = 0.f;
-  f32x4 o[DT];
+  float m[2] = {-FLT_MAX, -FLT_MAX}, l[2] = {0.f, 0.f};
+  f32x4 o[2][DT];
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[c][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  const int last_q = min(pos0 + 15, len - 1);
-  const int kt_hi = last_q / PAGE;
-  const int kt_lo = window > 0 ? max(0, pos0 - window + 1) / PAGE : 0;
+  const int blk_last = min(blk0 + 2 * PAGE - 1, len - 1);
+  const int kt_hi = blk_last / PAGE;
+  const int kt_lo = window > 0 ? max(0, blk0 - window + 1) / PAGE : 0;
+  const int wave_last = min(pos0 + 31, len - 1);
   const size_t tile_elems = (size_t)n_kv_heads * PAGE * HD;
 
-  bf16x8 kreg[4][KS];
-  {
-    const bf16* kp = k_stage + (tile0 + kt_lo) * tile_elems + (size_t)g * PAGE * HD;
-#pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) kreg[t][ks] = ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
-  }
-  for (int kt = kt_lo; kt <= kt_hi; ++kt) {
+  // global -> registers -> LDS; key rows are stored at the index the MFMA row reads them at
+  bf16x8 rk[NLOAD], rv[NLOAD];
+  auto load_tile = [&](int kt) {
+    const bf16* kp = k_stage + (tile0 + kt) * tile_elems + (size_t)g * PAGE * HD;
     const bf16* vp = v_stage + (tile0 + kt) * tile_elems + (size_t)g * PAGE * HD;
-    bf16x8 vreg[DT][2];
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-      for (int s = 0; s < 2; ++s) vreg[dt][s] = ld8(vp + (dt * 16 + j) * PAGE + s * 32 + qd * 8);
-
-    f32x4 sc[4];
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      sc[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[t][ks], qv[ks], sc[t], 0, 0, 0);
+    for (int p = 0; p < NLOAD; ++p) {
+      int c = tid + p * 256;
+      rk[p] = ld8(kp + (size_t)c * 8);
+      rv[p] = ld8(vp + (size_t)c * 8);
     }
-    if (kt < kt_hi) {
-      const bf16* kp = k_stage + (tile0 + kt + 1) * tile_elems + (size_t)g * PAGE * HD;
+  };
+  auto store_tile = [&](int buf) {
+    bf16* ks_l = smem + buf * (KTILE + VTILE);
+    bf16* vs_l = ks_l + KTILE;
+#pragma unroll
+    for (int p = 0; p < NLOAD; ++p) {
+      int c = tid + p * 256;
+      int row = c / (HD / 8), col = (c % (HD / 8)) * 8;              // key tile: [row][element]
+      int t = 2 * (row >> 5) + ((row >> 2) & 1), i = 4 * ((row >> 3) & 3) + (row & 3);
+      *reinterpret_cast<bf16x8*>(ks_l + (t * 16 + i) * KROW + col) = rk[p];
+      int vrow = c / 8, vcol = (c % 8) * 8;                            // value tile: [element][row]
+      *reinterpret_cast<bf16x8*>(vs_l + vrow * VROW + vcol) = rv[p];
+    }
+  };
+
+  load_tile(kt_lo);
+  store_tile(0);
+  __syncthreads();
+  for (int kt = kt_lo; kt <= kt_hi; ++kt) {
+    const int cur = (kt - kt_lo) & 1;
+    if (kt < kt_hi) load_tile(kt + 1);
+    const int base = kt * PAGE;
+    const bool visible = wave_live && base <= wave_last && (window == 0 || base + PAGE - 1 > pos0 - window);
+    if (visible) {
+      const bf16* ks_l = smem + cur * (KTILE + VTILE);
+      const bf16* vs_l = ks_l + KTILE;
+      f32x4 sc[2][4];
+#pragma unroll
+      for (int c = 0; c < 2; ++c)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) sc[c][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kreg[t][ks] = ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
-    }
-
-    const int base = kt * PAGE;
-    const bool edge = base + PAGE - 1 > pos0 || (window > 0 && base < pos0 + 15 - window + 1);
-    float mx = -FLT_MAX;
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks_l + (t * 16 + j) * KROW + ks * 32 + qd * 8);
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float v = sc[t][r] / root;
-        if (edge) {
-          int kpos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
-          bool vis = kpos <= pos_q && (window == 0 || pos_q - kpos < window) && q_ok;
-          if (!vis) v = -INFINITY;
+          for (int c = 0; c < 2; ++c)
+            sc[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qv[c][ks], sc[c][t], 0, 0, 0);
         }
-        sc[t][r] = v;
-        mx = fmaxf(mx, v);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-    const float m_new = fmaxf(m, mx);
-    const float corr = expf(m - m_new);
-    float psum = 0.f;
-    bf16x8 pb[2];
+      const bool edge = base + PAGE - 1 > pos0 || (window > 0 && base < pos0 + 31 - window + 1);
+      bf16x8 pb[2][2];
+      float corr[2];
 #pragma unroll
-    for (int s = 0; s < 2; ++s)
+      for (int c = 0; c < 2; ++c) {
+        float mx = -FLT_MAX;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float p = expf(sc[2 * s + (e >> 2)][e & 3] - m_new);
-        psum += p;
-        pb[s][e] = static_cast<bf16>(p);
-      }
-    l = l * corr + psum;
-    m = m_new;
-    if (base + PAGE > len) {                      // rows behind the sequence's end may hold anything
+        for (int t = 0; t < 4; ++t)
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
-#pragma unroll
-        for (int e = 0; e < 8; ++e)
-          if (base + 32 * s + 8 * qd + e >= len) {
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) vreg[dt][s][e] = static_cast<bf16>(0.f);
+          for (int r = 0; r < 4; ++r) {
+            float v = sc[c][t][r] * inv_root;
+            if (edge) {
+              int kpos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
+              bool vis = kpos <= pos_q[c] && (window == 0 || pos_q[c] - kpos < window) && q_ok[c];
+              if (!vis) v = -INFINITY;
+            }
+            sc[c][t][r] = v;
+            mx = fmaxf(mx, v);
           }
-    }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        const float m_new = fmaxf(m[c], mx);
+        corr[c] = fast_exp(m[c] - m_new);
+        float psum = 0.f;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      o[dt] *= corr;
+        for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt][s], pb[s], o[dt], 0, 0, 0);
+          for (int e = 0; e < 8; ++e) {
+            float p = fast_exp(sc[c][2 * s2 + (e >> 2)][e & 3] - m_new);
+            psum += p;
+            pb[c][s2][e] = static_cast<bf16>(p);
+          }
+        l[c] = l[c] * corr[c] + psum;
+        m[c] = m_new;
+      }
+      const bool tail = base + PAGE > len;        // rows behind the sequence's end may hold anything
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) o[c][dt] *= corr[c];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+          bf16x8 vf = *reinterpret_cast<const bf16x8*>(vs_l + (dt * 16 + j) * VROW + s2 * 32 + qd * 8);
+          if (tail) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (base + 32 * s2 + 8 * qd + e >= len) vf[e] = static_cast<bf16>(0.f);
+          }
+#pragma unroll
+          for (int c = 0; c < 2; ++c)
+            o[c][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[c][s2], o[c][dt], 0, 0, 0);
+        }
+      }
     }
+    if (kt < kt_hi) store_tile(cur ^ 1);
+    __syncthreads();
   }
-  l += __shfl_xor(l, 16, WAVE);
-  l += __shfl_xor(l, 32, WAVE);
-  if (q_ok) {
-    bf16* orow = out + ((size_t)(start + pos_q) * n_heads + h) * HD;
-    const float inv_l = 1.0f / l;
 #pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
+  for (int c = 0; c < 2; ++c) {
+    float lt = l[c];
+    lt += __shfl_xor(lt, 16, WAVE);
+    lt += __shfl_xor(lt, 32, WAVE);
+    if (q_ok[c]) {
+      bf16* orow = out + ((size_t)(start + pos_q[c]) * n_heads + h) * HD;
+      const float inv_l = 1.0f / lt;
 #pragma unroll
-      for (int r = 0; r < 4; ++r) orow[dt * 16 + 4 * qd + r] = static_cast<bf16>(o[dt][r] * inv_l);
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) orow[dt * 16 + 4 * qd + r] = static_cast<bf16>(o[c][dt][r] * inv_l);
+    }
   }
 }
 
@@ -351,12 +400,13 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
                                 int n_kv_heads, int head_dim, int window, hipStream_t stream) {
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim)) return YALM_ERR_ARG;
   dim3 grid(n_tiles, n_heads);
+  const size_t lds = 2 * ((size_t)PAGE * (head_dim + 8) + (size_t)head_dim * (PAGE + 8)) * sizeof(bf16);
   if (head_dim == 128)
-    attn_prefill_mfma_kernel<128><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,
+    attn_prefill_mfma_kernel<128><<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)k_stage,
                                                             (const bf16*)v_stage, (bf16*)out, cu_seqlens, seq_tile0,
                                                             B, n_heads, n_kv_heads, window);
   else
-    attn_prefill_mfma_kernel<64><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,
+    attn_prefill_mfma_kernel<64><<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)k_stage,
                                                            (const bf16*)v_stage, (bf16*)out, cu_seqlens, seq_tile0, B,
                                                            n_heads, n_kv_heads, window);
   return launch_status();

@@ -5,8 +5,8 @@
 //    chunks of 128, every lane streaming 64 contiguous bytes of a weight row per
 //    chunk; the batch is the other MFMA operand (16 rows a tile, up to 4 tiles);
 //    partial sums of the waves meet in LDS, then the epilogue runs once.
-//  * gemm_tiled   (M > 64, prefill): 128x128x64 tiles through LDS with a register
-//    prefetch of the next tile, 4 waves of 64x64, v_mfma_f32_32x32x16_bf16.
+//  * gemm_tiled   (M > 64, prefill): 128x128x64 or 256x128x64 tiles through LDS with a
+//    register prefetch of the next tile, 4 waves, v_mfma_f32_32x32x16_bf16.
 //
 // Both take any M and N and any K that is a multiple of 8 (rows must be 16-byte
 // aligned); other shapes are refused so that the caller runs the float32-arithmetic kernel.
@@ -187,120 +187,124 @@ int skinny_dispatch(const bf16* X, const bf16* W, void* C, int M, int N, int K, 
 // ---------------------------------------------------------------------------
 // tiled GEMM
 // ---------------------------------------------------------------------------
-constexpr int TM = 128, TN = 128, TK = 64;
+constexpr int TK = 64;
 constexpr int LDS_ROW = TK + 8;                  // bf16 elements; 16 bytes of padding keep b128 reads off each other's banks
 
 // MFMA 32x32x16: operand rows i/j = lane % 32, 8 k per lane at k offset 8 * (lane / 32);
 // C: lane holds column j = lane % 32 and rows 8 * (r / 4) + 4 * (lane / 32) + r % 4 for r < 16.
-template <int EPI>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
-                                                         void* __restrict__ Cv, int M, int N, int K, int H) {
-  __shared__ __attribute__((aligned(16))) bf16 As[2][TM * LDS_ROW];
-  __shared__ __attribute__((aligned(16))) bf16 Ws[2][TN * LDS_ROW];
+// A workgroup of 4 waves (2 x 2) owns a TM x TN tile; a wave owns (TM/2) x (TN/2).
+// One LDS buffer: the next k tile waits in registers while this one is multiplied.
+template <int EPI, int TM, int TN, int NWM, int NWN, int MINW>
+__global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_tiled_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                            void* __restrict__ Cv, int M, int N, int K, int H) {
+  constexpr int NT = NWM * NWN * WAVE;
+  constexpr int WM = TM / NWM, WN = TN / NWN, FA = WM / 32, FB = WN / 32;
+  constexpr int RPP = NT / 8;                    // rows covered by one pass of all threads
+  constexpr int LA = TM / RPP, LB = TN / RPP;    // 16-byte chunks per thread and k tile
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16* As = reinterpret_cast<bf16*>(smem_raw);  // [TM][LDS_ROW]
+  bf16* Ws = As + TM * LDS_ROW;                  // [TN][LDS_ROW]
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
-  const int wm = wave / 2, wn = wave % 2;       // the wave's 64x64 quadrant
+  const int wm = wave / NWN, wn = wave % NWN;
   const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
   const int li = lane % 32, lh = lane / 32;
 
-  // global -> LDS: thread t carries 16 bytes of row (t / 8) + 32 p, p < 4, at k offset 8 * (t % 8)
+  // global -> LDS: thread t carries 16 bytes of row (t / 8) + RPP p at k offset 8 * (t % 8)
   const int lrow = tid / 8, lk = (tid % 8) * 8;
-  const bf16* ap[4];
-  const bf16* wp[4];
-  bool aok[4], wok[4];
+  const bf16* ap[LA];
+  const bf16* wp[LB];
+  bool aok[LA], wok[LB];
 #pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    int m = m0 + lrow + 32 * p, n = n0 + lrow + 32 * p;
+  for (int p = 0; p < LA; ++p) {
+    int m = m0 + lrow + RPP * p;
     aok[p] = m < M;
-    wok[p] = n < N;
     ap[p] = A + (size_t)(aok[p] ? m : 0) * K + lk;
+  }
+#pragma unroll
+  for (int p = 0; p < LB; ++p) {
+    int n = n0 + lrow + RPP * p;
+    wok[p] = n < N;
     wp[p] = W + (size_t)(wok[p] ? n : 0) * K + lk;
   }
 
-  f32x16 acc[2][2];
+  f32x16 acc[FA][FB];
 #pragma unroll
-  for (int a = 0; a < 2; ++a)
+  for (int a = 0; a < FA; ++a)
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int b = 0; b < FB; ++b)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
-  // rows of the W tile that feed the wave's two column tiles: plain, or for the gated
-  // epilogue tile 0 = the gate rows and tile 1 = the up rows of the wave's two blocks
-  int wrow_lds[2];
+  // rows of the W tile that feed the wave's column tiles: plain, or for the gated epilogue
+  // even tiles = the gate rows and odd tiles = the up rows of two 16-row blocks
+  int wrow_lds[FB];
 #pragma unroll
-  for (int b = 0; b < 2; ++b) {
+  for (int b = 0; b < FB; ++b) {
     if (EPI == 3)
-      wrow_lds[b] = wn * 64 + (li / 16) * 32 + b * 16 + (li % 16);
+      wrow_lds[b] = wn * WN + (b / 2) * 64 + (li / 16) * 32 + (b % 2) * 16 + (li % 16);
     else
-      wrow_lds[b] = wn * 64 + b * 32 + li;
+      wrow_lds[b] = wn * WN + b * 32 + li;
   }
 
-  bf16x8 ra[4], rw[4];
+  bf16x8 ra[LA], rw[LB];
   const int nk = (K + TK - 1) / TK;
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {
+  {
     bool kok = lk < K;
-    ra[p] = load8(ap[p], aok[p] && kok);
-    rw[p] = load8(wp[p], wok[p] && kok);
-  }
 #pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    *reinterpret_cast<bf16x8*>(&As[0][(lrow + 32 * p) * LDS_ROW + lk]) = ra[p];
-    *reinterpret_cast<bf16x8*>(&Ws[0][(lrow + 32 * p) * LDS_ROW + lk]) = rw[p];
+    for (int p = 0; p < LA; ++p) ra[p] = load8(ap[p], aok[p] && kok);
+#pragma unroll
+    for (int p = 0; p < LB; ++p) rw[p] = load8(wp[p], wok[p] && kok);
   }
-  __syncthreads();
-
   for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) {
-      int k = (kt + 1) * TK + lk;
-      bool kok = k < K;
 #pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        ra[p] = load8(ap[p] + (size_t)(kt + 1) * TK, aok[p] && kok);
-        rw[p] = load8(wp[p] + (size_t)(kt + 1) * TK, wok[p] && kok);
-      }
+    for (int p = 0; p < LA; ++p) *reinterpret_cast<bf16x8*>(&As[(lrow + RPP * p) * LDS_ROW + lk]) = ra[p];
+#pragma unroll
+    for (int p = 0; p < LB; ++p) *reinterpret_cast<bf16x8*>(&Ws[(lrow + RPP * p) * LDS_ROW + lk]) = rw[p];
+    __syncthreads();
+    if (kt + 1 < nk) {
+      bool kok = (kt + 1) * TK + lk < K;
+#pragma unroll
+      for (int p = 0; p < LA; ++p) ra[p] = load8(ap[p] + (size_t)(kt + 1) * TK, aok[p] && kok);
+#pragma unroll
+      for (int p = 0; p < LB; ++p) rw[p] = load8(wp[p] + (size_t)(kt + 1) * TK, wok[p] && kok);
     }
 #pragma unroll
     for (int ks = 0; ks < TK / 16; ++ks) {
-      bf16x8 fa[2], fw[2];
+      bf16x8 fa[FA], fw[FB];
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
-        fa[a] = *reinterpret_cast<const bf16x8*>(&As[cur][(wm * 64 + a * 32 + li) * LDS_ROW + ks * 16 + lh * 8]);
+      for (int a = 0; a < FA; ++a)
+        fa[a] = *reinterpret_cast<const bf16x8*>(&As[(wm * WM + a * 32 + li) * LDS_ROW + ks * 16 + lh * 8]);
 #pragma unroll
-      for (int b = 0; b < 2; ++b)
-        fw[b] = *reinterpret_cast<const bf16x8*>(&Ws[cur][wrow_lds[b] * LDS_ROW + ks * 16 + lh * 8]);
+      for (int b = 0; b < FB; ++b)
+        fw[b] = *reinterpret_cast<const bf16x8*>(&Ws[wrow_lds[b] * LDS_ROW + ks * 16 + lh * 8]);
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
+      for (int a = 0; a < FA; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < FB; ++b)
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[a], fw[b], acc[a][b], 0, 0, 0);
-    }
-    if (kt + 1 < nk) {
-#pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        *reinterpret_cast<bf16x8*>(&As[cur ^ 1][(lrow + 32 * p) * LDS_ROW + lk]) = ra[p];
-        *reinterpret_cast<bf16x8*>(&Ws[cur ^ 1][(lrow + 32 * p) * LDS_ROW + lk]) = rw[p];
-      }
     }
     __syncthreads();
   }
 
   // epilogue
 #pragma unroll
-  for (int a = 0; a < 2; ++a) {
+  for (int a = 0; a < FA; ++a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      int m = m0 + wm * 64 + a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+      int m = m0 + wm * WM + a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
       if (m >= M) continue;
       if (EPI == 3) {
-        int hcol = (n0 + wn * 64) / 2 + li;
-        if (hcol < H)
-          ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(acc[a][0][r]) * acc[a][1][r]);
+#pragma unroll
+        for (int pp = 0; pp < FB / 2; ++pp) {
+          int hcol = (n0 + wn * WN + pp * 64) / 2 + li;
+          if (hcol < H)
+            ((bf16*)Cv)[(size_t)m * H + hcol] =
+                static_cast<bf16>(silu_f(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
+        }
       } else {
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-          int n = n0 + wn * 64 + b * 32 + li;
+        for (int b = 0; b < FB; ++b) {
+          int n = n0 + wn * WN + b * 32 + li;
           if (n >= N) continue;
           size_t o = (size_t)m * N + n;
           if (EPI == 0) ((float*)Cv)[o] = acc[a][b][r];
@@ -312,11 +316,20 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16* __restrict_
   }
 }
 
+template <int EPI, int TM, int TN, int NWM, int NWN, int MINW>
+int tiled_launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
+  dim3 grid(ceil_div(N, TN), ceil_div(M, TM));
+  size_t lds = (size_t)(TM + TN) * LDS_ROW * sizeof(bf16);
+  gemm_tiled_kernel<EPI, TM, TN, NWM, NWN, MINW><<<grid, NWM * NWN * WAVE, lds, stream>>>(A, W, C, M, N, K, H);
+  return launch_status();
+}
+
 template <int EPI>
 int tiled_launch(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
-  dim3 grid(ceil_div(N, TN), ceil_div(M, TM));
-  gemm_tiled_kernel<EPI><<<grid, 256, 0, stream>>>(A, W, C, M, N, K, H);
-  return launch_status();
+  // 256x128 tiles move fewer bytes per flop; 128x128 tiles where those would not fill the chip
+  if ((long)ceil_div(M, 256) * ceil_div(N, 128) > 1024)
+    return tiled_launch_shape<EPI, 256, 128, 2, 2, 2>(A, W, C, M, N, K, H, stream);
+  return tiled_launch_shape<EPI, 128, 128, 2, 2, 2>(A, W, C, M, N, K, H, stream);
 }
 
 }  // namespace
