@@ -479,3 +479,42 @@ def test_gemm_norm_qkv_rope(n_heads, n_kv, hd, rd, D):
         touched[page, r] = True
     assert (kp.float().abs().sum(dim=(1, 3)) > 0).equal(touched)
     assert (vp.float().abs().sum(dim=(1, 2)) > 0).equal(touched)
+
+
+@pytest.mark.parametrize("M,N,Kd", [(1, 64, 256), (8, 4096, 1000), (33, 80, 96), (64, 4096, 264), (5, 16400, 64)])
+def test_gemm_chain_producer_and_consumer(M, N, Kd):
+    """A residual-add GEMM that emits the next norm's activations and partial sums of squares,
+    and a consumer that scales by them: together they equal rmsnorm(x_new) @ W2^T."""
+    k = K()
+    a = rnd((M, Kd), 60, torch.bfloat16)
+    w = rnd((N, Kd), 61, torch.bfloat16, scale=1 / math.sqrt(Kd))
+    res = rnd((M, N), 62, scale=2.0)
+    nw = 1 + 0.1 * rnd((N,), 63)
+    x = res.to(DEV).clone()
+    if N >= 16384:                                      # too wide to emit: refused
+        with pytest.raises(Exception):
+            k.gemm_chain(a.to(DEV), w.to(DEV), x, k.EPI_ADD_F32,
+                         emit=(nw.to(DEV), torch.empty((M, N), dtype=torch.bfloat16, device=DEV),
+                               torch.empty((M, k.gemm_chain_parts(N)), device=DEV)))
+        return
+    xn = torch.zeros((M, N), dtype=torch.bfloat16, device=DEV)
+    ss = torch.zeros((M, k.gemm_chain_parts(N)), device=DEV)
+    k.gemm_chain(a.to(DEV), w.to(DEV), x, k.EPI_ADD_F32, emit=(nw.to(DEV), xn, ss))
+    x_want = res.double() + a.double() @ w.double().T
+    close(x, x_want, torch.float32, "residual")
+    close(xn, x_want * nw.double(), torch.bfloat16, "emitted activations")
+    assert torch.allclose(ss.sum(dim=1).cpu().double(), (x_want ** 2).sum(dim=1), rtol=1e-5)
+    # consumers: float32 store and gated
+    H = 48
+    from yalm_amd.parts.swiglu import interleave_gate_up
+    w2 = rnd((70, N), 64, torch.bfloat16, scale=1 / math.sqrt(N))
+    out = torch.empty((M, 70), device=DEV)
+    k.gemm_chain(xn, w2.to(DEV), out, k.EPI_STORE_F32, scale_from=(ss, 1e-5))
+    want = R.rmsnorm(x_want, nw, 1e-5) @ w2.double().T
+    close(out, want, torch.bfloat16, "chained consumer", factor=1.5)
+    wg = rnd((H, N), 65, torch.bfloat16, scale=1 / math.sqrt(N))
+    wu = rnd((H, N), 66, torch.bfloat16, scale=1 / math.sqrt(N))
+    outg = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
+    k.gemm_chain(xn, interleave_gate_up(wg, wu).to(DEV), outg, k.EPI_GATED, hidden=H, scale_from=(ss, 1e-5))
+    h = R.rmsnorm(x_want, nw, 1e-5)
+    close(outg, R.silu(h @ wg.double().T) * (h @ wu.double().T), torch.bfloat16, "chained gated", factor=2.0)

@@ -12,28 +12,14 @@
 // Same structure as gemm_skinny_kernel: 16 or 32 weight rows a workgroup, the
 // waves split K in chunks of 128, partial sums meet in LDS.
 #include "common.h"
+#include "skinny_gemm.h"
 #include "yalm_hip.h"
 
 namespace {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+using namespace skinny;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
-
-struct RopeArgs {
-  bf16* q_out;
-  bf16* k_pages;
-  bf16* v_pages;
-  const int* block_table;
-  const int* tok_pos;
-  const int* seq_slot;
-  const float2* cos_sin;
-  int table_stride, ring_pages, n_positions, n_heads, n_kv_heads, hd, rotary_dim, n_pages;
-};
-
-constexpr int EPI_F32 = 0, EPI_GATED = 3, EPI_ROPE = 4;
 constexpr int MAX_ROWS = 8;                      // rows of the step (sequences of a decode batch)
 
 // LDS: the normalised activations xs[M][K + 8] as bfloat16 (dynamic), then the partial sums.
@@ -227,7 +213,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_norm_kernel(const float* _
 }
 
 template <int EPI>
-int launch(const float* X, const float* norm_w, float eps, const bf16* W, void* C, int M, int N, int K, int H,
+int launch_norm(const float* X, const float* norm_w, float eps, const bf16* W, void* C, int M, int N, int K, int H,
            const RopeArgs& ra, hipStream_t stream) {
   bool wide = EPI == EPI_GATED || N >= 16384;
   size_t lds = (size_t)M * (K + 8) * sizeof(bf16);
@@ -249,10 +235,10 @@ extern "C" int yalm_gemm_norm(const float* x, const float* norm_w, float eps, co
                               int K, int epilogue, int H, hipStream_t stream) {
   if (!shape_ok(x, norm_w, W, M, N, K)) return YALM_ERR_ARG;
   RopeArgs ra = {};
-  if (epilogue == EPI_F32) return launch<EPI_F32>(x, norm_w, eps, (const bf16*)W, C, M, N, K, H, ra, stream);
+  if (epilogue == EPI_F32) return launch_norm<EPI_F32>(x, norm_w, eps, (const bf16*)W, C, M, N, K, H, ra, stream);
   if (epilogue == EPI_GATED) {
     if (H <= 0 || N != 32 * ((H + 15) / 16)) return YALM_ERR_ARG;
-    return launch<EPI_GATED>(x, norm_w, eps, (const bf16*)W, C, M, N, K, H, ra, stream);
+    return launch_norm<EPI_GATED>(x, norm_w, eps, (const bf16*)W, C, M, N, K, H, ra, stream);
   }
   return YALM_ERR_ARG;
 }
@@ -283,5 +269,77 @@ extern "C" int yalm_gemm_norm_qkv_rope(const float* x, const float* norm_w, floa
   ra.hd = head_dim;
   ra.rotary_dim = rotary_dim;
   ra.n_pages = n_pages;
-  return launch<EPI_ROPE>(x, norm_w, eps, (const bf16*)Wqkv, nullptr, M, N, K, 0, ra, stream);
+  return launch_norm<EPI_ROPE>(x, norm_w, eps, (const bf16*)Wqkv, nullptr, M, N, K, 0, ra, stream);
 }
+
+// ---------------------------------------------------------------------------
+// chained decode GEMMs (skinny_gemm.h): bfloat16 activations that a producer emitted
+// already multiplied by the norm weights, scaled here per row; and the producer side
+// ---------------------------------------------------------------------------
+extern "C" int yalm_gemm_chain(const void* X, const void* W, void* C, int M, int N, int K, int epilogue, int H,
+                               const float* ss_in, int n_parts_in, float eps, const float* emit_nw, void* emit_xn,
+                               float* emit_ss, hipStream_t stream) {
+  if (M < 1 || M > 64 || N <= 0 || K <= 0 || K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)W & 15))
+    return YALM_ERR_ARG;
+  if (ss_in != nullptr && n_parts_in <= 0) return YALM_ERR_ARG;
+  ChainArgs ca = {};
+  ca.ss_in = ss_in;
+  ca.n_parts_in = n_parts_in;
+  ca.eps = eps;
+  const bf16* x = (const bf16*)X;
+  const bf16* w = (const bf16*)W;
+  if (epilogue == EPI_ADD) {
+    if (emit_nw != nullptr) {
+      if (emit_xn == nullptr || emit_ss == nullptr || N >= 16384) return YALM_ERR_ARG;
+      ca.emit_nw = emit_nw;
+      ca.emit_xn = (bf16*)emit_xn;
+      ca.emit_ss = emit_ss;
+    }
+    return skinny::launch<EPI_ADD>(x, w, C, M, N, K, H, ca, stream);
+  }
+  if (emit_nw != nullptr) return YALM_ERR_ARG;
+  if (epilogue == EPI_F32) return skinny::launch<EPI_F32>(x, w, C, M, N, K, H, ca, stream);
+  if (epilogue == EPI_GATED) {
+    if (H <= 0 || N != 32 * ((H + 15) / 16)) return YALM_ERR_ARG;
+    return skinny::launch<EPI_GATED>(x, w, C, M, N, K, H, ca, stream);
+  }
+  return YALM_ERR_ARG;
+}
+
+extern "C" int yalm_gemm_chain_qkv_rope(const void* X, const float* ss_in, int n_parts_in, float eps,
+                                        const void* Wqkv, void* q_out, void* k_pages, void* v_pages,
+                                        const int* block_table, int table_stride, int ring_pages,
+                                        const int* tok_pos, const int* seq_slot, const float* cos_sin,
+                                        int n_positions, int M, int K, int n_heads, int n_kv_heads, int head_dim,
+                                        int rotary_dim, int n_pages, hipStream_t stream) {
+  const int N = (n_heads + 2 * n_kv_heads) * head_dim;
+  if (M < 1 || M > 64 || K <= 0 || K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wqkv & 15) || ss_in == nullptr ||
+      n_parts_in <= 0)
+    return YALM_ERR_ARG;
+  if (head_dim <= 0 || head_dim % 16 != 0 || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > head_dim ||
+      n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || n_pages <= 0)
+    return YALM_ERR_ARG;
+  ChainArgs ca = {};
+  ca.ss_in = ss_in;
+  ca.n_parts_in = n_parts_in;
+  ca.eps = eps;
+  RopeArgs& ra = ca.ra;
+  ra.q_out = (bf16*)q_out;
+  ra.k_pages = (bf16*)k_pages;
+  ra.v_pages = (bf16*)v_pages;
+  ra.block_table = block_table;
+  ra.tok_pos = tok_pos;
+  ra.seq_slot = seq_slot;
+  ra.cos_sin = (const float2*)cos_sin;
+  ra.table_stride = table_stride;
+  ra.ring_pages = ring_pages;
+  ra.n_positions = n_positions;
+  ra.n_heads = n_heads;
+  ra.n_kv_heads = n_kv_heads;
+  ra.hd = head_dim;
+  ra.rotary_dim = rotary_dim;
+  ra.n_pages = n_pages;
+  return skinny::launch<EPI_ROPE>((const bf16*)X, (const bf16*)Wqkv, nullptr, M, N, K, 0, ca, stream);
+}
+
+extern "C" int yalm_gemm_chain_parts(int N) { return skinny::parts_of(N); }

@@ -11,6 +11,7 @@
 // Both take any M and N and any K that is a multiple of 8 (rows must be 16-byte
 // aligned); other shapes are refused so that the caller runs the float32-arithmetic kernel.
 #include "common.h"
+#include "skinny_gemm.h"
 #include "yalm_hip.h"
 
 namespace {
@@ -27,161 +28,12 @@ __device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
 }
 
 // ---------------------------------------------------------------------------
-// skinny GEMM
+// skinny GEMM: see skinny_gemm.h
 // ---------------------------------------------------------------------------
-// MFMA 16x16x32: operand A = activations (row i = batch row, 8 k per lane), operand
-// B = weights (column j = weight row, 8 k per lane); C[i][j]: lane (q = lane/16,
-// j = lane%16) holds batch rows 4q..4q+3 of weight row j.  Which k a lane's slot
-// holds is the same for both operands, so any assignment of k to slots is right;
-// here step s of a chunk takes k = kc + 32 s + 8 q ... + 8, so that the four lane groups of
-// a weight row read 64 contiguous bytes per load.
-template <int MT, int NT, int NWAVES, int EPI, int KS>
-__global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ X,
-                                                                     const bf16* __restrict__ W,
-                                                                     void* __restrict__ Cv, int M, int N, int K,
-                                                                     int H) {
-  constexpr int KC = 32 * KS;                    // k per wave iteration
-  __shared__ f32x4 red[NWAVES][MT * NT][WAVE];
-  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  const int q = lane / 16, j = lane % 16;
-  const int n0 = blockIdx.x * 16 * NT;
-
-  const bf16* wrow[NT];
-  bool wok[NT];
-#pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    int n = n0 + t * 16 + j;
-    wok[t] = n < N;
-    wrow[t] = W + (size_t)(wok[t] ? n : 0) * K;
-  }
-  const bf16* xrow[MT];
-  bool xok[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    int m = mt * 16 + j;
-    xok[mt] = m < M;
-    xrow[mt] = X + (size_t)(xok[mt] ? m : 0) * K;
-  }
-
-  f32x4 acc[MT][NT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int t = 0; t < NT; ++t) acc[mt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-  bf16x8 wv[NT][KS], xv[MT][KS];
-  int kc = wave * KC;
-  if (kc < K) {
-#pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      int k = kc + s * 32 + q * 8;
-      bool ok = k < K;
-#pragma unroll
-      for (int t = 0; t < NT; ++t) wv[t][s] = load8(wrow[t] + k, ok && wok[t]);
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) xv[mt][s] = load8(xrow[mt] + k, ok && xok[mt]);
-    }
-  }
-  for (; kc < K; kc += NWAVES * KC) {
-    bf16x8 wn[NT][KS], xn[MT][KS];
-    int kn = kc + NWAVES * KC;
-    if (kn < K) {                                // prefetch the wave's next chunk
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        int k = kn + s * 32 + q * 8;
-        bool ok = k < K;
-#pragma unroll
-        for (int t = 0; t < NT; ++t) wn[t][s] = load8(wrow[t] + k, ok && wok[t]);
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xn[mt][s] = load8(xrow[mt] + k, ok && xok[mt]);
-      }
-    }
-#pragma unroll
-    for (int s = 0; s < KS; ++s)
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-        for (int t = 0; t < NT; ++t)
-          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
-    if (kn < K) {
-#pragma unroll
-      for (int s = 0; s < KS; ++s) {
-#pragma unroll
-        for (int t = 0; t < NT; ++t) wv[t][s] = wn[t][s];
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xv[mt][s] = xn[mt][s];
-      }
-    }
-  }
-
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int t = 0; t < NT; ++t) red[wave][mt * NT + t][lane] = acc[mt][t];
-  __syncthreads();
-
-  constexpr int NTP = (EPI == 3) ? NT / 2 : NT;  // gated: a gate tile and its up tile finish together
-  for (int idx = wave; idx < MT * NTP; idx += NWAVES) {
-    const int mt = idx / NTP, tp = idx % NTP;
-    if (EPI == 3) {
-      f32x4 g = (f32x4){0.f, 0.f, 0.f, 0.f}, u = g;
-#pragma unroll
-      for (int w = 0; w < NWAVES; ++w) {
-        g += red[w][mt * NT + 2 * tp][lane];
-        u += red[w][mt * NT + 2 * tp + 1][lane];
-      }
-      int hcol = (n0 / 32 + tp) * 16 + j;
-      bf16* C = (bf16*)Cv;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        int m = mt * 16 + 4 * q + r;
-        if (m < M && hcol < H) C[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(g[r]) * u[r]);
-      }
-    } else {
-      f32x4 v = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int w = 0; w < NWAVES; ++w) v += red[w][mt * NT + tp][lane];
-      int n = n0 + tp * 16 + j;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        int m = mt * 16 + 4 * q + r;
-        if (m < M && n < N) {
-          size_t o = (size_t)m * N + n;
-          if (EPI == 0) ((float*)Cv)[o] = v[r];
-          if (EPI == 1) ((bf16*)Cv)[o] = static_cast<bf16>(v[r]);
-          if (EPI == 2) ((float*)Cv)[o] += v[r];
-        }
-      }
-    }
-  }
-}
-
-template <int MT, int EPI>
-int skinny_launch(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
-  // few weight rows: 16 rows and 8 waves a workgroup, so that every CU has work;
-  // many: 64 rows (32 if the batch needs the registers) and 4 waves
-  bool wide = EPI == 3 || N >= 16384;
-  if (wide) {
-    if (MT <= 2)
-      gemm_skinny_kernel<MT, 4, 4, EPI, 4><<<ceil_div(N, 64), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H);
-    else
-      gemm_skinny_kernel<MT, 2, 4, EPI, 4><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H);
-  } else {
-    constexpr int E = EPI == 3 ? 0 : EPI;
-    gemm_skinny_kernel<MT, 1, 8, E, 4><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H);
-  }
-  return launch_status();
-}
-
 template <int EPI>
 int skinny_dispatch(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
-  switch ((M + 15) / 16) {
-    case 1: return skinny_launch<1, EPI>(X, W, C, M, N, K, H, stream);
-    case 2: return skinny_launch<2, EPI>(X, W, C, M, N, K, H, stream);
-    case 3: return skinny_launch<3, EPI>(X, W, C, M, N, K, H, stream);
-    case 4: return skinny_launch<4, EPI>(X, W, C, M, N, K, H, stream);
-  }
-  return YALM_ERR_ARG;
+  skinny::ChainArgs ca = {};
+  return skinny::launch<EPI>(X, W, C, M, N, K, H, ca, stream);
 }
 
 // ---------------------------------------------------------------------------

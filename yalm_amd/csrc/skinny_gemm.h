@@ -1,0 +1,299 @@
+// The decode GEMM (at most 64 rows) on the matrix cores, shared by gemm_mfma.hip and
+// gemm_fused.hip:  C = epilogue(row_scale * (X[M,K] * W[N,K]^T)), bfloat16 operands,
+// float32 accumulation.  It is bound by the one pass over the weights.  A workgroup owns
+// 16 * NT weight rows and all of K; its waves split K in chunks of 32 * KS, every lane
+// streaming 16 bytes of a weight row per load (the four lane groups of a row read 64
+// contiguous bytes); the batch is the other MFMA operand (16 rows a tile, MT tiles);
+// partial sums of the waves meet in LDS, then the epilogue runs once.
+//
+// Chaining norms through the GEMMs of a decode step: a producer with the residual-add
+// epilogue can also emit, for the NEXT RMSNorm, the activations bfloat16(x * w_norm) and
+// the partial sums of squares of its columns; a consumer given those scales its float32
+// sums by rsqrt(mean(x^2) + eps) per row.  No norm kernel runs in between, and the sums
+// are added in a fixed order.
+#pragma once
+#include "common.h"
+
+namespace skinny {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+__device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
+  bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+  return ok ? *reinterpret_cast<const bf16x8*>(p) : z;
+}
+
+constexpr int EPI_F32 = 0, EPI_STORE = 1, EPI_ADD = 2, EPI_GATED = 3, EPI_ROPE = 4;
+
+struct RopeArgs {                                // epilogue of the fused q/k/v projection
+  bf16* q_out;
+  bf16* k_pages;
+  bf16* v_pages;
+  const int* block_table;
+  const int* tok_pos;
+  const int* seq_slot;
+  const float2* cos_sin;
+  int table_stride, ring_pages, n_positions, n_heads, n_kv_heads, hd, rotary_dim, n_pages;
+};
+
+struct ChainArgs {
+  const float* ss_in;                            // [M][n_parts_in] partial sums of squares, or null: no row scale
+  int n_parts_in;
+  float eps;
+  const float* emit_nw;                          // EPI_ADD only: float32 norm weights [N], or null
+  bf16* emit_xn;                                 // [M][N] = bfloat16(x_new * emit_nw)
+  float* emit_ss;                                // [M][gridDim.x] sums of squares of this workgroup's columns
+  RopeArgs ra;
+};
+
+// MFMA 16x16x32: operand A = activations (row i = batch row, 8 k per lane), operand
+// B = weights (column j = weight row, 8 k per lane); C[i][j]: lane (q = lane/16,
+// j = lane%16) holds batch rows 4q..4q+3 of weight row j.  Which k a lane's slot
+// holds is the same for both operands, so any assignment of k to slots is right;
+// here step s of a chunk takes k = kc + 32 s + 8 q ... + 8.
+template <int MT, int NT, int NWAVES, int EPI, int KS>
+__global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ X,
+                                                                     const bf16* __restrict__ W,
+                                                                     void* __restrict__ Cv, int M, int N, int K,
+                                                                     int H, ChainArgs ca) {
+  constexpr int KC = 32 * KS;                    // k per wave iteration
+  __shared__ f32x4 red[NWAVES][MT * NT][WAVE];
+  __shared__ float sm_scale[MT * 16];
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const int q = lane / 16, j = lane % 16;
+  const int n0 = blockIdx.x * 16 * NT;
+
+  const bf16* wrow[NT];
+  bool wok[NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    int n = n0 + t * 16 + j;
+    wok[t] = n < N;
+    wrow[t] = W + (size_t)(wok[t] ? n : 0) * K;
+  }
+  const bf16* xrow[MT];
+  bool xok[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    int m = mt * 16 + j;
+    xok[mt] = m < M;
+    xrow[mt] = X + (size_t)(xok[mt] ? m : 0) * K;
+  }
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) acc[mt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  bf16x8 wv[NT][KS], xv[MT][KS];
+  int kc = wave * KC;
+  if (kc < K) {
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      int k = kc + s * 32 + q * 8;
+      bool ok = k < K;
+#pragma unroll
+      for (int t = 0; t < NT; ++t) wv[t][s] = load8(wrow[t] + k, ok && wok[t]);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) xv[mt][s] = load8(xrow[mt] + k, ok && xok[mt]);
+    }
+  }
+
+  // row scales from the producer's partial sums of squares (a wave per row, lanes over the parts)
+  if (ca.ss_in != nullptr) {
+    for (int m = wave; m < MT * 16; m += NWAVES) {
+      float s = 0.f;
+      if (m < M)
+        for (int p = lane; p < ca.n_parts_in; p += WAVE) s += ca.ss_in[(size_t)m * ca.n_parts_in + p];
+      s = wave_sum(s);
+      if (lane == 0) sm_scale[m] = 1.0f / sqrtf(s / (float)K + ca.eps);
+    }
+  }
+
+  for (; kc < K; kc += NWAVES * KC) {
+    bf16x8 wn[NT][KS], xn[MT][KS];
+    int kn = kc + NWAVES * KC;
+    if (kn < K) {                                // prefetch the wave's next chunk
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+        int k = kn + s * 32 + q * 8;
+        bool ok = k < K;
+#pragma unroll
+        for (int t = 0; t < NT; ++t) wn[t][s] = load8(wrow[t] + k, ok && wok[t]);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xn[mt][s] = load8(xrow[mt] + k, ok && xok[mt]);
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < KS; ++s)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
+    if (kn < K) {
+#pragma unroll
+      for (int s = 0; s < KS; ++s) {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) wv[t][s] = wn[t][s];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xv[mt][s] = xn[mt][s];
+      }
+    }
+  }
+
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NT; ++t) red[wave][mt * NT + t][lane] = acc[mt][t];
+  __syncthreads();
+
+  const bool scaled = ca.ss_in != nullptr;
+  constexpr int NTP = (EPI == EPI_GATED) ? NT / 2 : NT;  // gated: a gate tile and its up tile finish together
+  for (int idx = wave; idx < MT * NTP; idx += NWAVES) {
+    const int mt = idx / NTP, tp = idx % NTP;
+    float scale[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) scale[r] = scaled ? sm_scale[mt * 16 + 4 * q + r] : 1.0f;
+    if (EPI == EPI_GATED) {
+      f32x4 g = (f32x4){0.f, 0.f, 0.f, 0.f}, u = g;
+#pragma unroll
+      for (int w = 0; w < NWAVES; ++w) {
+        g += red[w][mt * NT + 2 * tp][lane];
+        u += red[w][mt * NT + 2 * tp + 1][lane];
+      }
+      int hcol = (n0 / 32 + tp) * 16 + j;
+      bf16* C = (bf16*)Cv;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        int m = mt * 16 + 4 * q + r;
+        if (m < M && hcol < H)
+          C[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(g[r] * scale[r]) * (u[r] * scale[r]));
+      }
+      continue;
+    }
+    f32x4 v = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < NWAVES; ++w) v += red[w][mt * NT + tp][lane];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) v[r] *= scale[r];
+    const int n = n0 + tp * 16 + j;
+    if (EPI == EPI_F32 || EPI == EPI_STORE) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        int m = mt * 16 + 4 * q + r;
+        if (m < M && n < N) {
+          size_t o = (size_t)m * N + n;
+          if (EPI == EPI_F32) ((float*)Cv)[o] = v[r];
+          if (EPI == EPI_STORE) ((bf16*)Cv)[o] = static_cast<bf16>(v[r]);
+        }
+      }
+    } else if (EPI == EPI_ADD) {
+      const bool emit = ca.emit_nw != nullptr;   // NT == 1 then (the launcher sees to it)
+      const float nw = (emit && n < N) ? ca.emit_nw[n] : 0.f;
+      float sq[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        int m = mt * 16 + 4 * q + r;
+        sq[r] = 0.f;
+        if (m < M && n < N) {
+          size_t o = (size_t)m * N + n;
+          float y = ((float*)Cv)[o] + v[r];
+          ((float*)Cv)[o] = y;
+          if (emit) {
+            ca.emit_xn[o] = static_cast<bf16>(y * nw);
+            sq[r] = y * y;
+          }
+        }
+      }
+      if (emit) {                                // sums over the 16 columns of the tile: lanes j of one lane group
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float t = sq[r];
+          t += __shfl_xor(t, 1, WAVE);
+          t += __shfl_xor(t, 2, WAVE);
+          t += __shfl_xor(t, 4, WAVE);
+          t += __shfl_xor(t, 8, WAVE);
+          int m = mt * 16 + 4 * q + r;
+          if (j == 0 && m < M) ca.emit_ss[(size_t)m * gridDim.x + blockIdx.x] = t;
+        }
+      }
+    } else {                                      // EPI_ROPE: n runs over [q heads | k heads | v heads]
+      const RopeArgs& ra = ca.ra;
+      f32x4 other;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) other[r] = __shfl_xor(v[r], 1, WAVE);   // the pair partner sits in the next lane
+      const int Q = ra.n_heads * ra.hd, KV = ra.n_kv_heads * ra.hd;
+      if (n < N) {
+        const int region = n < Q ? 0 : (n < Q + KV ? 1 : 2);
+        const int nn = n - (region == 0 ? 0 : (region == 1 ? Q : Q + KV));
+        const int head = nn / ra.hd, i = nn % ra.hd, p = i >> 1;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int m = mt * 16 + 4 * q + r;
+          if (m >= M) continue;
+          const int pos = ra.tok_pos[m];
+          float y = v[r];
+          if (region < 2 && ra.cos_sin != nullptr && p < ra.rotary_dim / 2 && pos >= 0 && pos < ra.n_positions) {
+            const float2 c = ra.cos_sin[(size_t)pos * (ra.rotary_dim / 2) + p];
+            y = (i & 1) ? other[r] * c.y + v[r] * c.x : v[r] * c.x - other[r] * c.y;
+          }
+          const bf16 yb = static_cast<bf16>(y);
+          if (region == 0) {
+            ra.q_out[(size_t)m * Q + n] = yb;
+          } else {
+            const int slot = ra.seq_slot[m];
+            if (slot < 0 || pos < 0) continue;
+            const int phys = ra.block_table[(size_t)slot * ra.table_stride + (pos / PAGE) % ra.ring_pages];
+            if (phys < 0 || phys >= ra.n_pages) continue;
+            const size_t base = ((size_t)phys * ra.n_kv_heads + head) * PAGE * ra.hd;
+            const int row = pos & (PAGE - 1);
+            if (region == 1)
+              ra.k_pages[base + (size_t)row * ra.hd + i] = yb;
+            else
+              ra.v_pages[base + (size_t)i * PAGE + row] = yb;
+          }
+        }
+      }
+    }
+  }
+}
+
+// few weight rows: 16 rows and 8 waves a workgroup, so that every CU has work;
+// many: 64 rows (32 if the batch needs the registers) and 4 waves
+template <int MT, int EPI>
+int launch_mt(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, const ChainArgs& ca,
+              hipStream_t stream) {
+  const bool wide = EPI == EPI_GATED || (N >= 16384 && ca.emit_nw == nullptr);
+  if (wide) {
+    if (MT <= 2)
+      gemm_skinny_kernel<MT, 4, 4, EPI, 4><<<ceil_div(N, 64), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
+    else
+      gemm_skinny_kernel<MT, 2, 4, EPI, 4><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
+  } else {
+    constexpr int E = EPI == EPI_GATED ? EPI_F32 : EPI;
+    gemm_skinny_kernel<MT, 1, 8, E, 4><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
+  }
+  return launch_status();
+}
+
+template <int EPI>
+int launch(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, const ChainArgs& ca,
+           hipStream_t stream) {
+  switch ((M + 15) / 16) {
+    case 1: return launch_mt<1, EPI>(X, W, C, M, N, K, H, ca, stream);
+    case 2: return launch_mt<2, EPI>(X, W, C, M, N, K, H, ca, stream);
+    case 3: return launch_mt<3, EPI>(X, W, C, M, N, K, H, ca, stream);
+    case 4: return launch_mt<4, EPI>(X, W, C, M, N, K, H, ca, stream);
+  }
+  return YALM_ERR_ARG;
+}
+
+// workgroups along N of a launch without the gated epilogue (the number of emitted parts)
+inline int parts_of(int N) { return ceil_div(N, 16); }
+
+}  // namespace skinny

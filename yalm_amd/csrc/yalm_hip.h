@@ -49,6 +49,23 @@ int yalm_gemm_norm_qkv_rope(const float* x, const float* norm_w, float eps, cons
                             int K, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, int n_pages,
                             hipStream_t stream);
 
+// Decode GEMMs (M <= 64, bfloat16) that chain norms without a norm kernel in between.
+// Producer: epilogue 2 (C float32 += product) with emit_nw given also writes
+// emit_xn[M,N] = bfloat16(C_new * emit_nw[n]) and emit_ss[M, parts] = sums of squares of
+// C_new over the columns of each workgroup (parts = yalm_gemm_chain_parts(N), N < 16384).
+// Consumer: X is such an emit_xn; with ss_in [M, n_parts_in] the float32 sums are scaled by
+// rsqrt(sum(ss_in[m, :]) / K + eps) per row before the epilogue (0: float32 store, 2, 3: gated).
+int yalm_gemm_chain(const void* X, const void* W, void* C, int M, int N, int K, int epilogue, int H,
+                    const float* ss_in, int n_parts_in, float eps, const float* emit_nw, void* emit_xn,
+                    float* emit_ss, hipStream_t stream);
+int yalm_gemm_chain_parts(int N);
+// The consumer form of the fused q/k/v projection with rotation and cache write (see yalm_gemm_norm_qkv_rope).
+int yalm_gemm_chain_qkv_rope(const void* X, const float* ss_in, int n_parts_in, float eps, const void* Wqkv,
+                             void* q_out, void* k_pages, void* v_pages, const int* block_table, int table_stride,
+                             int ring_pages, const int* tok_pos, const int* seq_slot, const float* cos_sin,
+                             int n_positions, int M, int K, int n_heads, int n_kv_heads, int head_dim,
+                             int rotary_dim, int n_pages, hipStream_t stream);
+
 // Rotates q and k of every token (adjacent pairs, angles from the table), writes q,
 // optionally k and v into a staging area in page format (for attention over the step's
 // own tokens: tile seq_tile0[sequence] + position / PAGE), and k and v into the pages

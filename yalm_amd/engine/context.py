@@ -61,6 +61,7 @@ class StepContext:
         self.tokens = self.tok_seq = self.tok_pos = self.seq_slot = self.seq_len = self.cu_seqlens = None
         self.seq_tile0 = None
         self.n_tiles = 0
+        self.normed = {}                  # id(norm part) -> (xn, ss, eps): activations a producer emitted for it
         self.pages_bucket = 1 << 30       # decode: no sequence of the step has more pages than this
         self.max_position = 0
         self.host_slots = []

@@ -37,6 +37,8 @@ class Model:
         self.final_norm = build_part("norm", spec.final_norm, spec.dim, "")
         self.head = build_part("head", spec.head, spec.dim, "", embedding=self.embedding)
         self.schedule = list(spec.schedule)
+        import inspect
+        self._takes_next_norm = ["next_norm" in inspect.signature(b.forward).parameters for b in self.blocks]
         readers = {}
         for e in self.schedule:
             if not e.writes_cache:
@@ -137,8 +139,16 @@ class Model:
         T = ctx.tokens.shape[0]
         x = ctx.ws.get("x", (T, self.dim), torch.float32)
         self.embedding.forward(ctx.tokens, x, ctx)
-        for e in self.schedule:
-            self.blocks[e.layer].forward(x, ctx, e.cache, e.writes_cache)
+        ctx.normed.clear()
+        n = len(self.schedule)
+        for i, e in enumerate(self.schedule):
+            block = self.blocks[e.layer]
+            if self._takes_next_norm[e.layer]:
+                nxt = self.blocks[self.schedule[i + 1].layer] if i + 1 < n else None
+                next_norm = getattr(nxt, "mixer_norm", None) if nxt is not None else self.final_norm
+                block.forward(x, ctx, e.cache, e.writes_cache, next_norm=next_norm)
+            else:
+                block.forward(x, ctx, e.cache, e.writes_cache)
         if logits is not None and logits.shape[0] > 0:
             R = logits.shape[0]
             if want_rows is None and R == T and self.head.fuses_norm(self.final_norm, x, ctx):

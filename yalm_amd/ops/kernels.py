@@ -165,6 +165,90 @@ def gemm_norm_qkv_rope(x, norm_w, eps, wqkv, q_out, k_pages, v_pages, block_tabl
         n_kv_heads, head_dim, rotary_dim, n_pages, _stream()), "gemm_norm_qkv_rope")
 
 
+CHAIN_MAX_ROWS = 16
+
+
+def can_chain(M, K, dtype):
+    """Whether gemm_chain / gemm_chain_qkv_rope take this shape."""
+    return dtype == torch.bfloat16 and 1 <= M <= CHAIN_MAX_ROWS and K % 8 == 0 and not FORCE_SIMPLE
+
+
+def gemm_chain_parts(N):
+    """Columns of the partial sums of squares that a producer with N output columns emits."""
+    return library.lib().yalm_gemm_chain_parts(int(N))
+
+
+def gemm_chain(x, w, out, epilogue, hidden=0, scale_from=None, emit=None):
+    """Decode GEMM (bfloat16; at most CHAIN_MAX_ROWS rows: beyond that the per-workgroup sum of the
+    partial sums costs more than a norm kernel) that chains norms.
+    scale_from = (ss float32 [M, parts], eps): x was emitted as bfloat16(residual * norm weight) and
+    the product is scaled by rsqrt(sum(ss[m]) / K + eps) per row.
+    emit = (norm_w float32 [N], xn bfloat16 [M, N], ss float32 [M, gemm_chain_parts(N)]), with
+    EPI_ADD_F32 only: also writes xn = bfloat16(out_new * norm_w) and the partial sums of squares."""
+    M, K = x.shape
+    N = w.shape[0]
+    p_x = _need(x, "x", torch.bfloat16, (M, K))
+    p_w = _need(w, "w", torch.bfloat16, (N, K))
+    if epilogue == EPI_GATED:
+        if hidden <= 0 or N != 32 * ((hidden + 15) // 16):
+            raise ValueError("gated gemm: weight rows %d do not match hidden %d" % (N, hidden))
+        p_o = _need(out, "out", torch.bfloat16, (M, hidden))
+    elif epilogue in (EPI_STORE_F32, EPI_ADD_F32):
+        p_o = _need(out, "out", torch.float32, (M, N))
+    else:
+        raise ValueError("gemm_chain: epilogue %r is not offered" % (epilogue,))
+    p_ss, n_parts, eps = None, 0, 0.0
+    if scale_from is not None:
+        ss, eps = scale_from
+        n_parts = ss.shape[1]
+        p_ss = _need(ss, "ss", torch.float32, (M, n_parts))
+    p_nw = p_xn = p_es = None
+    if emit is not None:
+        if epilogue != EPI_ADD_F32:
+            raise ValueError("gemm_chain: only the residual-add epilogue emits")
+        nw, xn, es = emit
+        p_nw = _need(nw, "emit norm_w", torch.float32, (N,))
+        p_xn = _need(xn, "emit xn", torch.bfloat16, (M, N))
+        p_es = _need(es, "emit ss", torch.float32, (M, gemm_chain_parts(N)))
+    library.check(library.lib().yalm_gemm_chain(p_x, p_w, p_o, M, N, K, epilogue, hidden, p_ss, n_parts, float(eps),
+                                                p_nw, p_xn, p_es, _stream()), "gemm_chain")
+    return out
+
+
+def gemm_chain_qkv_rope(xn, scale_from, wqkv, q_out, k_pages, v_pages, block_table, ring_pages, tok_pos, seq_slot,
+                        cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim):
+    """gemm_norm_qkv_rope for activations a producer emitted (see gemm_chain)."""
+    _check_heads(n_heads, n_kv_heads, head_dim)
+    if head_dim % 16:
+        raise ValueError("gemm_chain_qkv_rope needs a head_dim that is a multiple of 16")
+    M, K = xn.shape
+    Q, KV = n_heads * head_dim, n_kv_heads * head_dim
+    ss, eps = scale_from
+    n_parts = ss.shape[1]
+    p_x = _need(xn, "xn", torch.bfloat16, (M, K))
+    p_ss = _need(ss, "ss", torch.float32, (M, n_parts))
+    p_w = _need(wqkv, "wqkv", torch.bfloat16, (Q + 2 * KV, K))
+    p_q = _need(q_out, "q_out", torch.bfloat16, (M, Q))
+    n_pages = k_pages.shape[0]
+    p_kp = _need(k_pages, "k_pages", torch.bfloat16, (n_pages, n_kv_heads, PAGE, head_dim))
+    p_vp = _need(v_pages, "v_pages", torch.bfloat16, (n_pages, n_kv_heads, head_dim, PAGE))
+    p_bt = _need(block_table, "block_table", torch.int32, (None, None))
+    stride = block_table.shape[1]
+    if ring_pages <= 0 or ring_pages > stride:
+        raise ValueError("ring_pages %d does not fit the block table (%d columns)" % (ring_pages, stride))
+    p_tp = _need(tok_pos, "tok_pos", torch.int32, (M,))
+    p_sl = _need(seq_slot, "seq_slot", torch.int32, (M,))
+    n_pos, p_cs = 0, None
+    if cos_sin is not None:
+        n_pos = cos_sin.shape[0]
+        p_cs = _need(cos_sin, "cos_sin", torch.float32, (n_pos, rotary_dim // 2, 2))
+    else:
+        rotary_dim = 0
+    library.check(library.lib().yalm_gemm_chain_qkv_rope(
+        p_x, p_ss, n_parts, float(eps), p_w, p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_tp, p_sl, p_cs, n_pos, M, K,
+        n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, _stream()), "gemm_chain_qkv_rope")
+
+
 def _check_heads(n_heads, n_kv_heads, head_dim):
     if n_heads % n_kv_heads != 0:
         raise ValueError("n_heads %d is no multiple of n_kv_heads %d" % (n_heads, n_kv_heads))

@@ -23,6 +23,10 @@ _SIGNATURES = {
     "yalm_gemm_norm": (_I, [_P, _P, _F, _P, _P, _I, _I, _I, _I, _I, _P]),
     "yalm_gemm_norm_qkv_rope": (_I, [_P, _P, _F, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                      _I, _P]),
+    "yalm_gemm_chain": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _P, _I, _F, _P, _P, _P, _P]),
+    "yalm_gemm_chain_parts": (_I, [_I]),
+    "yalm_gemm_chain_qkv_rope": (_I, [_P, _P, _I, _F, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I,
+                                      _I, _I, _P]),
     "yalm_rope_kv_write": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                 _I, _I, _P]),
     "yalm_attn_prefill": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
@@ -33,7 +37,7 @@ _SIGNATURES = {
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
 }
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class KernelError(RuntimeError):

@@ -72,13 +72,16 @@ class GQAttention(Part):
         return max(1, min(max_pages, TARGET_WORKGROUPS // max(1, B * self.n_heads)))
 
     def fuses_norm(self, norm, x, ctx):
-        return hasattr(norm, "fused") and ctx.mode == "decode" and self.head_dim % 16 == 0 and \
-            kernels.can_fuse_norm(x.shape[0], self.dim, self.wo.dtype)
+        if not hasattr(norm, "fused") or ctx.mode != "decode" or self.head_dim % 16:
+            return False
+        return kernels.can_chain(x.shape[0], self.dim, self.wo.dtype)
 
-    def forward_prenorm(self, x, norm, ctx, line, writes_cache=True):
+    def forward_prenorm(self, x, norm, ctx, line, writes_cache=True, emit_for=None):
         """A decode step from the residual stream: norm, q/k/v, rotation and cache write in
-        one kernel, attention over the cache, output projection added to x."""
+        one kernel, attention over the cache, output projection added to x (which may
+        prepare the activations of the next norm, emit_for)."""
         if not writes_cache:                      # a reader of another entry's line: the plain way
+            ctx.normed.pop(id(norm), None)
             h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
             norm.forward(x, h, ctx)
             return self.forward(h, x, ctx, line, writes_cache)
@@ -87,16 +90,37 @@ class GQAttention(Part):
         if pos.table is not None and ctx.max_position >= pos.n_positions:
             raise ValueError("position %d is beyond the %d positions the rotation table holds"
                              % (ctx.max_position, pos.n_positions))
-        nw, eps = norm.fused()
         group = ctx.cache.group_of(line)
         k_pages, v_pages = group.line_pages(line)
         q = ctx.ws.get("attn.q", (T, self.q_dim), self.wo.dtype)
-        kernels.gemm_norm_qkv_rope(x, nw, eps, self.wqkv, q, k_pages, v_pages, group.table, group.ring_pages,
-                                   ctx.tok_pos, ctx.seq_slot, pos.table, self.n_heads, self.n_kv_heads,
-                                   self.head_dim, pos.rotary_dim)
+        src = ctx.normed.pop(id(norm), None)
+        if src is not None:
+            xn, ss, eps = src
+            kernels.gemm_chain_qkv_rope(xn, (ss, eps), self.wqkv, q, k_pages, v_pages, group.table, group.ring_pages,
+                                        ctx.tok_pos, ctx.seq_slot, pos.table, self.n_heads, self.n_kv_heads,
+                                        self.head_dim, pos.rotary_dim)
+        elif kernels.can_fuse_norm(T, self.dim, self.wo.dtype):
+            nw, eps = norm.fused()
+            kernels.gemm_norm_qkv_rope(x, nw, eps, self.wqkv, q, k_pages, v_pages, group.table, group.ring_pages,
+                                       ctx.tok_pos, ctx.seq_slot, pos.table, self.n_heads, self.n_kv_heads,
+                                       self.head_dim, pos.rotary_dim)
+        else:                                     # nothing prepared and too many rows for the one-kernel form
+            h = ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
+            norm.forward(x, h, ctx)
+            qkv = ctx.ws.get("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
+            kernels.gemm(h, self.wqkv, qkv, kernels.EPI_STORE_F32)
+            kernels.rope_kv_write(qkv, q, None, None, None, k_pages, v_pages, group.table, group.ring_pages,
+                                  ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads,
+                                  self.n_kv_heads, self.head_dim, pos.rotary_dim)
         o = ctx.ws.get("attn.o", (T, self.q_dim), self.wo.dtype)
         self._decode_attention(q, o, ctx, group, k_pages, v_pages)
-        kernels.gemm(o, self.wo, x, kernels.EPI_ADD_F32)
+        emit = self._emit_args(emit_for, ctx, T, self.dim)
+        if emit is not None and kernels.can_chain(T, self.q_dim, o.dtype):
+            nw2, xn2, ss2, eps2 = emit
+            kernels.gemm_chain(o, self.wo, x, kernels.EPI_ADD_F32, emit=(nw2, xn2, ss2))
+            ctx.normed[id(emit_for)] = (xn2, ss2, eps2)
+        else:
+            kernels.gemm(o, self.wo, x, kernels.EPI_ADD_F32)
 
     def _decode_attention(self, q, o, ctx, group, k_pages, v_pages):
         T = q.shape[0]

@@ -15,7 +15,10 @@ it is in.  Kinds of parts and the methods each must have:
 
 A mixer, feed-forward or head may fold the norm in front of it into its first
 product: fuses_norm(norm, x, ctx) says so for a step, and forward_prenorm(x, norm,
-...) then replaces norm.forward + forward.
+..., emit_for=next_norm) then replaces norm.forward + forward.  With emit_for it may
+also leave, in ctx.normed[id(next_norm)], the activations already multiplied by that
+norm's weights and the partial sums of squares (its residual-add GEMM writes them),
+which the next consumer takes instead of reading the residual stream.
 
 All of them: param_specs() -> [ParamSpec], load(get, compute_dtype, device),
 weight_bytes().  `h` is in the compute dtype (bfloat16 or float32); the
@@ -79,6 +82,20 @@ class Part:
 
     def children(self):
         return []
+
+    def _emit_args(self, emit_for, ctx, T, width):
+        """Operands for a residual-add GEMM that also prepares the activations of the norm
+        `emit_for` (the next norm on the residual stream), or None if that cannot be done."""
+        from ..ops import kernels
+        if emit_for is None or not hasattr(emit_for, "fused") or width >= 16384:
+            return None
+        if ctx.mode != "decode" or not kernels.can_chain(T, width, ctx.act_dtype):
+            return None
+        import torch
+        nw, eps = emit_for.fused()
+        xn = ctx.ws.get("chain.xn", (T, width), torch.bfloat16)
+        ss = ctx.ws.get("chain.ss", (T, kernels.gemm_chain_parts(width)), torch.float32)
+        return nw, xn, ss, eps
 
     def fuses_norm(self, norm, x, ctx):
         """True if this part can take the float32 residual stream x and do `norm` itself

@@ -52,11 +52,18 @@ class LMHead(Part):
         return self.weight.numel() * self.weight.element_size()
 
     def fuses_norm(self, norm, x, ctx):
-        return hasattr(norm, "fused") and ctx.mode == "decode" and \
-            kernels.can_fuse_norm(x.shape[0], self.dim, self.weight.dtype)
+        if not hasattr(norm, "fused") or ctx.mode != "decode":
+            return False
+        if id(norm) in ctx.normed:
+            return kernels.can_chain(x.shape[0], self.dim, self.weight.dtype)
+        return kernels.can_fuse_norm(x.shape[0], self.dim, self.weight.dtype)
 
     def forward_prenorm(self, x, norm, logits, ctx):
         """logits for every row of x (no row selection)."""
+        src = ctx.normed.pop(id(norm), None)
+        if src is not None:
+            xn, ss, eps = src
+            return kernels.gemm_chain(xn, self.weight, logits, kernels.EPI_STORE_F32, scale_from=(ss, eps))
         nw, eps = norm.fused()
         return kernels.gemm_norm(x, nw, eps, self.weight, logits, kernels.EPI_STORE_F32)
 

@@ -50,15 +50,31 @@ class SwiGLU(Part):
         return 3 * self.hidden * self.dim * self.w_down.element_size()
 
     def fuses_norm(self, norm, x, ctx):
-        return hasattr(norm, "fused") and ctx.mode == "decode" and \
-            kernels.can_fuse_norm(x.shape[0], self.dim, self.w_down.dtype)
+        if not hasattr(norm, "fused") or ctx.mode != "decode":
+            return False
+        return kernels.can_chain(x.shape[0], self.dim, self.w_down.dtype)
 
-    def forward_prenorm(self, x, norm, ctx):
-        nw, eps = norm.fused()
+    def forward_prenorm(self, x, norm, ctx, emit_for=None):
         T = x.shape[0]
         mid = ctx.ws.get("ffn.hidden", (T, self.hidden), self.w_down.dtype)
-        kernels.gemm_norm(x, nw, eps, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
-        kernels.gemm(mid, self.w_down, x, kernels.EPI_ADD_F32)
+        src = ctx.normed.pop(id(norm), None)
+        if src is not None:
+            xn, ss, eps = src
+            kernels.gemm_chain(xn, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden, scale_from=(ss, eps))
+        elif kernels.can_fuse_norm(T, self.dim, self.w_down.dtype):
+            nw, eps = norm.fused()
+            kernels.gemm_norm(x, nw, eps, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
+        else:
+            h = ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
+            norm.forward(x, h, ctx)
+            kernels.gemm(h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
+        emit = self._emit_args(emit_for, ctx, T, self.dim)
+        if emit is not None and kernels.can_chain(T, self.hidden, mid.dtype):
+            nw2, xn2, ss2, eps2 = emit
+            kernels.gemm_chain(mid, self.w_down, x, kernels.EPI_ADD_F32, emit=(nw2, xn2, ss2))
+            ctx.normed[id(emit_for)] = (xn2, ss2, eps2)
+        else:
+            kernels.gemm(mid, self.w_down, x, kernels.EPI_ADD_F32)
 
     def forward(self, h, x, ctx):
         T = h.shape[0]
