@@ -518,3 +518,40 @@ def test_gemm_chain_producer_and_consumer(M, N, Kd):
     k.gemm_chain(xn, interleave_gate_up(wg, wu).to(DEV), outg, k.EPI_GATED, hidden=H, scale_from=(ss, 1e-5))
     h = R.rmsnorm(x_want, nw, 1e-5)
     close(outg, R.silu(h @ wg.double().T) * (h @ wu.double().T), torch.bfloat16, "chained gated", factor=2.0)
+
+
+@pytest.mark.parametrize("with_workspace", [True, False])
+@pytest.mark.parametrize("M,N,Kd", [(17, 4096, 4096), (64, 100, 264), (48, 6144, 1000), (33, 4096, 14336)])
+def test_gemm_batches_of_17_to_64_rows(M, N, Kd, with_workspace):
+    """The kernel for 17..64 rows, with K split across workgroups (given scratch) and without."""
+    k = K()
+    a = rnd((M, Kd), 70, torch.bfloat16)
+    w = rnd((N, Kd), 71, torch.bfloat16, scale=1 / math.sqrt(Kd))
+    want = a.double() @ w.double().T
+    ws = torch.empty(k.gemm_workspace_floats(M, N), device=DEV) if with_workspace else None
+    out = torch.empty((M, N), device=DEV)
+    k.gemm(a.to(DEV), w.to(DEV), out, k.EPI_STORE_F32, workspace=ws)
+    close(out, want, torch.float32, "f32 out")
+    out2 = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+    k.gemm(a.to(DEV), w.to(DEV), out2, k.EPI_STORE, workspace=ws)
+    close(out2, want, torch.bfloat16, "bf16 out")
+    res = rnd((M, N), 72)
+    acc = res.to(DEV).clone()
+    k.gemm(a.to(DEV), w.to(DEV), acc, k.EPI_ADD_F32, workspace=ws)
+    close(acc, want + res.double(), torch.float32, "add")
+
+
+@pytest.mark.parametrize("with_workspace", [True, False])
+@pytest.mark.parametrize("M,H,D", [(64, 14336, 256), (20, 1000, 264), (40, 176, 4096)])
+def test_gemm_gated_batches_of_17_to_64_rows(M, H, D, with_workspace):
+    from yalm_amd.parts.swiglu import interleave_gate_up
+    k = K()
+    x = rnd((M, D), 73, torch.bfloat16)
+    wg = rnd((H, D), 74, torch.bfloat16, scale=1 / math.sqrt(D))
+    wu = rnd((H, D), 75, torch.bfloat16, scale=1 / math.sqrt(D))
+    want = R.silu(x.double() @ wg.double().T) * (x.double() @ wu.double().T)
+    w = interleave_gate_up(wg, wu).to(DEV)
+    ws = torch.empty(k.gemm_workspace_floats(M, w.shape[0]), device=DEV) if with_workspace else None
+    out = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
+    k.gemm(x.to(DEV), w, out, k.EPI_GATED, hidden=H, workspace=ws)
+    close(out, want, torch.bfloat16, "gated")

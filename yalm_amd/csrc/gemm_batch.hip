@@ -1,0 +1,265 @@
+// Decode GEMM for 17..64 rows, bfloat16: C = epilogue(X[M,K] * W[N,K]^T).
+//
+// With more than 16 rows the activations outweigh a workgroup's share of the weights,
+// so reading them once per 16 weight rows (as gemm_skinny does) makes L1, not HBM, the
+// limit.  Here K is split across workgroups and N across the 8 waves of a workgroup:
+// every wave owns 16 (32 for the gated epilogue) weight rows, the workgroup's chunk
+// of the activations [M x 128] goes through LDS once and all waves read it from there,
+// the weights go straight to registers, prefetched one chunk ahead.  Each K slice writes
+// its float32 partial product; a second kernel adds the slices in a fixed order and
+// applies the epilogue (one slice: the first kernel applies it itself).
+#include "common.h"
+#include "yalm_hip.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int NWAVES = 8;
+constexpr int KC = 128;                          // k per chunk
+constexpr int XROW = KC + 8;                     // LDS row stride (elements): 16 bytes of padding
+
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+__device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
+  bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+  return ok ? *reinterpret_cast<const bf16x8*>(p) : z;
+}
+
+// epilogue codes as in yalm_gemm: 0 float32 store, 1 bfloat16 store, 2 float32 add, 3 gated
+template <int EPI>
+__device__ __forceinline__ void store_tile(void* Cv, const f32x4& v, const f32x4& u, int m_base, int n, int hcol,
+                                           int M, int N, int H) {
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    int m = m_base + r;
+    if (m >= M) continue;
+    if (EPI == 3) {
+      if (hcol < H) ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(v[r]) * u[r]);
+    } else if (n < N) {
+      size_t o = (size_t)m * N + n;
+      if (EPI == 0) ((float*)Cv)[o] = v[r];
+      if (EPI == 1) ((bf16*)Cv)[o] = static_cast<bf16>(v[r]);
+      if (EPI == 2) ((float*)Cv)[o] += v[r];
+    }
+  }
+}
+
+// grid (row blocks of 128 * NTW weight rows, K slices).  partial: [slices][M][N] float32 when slices > 1.
+template <int MT, int NTW, int EPI>
+__global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_kernel(const bf16* __restrict__ X,
+                                                                    const bf16* __restrict__ W,
+                                                                    void* __restrict__ Cv,
+                                                                    float* __restrict__ partial, int M, int N, int K,
+                                                                    int H, int k_per_slice) {
+  __shared__ __attribute__((aligned(16))) bf16 xs[2][MT * 16 * XROW];
+  constexpr int NTHREADS = NWAVES * WAVE;
+  constexpr int XCHUNKS = MT * 16 * (KC / 8);    // 16-byte pieces of an activation chunk
+  constexpr int XPT = (XCHUNKS + NTHREADS - 1) / NTHREADS;
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int q = lane / 16, j = lane % 16;
+  const int n0 = (blockIdx.x * NWAVES + wave) * 16 * NTW;
+  const int k_begin = blockIdx.y * k_per_slice, k_end = min(K, k_begin + k_per_slice);
+
+  const bf16* wrow[NTW];
+  bool wok[NTW];
+#pragma unroll
+  for (int t = 0; t < NTW; ++t) {
+    int n = n0 + t * 16 + j;
+    wok[t] = n < N;
+    wrow[t] = W + (size_t)(wok[t] ? n : 0) * K;
+  }
+  f32x4 acc[MT][NTW];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) acc[mt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  bf16x8 wv[NTW][4], xr[XPT];
+  auto load_w = [&](int kc, bf16x8 (&dst)[NTW][4]) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      int k = kc + s * 32 + q * 8;
+      bool ok = k < k_end;
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) dst[t][s] = load8(wrow[t] + k, ok && wok[t]);
+    }
+  };
+  auto load_x = [&](int kc) {
+#pragma unroll
+    for (int p = 0; p < XPT; ++p) {
+      int c = tid + p * NTHREADS;
+      int row = c / (KC / 8), k = kc + (c % (KC / 8)) * 8;
+      xr[p] = load8(X + (size_t)min(row, M - 1) * K + k, c < XCHUNKS && row < M && k < k_end);
+    }
+  };
+  auto store_x = [&](int buf) {
+#pragma unroll
+    for (int p = 0; p < XPT; ++p) {
+      int c = tid + p * NTHREADS;
+      if (c < XCHUNKS) *reinterpret_cast<bf16x8*>(&xs[buf][(c / (KC / 8)) * XROW + (c % (KC / 8)) * 8]) = xr[p];
+    }
+  };
+
+  if (k_begin < k_end) {
+    load_w(k_begin, wv);
+    load_x(k_begin);
+    store_x(0);
+  }
+  __syncthreads();
+  int it = 0;
+  for (int kc = k_begin; kc < k_end; kc += KC, ++it) {
+    const int cur = it & 1;
+    const int kn = kc + KC;
+    bf16x8 wn[NTW][4];
+    if (kn < k_end) {
+      load_w(kn, wn);
+      load_x(kn);
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 xf = *reinterpret_cast<const bf16x8*>(&xs[cur][(mt * 16 + j) * XROW + s * 32 + q * 8]);
+#pragma unroll
+        for (int t = 0; t < NTW; ++t)
+          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf, wv[t][s], acc[mt][t], 0, 0, 0);
+      }
+    if (kn < k_end) {
+      store_x(cur ^ 1);
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) wv[t][s] = wn[t][s];
+    }
+    __syncthreads();
+  }
+
+  // C[m][n]: lane (q, j) holds rows 4q..4q+3 of column j of every tile
+  if (gridDim.y == 1) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      if (EPI == 3) {
+        store_tile<3>(Cv, acc[mt][0], acc[mt][NTW - 1], mt * 16 + 4 * q, 0, n0 / 2 + j, M, N, H);
+      } else {
+#pragma unroll
+        for (int t = 0; t < NTW; ++t)
+          store_tile<EPI>(Cv, acc[mt][t], acc[mt][t], mt * 16 + 4 * q, n0 + t * 16 + j, 0, M, N, H);
+      }
+    }
+  } else {
+    float* part = partial + (size_t)blockIdx.y * M * N;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) {
+        int n = n0 + t * 16 + j;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          int m = mt * 16 + 4 * q + r;
+          if (m < M && n < N) part[(size_t)m * N + n] = acc[mt][t][r];
+        }
+      }
+  }
+}
+
+// adds the K slices in order and applies the epilogue; a thread per (row, 4 columns)
+template <int EPI>
+__global__ void splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ Cv, int M, int N, int H,
+                                     int slices) {
+  const int cols4 = (EPI == 3) ? (N / 2) / 4 : (N + 3) / 4;     // gated: N = 32 * blocks, a thread per 4 hidden columns
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)M * cols4) return;
+  const int m = (int)(idx / cols4), c4 = (int)(idx % cols4) * 4;
+  const size_t plane = (size_t)M * N;
+  if (EPI == 3) {
+    const int blk = c4 / 16, off = c4 % 16;      // hidden column c4 = blk * 16 + off; gate at blk*32+off, up 16 further
+    const float* pg = partial + (size_t)m * N + blk * 32 + off;
+    float4 g = make_float4(0.f, 0.f, 0.f, 0.f), u = g;
+    for (int s = 0; s < slices; ++s) {
+      const float4 a = *reinterpret_cast<const float4*>(pg + s * plane);
+      const float4 b = *reinterpret_cast<const float4*>(pg + s * plane + 16);
+      g.x += a.x; g.y += a.y; g.z += a.z; g.w += a.w;
+      u.x += b.x; u.y += b.y; u.z += b.z; u.w += b.w;
+    }
+    bf16* C = (bf16*)Cv + (size_t)m * H;
+    const float gv[4] = {g.x, g.y, g.z, g.w}, uv[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (c4 + e < H) C[c4 + e] = static_cast<bf16>(silu_f(gv[e]) * uv[e]);
+  } else {
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    const float* p = partial + (size_t)m * N + c4;
+    if (c4 + 3 < N && (N & 3) == 0) {
+      for (int s = 0; s < slices; ++s) {
+        const float4 a = *reinterpret_cast<const float4*>(p + s * plane);
+        v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w;
+      }
+    } else {
+      for (int s = 0; s < slices; ++s)
+        for (int e = 0; e < 4; ++e)
+          if (c4 + e < N) v[e] += p[s * plane + e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (c4 + e >= N) continue;
+      size_t o = (size_t)m * N + c4 + e;
+      if (EPI == 0) ((float*)Cv)[o] = v[e];
+      if (EPI == 1) ((bf16*)Cv)[o] = static_cast<bf16>(v[e]);
+      if (EPI == 2) ((float*)Cv)[o] += v[e];
+    }
+  }
+}
+
+template <int MT, int EPI>
+int launch_mt(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
+              hipStream_t stream) {
+  constexpr int NTW = EPI == 3 ? 2 : 1;
+  const int rows_per_wg = NWAVES * 16 * NTW;
+  const int n_blocks = ceil_div(N, rows_per_wg);
+  const int chunks = ceil_div(K, KC);
+  // slices: until every CU has a workgroup, while the partial sums stay small beside the weights
+  // (slices * M * N * 4 bytes against N * K * 2) and a slice keeps at least 2 chunks
+  int slices = 1;
+  while (n_blocks * slices < 256 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
+    slices *= 2;
+  if (ws == nullptr || (long)slices * M * N > ws_floats) slices = 1;
+  const int k_per_slice = ceil_div(chunks, slices) * KC;
+  slices = ceil_div(K, k_per_slice);
+  dim3 grid(n_blocks, slices);
+  gemm_batch_kernel<MT, NTW, EPI><<<grid, NWAVES * WAVE, 0, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice);
+  int rc = launch_status();
+  if (rc != YALM_OK || slices == 1) return rc;
+  const long items = (long)M * (EPI == 3 ? (N / 2) / 4 : (N + 3) / 4);
+  splitk_reduce_kernel<EPI><<<ceil_div(items, 256), 256, 0, stream>>>(ws, C, M, N, H, slices);
+  return launch_status();
+}
+
+template <int EPI>
+int dispatch(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
+             hipStream_t stream) {
+  switch ((M + 15) / 16) {
+    case 2: return launch_mt<2, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+    case 3: return launch_mt<3, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+    case 4: return launch_mt<4, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+  }
+  return YALM_ERR_ARG;
+}
+}  // namespace
+
+// 17..64 rows; workspace: float32 scratch for the K slices (may be null: one slice then).
+// Refuses (YALM_ERR_ARG) what it does not take.
+int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
+                         int K, int epilogue, int H, hipStream_t stream) {
+  if (M <= 16 || M > 64 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  switch (epilogue) {
+    case 0: return dispatch<0>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+    case 1: return dispatch<1>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+    case 2: return dispatch<2>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+    case 3: return dispatch<3>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+  }
+  return YALM_ERR_ARG;
+}

@@ -186,11 +186,18 @@ int tiled_launch(const bf16* A, const bf16* W, void* C, int M, int N, int K, int
 
 }  // namespace
 
-int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, int M, int N, int K, int epilogue, int H,
-                        hipStream_t stream) {
+int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
+                         int K, int epilogue, int H, hipStream_t stream);   // gemm_batch.hip
+
+int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
+                        int K, int epilogue, int H, hipStream_t stream) {
   if (K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
+  if (M > 16 && M <= 64) {
+    int rc = yalm_gemm_bf16_batch(A, W, C, workspace, workspace_floats, M, N, K, epilogue, H, stream);
+    if (rc != YALM_ERR_ARG) return rc;
+  }
   if (M <= 64) {
     switch (epilogue) {
       case 0: return skinny_dispatch<0>(a, w, C, M, N, K, H, stream);

@@ -5,8 +5,8 @@
 #include "common.h"
 #include "yalm_hip.h"
 
-int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, int M, int N, int K, int epilogue, int H,
-                        hipStream_t stream);   // gemm_mfma.hip; returns YALM_ERR_ARG if it refuses the shape
+int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
+                        int K, int epilogue, int H, hipStream_t stream);   // gemm_mfma.hip; YALM_ERR_ARG: shape refused
 
 namespace {
 constexpr int BM = 64, BN = 64, BK = 16;
@@ -96,15 +96,15 @@ int gemm_simple(const void* A, const void* W, void* C, int M, int N, int K, int 
 }
 }  // namespace
 
-extern "C" int yalm_gemm(const void* A, const void* W, void* C, int M, int N, int K, int dtype, int epilogue, int H,
-                         int force_simple, hipStream_t stream) {
+extern "C" int yalm_gemm(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
+                         int K, int dtype, int epilogue, int H, int force_simple, hipStream_t stream) {
   if (M <= 0) return YALM_OK;
   if (N <= 0 || K <= 0 || epilogue < 0 || epilogue > 3) return YALM_ERR_ARG;
   if (epilogue == 3 && (H <= 0 || N != 32 * ((H + 15) / 16))) return YALM_ERR_ARG;
   if (dtype == YALM_F32) return gemm_simple<float>(A, W, C, M, N, K, epilogue, H, stream);
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
   if (!force_simple) {
-    int rc = yalm_gemm_bf16_mfma(A, W, C, M, N, K, epilogue, H, stream);
+    int rc = yalm_gemm_bf16_mfma(A, W, C, workspace, workspace_floats, M, N, K, epilogue, H, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   return gemm_simple<bf16>(A, W, C, M, N, K, epilogue, H, stream);

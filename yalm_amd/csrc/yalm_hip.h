@@ -32,8 +32,10 @@ int yalm_rmsnorm(const float* x, const void* w, int w_dtype, void* out, int out_
 //             C `dtype` [M,H] = silu(gate) * up
 // reference: matmul_wide, fused_matmul_add_residuals, fused_qkv_matmul_clip,
 // fused_ffn_w1_w3_glu_act (src/infer.cu:250-337, 610-634)
-int yalm_gemm(const void* A, const void* W, void* C, int M, int N, int K, int dtype, int epilogue, int H,
-              int force_simple, hipStream_t stream);
+// workspace: float32 scratch (may be null) for kernels that split K across workgroups; they
+// use as many slices as it holds (slices * M * N floats).
+int yalm_gemm(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N, int K,
+              int dtype, int epilogue, int H, int force_simple, hipStream_t stream);
 
 // Decode GEMMs from the float32 residual stream, M <= 8 rows (M * (K + 8) * 2 bytes <= 72 KB), bfloat16 weights:
 // C = epilogue(rmsnorm(x, norm_w, eps) * W^T); epilogue 0 (float32 store) or 3 (gated, as yalm_gemm).

@@ -76,11 +76,20 @@ def rmsnorm(x, weight, out, eps, row_index=None):
 EPI_STORE_F32, EPI_STORE, EPI_ADD_F32, EPI_GATED = 0, 1, 2, 3
 
 
-def gemm(a, w, out, epilogue, hidden=0):
+GEMM_SPLIT_MAX = 16          # most K slices a GEMM uses, given the workspace
+
+
+def gemm_workspace_floats(M, N):
+    """Floats of scratch with which gemm may split K across workgroups (17..64 rows)."""
+    return GEMM_SPLIT_MAX * M * N if 16 < M <= 64 else 0
+
+
+def gemm(a, w, out, epilogue, hidden=0, workspace=None):
     """out = a[M,K] @ w[N,K]^T with float32 accumulation and one of four epilogues:
     EPI_STORE_F32 (float32 out), EPI_STORE (out in a's dtype), EPI_ADD_F32
     (float32 out += product), EPI_GATED (w = gate/up rows interleaved in blocks of
-    16; out[M, hidden] = silu(gate) * up in a's dtype)."""
+    16; out[M, hidden] = silu(gate) * up in a's dtype).  workspace: float32 scratch of
+    gemm_workspace_floats(M, N) elements, with which batches of 17..64 rows split K."""
     M, K = a.shape
     N = w.shape[0]
     dt = a.dtype
@@ -96,7 +105,10 @@ def gemm(a, w, out, epilogue, hidden=0):
         p_o = _need(out, "out", torch.float32, (M, N))
     else:
         raise ValueError("unknown epilogue %r" % (epilogue,))
-    library.check(library.lib().yalm_gemm(p_a, p_w, p_o, M, N, K, dtype_code(dt), epilogue, hidden,
+    p_ws, n_ws = None, 0
+    if workspace is not None:
+        p_ws, n_ws = _need(workspace, "workspace", torch.float32), workspace.numel()
+    library.check(library.lib().yalm_gemm(p_a, p_w, p_o, p_ws, n_ws, M, N, K, dtype_code(dt), epilogue, hidden,
                                           1 if FORCE_SIMPLE else 0, _stream()), "gemm")
     return out
 

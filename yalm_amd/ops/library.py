@@ -19,7 +19,7 @@ _SIGNATURES = {
     "yalm_error_string": (ctypes.c_char_p, [_I]),
     "yalm_embed": (_I, [_P, _I, _P, _P, _I, _I, _I, _P]),
     "yalm_rmsnorm": (_I, [_P, _P, _I, _P, _I, _P, _I, _I, _F, _P]),
-    "yalm_gemm": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_gemm": (_I, [_P, _P, _P, _P, ctypes.c_long, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_gemm_norm": (_I, [_P, _P, _F, _P, _P, _I, _I, _I, _I, _I, _P]),
     "yalm_gemm_norm_qkv_rope": (_I, [_P, _P, _F, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
                                      _I, _P]),
@@ -37,7 +37,7 @@ _SIGNATURES = {
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
 }
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 
 class KernelError(RuntimeError):

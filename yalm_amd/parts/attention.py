@@ -108,7 +108,7 @@ class GQAttention(Part):
             h = ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
             norm.forward(x, h, ctx)
             qkv = ctx.ws.get("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
-            kernels.gemm(h, self.wqkv, qkv, kernels.EPI_STORE_F32)
+            self._gemm(ctx, h, self.wqkv, qkv, kernels.EPI_STORE_F32)
             kernels.rope_kv_write(qkv, q, None, None, None, k_pages, v_pages, group.table, group.ring_pages,
                                   ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads,
                                   self.n_kv_heads, self.head_dim, pos.rotary_dim)
@@ -120,7 +120,7 @@ class GQAttention(Part):
             kernels.gemm_chain(o, self.wo, x, kernels.EPI_ADD_F32, emit=(nw2, xn2, ss2))
             ctx.normed[id(emit_for)] = (xn2, ss2, eps2)
         else:
-            kernels.gemm(o, self.wo, x, kernels.EPI_ADD_F32)
+            self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)
 
     def _decode_attention(self, q, o, ctx, group, k_pages, v_pages):
         T = q.shape[0]
@@ -140,7 +140,7 @@ class GQAttention(Part):
             raise ValueError("position %d is beyond the %d positions the rotation table holds"
                              % (ctx.max_position, pos.n_positions))
         qkv = ws.get("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
-        kernels.gemm(h, self.wqkv, qkv, kernels.EPI_STORE_F32)
+        self._gemm(ctx, h, self.wqkv, qkv, kernels.EPI_STORE_F32)
         q = ws.get("attn.q", (T, self.q_dim), act)
         group = ctx.cache.group_of(line)
         k_pages, v_pages = group.line_pages(line)
@@ -167,4 +167,4 @@ class GQAttention(Part):
                                  self.n_heads, self.n_kv_heads, self.head_dim, self.window)
         else:
             self._decode_attention(q, o, ctx, group, k_pages, v_pages)
-        kernels.gemm(o, self.wo, x, kernels.EPI_ADD_F32)
+        self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)

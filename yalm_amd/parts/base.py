@@ -83,6 +83,17 @@ class Part:
     def children(self):
         return []
 
+    @staticmethod
+    def _gemm(ctx, a, w, out, epilogue, hidden=0):
+        """kernels.gemm with the scratch that lets batches of 17..64 rows split K."""
+        from ..ops import kernels
+        import torch
+        ws = None
+        n = kernels.gemm_workspace_floats(a.shape[0], w.shape[0]) if a.dtype == torch.bfloat16 else 0
+        if n and ctx is not None:
+            ws = ctx.ws.get("gemm.partial", (n,), torch.float32)
+        return kernels.gemm(a, w, out, epilogue, hidden=hidden, workspace=ws)
+
     def _emit_args(self, emit_for, ctx, T, width):
         """Operands for a residual-add GEMM that also prepares the activations of the norm
         `emit_for` (the next norm on the residual stream), or None if that cannot be done."""

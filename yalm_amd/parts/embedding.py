@@ -68,4 +68,4 @@ class LMHead(Part):
         return kernels.gemm_norm(x, nw, eps, self.weight, logits, kernels.EPI_STORE_F32)
 
     def forward(self, h, logits, ctx):
-        return kernels.gemm(h, self.weight, logits, kernels.EPI_STORE_F32)
+        return self._gemm(ctx, h, self.weight, logits, kernels.EPI_STORE_F32)

@@ -67,17 +67,17 @@ class SwiGLU(Part):
         else:
             h = ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
             norm.forward(x, h, ctx)
-            kernels.gemm(h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
+            self._gemm(ctx, h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
         emit = self._emit_args(emit_for, ctx, T, self.dim)
         if emit is not None and kernels.can_chain(T, self.hidden, mid.dtype):
             nw2, xn2, ss2, eps2 = emit
             kernels.gemm_chain(mid, self.w_down, x, kernels.EPI_ADD_F32, emit=(nw2, xn2, ss2))
             ctx.normed[id(emit_for)] = (xn2, ss2, eps2)
         else:
-            kernels.gemm(mid, self.w_down, x, kernels.EPI_ADD_F32)
+            self._gemm(ctx, mid, self.w_down, x, kernels.EPI_ADD_F32)
 
     def forward(self, h, x, ctx):
         T = h.shape[0]
         mid = ctx.ws.get("ffn.hidden", (T, self.hidden), h.dtype)
-        kernels.gemm(h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
-        kernels.gemm(mid, self.w_down, x, kernels.EPI_ADD_F32)
+        self._gemm(ctx, h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
+        self._gemm(ctx, mid, self.w_down, x, kernels.EPI_ADD_F32)
