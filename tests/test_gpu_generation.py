@@ -36,10 +36,11 @@ def plain_greedy(folder, prompt, n_new, stop=()):
     return seq[len(prompt):]
 
 
-def test_greedy_generation_matches_the_plain_implementation(folders):
-    """BASELINE configs[0]: prompts of 5, 17 and 1 tokens, then 8 greedy steps (float32)."""
+@pytest.mark.parametrize("name", ["tiny_llama", "tiny_mistral", "tiny_wide_heads"])
+def test_greedy_generation_matches_the_plain_implementation(folders, name):
+    """BASELINE configs[0]: prompts of 5, 17 and 1 tokens, then 8 greedy steps (float32); also
+    with untied heads, where the next token is not simply the last one again."""
     from yalm_amd import Engine, Model, generate
-    name = "tiny_llama"
     model = Model.from_folder(folders[name], dtype=torch.float32, device="cuda:0")
     engine = Engine(model, max_tokens=2048)
     prompts = list(helpers.random_requests(tiny_configs.ALL[name], [5, 17, 1], seed=1).values())

@@ -14,6 +14,7 @@
 // the keys of their KV head) or a query position (prefill: 16 positions a wave).
 #include <float.h>
 #include <math.h>
+#include <type_traits>
 #include "common.h"
 #include "yalm_hip.h"
 
@@ -206,8 +207,6 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 // per workgroup, double-buffered, rows stored in the order the MFMA operands read them.
 // grid (64-position tile, head): the workgroup of every second tile of a sequence works.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ float fast_exp(float x) { return __expf(x); }
-
 template <int HD>
 __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_stage, const bf16* __restrict__ v_stage,
@@ -237,7 +236,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
   if (tq & 1) return;                             // the workgroup of the even tile covers this one too
   const int start = cu_seqlens[b], len = cu_seqlens[b + 1] - start;
   const int g = h / (n_heads / n_kv_heads);
-  const float inv_root = 1.0f / sqrtf((float)HD);
+  const float score_scale = 1.4426950408889634f / sqrtf((float)HD);   // log2(e) / sqrt(head_dim)
 
   const int blk0 = tq * PAGE;                     // first position of the workgroup
   const int pos0 = blk0 + wave * 32;              // first position of the wave
@@ -320,43 +319,55 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
       const bool edge = base + PAGE - 1 > pos0 || (window > 0 && base < pos0 + 31 - window + 1);
       bf16x8 pb[2][2];
       float corr[2];
+      // scores in the base-2 domain: p = 2^(s * log2(e) / sqrt(hd) - m)
+      auto softmax_tile = [&](auto masked) {
 #pragma unroll
-      for (int c = 0; c < 2; ++c) {
-        float mx = -FLT_MAX;
+        for (int c = 0; c < 2; ++c) {
+          float mx = -FLT_MAX;
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+          for (int t = 0; t < 4; ++t)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            float v = sc[c][t][r] * inv_root;
-            if (edge) {
-              int kpos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
-              bool vis = kpos <= pos_q[c] && (window == 0 || pos_q[c] - kpos < window) && q_ok[c];
-              if (!vis) v = -INFINITY;
+            for (int r = 0; r < 4; ++r) {
+              float v = sc[c][t][r] * score_scale;
+              if (decltype(masked)::value) {
+                int kpos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
+                bool vis = kpos <= pos_q[c] && (window == 0 || pos_q[c] - kpos < window) && q_ok[c];
+                v = vis ? v : -INFINITY;
+              }
+              sc[c][t][r] = v;
+              mx = fmaxf(mx, v);
             }
-            sc[c][t][r] = v;
-            mx = fmaxf(mx, v);
-          }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-        const float m_new = fmaxf(m[c], mx);
-        corr[c] = fast_exp(m[c] - m_new);
-        float psum = 0.f;
+          mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+          mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+          const float m_new = fmaxf(m[c], mx);
+          corr[c] = __builtin_amdgcn_exp2f(m[c] - m_new);
+          float psum = 0.f;
 #pragma unroll
-        for (int s2 = 0; s2 < 2; ++s2)
+          for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            float p = fast_exp(sc[c][2 * s2 + (e >> 2)][e & 3] - m_new);
-            psum += p;
-            pb[c][s2][e] = static_cast<bf16>(p);
-          }
-        l[c] = l[c] * corr[c] + psum;
-        m[c] = m_new;
-      }
+            for (int e = 0; e < 8; ++e) {
+              float p = __builtin_amdgcn_exp2f(sc[c][2 * s2 + (e >> 2)][e & 3] - m_new);
+              psum += p;
+              pb[c][s2][e] = static_cast<bf16>(p);
+            }
+          l[c] = l[c] * corr[c] + psum;
+          m[c] = m_new;
+        }
+      };
+      if (edge)
+        softmax_tile(std::true_type{});
+      else
+        softmax_tile(std::false_type{});
+      const bool rescale = !__all(corr[0] == 1.0f && corr[1] == 1.0f);   // the maxima settle after a few tiles
       const bool tail = base + PAGE > len;        // rows behind the sequence's end may hold anything
+      if (rescale) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int c = 0; c < 2; ++c) o[c][dt] *= corr[c];
+      }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
-#pragma unroll
-        for (int c = 0; c < 2; ++c) o[c][dt] *= corr[c];
 #pragma unroll
         for (int s2 = 0; s2 < 2; ++s2) {
           bf16x8 vf = *reinterpret_cast<const bf16x8*>(vs_l + (dt * 16 + j) * VROW + s2 * 32 + qd * 8);

@@ -10,36 +10,47 @@ namespace {
 constexpr int NT = 256;
 constexpr int NW = NT / WAVE;
 
-__global__ __launch_bounds__(NT) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
-  __shared__ float bv[NT];
-  __shared__ int bi[NT];
+constexpr int NTA = 1024;                        // argmax: 1024 threads a row
+
+__global__ __launch_bounds__(NTA) void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int V) {
+  __shared__ float bv[NTA / WAVE];
+  __shared__ int bi[NTA / WAVE];
   const float* l = logits + (size_t)blockIdx.x * V;
   float best = -FLT_MAX;
   int arg = V;                                   // "none": larger than every index
-  for (int i = threadIdx.x; i < V; i += NT) {    // indices rise within a thread: strict '>' keeps its first maximum
+  for (int i = threadIdx.x; i < V; i += NTA) {   // indices rise within a thread: strict '>' keeps its first maximum
     float v = l[i];
     if (v > best) {
       best = v;
       arg = i;
     }
   }
-  bv[threadIdx.x] = best;
-  bi[threadIdx.x] = arg;
+  // the lowest index wins ties, in the wave and among the waves
+#pragma unroll
+  for (int o = WAVE / 2; o > 0; o >>= 1) {
+    float ov = __shfl_xor(best, o, WAVE);
+    int oi = __shfl_xor(arg, o, WAVE);
+    if (oi < V && (arg >= V || ov > best || (ov == best && oi < arg))) {
+      best = ov;
+      arg = oi;
+    }
+  }
+  if ((threadIdx.x & (WAVE - 1)) == 0) {
+    bv[threadIdx.x / WAVE] = best;
+    bi[threadIdx.x / WAVE] = arg;
+  }
   __syncthreads();
-  for (int stride = NT / 2; stride > 0; stride >>= 1) {
-    if (threadIdx.x < stride) {
-      float ov = bv[threadIdx.x + stride];
-      int oi = bi[threadIdx.x + stride];
-      float mv = bv[threadIdx.x];
-      int mi = bi[threadIdx.x];
-      if (oi < V && (mi >= V || ov > mv || (ov == mv && oi < mi))) {   // the lowest index wins ties
-        bv[threadIdx.x] = ov;
-        bi[threadIdx.x] = oi;
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < NTA / WAVE; ++w) {
+      float ov = bv[w];
+      int oi = bi[w];
+      if (oi < V && (arg >= V || ov > best || (ov == best && oi < arg))) {
+        best = ov;
+        arg = oi;
       }
     }
-    __syncthreads();
+    out[blockIdx.x] = arg < V ? arg : 0;
   }
-  if (threadIdx.x == 0) out[blockIdx.x] = bi[0] < V ? bi[0] : 0;
 }
 
 __global__ __launch_bounds__(NT) void sample_kernel(const float* __restrict__ logits, const float* __restrict__ u,
@@ -106,7 +117,7 @@ __global__ __launch_bounds__(NT) void token_prob_kernel(const float* __restrict_
 extern "C" int yalm_argmax(const float* logits, int* out, int R, int V, hipStream_t stream) {
   if (R <= 0) return YALM_OK;
   if (V <= 0) return YALM_ERR_ARG;
-  argmax_kernel<<<R, NT, 0, stream>>>(logits, out, V);
+  argmax_kernel<<<R, NTA, 0, stream>>>(logits, out, V);
   return launch_status();
 }
 
