@@ -426,3 +426,32 @@ def test_tokenizer(tmp_path):
     assert text == b"hello world!"                                 # the space after BOS is dropped
     assert t.encode("hé", False) == [3 + ord("h"), 3 + 0xC3, 3 + 0xA9]     # "he" does not match
     assert t.encode("he", False) == [263]
+
+
+def test_command_line_options_have_the_references_meanings():
+    """src/main.cpp:334-467: every option takes a value, -m and -d match by prefix,
+    -n sets the step count and the number of junk lines, one prompt source only."""
+    from yalm_amd.cli import parse_args
+    a = parse_args(["folder", "-m", "c", "-i", "hello", "-n", "12", "-t", "0.5", "-T", "64"])
+    assert (a["checkpoint"], a["mode"], a["prompt"], a["num_steps"], a["n_junk"], a["temperature"], a["context"]) == \
+        ("folder", "completion", "hello", 12, 12, 0.5, 64)
+    d = parse_args(["folder", "--tokens", "1,2"])
+    assert (d["mode"], d["num_steps"], d["n_junk"], d["temperature"], d["passkey_pos"], d["device"]) == \
+        ("completion", 256, 250, 1.0, -1, "hip")
+    assert parse_args(["folder", "-m", "perp", "-f", "x.txt"])["mode"] == "perplexity"
+    assert parse_args(["folder", "-m", "pass", "-n", "10", "-l", "9"])["passkey_pos"] == 9
+    r = parse_args(["--random", "cfg.json", "--weight-seed", "3", "--tokens", "1 2 3", "-d", "cuda"])
+    assert (r["checkpoint"], r["random"], r["weight_seed"], r["device"]) == ("", "cfg.json", 3, "cuda")
+    for bad in (["folder"],                                            # no prompt
+                ["folder", "-i", "a", "-f", "b"],                      # two prompts
+                ["folder", "-m", "x", "-i", "a"],                      # unknown mode
+                ["folder", "-d", "cpu", "-i", "a"],                    # no CPU path
+                ["folder", "-i"],                                      # option without value
+                ["folder", "-z", "1", "-i", "a"],                      # unknown option
+                ["folder", "-m", "pass", "-n", "10", "-l", "10"],      # passkey line out of range (main.cpp:455-458)
+                ["folder", "--random", "cfg.json", "-i", "a"],         # folder and --random
+                ["folder", "--dtype", "float16", "-i", "a"],
+                []):
+        with pytest.raises(SystemExit) as e:
+            parse_args(bad)
+        assert e.value.code == 1

@@ -209,6 +209,12 @@ def test_command_line(folders):
     want = plain_greedy(folder, prompt, 6, stop=(2,))
     assert [int(t) for t in first] == want
     assert "Generation stats:" in p.stdout and "throughput:" in p.stdout
+    # the same model made from its configuration and seed alone, without a folder
+    p = subprocess.run([sys.executable, "-m", "yalm_amd", "--random", os.path.join(folder, "config.json"),
+                        "--weight-seed", "6", "--tokens", ",".join(map(str, prompt)), "-n", "6", "-t", "0", "--dtype",
+                        "float32"], cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-3000:]
+    assert [int(t) for t in p.stdout.split("\n\n")[0].split()] == want
     toks = helpers.random_requests(tiny_configs.TINY_LLAMA, [30], seed=7)["r0"]
     p = subprocess.run([sys.executable, "-m", "yalm_amd", folder, "-m", "perp", "--tokens", " ".join(map(str, toks)),
                         "--dtype", "float32"], cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,

@@ -1,6 +1,7 @@
 """Command line in the reference's manner (src/main.cpp:17-40, 334-470):
 
     python -m yalm_amd <model folder> [options]
+    python -m yalm_amd --random <config.json> [--weight-seed <int>] [options]     (random weights, no folder)
       -h                 this text
       -d [hip,cuda]      device; there is no CPU path here (default - hip)
       -m [completion,passkey,perplexity]   mode, may be abbreviated (default - completion)
@@ -12,7 +13,8 @@
                          passkey: number of junk lines (default 250)
       -l <int>           passkey position (-1 - random)
     Additions: --tokens 1,2,3 (prompt as token ids; with --batch-file one prompt a line),
-      --batch-file <path>, --seed <int>, --dtype bfloat16|float32, --max-tokens <int>
+      --batch-file <path>, --seed <int>, --dtype bfloat16|float32, --max-tokens <int>,
+      --random <config.json> in place of the folder, --weight-seed <int> (default 0)
 
 Every option takes a value, as in the reference."""
 import math
@@ -41,11 +43,12 @@ def _prefix_choice(value, choices):
 def parse_args(argv):
     if len(argv) < 1 or argv[0] in ("-h", "--help"):
         error_usage()
-    a = {"checkpoint": argv[0], "device": "hip", "mode": "completion", "prompt": "", "prompt_path": "",
+    positional = not argv[0].startswith("--random")
+    a = {"checkpoint": argv[0] if positional else "", "random": "", "weight_seed": 0, "device": "hip", "mode": "completion", "prompt": "", "prompt_path": "",
          "context": 0, "num_steps": 256, "temperature": 1.0, "n_junk": 250, "passkey_pos": -1, "tokens": "",
          "batch_file": "", "seed": None, "dtype": "bfloat16", "max_tokens": 0}
-    i = 1
-    long_opts = {"--tokens": "tokens", "--batch-file": "batch_file", "--seed": "seed", "--dtype": "dtype",
+    i = 1 if positional else 0
+    long_opts = {"--random": "random", "--weight-seed": "weight_seed", "--tokens": "tokens", "--batch-file": "batch_file", "--seed": "seed", "--dtype": "dtype",
                  "--max-tokens": "max_tokens"}
     while i < len(argv):
         flag = argv[i]
@@ -54,7 +57,7 @@ def parse_args(argv):
         val = argv[i + 1]
         if flag in long_opts:
             key = long_opts[flag]
-            a[key] = int(val) if key in ("seed", "max_tokens") else val
+            a[key] = int(val) if key in ("seed", "max_tokens", "weight_seed") else val
         elif len(flag) != 2 or flag[0] != "-":
             error_usage("unknown option %s" % flag)
         elif flag[1] == "h":
@@ -84,6 +87,8 @@ def parse_args(argv):
         i += 2
     if a["dtype"] not in ("bfloat16", "float32"):
         error_usage("--dtype must be bfloat16 or float32")
+    if bool(a["random"]) == bool(a["checkpoint"]):
+        error_usage("give a model folder or --random <config.json>, not both")
     if a["mode"] in ("completion", "perplexity"):
         given = sum(1 for k in ("prompt", "prompt_path", "tokens", "batch_file") if a[k])
         if a["batch_file"] and a["tokens"] and not a["prompt"] and not a["prompt_path"]:
@@ -100,6 +105,14 @@ def _load(a):
     import torch
     from .engine import Engine, Model
     dtype = {"bfloat16": torch.bfloat16, "float32": torch.float32}[a["dtype"]]
+    if a["random"]:
+        import json
+        from .config import config_from_dict
+        with open(a["random"]) as f:
+            cfg = config_from_dict(json.load(f))
+        if a["context"]:
+            cfg = cfg.with_window(a["context"])
+        return Model.random(cfg, a["weight_seed"], dtype=dtype, device="cuda:0")
     model = Model.from_folder(a["checkpoint"], dtype=dtype, device="cuda:0", window=a["context"])
     return model
 
@@ -113,6 +126,8 @@ def _prompts(a, model):
     def tokenizer():
         nonlocal tok
         if tok is None:
+            if not a["checkpoint"]:
+                error_usage("a model made with --random has no tokenizer: give the prompt with --tokens")
             eos = cfg.eos_token_ids[0] if cfg.eos_token_ids else -1
             tok = Tokenizer.from_folder(a["checkpoint"], cfg.vocab_size,
                                         cfg.bos_token_id if cfg.bos_token_id is not None else -1, eos)

@@ -17,6 +17,7 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
 namespace {
 constexpr int MAX_HD = 256;              // head sizes up to 256 (4 output elements per lane)
 constexpr int ACC = MAX_HD / WAVE;
+constexpr int COMBINE_THREADS = 256;
 
 // ---------------------------------------------------------------------------
 // prefill: a step's tokens over the same step's keys
@@ -165,25 +166,53 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
 }
 
 template <typename T>
-__global__ void attn_decode_combine_kernel(const float* __restrict__ partial, T* __restrict__ out, int n_heads,
-                                           int hd, int n_splits) {
+__global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(const float* __restrict__ partial,
+                                                                             T* __restrict__ out, int n_heads, int hd,
+                                                                             int n_splits) {
+  // Every wave finds the maximum and the denominator for itself (lanes over splits);
+  // the four waves then share the splits of the weighted sum and add their parts in
+  // a fixed order, so that few loads wait on each other.
+  __shared__ float accs[COMBINE_THREADS / WAVE][MAX_HD];
   const int b = blockIdx.x, h = blockIdx.y;
-  const float* part = partial + ((size_t)b * n_heads + h) * n_splits * (hd + 2);
+  const int lane = threadIdx.x & (WAVE - 1), g = threadIdx.x / WAVE;
+  const int stride = hd + 2;
+  const float* part = partial + ((size_t)b * n_heads + h) * n_splits * stride;
   float m = -FLT_MAX;
-  for (int s = 0; s < n_splits; ++s) m = fmaxf(m, part[(size_t)s * (hd + 2) + hd]);
+  for (int s = lane; s < n_splits; s += WAVE) m = fmaxf(m, part[(size_t)s * stride + hd]);
+  m = wave_max(m);
   float l = 0.f;
-  for (int s = 0; s < n_splits; ++s) {
-    const float* ps = part + (size_t)s * (hd + 2);
+  for (int s = lane; s < n_splits; s += WAVE) {
+    const float* ps = part + (size_t)s * stride;
     l += ps[hd + 1] * expf(ps[hd] - m);
   }
+  l = wave_sum(l);
   const float inv_l = l > 0.f ? 1.0f / l : 0.f;
-  for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-    float a = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
-      const float* ps = part + (size_t)s * (hd + 2);
-      a += ps[d] * expf(ps[hd] - m);
+  float a[ACC];
+#pragma unroll
+  for (int j = 0; j < ACC; ++j) a[j] = 0.f;
+#pragma unroll 4
+  for (int s = g; s < n_splits; s += COMBINE_THREADS / WAVE) {
+    const float* ps = part + (size_t)s * stride;
+    const float w = expf(ps[hd] - m);
+#pragma unroll
+    for (int j = 0; j < ACC; ++j) {
+      const int d = lane + j * WAVE;
+      if (d < hd) a[j] += ps[d] * w;
     }
-    out[((size_t)b * n_heads + h) * hd + d] = from_f32<T>(a * inv_l);
+  }
+#pragma unroll
+  for (int j = 0; j < ACC; ++j) accs[g][lane + j * WAVE] = a[j];
+  __syncthreads();
+  if (g == 0) {
+#pragma unroll
+    for (int j = 0; j < ACC; ++j) {
+      const int d = lane + j * WAVE;
+      if (d >= hd) continue;
+      float t = accs[0][d];
+#pragma unroll
+      for (int w = 1; w < COMBINE_THREADS / WAVE; ++w) t += accs[w][d];
+      out[((size_t)b * n_heads + h) * hd + d] = from_f32<T>(t * inv_l);
+    }
   }
 }
 
@@ -222,8 +251,7 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
 int yalm_attn_decode_combine_bf16(const float* partial, void* out, int B, int n_heads, int head_dim, int n_splits,
                                   hipStream_t stream) {
   dim3 cgrid(B, n_heads);
-  int threads = head_dim > 64 ? 128 : 64;
-  attn_decode_combine_kernel<bf16><<<cgrid, threads, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
+  attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
   return launch_status();
 }
 
@@ -243,7 +271,7 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
     attn_decode_simple_kernel<float><<<grid, WAVE, 0, stream>>>(
         (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
         seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
-    attn_decode_combine_kernel<float><<<cgrid, WAVE, 0, stream>>>(partial, (float*)out, n_heads, head_dim, n_splits);
+    attn_decode_combine_kernel<float><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (float*)out, n_heads, head_dim, n_splits);
     return launch_status();
   }
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
@@ -256,6 +284,6 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
   attn_decode_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
       seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
-  attn_decode_combine_kernel<bf16><<<cgrid, WAVE, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
+  attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
   return launch_status();
 }

@@ -25,6 +25,14 @@ __device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
   bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
   return ok ? *reinterpret_cast<const bf16x8*>(p) : z;
 }
+// A load that every lane makes (from an address kept inside the matrix), zeroed afterwards
+// where it does not count.  Loads under a branch make the compiler wait for all loads in
+// flight before the next arithmetic, which undoes the prefetch.
+__device__ __forceinline__ bf16x8 load8_always(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ bf16x8 zero_unless(bf16x8 v, bool ok) {
+  bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+  return ok ? v : z;
+}
 
 constexpr int EPI_F32 = 0, EPI_STORE = 1, EPI_ADD = 2, EPI_GATED = 3, EPI_ROPE = 4;
 
@@ -54,7 +62,7 @@ struct ChainArgs {
 // j = lane%16) holds batch rows 4q..4q+3 of weight row j.  Which k a lane's slot
 // holds is the same for both operands, so any assignment of k to slots is right;
 // here step s of a chunk takes k = kc + 32 s + 8 q ... + 8.
-template <int MT, int NT, int NWAVES, int EPI, int KS>
+template <int MT, int NT, int NWAVES, int EPI, int KS, bool PREFETCH = true>
 __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ X,
                                                                      const bf16* __restrict__ W,
                                                                      void* __restrict__ Cv, int M, int N, int K,
@@ -89,22 +97,41 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
 #pragma unroll
     for (int t = 0; t < NT; ++t) acc[mt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  bf16x8 wv[NT][KS], xv[MT][KS];
-  int kc = wave * KC;
-  if (kc < K) {
+  // Workgroups start at different chunks of K (and wrap around): with all of them on the
+  // same columns at the same time, the rows' 8 KB-strided pieces crowd few memory channels.
+  const int n_chunks = (K + KC - 1) / KC;
+  const int rot = (int)((blockIdx.x * 5u) % (unsigned)n_chunks);
+  auto chunk_k = [&](int c) {
+    int cc = c + rot;
+    if (cc >= n_chunks) cc -= n_chunks;
+    return cc * KC;
+  };
+  // the residual values of the epilogue's first tile are asked for now, not after the sums
+  f32x4 c_old = (f32x4){0.f, 0.f, 0.f, 0.f};
+  if (EPI == EPI_ADD && wave < MT * NT) {
+    const int n = min(n0 + (wave % NT) * 16 + j, N - 1);
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-      int k = kc + s * 32 + q * 8;
-      bool ok = k < K;
-#pragma unroll
-      for (int t = 0; t < NT; ++t) wv[t][s] = load8(wrow[t] + k, ok && wok[t]);
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) xv[mt][s] = load8(xrow[mt] + k, ok && xok[mt]);
+    for (int r = 0; r < 4; ++r) {
+      const int m = min((wave / NT) * 16 + 4 * q + r, M - 1);
+      c_old[r] = ((const float*)Cv)[(size_t)m * N + n];
     }
   }
 
-  // row scales from the producer's partial sums of squares (a wave per row, lanes over the parts)
-  if (ca.ss_in != nullptr) {
+  auto load_chunk = [&](int c, bf16x8 (&w)[NT][KS], bf16x8 (&x)[MT][KS]) {
+    const int kc = chunk_k(c);
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+      const int k = kc + s * 32 + q * 8;
+      const bool ok = k < K;
+      const int kk = ok ? k : K - 8;               // rows beyond N or M are clamped too and never stored
+#pragma unroll
+      for (int t = 0; t < NT; ++t) w[t][s] = load8_always(wrow[t] + kk);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) x[mt][s] = zero_unless(load8_always(xrow[mt] + kk), ok);
+    }
+  };
+  auto row_scales = [&]() {   // from the producer's partial sums of squares (a wave per row, lanes over the parts)
+    if (ca.ss_in == nullptr) return;
     for (int m = wave; m < MT * 16; m += NWAVES) {
       float s = 0.f;
       if (m < M)
@@ -112,36 +139,49 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
       s = wave_sum(s);
       if (lane == 0) sm_scale[m] = 1.0f / sqrtf(s / (float)K + ca.eps);
     }
-  }
+  };
 
-  for (; kc < K; kc += NWAVES * KC) {
-    bf16x8 wn[NT][KS], xn[MT][KS];
-    int kn = kc + NWAVES * KC;
-    if (kn < K) {                                // prefetch the wave's next chunk
+  bf16x8 wv[NT][KS], xv[MT][KS];
+  if (!PREFETCH) {
+    // few, large chunks: all loads of a chunk are in flight at once and the products
+    // start as the first arrive (K <= 512 * NWAVES is one round trip to memory)
+    bool first = true;
+    for (int c = wave; c < n_chunks; c += NWAVES) {
+      load_chunk(c, wv, xv);
+      if (first) row_scales();
+      first = false;
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
-        int k = kn + s * 32 + q * 8;
-        bool ok = k < K;
+      for (int s = 0; s < KS; ++s)
 #pragma unroll
-        for (int t = 0; t < NT; ++t) wn[t][s] = load8(wrow[t] + k, ok && wok[t]);
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xn[mt][s] = load8(xrow[mt] + k, ok && xok[mt]);
-      }
+          for (int t = 0; t < NT; ++t)
+            acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
     }
+    if (first) row_scales();
+  } else {
+    int c = wave;
+    if (c < n_chunks) load_chunk(c, wv, xv);
+    row_scales();
+    for (; c < n_chunks; c += NWAVES) {
+      bf16x8 wn[NT][KS], xn[MT][KS];
+      const bool more = c + NWAVES < n_chunks;
+      if (more) load_chunk(c + NWAVES, wn, xn);    // prefetch the wave's next chunk
 #pragma unroll
-    for (int s = 0; s < KS; ++s)
+      for (int s = 0; s < KS; ++s)
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt)
+        for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
-    if (kn < K) {
+          for (int t = 0; t < NT; ++t)
+            acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
+      if (more) {
 #pragma unroll
-      for (int s = 0; s < KS; ++s) {
+        for (int s = 0; s < KS; ++s) {
 #pragma unroll
-        for (int t = 0; t < NT; ++t) wv[t][s] = wn[t][s];
+          for (int t = 0; t < NT; ++t) wv[t][s] = wn[t][s];
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) xv[mt][s] = xn[mt][s];
+          for (int mt = 0; mt < MT; ++mt) xv[mt][s] = xn[mt][s];
+        }
       }
     }
   }
@@ -202,7 +242,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
         sq[r] = 0.f;
         if (m < M && n < N) {
           size_t o = (size_t)m * N + n;
-          float y = ((float*)Cv)[o] + v[r];
+          float y = (idx == wave ? c_old[r] : ((float*)Cv)[o]) + v[r];
           ((float*)Cv)[o] = y;
           if (emit) {
             ca.emit_xn[o] = static_cast<bf16>(y * nw);
@@ -263,20 +303,32 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
   }
 }
 
-// few weight rows: 16 rows and 8 waves a workgroup, so that every CU has work;
-// many: 64 rows (32 if the batch needs the registers) and 4 waves
+// Up to 16 batch rows (measured at 4096..32000 weight rows, K 4096 and 14336): many
+// weight rows, or the gated epilogue, take 32 rows and 4 waves a workgroup with all loads
+// of a 256-wide chunk in flight at once; a long K takes 16 rows, 8 waves and 512-wide
+// chunks; the small projections 16 rows, 8 waves and prefetched 128-wide chunks.  A producer
+// of the norm chain always owns 16 rows (one emitted part a workgroup).  More batch rows
+// (only when the split-K kernel refused the shape) keep 128-wide chunks for the registers.
 template <int MT, int EPI>
 int launch_mt(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, const ChainArgs& ca,
               hipStream_t stream) {
-  const bool wide = EPI == EPI_GATED || (N >= 16384 && ca.emit_nw == nullptr);
-  if (wide) {
-    if (MT <= 2)
-      gemm_skinny_kernel<MT, 4, 4, EPI, 4><<<ceil_div(N, 64), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
+  constexpr int E = EPI == EPI_GATED ? EPI_F32 : EPI;   // the gated epilogue needs pairs of tiles
+  const bool emit = ca.emit_nw != nullptr;
+  if constexpr (MT == 1) {
+    if (EPI == EPI_GATED || (!emit && N > 4096 && K < 8192))
+      gemm_skinny_kernel<1, 2, 4, EPI, 8, false><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
+    else if (K >= 8192)
+      gemm_skinny_kernel<1, 1, 8, E, 16, false><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
     else
-      gemm_skinny_kernel<MT, 2, 4, EPI, 4><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
+      gemm_skinny_kernel<1, 1, 8, E, 4><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
   } else {
-    constexpr int E = EPI == EPI_GATED ? EPI_F32 : EPI;
-    gemm_skinny_kernel<MT, 1, 8, E, 4><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
+    const bool wide = EPI == EPI_GATED || (N >= 16384 && !emit);
+    if (wide && MT <= 2)
+      gemm_skinny_kernel<MT, 4, 4, EPI, 4><<<ceil_div(N, 64), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
+    else if (wide)
+      gemm_skinny_kernel<MT, 2, 4, EPI, 4><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
+    else
+      gemm_skinny_kernel<MT, 1, 8, E, 4><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
   }
   return launch_status();
 }
