@@ -314,7 +314,7 @@ extern "C" int yalm_gemm_chain_qkv_rope(const void* X, const float* ss_in, int n
                                         int rotary_dim, int n_pages, hipStream_t stream) {
   const int N = (n_heads + 2 * n_kv_heads) * head_dim;
   if (M < 1 || M > 64 || K <= 0 || K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wqkv & 15) || ss_in == nullptr ||
-      n_parts_in <= 0)
+      n_parts_in <= 0 || block_table == nullptr || tok_pos == nullptr || seq_slot == nullptr)
     return YALM_ERR_ARG;
   if (head_dim <= 0 || head_dim % 16 != 0 || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > head_dim ||
       n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || n_pages <= 0)
