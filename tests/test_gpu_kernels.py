@@ -82,8 +82,10 @@ def test_rmsnorm(D, w_dtype, out_dtype):
 
 # ------------------------------------------------------------------ GEMM
 
+# more than 64 rows: K a multiple of 64 takes the kernel that loads straight into LDS (128x128 tiles,
+# or 256x256 where 160 of them exist), any other K the register-staged one
 GEMM_SHAPES = [(1, 16, 256), (3, 70, 96), (64, 130, 264), (65, 64, 80), (200, 333, 1000), (8, 4096 + 16, 136),
-               (130, 100, 50)]
+               (130, 100, 50), (65, 64, 64), (200, 333, 1024), (300, 20480 + 8, 128), (513, 130, 192)]
 
 
 @pytest.mark.parametrize("simple", [False, True])
@@ -112,7 +114,8 @@ def test_gemm_store_and_add(M, N, Kd, dtype, simple):
 
 @pytest.mark.parametrize("simple", [False, True])
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("M,H,D", [(1, 16, 64), (5, 176, 64), (70, 100, 96), (64, 1000, 264), (3, 14336, 128)])
+@pytest.mark.parametrize("M,H,D", [(1, 16, 64), (5, 176, 64), (70, 100, 96), (64, 1000, 264), (3, 14336, 128),
+                                   (70, 100, 128), (300, 10300, 64), (260, 1000, 256)])
 def test_gemm_gated(M, H, D, dtype, simple):
     from yalm_amd.parts.swiglu import interleave_gate_up
     k = K()

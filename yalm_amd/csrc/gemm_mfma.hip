@@ -5,8 +5,9 @@
 //    chunks of 128, every lane streaming 64 contiguous bytes of a weight row per
 //    chunk; the batch is the other MFMA operand (16 rows a tile, up to 4 tiles);
 //    partial sums of the waves meet in LDS, then the epilogue runs once.
-//  * gemm_tiled   (M > 64, prefill): 128x128x64 or 256x128x64 tiles through LDS with a
-//    register prefetch of the next tile, 4 waves, v_mfma_f32_32x32x16_bf16.
+//  * gemm_tiled   (M > 64, prefill, K not a multiple of 64; otherwise gemm_dma.hip runs):
+//    128x128x64 or 256x128x64 tiles through LDS with a register prefetch of the next
+//    tile, 4 waves, v_mfma_f32_32x32x16_bf16.
 //
 // Both take any M and N and any K that is a multiple of 8 (rows must be 16-byte
 // aligned); other shapes are refused so that the caller runs the float32-arithmetic kernel.
@@ -189,6 +190,9 @@ int tiled_launch(const bf16* A, const bf16* W, void* C, int M, int N, int K, int
 int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
                          int K, int epilogue, int H, hipStream_t stream);   // gemm_batch.hip
 
+int yalm_gemm_bf16_dma(const void* A, const void* W, void* C, int M, int N, int K, int epilogue, int H,
+                       hipStream_t stream);                                  // gemm_dma.hip
+
 int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
                         int K, int epilogue, int H, hipStream_t stream) {
   if (K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
@@ -206,6 +210,10 @@ int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, float* workspace,
       case 3: return skinny_dispatch<3>(a, w, C, M, N, K, H, stream);
     }
     return YALM_ERR_ARG;
+  }
+  {
+    int rc = yalm_gemm_bf16_dma(A, W, C, M, N, K, epilogue, H, stream);      // K a multiple of 64
+    if (rc != YALM_ERR_ARG) return rc;
   }
   switch (epilogue) {
     case 0: return tiled_launch<0>(a, w, C, M, N, K, H, stream);
