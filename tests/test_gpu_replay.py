@@ -20,6 +20,7 @@ LENGTHS = {
     "tiny_llama3": [3, 70, 200, 33],
     "tiny_wide_heads": [150, 33, 260, 64, 65],
     "tiny_long": [700, 64, 129],
+    "small_windowed": [300, 97, 64, 200, 31],
 }
 # batches: (request indices, first-step lengths)
 GROUPS = {
@@ -28,6 +29,7 @@ GROUPS = {
     "tiny_llama3": [([0, 1], [1, 33]), ([2, 3], [130, 20]), ([1], [64])],
     "tiny_wide_heads": [([0, 1, 2], [120, 3, 101]), ([3, 4], [63, 64]), ([1, 0], [32, 100])],
     "tiny_long": [([0, 1, 2], [500, 1, 100]), ([2, 1], [128, 63])],
+    "small_windowed": [([0, 1, 2], [250, 96, 1]), ([3, 4, 1], [97, 30, 60])],
 }
 
 _engines = {}
@@ -41,7 +43,7 @@ def folders(tmp_path_factory):
 
 def engine_for(folders, name, dtype, max_tokens=4096):
     from yalm_amd.engine import Engine, Model
-    key = (name, dtype)
+    key = (name, dtype, max_tokens)
     if key not in _engines:
         model = Model.from_folder(folders[name], dtype=helpers.torch_dtype(dtype), device="cuda:0")
         _engines[key] = Engine(model, max_tokens=max_tokens)
@@ -101,6 +103,24 @@ def test_unequal_batches_with_reuse(folders, name, dtype):
         groups.append(ids)
     steps = schedules.batches(requests, groups, prompt_lens)
     compare(folders, name, dtype, steps, requests, engine_for(folders, name, dtype), "batches")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,n_requests", [("tiny_llama", 20), ("tiny_mistral", 40), ("tiny_wide_heads", 70),
+                                             ("tiny_llama", 130), ("small_windowed", 24), ("small_windowed", 66)])
+def test_batches_of_many_requests(folders, name, n_requests, dtype):
+    """Decode batches beyond 16, 64 and 128 rows take other GEMM kernels (split-K, tiled), norm and
+    rotation kernels of their own and other graph buckets than the small batches; the requests have
+    unequal lengths and end one after another, so the batch passes through the smaller buckets too."""
+    cfg = tiny_configs.ALL[name]
+    rng = np.random.default_rng(n_requests)
+    lengths = [int(x) for x in rng.integers(2, 15, size=n_requests)]
+    lengths[0], lengths[1] = 40, 33                      # two that outlive the others
+    requests = helpers.random_requests(cfg, lengths, seed=11)
+    first = {rid: int(rng.integers(1, len(t) + 1)) for rid, t in requests.items()}
+    first["r1"] = 1
+    steps = schedules.batches(requests, [list(requests)], first)
+    compare(folders, name, dtype, steps, requests, engine_for(folders, name, dtype, max_tokens=16384), "many requests")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -86,7 +86,24 @@ TINY_LONG.update({
     "tie_word_embeddings": False,
 })
 
+# the head size of the big models (128) with a window that prompts and decoding cross:
+# the matrix-core attention kernels over a ring of cache pages
+SMALL_WINDOWED = copy.deepcopy(TINY_MISTRAL)
+SMALL_WINDOWED.update({
+    "hidden_size": 256,
+    "intermediate_size": 640,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 2,
+    "head_dim": 128,
+    "vocab_size": 512,
+    "num_hidden_layers": 2,
+    "sliding_window": 96,
+    "max_position_embeddings": 512,
+    "rms_norm_eps": 1e-5,
+})
+
 ALL = {
+    "small_windowed": SMALL_WINDOWED,
     "tiny_llama": TINY_LLAMA,
     "tiny_mistral": TINY_MISTRAL,
     "tiny_llama3": TINY_LLAMA3,
