@@ -202,12 +202,16 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
 }
 
 // ---------------------------------------------------------------------------
-// prefill: a workgroup takes 128 query positions of one head (4 waves x 32 positions,
-// two 16-position column tiles a wave); key/value tiles of 64 rows go through LDS once
-// per workgroup, double-buffered, rows stored in the order the MFMA operands read them.
-// grid (64-position tile, head): the workgroup of every second tile of a sequence works.
+// prefill: a workgroup takes 64 * NC query positions of one head (4 waves x NC 16-position
+// column tiles); key/value tiles of 64 rows go through LDS once per workgroup, double-
+// buffered, rows stored in the order the MFMA operands read them.  grid (head, 64-position
+// tile): with NC = 2 (the one in use: each key tile read from LDS serves more queries; NC = 1
+// measured no faster at 2,048 tokens and slower beyond) the workgroup of every second tile of
+// a sequence works.  The heads of a tile are neighbours in the launch order, so that the
+// workgroups running together cost the same and the heads of a group share their keys in the
+// cache; a prompt's last tiles, which see the most keys, start first.
 // ---------------------------------------------------------------------------
-template <int HD>
+template <int HD, int NC>
 __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_stage, const bf16* __restrict__ v_stage,
     bf16* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_tile0, int B, int n_heads,
@@ -220,7 +224,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16* smem = reinterpret_cast<bf16*>(smem_raw);   // [2][KTILE + VTILE]
 
-  const int gt = blockIdx.x, h = blockIdx.y;
+  // heads run fastest and tiles from the last to the first: within a sequence the last tiles see
+  // the most keys, and workgroups that start first should be the long ones
+  const int h = blockIdx.x, gt = (int)gridDim.y - 1 - (int)blockIdx.y;
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE, qd = lane / 16, j = lane % 16;
   int b = 0;
   {
@@ -233,36 +239,41 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
   }
   const int tile0 = seq_tile0[b];
   const int tq = gt - tile0;
-  if (tq & 1) return;                             // the workgroup of the even tile covers this one too
+  if (NC == 2 && (tq & 1)) return;                // the workgroup of the even tile covers this one too
   const int start = cu_seqlens[b], len = cu_seqlens[b + 1] - start;
   const int g = h / (n_heads / n_kv_heads);
   const float score_scale = 1.4426950408889634f / sqrtf((float)HD);   // log2(e) / sqrt(head_dim)
 
   const int blk0 = tq * PAGE;                     // first position of the workgroup
-  const int pos0 = blk0 + wave * 32;              // first position of the wave
+  const int pos0 = blk0 + wave * 16 * NC;         // first position of the wave
   const bool wave_live = pos0 < len;
-  bf16x8 qv[2][KS];
-  bool q_ok[2];
-  int pos_q[2];
+  bf16x8 qv[NC][KS];
+  bool q_ok[NC];
+  int pos_q[NC];
 #pragma unroll
-  for (int c = 0; c < 2; ++c) {
+  for (int c = 0; c < NC; ++c) {
     pos_q[c] = pos0 + c * 16 + j;
     q_ok[c] = pos_q[c] < len;
     const bf16* qrow = q + ((size_t)(start + (q_ok[c] ? pos_q[c] : 0)) * n_heads + h) * HD;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) qv[c][ks] = q_ok[c] ? ld8(qrow + ks * 32 + qd * 8) : zero8();
   }
-  float m[2] = {-FLT_MAX, -FLT_MAX}, l[2] = {0.f, 0.f};
-  f32x4 o[2][DT];
+  float m[NC], l[NC];
+  f32x4 o[NC][DT];
 #pragma unroll
-  for (int c = 0; c < 2; ++c)
+  for (int c = 0; c < NC; ++c) {
+    m[c] = -FLT_MAX;
+    l[c] = 0.f;
+  }
+#pragma unroll
+  for (int c = 0; c < NC; ++c)
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) o[c][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  const int blk_last = min(blk0 + 2 * PAGE - 1, len - 1);
+  const int blk_last = min(blk0 + NC * PAGE - 1, len - 1);
   const int kt_hi = blk_last / PAGE;
   const int kt_lo = window > 0 ? max(0, blk0 - window + 1) / PAGE : 0;
-  const int wave_last = min(pos0 + 31, len - 1);
+  const int wave_last = min(pos0 + 16 * NC - 1, len - 1);
   const size_t tile_elems = (size_t)n_kv_heads * PAGE * HD;
 
   // global -> registers -> LDS; key rows are stored at the index the MFMA row reads them at
@@ -302,9 +313,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     if (visible) {
       const bf16* ks_l = smem + cur * (KTILE + VTILE);
       const bf16* vs_l = ks_l + KTILE;
-      f32x4 sc[2][4];
+      f32x4 sc[NC][4];
 #pragma unroll
-      for (int c = 0; c < 2; ++c)
+      for (int c = 0; c < NC; ++c)
 #pragma unroll
         for (int t = 0; t < 4; ++t) sc[c][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -313,16 +324,16 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
         for (int ks = 0; ks < KS; ++ks) {
           const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks_l + (t * 16 + j) * KROW + ks * 32 + qd * 8);
 #pragma unroll
-          for (int c = 0; c < 2; ++c)
+          for (int c = 0; c < NC; ++c)
             sc[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qv[c][ks], sc[c][t], 0, 0, 0);
         }
-      const bool edge = base + PAGE - 1 > pos0 || (window > 0 && base < pos0 + 31 - window + 1);
-      bf16x8 pb[2][2];
-      float corr[2];
+      const bool edge = base + PAGE - 1 > pos0 || (window > 0 && base < pos0 + 16 * NC - 1 - window + 1);
+      bf16x8 pb[NC][2];
+      float corr[NC];
       // scores in the base-2 domain: p = 2^(s * log2(e) / sqrt(hd) - m)
       auto softmax_tile = [&](auto masked) {
 #pragma unroll
-        for (int c = 0; c < 2; ++c) {
+        for (int c = 0; c < NC; ++c) {
           float mx = -FLT_MAX;
 #pragma unroll
           for (int t = 0; t < 4; ++t)
@@ -358,13 +369,16 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
         softmax_tile(std::true_type{});
       else
         softmax_tile(std::false_type{});
-      const bool rescale = !__all(corr[0] == 1.0f && corr[1] == 1.0f);   // the maxima settle after a few tiles
+      bool settled = true;                        // the maxima settle after a few tiles
+#pragma unroll
+      for (int c = 0; c < NC; ++c) settled = settled && corr[c] == 1.0f;
+      const bool rescale = !__all(settled);
       const bool tail = base + PAGE > len;        // rows behind the sequence's end may hold anything
       if (rescale) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-          for (int c = 0; c < 2; ++c) o[c][dt] *= corr[c];
+          for (int c = 0; c < NC; ++c) o[c][dt] *= corr[c];
       }
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
@@ -377,7 +391,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
               if (base + 32 * s2 + 8 * qd + e >= len) vf[e] = static_cast<bf16>(0.f);
           }
 #pragma unroll
-          for (int c = 0; c < 2; ++c)
+          for (int c = 0; c < NC; ++c)
             o[c][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[c][s2], o[c][dt], 0, 0, 0);
         }
       }
@@ -386,7 +400,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     __syncthreads();
   }
 #pragma unroll
-  for (int c = 0; c < 2; ++c) {
+  for (int c = 0; c < NC; ++c) {
     float lt = l[c];
     lt += __shfl_xor(lt, 16, WAVE);
     lt += __shfl_xor(lt, 32, WAVE);
@@ -409,17 +423,16 @@ bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
 int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out,
                                 const int* cu_seqlens, const int* seq_tile0, int T, int B, int n_tiles, int n_heads,
                                 int n_kv_heads, int head_dim, int window, hipStream_t stream) {
-  if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim)) return YALM_ERR_ARG;
-  dim3 grid(n_tiles, n_heads);
+  if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_tiles > 65535) return YALM_ERR_ARG;
+  dim3 grid(n_heads, n_tiles);
   const size_t lds = 2 * ((size_t)PAGE * (head_dim + 8) + (size_t)head_dim * (PAGE + 8)) * sizeof(bf16);
+  const bf16 *qp = (const bf16*)q, *kp = (const bf16*)k_stage, *vp = (const bf16*)v_stage;
   if (head_dim == 128)
-    attn_prefill_mfma_kernel<128><<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)k_stage,
-                                                            (const bf16*)v_stage, (bf16*)out, cu_seqlens, seq_tile0,
-                                                            B, n_heads, n_kv_heads, window);
+    attn_prefill_mfma_kernel<128, 2><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, cu_seqlens, seq_tile0, B,
+                                                                n_heads, n_kv_heads, window);
   else
-    attn_prefill_mfma_kernel<64><<<grid, 256, lds, stream>>>((const bf16*)q, (const bf16*)k_stage,
-                                                           (const bf16*)v_stage, (bf16*)out, cu_seqlens, seq_tile0, B,
-                                                           n_heads, n_kv_heads, window);
+    attn_prefill_mfma_kernel<64, 2><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, cu_seqlens, seq_tile0, B,
+                                                               n_heads, n_kv_heads, window);
   return launch_status();
 }
 
