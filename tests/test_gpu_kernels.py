@@ -357,6 +357,61 @@ def test_attn_decode_finds_a_far_key(dtype):
         got = out.cpu().double().reshape(n_heads, hd)
         assert (got - vals[0][far, 0].double()).abs().max() < 0.05, far
 
+@pytest.mark.parametrize("simple", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hd,window,n", [(64, 70, 300), (128, 64, 200), (128, 100, 513), (32, 16, 90)])
+def test_attn_window_edge_decides(hd, window, n, dtype, simple):
+    """The key just outside the window has by far the largest score and a value of 1000; the key
+    just inside has the next largest and a value of 7.  A window off by one, in either kernel,
+    gives 1000 or loses the 7: among a hundred random keys it would hide in the rounding."""
+    k = K()
+    n_heads, n_kv = 4, 2
+    unit = torch.zeros(hd, dtype=torch.float64)
+    unit[3] = 1.0
+    k.FORCE_SIMPLE = simple
+    try:
+        # decode: the query at position n - 1 sees positions n - window ... n - 1
+        kp, vp, bt, slots, ring, keys, vals = paged_case([n], n_kv, hd, window, dtype, 40)
+        inside, outside = n - window, n - window - 1
+        PAGE = k.PAGE
+        for pos, strength, value in ((inside, 30.0, 7.0), (outside, 60.0, 1000.0)):
+            page = int(bt[slots[0], (pos // PAGE) % ring])
+            if pos // PAGE > (n - 1) // PAGE - ring:          # the ring still holds this position's page
+                kp[page, :, pos % PAGE, :] = (unit * strength).to(dtype)
+                vp[page, :, :, pos % PAGE] = value
+        q = (unit * 8.0).to(dtype).repeat(n_heads)[None]
+        out = torch.empty((1, n_heads * hd), dtype=dtype, device=DEV)
+        partial = torch.empty(k.attn_decode_workspace_floats(1, n_heads, hd, 3), device=DEV)
+        k.attn_decode(q.to(DEV), kp.to(DEV), vp.to(DEV), bt.to(DEV), ring, i32(slots), i32([n]), out, partial, n_heads,
+                      n_kv, hd, window, 3)
+        assert (out.cpu().double() - 7.0).abs().max() < 0.1, "decode"
+
+        # prefill: keys grow stronger towards the past, so that for query i the strongest visible key is the
+        # oldest one, i - window + 1, and the one before it would be stronger still.  The strength T - j is
+        # split over two elements (16 a + b) so that bfloat16 holds it exactly; scores of neighbours differ by 16.
+        T = n
+        s_q = 16.0 * math.sqrt(hd)
+        qrow = torch.zeros(hd, dtype=torch.float64)
+        qrow[3], qrow[4] = 16.0 * s_q, s_q
+        qq = qrow.to(dtype).repeat(T, n_heads)
+        kk = torch.zeros((T, n_kv * hd), dtype=dtype)
+        v = torch.zeros((T, n_kv * hd), dtype=dtype)
+        for j in range(T):
+            krow = torch.zeros(hd, dtype=torch.float64)
+            krow[3], krow[4] = (T - j) // 16, (T - j) % 16
+            kk[j] = krow.to(dtype).repeat(n_kv)
+            v[j] = float(j % 50)
+        ks, vs, tile0 = stage(kk, v, [T], n_kv, hd, dtype)
+        out = torch.empty((T, n_heads * hd), dtype=dtype, device=DEV)
+        k.attn_prefill(qq.to(DEV), ks.to(DEV), vs.to(DEV), out, i32([0, T]), i32(tile0), i32([0] * T),
+                       i32(list(range(T))), n_heads, n_kv, hd, window)
+        got = out.cpu().double()[:, 0]
+        want = torch.tensor([float(max(0, i - window + 1) % 50) for i in range(T)], dtype=torch.float64)
+        assert (got - want).abs().max() < 0.1, "prefill, first bad position %d" % int(((got - want).abs() >= 0.1).nonzero()[0])
+    finally:
+        k.FORCE_SIMPLE = False
+
+
 
 def test_attn_vector_of_the_reference():
     """src/test.cpp:67-126 through both attention kernels (head size padded from 3 to 16 with zeros)."""
