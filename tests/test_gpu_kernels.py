@@ -197,6 +197,52 @@ def test_rope_kv_write(n_heads, n_kv, hd, rd, dtype):
     assert (kp.float().abs().sum(dim=(1, 3)) > 0).equal(touched)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,rd,lens,ring", [(4, 2, 16, 16, [5, 130, 64], 3), (3, 1, 48, 24, [200, 1], 2),
+                                                          (8, 2, 128, 128, [70, 257], 8), (2, 2, 64, 64, [300], 3)])
+def test_rope_kv_write_tiles(n_heads, n_kv, hd, rd, lens, ring, dtype):
+    """Whole prompts, a tile of 64 positions at a time: the same q, staging area and cache pages as the
+    per-token kernel (which the tests above pin to the plain rotation), also where a prompt ends inside a
+    tile and where a ring keeps the last pages only."""
+    k = K()
+    PAGE = k.PAGE
+    B, T = len(lens), sum(lens)
+    Q, KV = n_heads * hd, n_kv * hd
+    qkv = rnd((T, Q + 2 * KV), 21).to(DEV)
+    table = make_table(max(lens) + 3, hd, rd, 10000.0).to(DEV)
+    tiles = [(n + PAGE - 1) // PAGE for n in lens]
+    tile0 = np.concatenate([[0], np.cumsum(tiles)])
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    n_tiles, n_pages = int(tile0[-1]), B * ring + 2
+    order = np.random.default_rng(5).permutation(n_pages)
+    bt = torch.full((B + 1, ring), -1, dtype=torch.int32)
+    slots = [B - b for b in range(B)]                         # slots B, B-1, ..., 1
+    nxt = 0
+    for b in range(B):
+        for c in range(min(ring, tiles[b])):
+            bt[slots[b], c] = int(order[nxt])
+            nxt += 1
+    seq = np.repeat(np.arange(B), lens)
+    pos = np.concatenate([np.arange(n) for n in lens])
+
+    def buffers():
+        return (torch.zeros((n_pages, n_kv, PAGE, hd), dtype=dtype, device=DEV),
+                torch.zeros((n_pages, n_kv, hd, PAGE), dtype=dtype, device=DEV),
+                torch.zeros((n_tiles, n_kv, PAGE, hd), dtype=dtype, device=DEV),
+                torch.zeros((n_tiles, n_kv, hd, PAGE), dtype=dtype, device=DEV),
+                torch.zeros((T, Q), dtype=dtype, device=DEV))
+    kp0, vp0, ks0, vs0, q0 = buffers()
+    k.rope_kv_write(qkv, q0, ks0, vs0, i32(tile0), kp0, vp0, bt.to(DEV), ring, i32(seq), i32(pos), i32(slots),
+                    i32(lens), table, n_heads, n_kv, hd, rd)
+    kp1, vp1, ks1, vs1, q1 = buffers()
+    assert k.rope_kv_write_tiles(qkv, q1, ks1, vs1, i32(cu), i32(tile0), kp1, vp1, bt.to(DEV), ring, i32(slots),
+                                 i32(lens), table, n_heads, n_kv, hd, rd)
+    for a, b, what in ((q0, q1, "q"), (ks0, ks1, "staged k"), (vs0, vs1, "staged v"), (kp0, kp1, "k pages"),
+                       (vp0, vp1, "v pages")):
+        assert torch.equal(a, b), what
+    assert q0.abs().sum() > 0 and kp0.abs().sum() > 0
+
+
 def test_rope_kv_write_ring_keeps_the_last_pages_only():
     k = K()
     PAGE = k.PAGE

@@ -179,6 +179,140 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same for whole prompts (every sequence from position 0), a workgroup per
+// (64-position tile, job): job < n_kv_heads: the keys and values of one KV head, whole
+// page-shaped tiles at once (the values transposed through LDS, so that staging area and
+// cache page are written in 16-byte pieces); the other jobs: one query head of the tile's
+// positions.  A thread takes a pair of a row at a time: 512 contiguous bytes a wave.
+// ---------------------------------------------------------------------------
+constexpr int VT_ROW = PAGE + 8;                  // LDS row of the transposed values (elements)
+
+__device__ __forceinline__ void store_pair(float* dst, float a, float b) {
+  *reinterpret_cast<float2*>(dst) = make_float2(a, b);
+}
+__device__ __forceinline__ void store_pair(bf16* dst, float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  bf16x2 v = {static_cast<bf16>(a), static_cast<bf16>(b)};
+  *reinterpret_cast<bf16x2*>(dst) = v;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_tiles_kernel(
+    const float* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_stage, T* __restrict__ v_stage,
+    const int* __restrict__ cu_seqlens, const int* __restrict__ seq_tile0, T* __restrict__ k_pages,
+    T* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride, int ring_pages,
+    const int* __restrict__ seq_slot, const int* __restrict__ seq_len, const float2* __restrict__ cos_sin,
+    int n_positions, int B, int n_heads, int n_kv_heads, int hd, int rotary_dim, int n_pages) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char vt_raw[];
+  T* vt = reinterpret_cast<T*>(vt_raw);           // [hd][VT_ROW]
+  const int gt = blockIdx.x, job = blockIdx.y, tid = threadIdx.x;
+  int b = 0;
+  {
+    int lo = 0, hi = B - 1;
+    while (lo < hi) {
+      int mid = (lo + hi + 1) >> 1;
+      if (seq_tile0[mid] <= gt) lo = mid; else hi = mid - 1;
+    }
+    b = lo;
+  }
+  const int ap = gt - seq_tile0[b];               // page of the sequence
+  const int start = cu_seqlens[b], len = cu_seqlens[b + 1] - start;
+  const int p0 = ap * PAGE;
+  const int rows = min(PAGE, len - p0);           // positions of this tile
+  if (rows <= 0) return;
+  const int Q = n_heads * hd, KV = n_kv_heads * hd, W = Q + 2 * KV;
+  const int half_rot = rotary_dim / 2, pairs = hd / 2;
+  const float* src0 = qkv + (size_t)(start + p0) * W;
+
+  auto rotated = [&](const float* row, int pos, int p) {
+    float2 x = *reinterpret_cast<const float2*>(row + 2 * p);
+    if (cos_sin != nullptr && p < half_rot && pos < n_positions) {
+      const float2 c = cos_sin[(size_t)pos * half_rot + p];
+      x = make_float2(x.x * c.x - x.y * c.y, x.x * c.y + x.y * c.x);
+    }
+    return x;
+  };
+
+  if (job >= n_kv_heads) {                        // a query head
+    const int h = job - n_kv_heads;
+    for (int e = tid; e < rows * pairs; e += 256) {
+      const int r = e / pairs, p = e % pairs;
+      const float2 y = rotated(src0 + (size_t)r * W + h * hd, p0 + r, p);
+      store_pair(q_out + (size_t)(start + p0 + r) * Q + h * hd + 2 * p, y.x, y.y);
+    }
+    return;
+  }
+
+  const int g = job;
+  T* kst = k_stage + ((size_t)gt * n_kv_heads + g) * PAGE * hd;
+  T* vst = v_stage + ((size_t)gt * n_kv_heads + g) * PAGE * hd;
+  T* kpage = nullptr;
+  T* vpage = nullptr;
+  const int slot = seq_slot[b];
+  if (k_pages != nullptr && slot >= 0) {          // a page is kept iff it is among the last ring_pages of its sequence
+    const int last_ap = (seq_len[b] - 1) / PAGE;
+    if (ap > last_ap - ring_pages) {
+      const int phys = block_table[(size_t)slot * table_stride + (ap % ring_pages)];
+      if (phys >= 0 && phys < n_pages) {
+        kpage = k_pages + ((size_t)phys * n_kv_heads + g) * PAGE * hd;
+        vpage = v_pages + ((size_t)phys * n_kv_heads + g) * PAGE * hd;
+      }
+    }
+  }
+  for (int e = tid; e < rows * pairs; e += 256) {
+    const int r = e / pairs, p = e % pairs;
+    const float2 y = rotated(src0 + (size_t)r * W + Q + g * hd, p0 + r, p);
+    store_pair(kst + r * hd + 2 * p, y.x, y.y);
+    if (kpage) store_pair(kpage + r * hd + 2 * p, y.x, y.y);
+    const float2 v = *reinterpret_cast<const float2*>(src0 + (size_t)r * W + Q + KV + g * hd + 2 * p);
+    vt[(2 * p) * VT_ROW + r] = from_f32<T>(v.x);
+    vt[(2 * p + 1) * VT_ROW + r] = from_f32<T>(v.y);
+  }
+  __syncthreads();
+  // values, transposed: element i of the head is a row of 64 positions; positions behind the prompt's end get zeros
+  constexpr int PER = 16 / sizeof(T);             // elements in 16 bytes
+  for (int e = tid; e < hd * (PAGE / PER); e += 256) {
+    const int i = e / (PAGE / PER), c0 = (e % (PAGE / PER)) * PER;
+    T piece[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u) piece[u] = c0 + u < rows ? vt[i * VT_ROW + c0 + u] : from_f32<T>(0.f);
+    *reinterpret_cast<uint4*>(vst + (size_t)i * PAGE + c0) = *reinterpret_cast<const uint4*>(piece);
+    if (vpage) *reinterpret_cast<uint4*>(vpage + (size_t)i * PAGE + c0) = *reinterpret_cast<const uint4*>(piece);
+  }
+}
+
+extern "C" int yalm_rope_kv_write_tiles(const float* qkv, void* q_out, void* k_stage, void* v_stage,
+                                        const int* cu_seqlens, const int* seq_tile0, void* k_pages, void* v_pages,
+                                        const int* block_table, int table_stride, int ring_pages,
+                                        const int* seq_slot, const int* seq_len, const float* cos_sin,
+                                        int n_positions, int T, int B, int n_tiles, int n_heads, int n_kv_heads,
+                                        int head_dim, int rotary_dim, int n_pages, int dtype, hipStream_t stream) {
+  if (T <= 0 || B <= 0 || n_tiles <= 0) return YALM_OK;
+  if (head_dim <= 0 || (head_dim & 1) || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > head_dim ||
+      n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || k_stage == nullptr || v_stage == nullptr ||
+      cu_seqlens == nullptr || seq_tile0 == nullptr || n_heads + n_kv_heads > 65535 ||
+      ((n_heads + 2 * n_kv_heads) * head_dim) % 2 != 0)
+    return YALM_ERR_ARG;
+  const size_t esize = dtype == YALM_F32 ? 4 : 2;
+  const size_t lds = (size_t)head_dim * VT_ROW * esize;
+  if (lds > 64 * 1024) return YALM_ERR_ARG;
+  dim3 grid(n_tiles, n_kv_heads + n_heads);
+  if (dtype == YALM_F32)
+    rope_kv_tiles_kernel<float><<<grid, 256, lds, stream>>>(
+        qkv, (float*)q_out, (float*)k_stage, (float*)v_stage, cu_seqlens, seq_tile0, (float*)k_pages, (float*)v_pages,
+        block_table, table_stride, ring_pages, seq_slot, seq_len, (const float2*)cos_sin, n_positions, B, n_heads,
+        n_kv_heads, head_dim, rotary_dim, n_pages);
+  else if (dtype == YALM_BF16)
+    rope_kv_tiles_kernel<bf16><<<grid, 256, lds, stream>>>(
+        qkv, (bf16*)q_out, (bf16*)k_stage, (bf16*)v_stage, cu_seqlens, seq_tile0, (bf16*)k_pages, (bf16*)v_pages,
+        block_table, table_stride, ring_pages, seq_slot, seq_len, (const float2*)cos_sin, n_positions, B, n_heads,
+        n_kv_heads, head_dim, rotary_dim, n_pages);
+  else
+    return YALM_ERR_DTYPE;
+  return launch_status();
+}
+
 extern "C" int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_stage, void* v_stage,
                                   const int* seq_tile0, void* k_pages, void* v_pages, const int* block_table, int table_stride, int ring_pages,
                                   const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_len,

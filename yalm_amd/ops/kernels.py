@@ -315,6 +315,52 @@ def rope_kv_write(qkv, q_out, k_stage, v_stage, seq_tile0, k_pages, v_pages, blo
         n_pos, T, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, dtype_code(dt), _stream()), "rope_kv_write")
 
 
+def rope_kv_write_tiles(qkv, q_out, k_stage, v_stage, cu_seqlens, seq_tile0, k_pages, v_pages, block_table, ring_pages,
+                        seq_slot, seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim):
+    """rope_kv_write for a step of whole prompts (every sequence from position 0), a page-shaped
+    tile of 64 positions at a time.  False if the kernel refuses the head size (the caller then
+    uses rope_kv_write)."""
+    _check_heads(n_heads, n_kv_heads, head_dim)
+    T = qkv.shape[0]
+    Q, KV = n_heads * head_dim, n_kv_heads * head_dim
+    dt = q_out.dtype
+    if head_dim * (PAGE + 8) * dt.itemsize > 64 * 1024:
+        return False
+    B = seq_slot.shape[0]
+    n_tiles = k_stage.shape[0]
+    p_qkv = _need(qkv, "qkv", torch.float32, (T, Q + 2 * KV))
+    p_q = _need(q_out, "q_out", dt, (T, Q))
+    p_ks = _need(k_stage, "k_stage", dt, (n_tiles, n_kv_heads, PAGE, head_dim))
+    p_vs = _need(v_stage, "v_stage", dt, (n_tiles, n_kv_heads, head_dim, PAGE))
+    p_cu = _need(cu_seqlens, "cu_seqlens", torch.int32, (B + 1,))
+    p_t0 = _need(seq_tile0, "seq_tile0", torch.int32, (B + 1,))
+    n_pages, stride = 0, 0
+    p_kp = p_vp = p_bt = None
+    if k_pages is not None:
+        n_pages = k_pages.shape[0]
+        p_kp = _need(k_pages, "k_pages", dt, (n_pages, n_kv_heads, PAGE, head_dim))
+        p_vp = _need(v_pages, "v_pages", dt, (n_pages, n_kv_heads, head_dim, PAGE))
+        p_bt = _need(block_table, "block_table", torch.int32, (None, None))
+        stride = block_table.shape[1]
+        if ring_pages <= 0 or ring_pages > stride:
+            raise ValueError("ring_pages %d does not fit the block table (%d columns)" % (ring_pages, stride))
+    p_ss = _need(seq_slot, "seq_slot", torch.int32, (B,))
+    p_sl = _need(seq_len, "seq_len", torch.int32, (B,))
+    n_pos = 0
+    p_cs = None
+    if cos_sin is not None:
+        if rotary_dim % 2 != 0 or rotary_dim > head_dim or rotary_dim <= 0:
+            raise ValueError("rotary_dim %d does not fit head_dim %d" % (rotary_dim, head_dim))
+        n_pos = cos_sin.shape[0]
+        p_cs = _need(cos_sin, "cos_sin", torch.float32, (n_pos, rotary_dim // 2, 2))
+    else:
+        rotary_dim = 0
+    library.check(library.lib().yalm_rope_kv_write_tiles(
+        p_qkv, p_q, p_ks, p_vs, p_cu, p_t0, p_kp, p_vp, p_bt, stride, max(ring_pages, 1), p_ss, p_sl, p_cs, n_pos, T, B,
+        n_tiles, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, dtype_code(dt), _stream()), "rope_kv_write_tiles")
+    return True
+
+
 def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
                  window):
     """Causal (and windowed) attention of packed sequences that start at position 0, over

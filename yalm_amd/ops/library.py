@@ -29,6 +29,8 @@ _SIGNATURES = {
                                       _I, _I, _P]),
     "yalm_rope_kv_write": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                 _I, _I, _P]),
+    "yalm_rope_kv_write_tiles": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I,
+                                      _I, _I, _I, _I, _P]),
     "yalm_attn_prefill": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_workspace": (ctypes.c_long, [_I, _I, _I, _I]),
@@ -37,7 +39,7 @@ _SIGNATURES = {
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
 }
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 class KernelError(RuntimeError):

@@ -154,9 +154,13 @@ class GQAttention(Part):
         else:
             kst = vst = None
         if writes_cache:
-            kernels.rope_kv_write(qkv, q, kst, vst, ctx.seq_tile0, k_pages, v_pages, group.table, group.ring_pages,
-                                  ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads,
-                                  self.n_kv_heads, self.head_dim, pos.rotary_dim)
+            done = prefill and kernels.rope_kv_write_tiles(
+                qkv, q, kst, vst, ctx.cu_seqlens, ctx.seq_tile0, k_pages, v_pages, group.table, group.ring_pages,
+                ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads, self.head_dim, pos.rotary_dim)
+            if not done:
+                kernels.rope_kv_write(qkv, q, kst, vst, ctx.seq_tile0, k_pages, v_pages, group.table,
+                                      group.ring_pages, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table,
+                                      self.n_heads, self.n_kv_heads, self.head_dim, pos.rotary_dim)
         else:
             kernels.rope_kv_write(qkv, q, None, None, None, None, None, None, 0, ctx.tok_seq, ctx.tok_pos,
                                   ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads, self.head_dim,
