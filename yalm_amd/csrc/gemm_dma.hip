@@ -185,7 +185,7 @@ int launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int
 template <int EPI>
 int launch(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
   if ((long)ceil_div(M, 256) * ceil_div(N, 256) >= 160)
-    return launch_shape<EPI, 256, 256, 2, 2, 4, 1>(A, W, C, M, N, K, H, stream);
+    return launch_shape<EPI, 256, 256, 2, 4, 2, 1>(A, W, C, M, N, K, H, stream);
   return launch_shape<EPI, 128, 128, 2, 2, 2, 2>(A, W, C, M, N, K, H, stream);
 }
 
