@@ -228,3 +228,47 @@ def test_command_line(folders):
     bad = subprocess.run([sys.executable, "-m", "yalm_amd", folder, "-d", "cpu", "--tokens", "1"], cwd=ROOT,
                          stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=120)
     assert bad.returncode == 1 and "no CPU path" in bad.stderr
+
+
+def test_command_line_with_a_tokenizer(folders, tmp_path):
+    """Text prompts and the passkey mode (src/main.cpp:237-332) need tokenizer.json: a byte-level one with a
+    few words is written next to the random model; what the program prints is the plain implementation's
+    greedy continuation, decoded."""
+    import json
+    import shutil
+    from yalm_amd.tokenizer import Tokenizer
+    name = "tiny_wide_heads"
+    cfg = tiny_configs.ALL[name]
+    folder = str(tmp_path / "with_tokenizer")
+    shutil.copytree(folders[name], folder)
+    vocab = {"<unk>": 0, "<s>": 1, "</s>": 2}
+    for i in range(256):
+        vocab["<0x%02X>" % i] = 3 + i
+    for i, t in enumerate(["\u2581The", "\u2581pass", "\u2581key", "\u2581is", "\u2581the", "\u2581green", "."]):
+        vocab[t] = 259 + i
+    assert max(vocab.values()) < cfg["vocab_size"]
+    with open(os.path.join(folder, "tokenizer.json"), "w") as f:
+        json.dump({"model": {"vocab": vocab, "byte_fallback": True}, "added_tokens": []}, f)
+    tok = Tokenizer.from_folder(folder, cfg["vocab_size"], cfg["bos_token_id"], cfg["eos_token_id"])
+
+    def printed(tokens, last):
+        out = b""
+        for t in tokens:
+            out += tok.decode_one(last, t)
+            last = t
+        return out
+
+    text = "The pass key is green."
+    p = subprocess.run([sys.executable, "-m", "yalm_amd", folder, "-i", text, "-n", "5", "-t", "0", "--dtype", "float32"],
+                       cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=300)
+    assert p.returncode == 0, p.stderr[-3000:]
+    prompt = tok.encode(text, True)
+    assert prompt[:6] == [1, 3 + ord("T"), 3 + ord("h"), 3 + ord("e"), 260, 261]     # no space is put before the text
+    want = plain_greedy(folder, prompt, 5, stop=(cfg["eos_token_id"],))
+    assert p.stdout.startswith(printed(want, prompt[-1])), (p.stdout[:80], printed(want, prompt[-1]))
+
+    p = subprocess.run([sys.executable, "-m", "yalm_amd", folder, "-m", "passkey", "-n", "2", "-l", "1", "--seed", "4",
+                        "--dtype", "float32"], cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=300)
+    assert p.returncode == 0, p.stderr[-3000:]
+    out = p.stdout.decode("utf-8", "replace")
+    assert "Passkey test:" in out and "passkey:" in out and " What is the pass key? The pass key is" in out
