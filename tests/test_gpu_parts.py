@@ -320,3 +320,178 @@ def test_toy_mixer_and_architecture_from_outside(tmp_path):
     finally:
         unregister_architecture("ToyForCausalLM")
         unregister_part("mixer", "toy_running_mean")
+
+
+# ---------------------------------------------------------------------------
+# a toy feed-forward with routing and a toy position encoding, in a second toy architecture
+# ---------------------------------------------------------------------------
+
+def define_routed_and_linear_parts():
+    from yalm_amd.ops import kernels
+    from yalm_amd.parts import Part, register_part
+    from yalm_amd.weights import ParamSpec
+
+    class Top1Experts(Part):
+        """x += p_e * W2_e silu(W1_e h) with e = argmax of the router's logits and p_e its softmax
+        probability (float32).  Rows are gathered per expert in front of the framework's GEMM and
+        scattered back behind it."""
+        graph_safe = False
+
+        def __init__(self, spec, dim, prefix):
+            super().__init__(spec, dim, prefix)
+            self.n_experts, self.hidden = int(spec.params["n_experts"]), int(spec.params["hidden"])
+
+        def param_specs(self):
+            out = [ParamSpec(self.prefix + "router.weight", (self.n_experts, self.dim), fan_in=self.dim)]
+            for e in range(self.n_experts):
+                out.append(ParamSpec("%sexperts.%d.w1.weight" % (self.prefix, e), (self.hidden, self.dim), fan_in=self.dim))
+                out.append(ParamSpec("%sexperts.%d.w2.weight" % (self.prefix, e), (self.dim, self.hidden),
+                                     fan_in=self.hidden))
+            return out
+
+        def load(self, get, compute_dtype, device):
+            self.router = get(self.prefix + "router.weight").to(device, torch.float32)
+            self.w1 = [get("%sexperts.%d.w1.weight" % (self.prefix, e)).to(device, compute_dtype)
+                       for e in range(self.n_experts)]
+            self.w2 = [get("%sexperts.%d.w2.weight" % (self.prefix, e)).to(device, compute_dtype)
+                       for e in range(self.n_experts)]
+
+        def forward(self, h, x, ctx):
+            logits = torch.empty((h.shape[0], self.n_experts), dtype=torch.float32, device=h.device)
+            kernels.gemm(h.float().contiguous(), self.router, logits, kernels.EPI_STORE_F32)     # router in 32-bit
+            prob, chosen = torch.softmax(logits, dim=-1).max(dim=-1)
+            for e in range(self.n_experts):
+                rows = (chosen == e).nonzero()[:, 0]
+                if rows.numel() == 0:
+                    continue
+                he = h.index_select(0, rows).contiguous()
+                mid = torch.empty((rows.numel(), self.hidden), dtype=torch.float32, device=h.device)
+                self._gemm(ctx, he, self.w1[e], mid, kernels.EPI_STORE_F32)
+                act = torch.nn.functional.silu(mid).to(h.dtype)
+                y = torch.zeros((rows.numel(), self.dim), dtype=torch.float32, device=h.device)
+                self._gemm(ctx, act, self.w2[e], y, kernels.EPI_ADD_F32)
+                x.index_add_(0, rows, y * prob[rows][:, None])
+
+    class LinearFrequencies(Part):
+        """Rotation whose pair p turns by pos * step * (p + 1): the same table interface as the
+        framework's rotary encoding, another law of frequencies."""
+
+        def __init__(self, spec, dim, prefix):
+            super().__init__(spec, dim, prefix)
+            self.head_dim = int(spec.params["head_dim"])
+            self.rotary_dim = int(spec.params["rotary_dim"])
+            self.step = float(spec.params["step"])
+            self.table = None
+
+        def prepare(self, n_positions, device):
+            f = self.step * torch.arange(1, self.rotary_dim // 2 + 1, dtype=torch.float64)
+            ang = torch.arange(n_positions, dtype=torch.float64)[:, None] * f[None, :]
+            self.table = torch.stack([torch.cos(ang), torch.sin(ang)], dim=-1).float().contiguous().to(device)
+
+        @property
+        def n_positions(self):
+            return 0 if self.table is None else self.table.shape[0]
+
+        def arrange_projection_rows(self, w, n_heads):
+            return w
+
+    register_part("feed_forward", "toy_top1_experts", Top1Experts, replace=True)
+    register_part("position", "toy_linear_frequencies", LinearFrequencies, replace=True)
+
+
+class RoutedToyConfig:
+    """Layer 0: attention with the linear-frequency rotation (half of each head rotated) and a dense
+    feed-forward; layer 1: the same attention kind with a window and the routed feed-forward."""
+
+    def __init__(self, d):
+        self.d = d
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d)
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def to_spec(self):
+        from yalm_amd.config import LayerSpec, ModelSpec, PartSpec
+        d = self.d
+        norm = {"eps": d["eps"]}
+        pos = PartSpec("toy_linear_frequencies", {"head_dim": 32, "rotary_dim": 16, "step": d["step"]})
+
+        def attn(window):
+            return PartSpec("gqa_attention", {"n_heads": 3, "n_kv_heads": 3, "head_dim": 32, "window": window,
+                                              "position": pos}, prefix="attn.")
+        ffs = [PartSpec("swiglu", {"hidden": d["hidden"]}, prefix="ff."),
+               PartSpec("toy_top1_experts", {"n_experts": d["experts"], "hidden": d["hidden"]}, prefix="moe.")]
+        layers = [LayerSpec("prenorm_residual", attn(w), ff, PartSpec("rmsnorm", norm, prefix="n1."),
+                            PartSpec("rmsnorm", norm, prefix="n2."), "toy.%d." % i)
+                  for i, (w, ff) in enumerate(zip((0, 9), ffs))]
+        return ModelSpec("RoutedToyForCausalLM", d["width"], d["vocab"], d["positions"],
+                         PartSpec("token_embedding", {"vocab_size": d["vocab"]}, prefix="toy.emb."), layers,
+                         PartSpec("rmsnorm", norm, prefix="toy.norm."),
+                         PartSpec("lm_head", {"vocab_size": d["vocab"], "tied": False}, prefix="toy.head."))
+
+
+def routed_toy_plain_forward(w, d, tokens):
+    T = len(tokens)
+    x = R.embedding(w["toy.emb.weight"], torch.tensor(tokens))
+    f = torch.cat([d["step"] * torch.arange(1, 9, dtype=torch.float64), torch.zeros(8, dtype=torch.float64)])
+    pos = torch.arange(T)
+    for i, window in enumerate((0, 9)):
+        p = "toy.%d." % i
+        h = R.rmsnorm(x, w[p + "n1.weight"], d["eps"])
+        q = (h @ w[p + "attn.q_proj.weight"].double().T).reshape(T, 3, 32)
+        k = (h @ w[p + "attn.k_proj.weight"].double().T).reshape(T, 3, 32)
+        v = (h @ w[p + "attn.v_proj.weight"].double().T).reshape(T, 3, 32)
+        a = R.attention(R.rope_interleaved(q, pos, f), R.rope_interleaved(k, pos, f), v, window)
+        x = x + a.reshape(T, 96) @ w[p + "attn.o_proj.weight"].double().T
+        h = R.rmsnorm(x, w[p + "n2.weight"], d["eps"])
+        if i == 0:
+            x = x + R.swiglu_ffn(h, w[p + "ff.gate_proj.weight"], w[p + "ff.down_proj.weight"], w[p + "ff.up_proj.weight"])
+        else:
+            probs = torch.softmax(h @ w[p + "moe.router.weight"].double().T, dim=-1)
+            for t in range(T):
+                e = int(torch.argmax(probs[t]))
+                mid = R.silu(w["%smoe.experts.%d.w1.weight" % (p, e)].double() @ h[t])
+                x[t] = x[t] + probs[t, e] * (w["%smoe.experts.%d.w2.weight" % (p, e)].double() @ mid)
+    return R.rmsnorm(x, w["toy.norm.weight"], d["eps"]) @ w["toy.head.weight"].double().T
+
+
+def test_toy_routed_feed_forward_and_position_encoding_from_outside(tmp_path):
+    """A feed-forward that routes rows to experts and a position encoding with its own law of angles,
+    both defined above, take their places in a layer by configuration alone; every way of cutting the
+    requests agrees with the toy written out in float64."""
+    from yalm_amd import Engine, Model, register_architecture, write_random_model
+    from yalm_amd.config import unregister_architecture
+    from yalm_amd.parts import unregister_part
+    define_routed_and_linear_parts()
+    register_architecture("RoutedToyForCausalLM", RoutedToyConfig, replace=True)
+    try:
+        d = {"architectures": ["RoutedToyForCausalLM"], "width": 56, "hidden": 72, "vocab": 83, "positions": 128,
+             "eps": 1e-6, "experts": 3, "step": 0.37}
+        folder = write_random_model(str(tmp_path / "routed_toy"), d, seed=4)
+        model = Model.from_folder(folder, dtype=torch.float32, device=DEV)
+        assert not model.graph_safe()
+        engine = Engine(model, max_tokens=1024)
+        assert len(engine.cache.kv_groups) == 2                # all keys for layer 0, a window's ring for layer 1
+        cfg, w = R.read_folder(folder)
+        rng = np.random.default_rng(3)
+        requests = {rid: [int(t) for t in rng.integers(0, d["vocab"], size=n)]
+                    for rid, n in (("a", 30), ("b", 3), ("c", 70), ("d", 12))}
+        used = set()
+        probs = torch.softmax(R.rmsnorm(R.embedding(w["toy.emb.weight"], torch.tensor(requests["c"])),
+                                        w["toy.1.n2.weight"], d["eps"]) @ w["toy.1.moe.router.weight"].double().T, -1)
+        used.update(int(e) for e in probs.argmax(-1))
+        assert len(used) > 1                                    # the routing has something to decide
+        for steps in (schedules.whole(requests), schedules.tail_one_by_one(requests, 6),
+                      schedules.batches(requests, [["a", "b"], ["c", "d"]], {"a": 11, "b": 1, "c": 64, "d": 2})):
+            out = schedules.replay_in_process(engine, steps)
+            got = schedules.per_request(steps, out, requests)
+            for rid, toks in requests.items():
+                want = routed_toy_plain_forward(w, d, toks).float().numpy()
+                helpers.check_logits(got[rid], want, "float32", "routed toy %s" % rid)
+    finally:
+        unregister_architecture("RoutedToyForCausalLM")
+        unregister_part("feed_forward", "toy_top1_experts")
+        unregister_part("position", "toy_linear_frequencies")
