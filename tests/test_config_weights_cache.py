@@ -387,6 +387,18 @@ def test_generation_loop_decisions():
     assert generate(e2, [[1]], max_new_tokens=0, sampler=ArgmaxSampler()) == [[]]
 
 
+def test_a_failed_step_gives_the_slots_back():
+    class Failing(ScriptedEngine):
+        def step(self, slots, tokens, want=None):
+            if len(self.log) == 3:
+                raise RuntimeError("step failed")
+            return super().step(slots, tokens, want)
+    eng = Failing()
+    with pytest.raises(RuntimeError, match="step failed"):
+        generate(eng, [[1], [7, 8], [3]], max_new_tokens=6, sampler=ArgmaxSampler())
+    assert sorted(eng.free) == [0, 1, 2] and not eng.lens          # also the one that had ended before
+
+
 def test_plan_batches():
     assert plan_batches([5, 17, 1, 300, 64], 8, 2, 1024, 8, 512) == [[0, 1], [2, 3], [4]]
     # the cache bounds a batch: 3 requests of 100 + 28 tokens = 2 pages each, 4 pages in all

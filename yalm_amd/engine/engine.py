@@ -111,9 +111,10 @@ class Engine:
             starts.append(self.cache.seq_len[s])
         V = self.model.vocab_size
         for t in tokens:
-            for tok in t:
-                if not 0 <= tok < V:
-                    raise StepError("token id %r is outside the vocabulary of %d" % (tok, V))
+            ids = np.asarray(t, dtype=np.int64)
+            if ids.ndim != 1 or ids.min() < 0 or ids.max() >= V:
+                bad = [tok for tok in t if not 0 <= tok < V]
+                raise StepError("token id %r is outside the vocabulary of %d" % (bad[0] if bad else t, V))
         if want is None:
             want = [[n - 1] for n in n_tok]
         for w, n in zip(want, n_tok):

@@ -82,34 +82,40 @@ def generate(engine, prompts, max_new_tokens=256, temperature=0.0, seed=0, stop_
         stats.batch_sizes.append(len(batch))
         slots = engine.start(len(batch))
         live = list(zip(batch, slots))
-        t0 = time.perf_counter()
-        logits = engine.step(slots, [prompts[i] for i in batch])
-        tokens = sampler.sample(logits, temperature, [ids[i] for i, _ in live], [0] * len(live))
-        stats.prefill_seconds += time.perf_counter() - t0
-        stats.prompt_tokens += sum(len(prompts[i]) for i in batch)
-        stats.batches_first_tokens += len(batch)
-        t0 = time.perf_counter()
-        while True:
-            still = []
-            ended = []
-            for (i, slot), tok in zip(live, tokens):
-                results[i].append(tok)
-                stats.new_tokens += 1
-                if on_token is not None:
-                    on_token(i, tok)
-                full = len(prompts[i]) + len(results[i]) >= max_len        # no room for the token just sampled
-                if tok in stop or len(results[i]) >= max_new_tokens or full:
-                    ended.append(slot)
-                else:
-                    still.append((i, slot))
-            if ended:
-                engine.release(ended)
-            live = still
-            if not live:
-                break
-            logits = engine.step([s for _, s in live], [[results[i][-1]] for i, _ in live])
-            tokens = sampler.sample(logits, temperature, [ids[i] for i, _ in live],
-                                    [len(results[i]) for i, _ in live])
-            stats.decode_steps += 1
+        held = set(slots)
+        try:
+            t0 = time.perf_counter()
+            logits = engine.step(slots, [prompts[i] for i in batch])
+            tokens = sampler.sample(logits, temperature, [ids[i] for i, _ in live], [0] * len(live))
+            stats.prefill_seconds += time.perf_counter() - t0
+            stats.prompt_tokens += sum(len(prompts[i]) for i in batch)
+            stats.batches_first_tokens += len(batch)
+            t0 = time.perf_counter()
+            while True:
+                still = []
+                ended = []
+                for (i, slot), tok in zip(live, tokens):
+                    results[i].append(tok)
+                    stats.new_tokens += 1
+                    if on_token is not None:
+                        on_token(i, tok)
+                    full = len(prompts[i]) + len(results[i]) >= max_len        # no room for the token just sampled
+                    if tok in stop or len(results[i]) >= max_new_tokens or full:
+                        ended.append(slot)
+                    else:
+                        still.append((i, slot))
+                if ended:
+                    engine.release(ended)
+                    held.difference_update(ended)
+                live = still
+                if not live:
+                    break
+                logits = engine.step([s for _, s in live], [[results[i][-1]] for i, _ in live])
+                tokens = sampler.sample(logits, temperature, [ids[i] for i, _ in live],
+                                        [len(results[i]) for i, _ in live])
+                stats.decode_steps += 1
+        except BaseException:
+            engine.release(sorted(held))                  # a failed batch gives back what it still holds
+            raise
         stats.decode_seconds += time.perf_counter() - t0
     return results
