@@ -186,3 +186,32 @@ def test_trace_run_program(folders, tmp_path):
             keep = ~np.isnan(got[rid]).any(axis=1)
             assert keep.sum() >= len(toks) - 1
             helpers.check_logits(got[rid][keep], want[keep], dtype, "trace_run %s %s" % (dtype, rid))
+
+
+FULL_WIDTH = {"architectures": ["MistralForCausalLM"], "hidden_size": 4096, "intermediate_size": 14336,
+              "num_hidden_layers": 1, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
+              "vocab_size": 4096, "max_position_embeddings": 4096, "rope_theta": 1e6, "rms_norm_eps": 1e-5,
+              "hidden_act": "silu", "tie_word_embeddings": False, "bos_token_id": 1, "eos_token_id": 2}
+
+
+def test_one_layer_at_the_width_of_the_big_models(tmp_path_factory):
+    """One layer with the sizes of Mistral-7B (a small vocabulary): the kernels take their big-shape paths
+    (256x256 and 128x128 GEMM tiles in the prompt step, 256 parts in the norm chain, split-K for 20 rows,
+    matrix-core attention with 4 heads a group), and the logits still follow the plain implementation."""
+    from yalm_amd.engine import Engine, Model
+    folder = helpers.make_folder(tmp_path_factory.mktemp("wide"), "full_width", FULL_WIDTH, seed=1,
+                                 stored=torch.bfloat16)
+    model = Model.from_folder(folder, dtype=torch.bfloat16, device="cuda:0")
+    engine = Engine(model, max_tokens=4096)
+    requests = helpers.random_requests(FULL_WIDTH, [200, 70, 33] + [6 + (i % 5) for i in range(17)], seed=12)
+    ids = list(requests)
+    three = {rid: requests[rid] for rid in ids[:3]}
+    first = {rid: max(1, len(requests[rid]) - 3) for rid in ids}
+    first[ids[0]] = 180
+    for reqs, steps in ((three, schedules.batches(three, [ids[:3]], {ids[0]: 200 - 32, ids[1]: 70, ids[2]: 1})),
+                        (requests, schedules.batches(requests, [ids], first))):               # 3 rows, then 20 rows
+        got = schedules.per_request(steps, schedules.replay_in_process(engine, steps), reqs)
+        for rid, toks in reqs.items():
+            want = helpers.plain_logits(folder, tuple(toks), "bfloat16")
+            helpers.check_logits(got[rid], want, "bfloat16", "full width, request %s (%d tokens)" % (rid, len(toks)))
+    assert not engine.cache.slots.held
