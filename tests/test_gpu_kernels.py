@@ -659,3 +659,24 @@ def test_gemm_gated_batches_of_17_to_64_rows(M, H, D, with_workspace):
     out = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
     k.gemm(x.to(DEV), w, out, k.EPI_GATED, hidden=H, workspace=ws)
     close(out, want, torch.bfloat16, "gated")
+
+
+@pytest.mark.parametrize("small_workspace", [False, True])
+@pytest.mark.parametrize("M,N,Kd", [(17, 4096, 4096), (64, 100, 264), (40, 4096, 14336), (33, 96, 64)])
+def test_gemm_add_norm(M, N, Kd, small_workspace):
+    """Residual add and the next RMSNorm in one, 17..64 rows: x += a W^T; h = rmsnorm(x) * w."""
+    k = K()
+    a = rnd((M, Kd), 80, torch.bfloat16)
+    w = rnd((N, Kd), 81, torch.bfloat16, scale=1 / math.sqrt(Kd))
+    x0 = rnd((M, N), 82, scale=2.0)
+    nw = (1 + 0.1 * rnd((N,), 83)).float()
+    eps = 1e-5
+    x = x0.clone().to(DEV)
+    h = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+    ws = torch.empty(M * N if small_workspace else k.gemm_workspace_floats(M, N), device=DEV)
+    k.gemm_add_norm(a.to(DEV), w.to(DEV), x, nw.to(DEV), eps, h, ws)
+    want_x = x0.double() + a.double() @ w.double().T
+    close(x, want_x, torch.float32, "residual", factor=4)
+    close(h, R.rmsnorm(want_x, nw, eps), torch.bfloat16, "normed")
+    with pytest.raises(ValueError):
+        k.gemm_add_norm(a.to(DEV), w.to(DEV), x, nw.to(DEV), eps, h, torch.empty(M * N - 1, device=DEV))

@@ -52,7 +52,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_kernel(const bf16* _
                                                                     const bf16* __restrict__ W,
                                                                     void* __restrict__ Cv,
                                                                     float* __restrict__ partial, int M, int N, int K,
-                                                                    int H, int k_per_slice) {
+                                                                    int H, int k_per_slice, int always_partial) {
   __shared__ __attribute__((aligned(16))) bf16 xs[2][MT * 16 * XROW];
   constexpr int NTHREADS = NWAVES * WAVE;
   constexpr int XCHUNKS = MT * 16 * (KC / 8);    // 16-byte pieces of an activation chunk
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_kernel(const bf16* _
   }
 
   // C[m][n]: lane (q, j) holds rows 4q..4q+3 of column j of every tile
-  if (gridDim.y == 1) {
+  if (gridDim.y == 1 && !always_partial) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       if (EPI == 3) {
@@ -228,11 +228,91 @@ int launch_mt(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, 
   const int k_per_slice = ceil_div(chunks, slices) * KC;
   slices = ceil_div(K, k_per_slice);
   dim3 grid(n_blocks, slices);
-  gemm_batch_kernel<MT, NTW, EPI><<<grid, NWAVES * WAVE, 0, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice);
+  gemm_batch_kernel<MT, NTW, EPI><<<grid, NWAVES * WAVE, 0, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice, 0);
   int rc = launch_status();
   if (rc != YALM_OK || slices == 1) return rc;
   const long items = (long)M * (EPI == 3 ? (N / 2) / 4 : (N + 3) / 4);
   splitk_reduce_kernel<EPI><<<ceil_div(items, 256), 256, 0, stream>>>(ws, C, M, N, H, slices);
+  return launch_status();
+}
+
+// The residual add that also does the NEXT RMSNorm: a workgroup per row adds the K slices to
+// the float32 residual stream, sums the squares of the new row, and writes the normalised
+// activations h = bfloat16(x * rsqrt(mean(x^2) + eps) * w).  No norm kernel runs afterwards.
+constexpr int RN_THREADS = 1024;
+__global__ __launch_bounds__(RN_THREADS) void reduce_add_norm_kernel(const float* __restrict__ partial,
+                                                                     float* __restrict__ C,
+                                                                     const float* __restrict__ norm_w, float eps,
+                                                                     bf16* __restrict__ h, int M, int N, int slices) {
+  __shared__ float red[RN_THREADS / WAVE];
+  const int m = blockIdx.x;
+  const size_t plane = (size_t)M * N;
+  float* row = C + (size_t)m * N;
+  const float* prow = partial + (size_t)m * N;
+  float ss = 0.f;
+  if ((N & 3) == 0) {                             // four columns a thread, the slices' loads four at a time
+    for (int c = threadIdx.x * 4; c < N; c += RN_THREADS * 4) {
+      float4 y = *reinterpret_cast<const float4*>(row + c);
+      int s = 0;
+      for (; s + 4 <= slices; s += 4) {
+        float4 p[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) p[u] = *reinterpret_cast<const float4*>(prow + (size_t)(s + u) * plane + c);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {             // added in the order of the slices
+          y.x += p[u].x; y.y += p[u].y; y.z += p[u].z; y.w += p[u].w;
+        }
+      }
+      for (; s < slices; ++s) {
+        const float4 p = *reinterpret_cast<const float4*>(prow + (size_t)s * plane + c);
+        y.x += p.x; y.y += p.y; y.z += p.z; y.w += p.w;
+      }
+      *reinterpret_cast<float4*>(row + c) = y;
+      ss += y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w;
+    }
+  } else {
+    for (int c = threadIdx.x; c < N; c += RN_THREADS) {
+      float y = row[c];
+      for (int s = 0; s < slices; ++s) y += prow[(size_t)s * plane + c];
+      row[c] = y;
+      ss += y * y;
+    }
+  }
+  ss = block_sum<RN_THREADS / WAVE>(ss, red);
+  const float scale = 1.0f / sqrtf(ss / (float)N + eps);
+  // every thread reads back what it wrote itself
+  if ((N & 3) == 0) {
+    for (int c = threadIdx.x * 4; c < N; c += RN_THREADS * 4) {
+      const float4 y = *reinterpret_cast<const float4*>(row + c);
+      const float4 w = *reinterpret_cast<const float4*>(norm_w + c);
+      typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+      bf16x4 o = {static_cast<bf16>(y.x * scale * w.x), static_cast<bf16>(y.y * scale * w.y),
+                  static_cast<bf16>(y.z * scale * w.z), static_cast<bf16>(y.w * scale * w.w)};
+      *reinterpret_cast<bf16x4*>(h + (size_t)m * N + c) = o;
+    }
+  } else {
+    for (int c = threadIdx.x; c < N; c += RN_THREADS)
+      h[(size_t)m * N + c] = static_cast<bf16>(row[c] * scale * norm_w[c]);
+  }
+}
+
+template <int MT>
+int launch_add_norm(const bf16* X, const bf16* W, float* C, float* ws, long ws_floats, int M, int N, int K,
+                    const float* norm_w, float eps, bf16* h, hipStream_t stream) {
+  const int n_blocks = ceil_div(N, NWAVES * 16);
+  const int chunks = ceil_div(K, KC);
+  int slices = 1;
+  while (n_blocks * slices < 256 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
+    slices *= 2;
+  while (slices > 1 && (long)slices * M * N > ws_floats) slices /= 2;
+  if (ws == nullptr || (long)slices * M * N > ws_floats) return YALM_ERR_ARG;
+  const int k_per_slice = ceil_div(chunks, slices) * KC;
+  slices = ceil_div(K, k_per_slice);
+  dim3 grid(n_blocks, slices);
+  gemm_batch_kernel<MT, 1, 2><<<grid, NWAVES * WAVE, 0, stream>>>(X, W, C, ws, M, N, K, 0, k_per_slice, 1);
+  int rc = launch_status();
+  if (rc != YALM_OK) return rc;
+  reduce_add_norm_kernel<<<M, RN_THREADS, 0, stream>>>(ws, C, norm_w, eps, h, M, N, slices);
   return launch_status();
 }
 
@@ -260,6 +340,24 @@ int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace
     case 1: return dispatch<1>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
     case 2: return dispatch<2>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
     case 3: return dispatch<3>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+  }
+  return YALM_ERR_ARG;
+}
+
+// C (float32 residual stream) += A * W^T for 17..64 rows, and h = RMSNorm(C_new) * norm_w in bfloat16
+// for the next consumer.  Needs scratch for at least M * N floats; refuses (YALM_ERR_ARG) other shapes.
+extern "C" int yalm_gemm_add_norm(const void* A, const void* W, float* C, float* workspace, long workspace_floats,
+                                  int M, int N, int K, const float* norm_w, float eps, void* h_out,
+                                  hipStream_t stream) {
+  if (M <= 16 || M > 64 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || norm_w == nullptr ||
+      h_out == nullptr)
+    return YALM_ERR_ARG;
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  switch ((M + 15) / 16) {
+    case 2: return launch_add_norm<2>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
+    case 3: return launch_add_norm<3>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
+    case 4: return launch_add_norm<4>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
   }
   return YALM_ERR_ARG;
 }

@@ -51,6 +51,12 @@ int yalm_gemm_norm_qkv_rope(const float* x, const float* norm_w, float eps, cons
                             int K, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, int n_pages,
                             hipStream_t stream);
 
+// Residual add and the next RMSNorm in one for 17..64 rows (bfloat16): C float32 [M,N] += A[M,K] * W[N,K]^T, then
+// h_out bfloat16 [M,N] = C_new * rsqrt(mean(C_new^2) + eps) * norm_w.  workspace: at least M * N floats (more lets
+// it split K).  Refuses (YALM_ERR_ARG) other shapes.
+int yalm_gemm_add_norm(const void* A, const void* W, float* C, float* workspace, long workspace_floats, int M, int N,
+                       int K, const float* norm_w, float eps, void* h_out, hipStream_t stream);
+
 // Decode GEMMs (M <= 64, bfloat16) that chain norms without a norm kernel in between.
 // Producer: epilogue 2 (C float32 += product) with emit_nw given also writes
 // emit_xn[M,N] = bfloat16(C_new * emit_nw[n]) and emit_ss[M, parts] = sums of squares of

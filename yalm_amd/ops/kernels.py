@@ -185,6 +185,30 @@ def can_chain(M, K, dtype):
     return dtype == torch.bfloat16 and 1 <= M <= CHAIN_MAX_ROWS and K % 8 == 0 and not FORCE_SIMPLE
 
 
+def can_add_norm(M, K, dtype):
+    """Whether gemm_add_norm takes this shape (the batches that gemm_chain leaves out)."""
+    return dtype == torch.bfloat16 and CHAIN_MAX_ROWS < M <= 64 and K % 8 == 0 and not FORCE_SIMPLE
+
+
+def gemm_add_norm(a, w, x, norm_w, eps, h_out, workspace):
+    """x float32 [M, N] += a[M, K] @ w[N, K]^T for 17..64 bfloat16 rows, and h_out bfloat16 [M, N] =
+    RMSNorm(x_new) with the weights norm_w (float32 [N]): the residual add and the next norm in one.
+    workspace: float32 scratch of gemm_workspace_floats(M, N) elements."""
+    M, K = a.shape
+    N = w.shape[0]
+    p_a = _need(a, "a", torch.bfloat16, (M, K))
+    p_w = _need(w, "w", torch.bfloat16, (N, K))
+    p_x = _need(x, "x", torch.float32, (M, N))
+    p_nw = _need(norm_w, "norm_w", torch.float32, (N,))
+    p_h = _need(h_out, "h_out", torch.bfloat16, (M, N))
+    if workspace is None or workspace.numel() < M * N:
+        raise ValueError("gemm_add_norm needs a workspace of at least M * N floats")
+    p_ws = _need(workspace, "workspace", torch.float32, None)
+    library.check(library.lib().yalm_gemm_add_norm(p_a, p_w, p_x, p_ws, workspace.numel(), M, N, K, p_nw, float(eps),
+                                                   p_h, _stream()), "gemm_add_norm")
+    return h_out
+
+
 def gemm_chain_parts(N):
     """Columns of the partial sums of squares that a producer with N output columns emits."""
     return library.lib().yalm_gemm_chain_parts(int(N))

@@ -74,7 +74,8 @@ class GQAttention(Part):
     def fuses_norm(self, norm, x, ctx):
         if not hasattr(norm, "fused") or ctx.mode != "decode" or self.head_dim % 16:
             return False
-        return kernels.can_chain(x.shape[0], self.dim, self.wo.dtype)
+        T = x.shape[0]
+        return kernels.can_chain(T, self.dim, self.wo.dtype) or kernels.can_add_norm(T, self.dim, self.wo.dtype)
 
     def forward_prenorm(self, x, norm, ctx, line, writes_cache=True, emit_for=None):
         """A decode step from the residual stream: norm, q/k/v, rotation and cache write in
@@ -94,19 +95,22 @@ class GQAttention(Part):
         k_pages, v_pages = group.line_pages(line)
         q = ctx.ws.get("attn.q", (T, self.q_dim), self.wo.dtype)
         src = ctx.normed.pop(id(norm), None)
-        if src is not None:
+        if src is not None and src[1] is not None:
             xn, ss, eps = src
             kernels.gemm_chain_qkv_rope(xn, (ss, eps), self.wqkv, q, k_pages, v_pages, group.table, group.ring_pages,
                                         ctx.tok_pos, ctx.seq_slot, pos.table, self.n_heads, self.n_kv_heads,
                                         self.head_dim, pos.rotary_dim)
-        elif kernels.can_fuse_norm(T, self.dim, self.wo.dtype):
+        elif src is None and kernels.can_fuse_norm(T, self.dim, self.wo.dtype):
             nw, eps = norm.fused()
             kernels.gemm_norm_qkv_rope(x, nw, eps, self.wqkv, q, k_pages, v_pages, group.table, group.ring_pages,
                                        ctx.tok_pos, ctx.seq_slot, pos.table, self.n_heads, self.n_kv_heads,
                                        self.head_dim, pos.rotary_dim)
-        else:                                     # nothing prepared and too many rows for the one-kernel form
-            h = ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
-            norm.forward(x, h, ctx)
+        else:             # the norm's output is ready, or nothing is prepared and the rows are too many for one kernel
+            if src is not None:
+                h = src[0]
+            else:
+                h = ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
+                norm.forward(x, h, ctx)
             qkv = ctx.ws.get("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
             self._gemm(ctx, h, self.wqkv, qkv, kernels.EPI_STORE_F32)
             kernels.rope_kv_write(qkv, q, None, None, None, k_pages, v_pages, group.table, group.ring_pages,
@@ -115,10 +119,15 @@ class GQAttention(Part):
         o = ctx.ws.get("attn.o", (T, self.q_dim), self.wo.dtype)
         self._decode_attention(q, o, ctx, group, k_pages, v_pages)
         emit = self._emit_args(emit_for, ctx, T, self.dim)
+        ready = self._add_norm_args(emit_for, ctx, T, self.dim) if emit is None else None
         if emit is not None and kernels.can_chain(T, self.q_dim, o.dtype):
             nw2, xn2, ss2, eps2 = emit
             kernels.gemm_chain(o, self.wo, x, kernels.EPI_ADD_F32, emit=(nw2, xn2, ss2))
             ctx.normed[id(emit_for)] = (xn2, ss2, eps2)
+        elif ready is not None and kernels.can_add_norm(T, self.q_dim, o.dtype):
+            nw2, eps2, h2, ws2 = ready
+            kernels.gemm_add_norm(o, self.wo, x, nw2, eps2, h2, ws2)
+            ctx.normed[id(emit_for)] = (h2, None, None)
         else:
             self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)
 

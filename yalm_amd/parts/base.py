@@ -16,8 +16,9 @@ it is in.  Kinds of parts and the methods each must have:
 A mixer, feed-forward or head may fold the norm in front of it into its first
 product: fuses_norm(norm, x, ctx) says so for a step, and forward_prenorm(x, norm,
 ..., emit_for=next_norm) then replaces norm.forward + forward.  With emit_for it may
-also leave, in ctx.normed[id(next_norm)], the activations already multiplied by that
-norm's weights and the partial sums of squares (its residual-add GEMM writes them),
+also leave, in ctx.normed[id(next_norm)], either (xn, ss, eps): the activations already
+multiplied by that norm's weights and the partial sums of squares (its residual-add GEMM
+writes them; up to 16 rows), or (h, None, None): the norm's finished output (17..64 rows),
 which the next consumer takes instead of reading the residual stream.
 
 All of them: param_specs() -> [ParamSpec], load(get, compute_dtype, device),
@@ -107,6 +108,20 @@ class Part:
         xn = ctx.ws.get("chain.xn", (T, width), torch.bfloat16)
         ss = ctx.ws.get("chain.ss", (T, kernels.gemm_chain_parts(width)), torch.float32)
         return nw, xn, ss, eps
+
+    def _add_norm_args(self, emit_for, ctx, T, width):
+        """Operands for a residual-add GEMM of 17..64 rows that also does the norm `emit_for` (the next
+        one on the residual stream) and leaves its activations ready, or None."""
+        from ..ops import kernels
+        if emit_for is None or not hasattr(emit_for, "fused") or ctx.mode != "decode":
+            return None
+        if not kernels.can_add_norm(T, width, ctx.act_dtype):
+            return None
+        import torch
+        nw, eps = emit_for.fused()
+        h = ctx.ws.get("chain.h", (T, width), torch.bfloat16)          # read by the consumer before the next is written
+        ws = ctx.ws.get("gemm.partial", (kernels.gemm_workspace_floats(T, width),), torch.float32)
+        return nw, eps, h, ws
 
     def fuses_norm(self, norm, x, ctx):
         """True if this part can take the float32 residual stream x and do `norm` itself

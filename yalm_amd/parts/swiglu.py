@@ -52,15 +52,18 @@ class SwiGLU(Part):
     def fuses_norm(self, norm, x, ctx):
         if not hasattr(norm, "fused") or ctx.mode != "decode":
             return False
-        return kernels.can_chain(x.shape[0], self.dim, self.w_down.dtype)
+        T = x.shape[0]
+        return kernels.can_chain(T, self.dim, self.w_down.dtype) or kernels.can_add_norm(T, self.dim, self.w_down.dtype)
 
     def forward_prenorm(self, x, norm, ctx, emit_for=None):
         T = x.shape[0]
         mid = ctx.ws.get("ffn.hidden", (T, self.hidden), self.w_down.dtype)
         src = ctx.normed.pop(id(norm), None)
-        if src is not None:
+        if src is not None and src[1] is not None:
             xn, ss, eps = src
             kernels.gemm_chain(xn, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden, scale_from=(ss, eps))
+        elif src is not None:                     # the norm's output is ready
+            self._gemm(ctx, src[0], self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
         elif kernels.can_fuse_norm(T, self.dim, self.w_down.dtype):
             nw, eps = norm.fused()
             kernels.gemm_norm(x, nw, eps, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
@@ -69,10 +72,15 @@ class SwiGLU(Part):
             norm.forward(x, h, ctx)
             self._gemm(ctx, h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
         emit = self._emit_args(emit_for, ctx, T, self.dim)
+        ready = self._add_norm_args(emit_for, ctx, T, self.dim) if emit is None else None
         if emit is not None and kernels.can_chain(T, self.hidden, mid.dtype):
             nw2, xn2, ss2, eps2 = emit
             kernels.gemm_chain(mid, self.w_down, x, kernels.EPI_ADD_F32, emit=(nw2, xn2, ss2))
             ctx.normed[id(emit_for)] = (xn2, ss2, eps2)
+        elif ready is not None and kernels.can_add_norm(T, self.hidden, mid.dtype):
+            nw2, eps2, h2, ws2 = ready
+            kernels.gemm_add_norm(mid, self.w_down, x, nw2, eps2, h2, ws2)
+            ctx.normed[id(emit_for)] = (h2, None, None)
         else:
             self._gemm(ctx, mid, self.w_down, x, kernels.EPI_ADD_F32)
 
