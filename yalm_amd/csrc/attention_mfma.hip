@@ -36,7 +36,7 @@ __device__ __forceinline__ int key_row(int t, int i) { return 32 * (t >> 1) + 8 
 // decode: grid (split, kv head, sequence); 4 waves take the pages of the split in turn
 // ---------------------------------------------------------------------------
 template <int HD>
-__global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
+__global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(   // two workgroups a CU: without the bound head size 128 takes the registers of both
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out,
