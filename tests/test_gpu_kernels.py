@@ -632,7 +632,7 @@ def test_gemm_batches_of_17_to_64_rows(M, N, Kd, with_workspace):
     a = rnd((M, Kd), 70, torch.bfloat16)
     w = rnd((N, Kd), 71, torch.bfloat16, scale=1 / math.sqrt(Kd))
     want = a.double() @ w.double().T
-    ws = torch.empty(k.gemm_workspace_floats(M, N), device=DEV) if with_workspace else None
+    ws = torch.empty(k.gemm_workspace_floats(M, N, Kd), device=DEV) if with_workspace else None
     out = torch.empty((M, N), device=DEV)
     k.gemm(a.to(DEV), w.to(DEV), out, k.EPI_STORE_F32, workspace=ws)
     close(out, want, torch.float32, "f32 out")
@@ -655,9 +655,51 @@ def test_gemm_gated_batches_of_17_to_64_rows(M, H, D, with_workspace):
     wu = rnd((H, D), 75, torch.bfloat16, scale=1 / math.sqrt(D))
     want = R.silu(x.double() @ wg.double().T) * (x.double() @ wu.double().T)
     w = interleave_gate_up(wg, wu).to(DEV)
-    ws = torch.empty(k.gemm_workspace_floats(M, w.shape[0]), device=DEV) if with_workspace else None
+    ws = torch.empty(k.gemm_workspace_floats(M, w.shape[0], D), device=DEV) if with_workspace else None
     out = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
     k.gemm(x.to(DEV), w, out, k.EPI_GATED, hidden=H, workspace=ws)
+    close(out, want, torch.bfloat16, "gated")
+
+
+@pytest.mark.parametrize("M,N,Kd", [(65, 4096, 4096), (128, 1000, 14336), (130, 333, 1024), (256, 4096, 1088),
+                                    (70, 100, 4160)])
+def test_gemm_of_more_than_64_rows_splits_k(M, N, Kd):
+    """A batch of more than 64 rows whose output has few tiles: K in slices, given the scratch (whole, and
+    too small for all the slices the kernel would like), and the same products without it."""
+    k = K()
+    a = rnd((M, Kd), 76, torch.bfloat16)
+    w = rnd((N, Kd), 77, torch.bfloat16, scale=1 / math.sqrt(Kd))
+    want = a.double() @ w.double().T
+    res = rnd((M, N), 78)
+    full = k.gemm_workspace_floats(M, N, Kd)
+    assert full >= 2 * M * N and full % (M * N) == 0
+    for floats in (full, 2 * M * N, 0):
+        ws = torch.full((floats,), float("nan"), device=DEV) if floats else None
+        out = torch.empty((M, N), device=DEV)
+        k.gemm(a.to(DEV), w.to(DEV), out, k.EPI_STORE_F32, workspace=ws)
+        close(out, want, torch.float32, "f32 out, %d floats" % floats)
+        out2 = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+        k.gemm(a.to(DEV), w.to(DEV), out2, k.EPI_STORE, workspace=ws)
+        close(out2, want, torch.bfloat16, "bf16 out, %d floats" % floats)
+        acc = res.to(DEV).clone()
+        k.gemm(a.to(DEV), w.to(DEV), acc, k.EPI_ADD_F32, workspace=ws)
+        close(acc, want + res.double(), torch.float32, "add, %d floats" % floats)
+    assert k.gemm_workspace_floats(2048, 4096, 4096) == 0       # enough tiles: no slices
+
+
+@pytest.mark.parametrize("M,H,D", [(100, 1000, 4096), (128, 176, 2048), (65, 3000, 1024)])
+def test_gemm_gated_of_more_than_64_rows_splits_k(M, H, D):
+    from yalm_amd.parts.swiglu import interleave_gate_up
+    k = K()
+    x = rnd((M, D), 79, torch.bfloat16)
+    wg = rnd((H, D), 84, torch.bfloat16, scale=1 / math.sqrt(D))
+    wu = rnd((H, D), 85, torch.bfloat16, scale=1 / math.sqrt(D))
+    want = R.silu(x.double() @ wg.double().T) * (x.double() @ wu.double().T)
+    w = interleave_gate_up(wg, wu).to(DEV)
+    floats = k.gemm_workspace_floats(M, w.shape[0], D)
+    assert floats >= 2 * M * w.shape[0]
+    out = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
+    k.gemm(x.to(DEV), w, out, k.EPI_GATED, hidden=H, workspace=torch.full((floats,), float("nan"), device=DEV))
     close(out, want, torch.bfloat16, "gated")
 
 
@@ -673,7 +715,7 @@ def test_gemm_add_norm(M, N, Kd, small_workspace):
     eps = 1e-5
     x = x0.clone().to(DEV)
     h = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
-    ws = torch.empty(M * N if small_workspace else k.gemm_workspace_floats(M, N), device=DEV)
+    ws = torch.empty(M * N if small_workspace else k.gemm_workspace_floats(M, N, Kd), device=DEV)
     k.gemm_add_norm(a.to(DEV), w.to(DEV), x, nw.to(DEV), eps, h, ws)
     want_x = x0.double() + a.double() @ w.double().T
     close(x, want_x, torch.float32, "residual", factor=4)

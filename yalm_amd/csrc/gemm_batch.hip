@@ -361,3 +361,19 @@ extern "C" int yalm_gemm_add_norm(const void* A, const void* W, float* C, float*
   }
   return YALM_ERR_ARG;
 }
+
+// Adds `slices` float32 partial products [slices][M][N] in order and applies the epilogue (for the
+// kernels that split K: this file's and the tiled one of gemm_dma.hip).
+int yalm_splitk_reduce(const float* partial, void* C, int M, int N, int H, int slices, int epilogue,
+                       hipStream_t stream) {
+  const long items = (long)M * (epilogue == 3 ? (N / 2) / 4 : (N + 3) / 4);
+  const int blocks = ceil_div(items, 256);
+  switch (epilogue) {
+    case 0: splitk_reduce_kernel<0><<<blocks, 256, 0, stream>>>(partial, C, M, N, H, slices); break;
+    case 1: splitk_reduce_kernel<1><<<blocks, 256, 0, stream>>>(partial, C, M, N, H, slices); break;
+    case 2: splitk_reduce_kernel<2><<<blocks, 256, 0, stream>>>(partial, C, M, N, H, slices); break;
+    case 3: splitk_reduce_kernel<3><<<blocks, 256, 0, stream>>>(partial, C, M, N, H, slices); break;
+    default: return YALM_ERR_ARG;
+  }
+  return launch_status();
+}

@@ -11,10 +11,16 @@
 // kernel waits for them itself (s_waitcnt vmcnt) and uses the bare s_barrier, because
 // __syncthreads() carries a fence that would wait for the loads of all stages.
 //
+// With few tiles (a decode batch of more than 64 rows) K is split over grid z as well: every slice
+// writes its float32 partial product and yalm_splitk_reduce adds them in order and applies the epilogue.
+//
 // Takes any M and N and K % 64 == 0; other shapes are refused (YALM_ERR_ARG) and the
 // caller runs the kernel of gemm_mfma.hip.  Sums are in a fixed order for a given shape.
 #include "common.h"
 #include "yalm_hip.h"
+
+int yalm_splitk_reduce(const float* partial, void* C, int M, int N, int H, int slices, int epilogue,
+                       hipStream_t stream);                                  // gemm_batch.hip
 
 namespace {
 
@@ -40,7 +46,8 @@ template <int EPI, int TM, int TN, int S, int NWM, int NWN, int MINW>
 __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const bf16* __restrict__ A,
                                                                          const bf16* __restrict__ W,
                                                                          void* __restrict__ Cv, int M, int N, int K,
-                                                                         int H) {
+                                                                         int H, float* __restrict__ partial,
+                                                                         int tiles_per_slice) {
   constexpr int NW = NWM * NWN;
   constexpr int ROWS = TM + TN;                    // A rows, then W rows
   constexpr int STAGE_B = ROWS * ROWB;
@@ -101,7 +108,11 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const 
     w_swz[b] = swizzle_of(row);
   }
 
-  const int nk = K / TK;
+  // grid z: slices of K (each writes its float32 partial product; a second kernel adds them)
+  const int kt0 = blockIdx.z * tiles_per_slice;
+  const int nk = min(K / TK - kt0, tiles_per_slice);
+#pragma unroll
+  for (int i = 0; i < L; ++i) gp[i] += (size_t)kt0 * TK;
 #pragma unroll
   for (int s = 0; s < S - 1; ++s)
     if (s < nk) issue(s, s);
@@ -136,6 +147,23 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const 
     }
   }
 
+  if (gridDim.z > 1) {                             // a slice of K: the plain sums, column n = weight row n
+    float* plane = partial + (size_t)blockIdx.z * M * N;
+#pragma unroll
+    for (int a = 0; a < FA; ++a)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * WM + a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+        if (m >= M) continue;
+#pragma unroll
+        for (int b = 0; b < FB; ++b) {
+          const int wr = (EPI == 3) ? wn * WN + (b / 2) * 64 + (li / 16) * 32 + (b % 2) * 16 + (li % 16) : wn * WN + b * 32 + li;
+          const int n = n0 + wr;
+          if (n < N) plane[(size_t)m * N + n] = acc[a][b][r];
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int a = 0; a < FA; ++a) {
 #pragma unroll
@@ -165,8 +193,10 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const 
 }
 
 template <int EPI, int TM, int TN, int S, int NWM, int NWN, int MINW>
-int launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
-  const dim3 grid(ceil_div(N, TN), ceil_div(M, TM));
+int launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, float* partial, int slices,
+                 hipStream_t stream) {
+  const int tiles_per_slice = ceil_div(K / TK, slices);
+  const dim3 grid(ceil_div(N, TN), ceil_div(M, TM), ceil_div(K / TK, tiles_per_slice));
   const size_t lds = (size_t)S * (TM + TN) * ROWB;
   static bool allowed = false;                     // more than 64 KB of LDS has to be asked for once
   if (!allowed) {
@@ -175,32 +205,55 @@ int launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int
     if (e != hipSuccess) return (int)e;
     allowed = true;
   }
-  gemm_dma_kernel<EPI, TM, TN, S, NWM, NWN, MINW><<<grid, NWM * NWN * WAVE, lds, stream>>>(A, W, C, M, N, K, H);
-  return launch_status();
+  gemm_dma_kernel<EPI, TM, TN, S, NWM, NWN, MINW><<<grid, NWM * NWN * WAVE, lds, stream>>>(A, W, C, M, N, K, H, partial,
+                                                                                       tiles_per_slice);
+  int rc = launch_status();
+  if (rc != YALM_OK || grid.z == 1) return rc;
+  return yalm_splitk_reduce(partial, C, M, N, H, (int)grid.z, EPI, stream);
+}
+
+// slices of K for the 128x128 tiles: with few rows (a big decode batch) the tiles alone leave most CUs
+// without work and the weights would stream through a few of them
+int slices_for(int M, int N, int K, long workspace_floats) {
+  const long tiles = (long)ceil_div(M, 128) * ceil_div(N, 128);
+  int slices = 1;
+  while (tiles * slices < 384 && slices * 2 <= (K / TK) / 8 && slices < 16 &&
+         (long)slices * 2 * M * N <= workspace_floats)
+    slices *= 2;
+  return slices;
 }
 
 // 256x256 tiles (8 waves, two stages of 64 KB, one workgroup a CU) ask the caches for the
 // fewest bytes per product; 128x128 tiles (4 waves, two workgroups a CU) where those would
 // leave CUs without work.
 template <int EPI>
-int launch(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
+int launch(const bf16* A, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
+           hipStream_t stream) {
   if ((long)ceil_div(M, 256) * ceil_div(N, 256) >= 160)
-    return launch_shape<EPI, 256, 256, 2, 4, 2, 1>(A, W, C, M, N, K, H, stream);
-  return launch_shape<EPI, 128, 128, 2, 2, 2, 2>(A, W, C, M, N, K, H, stream);
+    return launch_shape<EPI, 256, 256, 2, 4, 2, 1>(A, W, C, M, N, K, H, nullptr, 1, stream);
+  const int slices = ws != nullptr ? slices_for(M, N, K, ws_floats) : 1;
+  return launch_shape<EPI, 128, 128, 2, 2, 2, 2>(A, W, C, M, N, K, H, ws, slices, stream);
 }
 
 }  // namespace
 
-int yalm_gemm_bf16_dma(const void* A, const void* W, void* C, int M, int N, int K, int epilogue, int H,
-                       hipStream_t stream) {
+// floats of scratch with which yalm_gemm_bf16_dma would split K (0: it would not)
+long yalm_gemm_bf16_dma_workspace(int M, int N, int K) {
+  if (M <= 64 || K < TK || K % TK != 0 || (long)ceil_div(M, 256) * ceil_div(N, 256) >= 160) return 0;
+  const int slices = slices_for(M, N, K, (long)1 << 40);
+  return slices > 1 ? (long)slices * M * N : 0;
+}
+
+int yalm_gemm_bf16_dma(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
+                       int K, int epilogue, int H, hipStream_t stream) {
   if (M <= 64 || K < TK || K % TK != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   switch (epilogue) {
-    case 0: return launch<0>(a, w, C, M, N, K, H, stream);
-    case 1: return launch<1>(a, w, C, M, N, K, H, stream);
-    case 2: return launch<2>(a, w, C, M, N, K, H, stream);
-    case 3: return launch<3>(a, w, C, M, N, K, H, stream);
+    case 0: return launch<0>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+    case 1: return launch<1>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+    case 2: return launch<2>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+    case 3: return launch<3>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
   }
   return YALM_ERR_ARG;
 }

@@ -190,8 +190,8 @@ int tiled_launch(const bf16* A, const bf16* W, void* C, int M, int N, int K, int
 int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
                          int K, int epilogue, int H, hipStream_t stream);   // gemm_batch.hip
 
-int yalm_gemm_bf16_dma(const void* A, const void* W, void* C, int M, int N, int K, int epilogue, int H,
-                       hipStream_t stream);                                  // gemm_dma.hip
+int yalm_gemm_bf16_dma(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
+                       int K, int epilogue, int H, hipStream_t stream);      // gemm_dma.hip
 
 int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
                         int K, int epilogue, int H, hipStream_t stream) {
@@ -212,7 +212,7 @@ int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, float* workspace,
     return YALM_ERR_ARG;
   }
   {
-    int rc = yalm_gemm_bf16_dma(A, W, C, M, N, K, epilogue, H, stream);      // K a multiple of 64
+    int rc = yalm_gemm_bf16_dma(A, W, C, workspace, workspace_floats, M, N, K, epilogue, H, stream);   // K % 64 == 0
     if (rc != YALM_ERR_ARG) return rc;
   }
   switch (epilogue) {

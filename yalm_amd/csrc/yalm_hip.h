@@ -37,6 +37,10 @@ int yalm_rmsnorm(const float* x, const void* w, int w_dtype, void* out, int out_
 int yalm_gemm(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N, int K,
               int dtype, int epilogue, int H, int force_simple, hipStream_t stream);
 
+// Floats of workspace with which the tiled bfloat16 kernel for more than 64 rows splits K (0: it does
+// not; the output's tiles fill the chip).
+long yalm_gemm_bf16_dma_workspace(int M, int N, int K);
+
 // Decode GEMMs from the float32 residual stream, M <= 8 rows (M * (K + 8) * 2 bytes <= 72 KB), bfloat16 weights:
 // C = epilogue(rmsnorm(x, norm_w, eps) * W^T); epilogue 0 (float32 store) or 3 (gated, as yalm_gemm).
 // norm_w is float32 [K].  Refuses (YALM_ERR_ARG) other shapes: use yalm_rmsnorm + yalm_gemm then.

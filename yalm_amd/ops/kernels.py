@@ -79,9 +79,14 @@ EPI_STORE_F32, EPI_STORE, EPI_ADD_F32, EPI_GATED = 0, 1, 2, 3
 GEMM_SPLIT_MAX = 16          # most K slices a GEMM uses, given the workspace
 
 
-def gemm_workspace_floats(M, N):
-    """Floats of scratch with which gemm may split K across workgroups (17..64 rows)."""
-    return GEMM_SPLIT_MAX * M * N if 16 < M <= 64 else 0
+def gemm_workspace_floats(M, N, K):
+    """Floats of scratch with which a bfloat16 gemm splits K across workgroups: 17..64 rows, and
+    more rows than that while the output's tiles alone would leave most of the chip idle."""
+    if 16 < M <= 64:
+        return GEMM_SPLIT_MAX * M * N
+    if M > 64:
+        return int(library.lib().yalm_gemm_bf16_dma_workspace(M, N, K))
+    return 0
 
 
 def gemm(a, w, out, epilogue, hidden=0, workspace=None):
@@ -89,7 +94,7 @@ def gemm(a, w, out, epilogue, hidden=0, workspace=None):
     EPI_STORE_F32 (float32 out), EPI_STORE (out in a's dtype), EPI_ADD_F32
     (float32 out += product), EPI_GATED (w = gate/up rows interleaved in blocks of
     16; out[M, hidden] = silu(gate) * up in a's dtype).  workspace: float32 scratch of
-    gemm_workspace_floats(M, N) elements, with which batches of 17..64 rows split K."""
+    gemm_workspace_floats(M, N, K) elements, with which small batches split K."""
     M, K = a.shape
     N = w.shape[0]
     dt = a.dtype
@@ -193,7 +198,7 @@ def can_add_norm(M, K, dtype):
 def gemm_add_norm(a, w, x, norm_w, eps, h_out, workspace):
     """x float32 [M, N] += a[M, K] @ w[N, K]^T for 17..64 bfloat16 rows, and h_out bfloat16 [M, N] =
     RMSNorm(x_new) with the weights norm_w (float32 [N]): the residual add and the next norm in one.
-    workspace: float32 scratch of gemm_workspace_floats(M, N) elements."""
+    workspace: float32 scratch of gemm_workspace_floats(M, N, K) elements."""
     M, K = a.shape
     N = w.shape[0]
     p_a = _need(a, "a", torch.bfloat16, (M, K))

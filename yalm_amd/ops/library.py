@@ -29,6 +29,7 @@ _SIGNATURES = {
                                       _I, _I, _P]),
     "yalm_rope_kv_write": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                 _I, _I, _P]),
+    "yalm_gemm_bf16_dma_workspace": (ctypes.c_long, [_I, _I, _I]),
     "yalm_gemm_add_norm": (_I, [_P, _P, _P, _P, ctypes.c_long, _I, _I, _I, _P, _F, _P, _P]),
     "yalm_rope_kv_write_tiles": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                       _I, _I, _I, _I, _P]),
@@ -40,7 +41,7 @@ _SIGNATURES = {
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
 }
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 
 class KernelError(RuntimeError):

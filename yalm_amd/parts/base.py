@@ -86,11 +86,11 @@ class Part:
 
     @staticmethod
     def _gemm(ctx, a, w, out, epilogue, hidden=0):
-        """kernels.gemm with the scratch that lets batches of 17..64 rows split K."""
+        """kernels.gemm with the scratch that lets small batches split K."""
         from ..ops import kernels
         import torch
         ws = None
-        n = kernels.gemm_workspace_floats(a.shape[0], w.shape[0]) if a.dtype == torch.bfloat16 else 0
+        n = kernels.gemm_workspace_floats(a.shape[0], w.shape[0], a.shape[1]) if a.dtype == torch.bfloat16 else 0
         if n and ctx is not None:
             ws = ctx.ws.get("gemm.partial", (n,), torch.float32)
         return kernels.gemm(a, w, out, epilogue, hidden=hidden, workspace=ws)
@@ -120,7 +120,7 @@ class Part:
         import torch
         nw, eps = emit_for.fused()
         h = ctx.ws.get("chain.h", (T, width), torch.bfloat16)          # read by the consumer before the next is written
-        ws = ctx.ws.get("gemm.partial", (kernels.gemm_workspace_floats(T, width),), torch.float32)
+        ws = ctx.ws.get("gemm.partial", (kernels.gemm_workspace_floats(T, width, width),), torch.float32)
         return nw, eps, h, ws
 
     def fuses_norm(self, norm, x, ctx):
