@@ -279,6 +279,23 @@ def test_cache_groups_and_page_accounting():
     assert c.tokens_held() == 0
 
 
+def test_a_batch_takes_its_pages_in_turn():
+    """Sequences that start together take their pages a page each in turn: page p of all of them lies
+    together, not every sequence's pages in a run of its own."""
+    c = make_cache()
+    full = c.group_of(0)
+    s = c.acquire(3)
+    c.extend(s, [130, 64, 70])                                       # 3, 1 and 2 pages
+    t = full.table_host
+    assert [int(t[x, 0]) for x in s] == [0, 1, 2]
+    assert [int(t[s[0], 1]), int(t[s[2], 1])] == [3, 4] and int(t[s[1], 1]) == -1
+    assert int(t[s[0], 2]) == 5 and full.pool.n_free == 10 - 6
+    c.extend(s, [1, 1, 58])                                          # only the second crosses into a new page
+    assert int(t[s[1], 1]) == 6 and int(t[s[2], 2]) == -1
+    c.release(s)
+    assert full.pool.n_free == 10
+
+
 def test_cache_state_is_cleared_on_acquire_and_random_use_keeps_the_books():
     c = make_cache(max_tokens=64 * 40, n_slots=6)
     st = c.state_groups[0]

@@ -146,12 +146,25 @@ class KVGroup:
         need = min(pages_for(new_len), self.ring_pages)
         return max(0, need - have)
 
-    def grow(self, slot, old_len, new_len):
-        have = min(pages_for(old_len), self.ring_pages)
-        need = min(pages_for(new_len), self.ring_pages)
-        for col in range(have, need):
-            self.table_host[slot, col] = self.pool.take()
-            self._dirty.add(slot)
+    def grow(self, slots, old_lens, new_lens):
+        """Takes the pages that the sequences in `slots` need to grow from old_lens to new_lens.
+        The sequences take their pages in turn, a page each: a batch that advances together then
+        reads neighbouring pages at the same time.  (Handing every sequence a run of its own puts
+        equally long prompts a power of two apart, and the attention kernel's reads, which walk
+        all sequences in step, crowd into few memory channels: measured 4.8 against 5.8 TB/s.)"""
+        spans = []
+        for slot, old_len, new_len in zip(slots, old_lens, new_lens):
+            have = min(pages_for(old_len), self.ring_pages)
+            need = min(pages_for(new_len), self.ring_pages)
+            if need > have:
+                spans.append((slot, have, need))
+        if not spans:
+            return
+        for col in range(min(h for _, h, _ in spans), max(n for _, _, n in spans)):
+            for slot, have, need in spans:
+                if have <= col < need:
+                    self.table_host[slot, col] = self.pool.take()
+                    self._dirty.add(slot)
 
     def free_slot(self, slot):
         row = self.table_host[slot]
@@ -268,8 +281,7 @@ class CacheManager:
                 raise CacheFull("the step needs %d more cache pages, %d are free of %d (max_tokens too small)"
                                 % (need, g.pool.n_free, g.n_pages))
         for g in self.kv_groups:
-            for s, nl in zip(slots, new_lens):
-                g.grow(s, self.seq_len[s], nl)
+            g.grow(slots, [self.seq_len[s] for s in slots], new_lens)
             g.flush()
         for s, nl in zip(slots, new_lens):
             self.seq_len[s] = nl

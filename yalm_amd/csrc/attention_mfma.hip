@@ -18,8 +18,9 @@
 #include "common.h"
 #include "yalm_hip.h"
 
+// attention_simple.hip; base2: the partial results' maxima are exponents of 2, not of e
 int yalm_attn_decode_combine_bf16(const float* partial, void* out, int B, int n_heads, int head_dim, int n_splits,
-                                  hipStream_t stream);   // attention_simple.hip
+                                  int base2, hipStream_t stream);
 
 namespace {
 
@@ -63,7 +64,8 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(   // two work
     const int per = (total + n_splits - 1) / n_splits;
     const int p_begin = first_page + split * per;
     const int p_end = min(last_page + 1, p_begin + per);
-    const float root = sqrtf((float)HD);
+    // scores and the running maximum are kept in units of log2(e) / sqrt(head_dim): one multiply, and 2^x is one instruction
+    const float score_scale = 1.4426950408889634f / sqrtf((float)HD);
     const size_t page_elems = (size_t)n_kv_heads * PAGE * HD;
     const int* table = block_table + (size_t)slot * table_stride;
 
@@ -119,7 +121,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(   // two work
       for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          float v = sc[t][r] / root;
+          float v = sc[t][r] * score_scale;
           if (edge) {
             int pos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
             if (pos < lo || pos >= L) v = -INFINITY;
@@ -130,14 +132,14 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(   // two work
       mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
       mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
       const float m_new = fmaxf(m, mx);
-      const float corr = expf(m - m_new);
+      const float corr = __builtin_amdgcn_exp2f(m - m_new);
       float psum = 0.f;
       bf16x8 pb[2];
 #pragma unroll
       for (int s = 0; s < 2; ++s)
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          float p = expf(sc[2 * s + (e >> 2)][e & 3] - m_new);
+          float p = __builtin_amdgcn_exp2f(sc[2 * s + (e >> 2)][e & 3] - m_new);
           psum += p;
           pb[s][e] = static_cast<bf16>(p);
         }
@@ -169,7 +171,7 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(   // two work
   if (qd == 0) sm_m[wave][j] = m;
   __syncthreads();
   float m_all = fmaxf(fmaxf(sm_m[0][j], sm_m[1][j]), fmaxf(sm_m[2][j], sm_m[3][j]));
-  const float scale = expf(m - m_all);
+  const float scale = __builtin_amdgcn_exp2f(m - m_all);
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) sm_o[wave][dt][lane] = o[dt] * scale;
   if (qd == 0) sm_l[wave][j] = l * scale;
@@ -455,5 +457,5 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
                                                           n_splits, n_pages);
   int rc = launch_status();
   if (rc != YALM_OK || n_splits == 1) return rc;   // one split writes the result itself
-  return yalm_attn_decode_combine_bf16(partial, out, B, n_heads, head_dim, n_splits, stream);
+  return yalm_attn_decode_combine_bf16(partial, out, B, n_heads, head_dim, n_splits, 1, stream);
 }

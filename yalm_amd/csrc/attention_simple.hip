@@ -165,7 +165,8 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
   }
 }
 
-template <typename T>
+// BASE2: the maxima of the partial results are exponents of 2 (the matrix-core kernel's), else of e
+template <typename T, bool BASE2 = false>
 __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(const float* __restrict__ partial,
                                                                              T* __restrict__ out, int n_heads, int hd,
                                                                              int n_splits) {
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(co
   float l = 0.f;
   for (int s = lane; s < n_splits; s += WAVE) {
     const float* ps = part + (size_t)s * stride;
-    l += ps[hd + 1] * expf(ps[hd] - m);
+    l += ps[hd + 1] * (BASE2 ? exp2f(ps[hd] - m) : expf(ps[hd] - m));
   }
   l = wave_sum(l);
   const float inv_l = l > 0.f ? 1.0f / l : 0.f;
@@ -193,7 +194,7 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(co
 #pragma unroll 4
   for (int s = g; s < n_splits; s += COMBINE_THREADS / WAVE) {
     const float* ps = part + (size_t)s * stride;
-    const float w = expf(ps[hd] - m);
+    const float w = BASE2 ? exp2f(ps[hd] - m) : expf(ps[hd] - m);
 #pragma unroll
     for (int j = 0; j < ACC; ++j) {
       const int d = lane + j * WAVE;
@@ -249,9 +250,12 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
 
 // merges the partial results of the splits (also used by the MFMA kernel)
 int yalm_attn_decode_combine_bf16(const float* partial, void* out, int B, int n_heads, int head_dim, int n_splits,
-                                  hipStream_t stream) {
+                                  int base2, hipStream_t stream) {
   dim3 cgrid(B, n_heads);
-  attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
+  if (base2)
+    attn_decode_combine_kernel<bf16, true><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
+  else
+    attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
   return launch_status();
 }
 

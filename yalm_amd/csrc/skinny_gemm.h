@@ -62,23 +62,31 @@ struct ChainArgs {
 // j = lane%16) holds batch rows 4q..4q+3 of weight row j.  Which k a lane's slot
 // holds is the same for both operands, so any assignment of k to slots is right;
 // here step s of a chunk takes k = kc + 32 s + 8 q ... + 8.
-template <int MT, int NT, int NWAVES, int EPI, int KS, bool PREFETCH = true>
+//
+// A wave multiplies TW of the workgroup's NT tiles: with TW < NT the waves form NT / TW groups, each
+// with its own tiles and the chunks of K split over the waves of the group (less to keep in flight per
+// wave and more waves, at the price of one more load of the activations per group).
+template <int MT, int NT, int NWAVES, int EPI, int KS, bool PREFETCH = true, int TW = NT>
 __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ X,
                                                                      const bf16* __restrict__ W,
                                                                      void* __restrict__ Cv, int M, int N, int K,
                                                                      int H, ChainArgs ca) {
   constexpr int KC = 32 * KS;                    // k per wave iteration
-  __shared__ f32x4 red[NWAVES][MT * NT][WAVE];
+  constexpr int G = NT / TW;                     // groups of waves, each with TW tiles
+  constexpr int KW = NWAVES / G;                 // waves of a group: they split K
+  static_assert(NT % TW == 0 && NWAVES % G == 0, "tiles and waves divide evenly");
+  __shared__ f32x4 red[NWAVES][MT * TW][WAVE];
   __shared__ float sm_scale[MT * 16];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int q = lane / 16, j = lane % 16;
   const int n0 = blockIdx.x * 16 * NT;
 
-  const bf16* wrow[NT];
-  bool wok[NT];
+  const int grp = wave % G, kw = wave / G;
+  const bf16* wrow[TW];
+  bool wok[TW];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    int n = n0 + t * 16 + j;
+  for (int t = 0; t < TW; ++t) {
+    int n = n0 + (grp * TW + t) * 16 + j;
     wok[t] = n < N;
     wrow[t] = W + (size_t)(wok[t] ? n : 0) * K;
   }
@@ -91,11 +99,11 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
     xrow[mt] = X + (size_t)(xok[mt] ? m : 0) * K;
   }
 
-  f32x4 acc[MT][NT];
+  f32x4 acc[MT][TW];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) acc[mt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < TW; ++t) acc[mt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   // Workgroups start at different chunks of K (and wrap around): with all of them on the
   // same columns at the same time, the rows' 8 KB-strided pieces crowd few memory channels.
@@ -117,7 +125,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
     }
   }
 
-  auto load_chunk = [&](int c, bf16x8 (&w)[NT][KS], bf16x8 (&x)[MT][KS]) {
+  auto load_chunk = [&](int c, bf16x8 (&w)[TW][KS], bf16x8 (&x)[MT][KS]) {
     const int kc = chunk_k(c);
 #pragma unroll
     for (int s = 0; s < KS; ++s) {
@@ -125,7 +133,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
       const bool ok = k < K;
       const int kk = ok ? k : K - 8;               // rows beyond N or M are clamped too and never stored
 #pragma unroll
-      for (int t = 0; t < NT; ++t) w[t][s] = load8_always(wrow[t] + kk);
+      for (int t = 0; t < TW; ++t) w[t][s] = load8_always(wrow[t] + kk);
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) x[mt][s] = zero_unless(load8_always(xrow[mt] + kk), ok);
     }
@@ -141,12 +149,12 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
     }
   };
 
-  bf16x8 wv[NT][KS], xv[MT][KS];
+  bf16x8 wv[TW][KS], xv[MT][KS];
   if (!PREFETCH) {
     // few, large chunks: all loads of a chunk are in flight at once and the products
     // start as the first arrive (K <= 512 * NWAVES is one round trip to memory)
     bool first = true;
-    for (int c = wave; c < n_chunks; c += NWAVES) {
+    for (int c = kw; c < n_chunks; c += KW) {
       load_chunk(c, wv, xv);
       if (first) row_scales();
       first = false;
@@ -155,30 +163,30 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-          for (int t = 0; t < NT; ++t)
+          for (int t = 0; t < TW; ++t)
             acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
     }
     if (first) row_scales();
   } else {
-    int c = wave;
+    int c = kw;
     if (c < n_chunks) load_chunk(c, wv, xv);
     row_scales();
-    for (; c < n_chunks; c += NWAVES) {
-      bf16x8 wn[NT][KS], xn[MT][KS];
-      const bool more = c + NWAVES < n_chunks;
-      if (more) load_chunk(c + NWAVES, wn, xn);    // prefetch the wave's next chunk
+    for (; c < n_chunks; c += KW) {
+      bf16x8 wn[TW][KS], xn[MT][KS];
+      const bool more = c + KW < n_chunks;
+      if (more) load_chunk(c + KW, wn, xn);        // prefetch the wave's next chunk
 #pragma unroll
       for (int s = 0; s < KS; ++s)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-          for (int t = 0; t < NT; ++t)
+          for (int t = 0; t < TW; ++t)
             acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
       if (more) {
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
 #pragma unroll
-          for (int t = 0; t < NT; ++t) wv[t][s] = wn[t][s];
+          for (int t = 0; t < TW; ++t) wv[t][s] = wn[t][s];
 #pragma unroll
           for (int mt = 0; mt < MT; ++mt) xv[mt][s] = xn[mt][s];
         }
@@ -189,8 +197,15 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) red[wave][mt * NT + t][lane] = acc[mt][t];
+    for (int t = 0; t < TW; ++t) red[wave][mt * TW + t][lane] = acc[mt][t];
   __syncthreads();
+  // tile t of the workgroup: the sums of the waves of group t / TW, in their slot t % TW
+  auto tile_sum = [&](int mt, int t) {
+    f32x4 v = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int w = 0; w < KW; ++w) v += red[w * G + t / TW][mt * TW + t % TW][lane];
+    return v;
+  };
 
   const bool scaled = ca.ss_in != nullptr;
   constexpr int NTP = (EPI == EPI_GATED) ? NT / 2 : NT;  // gated: a gate tile and its up tile finish together
@@ -200,12 +215,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
 #pragma unroll
     for (int r = 0; r < 4; ++r) scale[r] = scaled ? sm_scale[mt * 16 + 4 * q + r] : 1.0f;
     if (EPI == EPI_GATED) {
-      f32x4 g = (f32x4){0.f, 0.f, 0.f, 0.f}, u = g;
-#pragma unroll
-      for (int w = 0; w < NWAVES; ++w) {
-        g += red[w][mt * NT + 2 * tp][lane];
-        u += red[w][mt * NT + 2 * tp + 1][lane];
-      }
+      const f32x4 g = tile_sum(mt, 2 * tp), u = tile_sum(mt, 2 * tp + 1);
       int hcol = (n0 / 32 + tp) * 16 + j;
       bf16* C = (bf16*)Cv;
 #pragma unroll
@@ -216,9 +226,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
       }
       continue;
     }
-    f32x4 v = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int w = 0; w < NWAVES; ++w) v += red[w][mt * NT + tp][lane];
+    f32x4 v = tile_sum(mt, tp);
 #pragma unroll
     for (int r = 0; r < 4; ++r) v[r] *= scale[r];
     const int n = n0 + tp * 16 + j;
@@ -303,9 +311,10 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
   }
 }
 
-// Up to 16 batch rows (measured at 4096..32000 weight rows, K 4096 and 14336): many
-// weight rows, or the gated epilogue, take 32 rows and 4 waves a workgroup with all loads
-// of a 256-wide chunk in flight at once; a long K takes 16 rows, 8 waves and 512-wide
+// Up to 16 batch rows (measured at 4096..32000 weight rows, K 4096 and 14336): the gated
+// epilogue takes 32 rows and 4 waves a workgroup with all loads of a 256-wide chunk in flight
+// at once; other wide matrices 32 rows and 16 waves, a tile each for half of them (14.9 against
+// 17.0 us for the q/k/v projection of 6144 rows); a long K takes 16 rows, 8 waves and 512-wide
 // chunks; the small projections 16 rows, 8 waves and prefetched 128-wide chunks.  A producer
 // of the norm chain always owns 16 rows (one emitted part a workgroup).  More batch rows
 // (only when the split-K kernel refused the shape) keep 128-wide chunks for the registers.
@@ -315,8 +324,10 @@ int launch_mt(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H,
   constexpr int E = EPI == EPI_GATED ? EPI_F32 : EPI;   // the gated epilogue needs pairs of tiles
   const bool emit = ca.emit_nw != nullptr;
   if constexpr (MT == 1) {
-    if (EPI == EPI_GATED || (!emit && N > 4096 && K < 8192))
+    if (EPI == EPI_GATED)
       gemm_skinny_kernel<1, 2, 4, EPI, 8, false><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
+    else if (!emit && N > 4096 && K < 8192)
+      gemm_skinny_kernel<1, 2, 16, EPI, 8, false, 1><<<ceil_div(N, 32), 16 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
     else if (K >= 8192)
       gemm_skinny_kernel<1, 1, 8, E, 16, false><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
     else
