@@ -34,20 +34,24 @@ __device__ __forceinline__ bf16x8 zero8() { return (bf16x8){0, 0, 0, 0, 0, 0, 0,
 __device__ __forceinline__ int key_row(int t, int i) { return 32 * (t >> 1) + 8 * (i >> 2) + 4 * (t & 1) + (i & 3); }
 
 // ---------------------------------------------------------------------------
-// decode: grid (split, kv head, sequence); 4 waves take the pages of the split in turn
+// decode: grid (split, kv head, sequence); NW waves take the pages of the split in turn.
+// The keys of a wave's next page stay in flight while this page is mixed: the loop's loads stand
+// under no branch (the last page is done by a copy of the body without them), else the compiler
+// waits for every load in flight at each use.
 // ---------------------------------------------------------------------------
-template <int HD>
-__global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(   // two workgroups a CU: without the bound head size 128 takes the registers of both
+template <int HD, int NW>
+__global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_kernel(   // 2 waves a SIMD: head size 128 needs their registers
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out,
     int n_heads, int n_kv_heads, int window, int n_splits, int n_pages) {
   constexpr int KS = HD / 32, DT = HD / 16;
-  __shared__ float sm_m[4][16];
-  __shared__ float sm_l[4][16];
-  __shared__ f32x4 sm_o[4][DT][WAVE];
+  __shared__ float sm_m[NW][16];
+  __shared__ float sm_l[NW][16];
+  __shared__ f32x4 sm_o[NW][DT][WAVE];
   const int split = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
-  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE, qd = lane / 16, j = lane % 16;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE, qd = lane / 16,
+            j = lane % 16;
   const int G = n_heads / n_kv_heads;
   const int slot = seq_slot[b];
   const int L = slot >= 0 ? seq_len[b] : 0;
@@ -78,23 +82,29 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(   // two work
     }
 
     bf16x8 kreg[4][KS];
-    int ap = p_begin + wave;
-    if (ap < p_end) {
-      int phys = min(max(table[ap % ring_pages], 0), n_pages - 1);
+    auto page_of = [&](int a) { return min(max(table[a % ring_pages], 0), n_pages - 1); };
+    auto load_keys = [&](int phys) {
       const bf16* kp = k_pages + phys * page_elems + (size_t)g * PAGE * HD;
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) kreg[t][ks] = ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
-    }
-    for (; ap < p_end; ap += 4) {
-      int phys = min(max(table[ap % ring_pages], 0), n_pages - 1);
+    };
+    int ap = p_begin + wave;
+    int phys = ap < p_end ? page_of(ap) : 0;
+    if (ap < p_end) load_keys(phys);
+
+    // one page: has_next is a compile-time tag (std::true_type: the next page's keys are asked for)
+    auto one_page = [&](auto has_next) {
       const bf16* vp = v_pages + phys * page_elems + (size_t)g * PAGE * HD;
       bf16x8 vreg[DT][2];
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int s = 0; s < 2; ++s) vreg[dt][s] = ld8(vp + (dt * 16 + j) * PAGE + s * 32 + qd * 8);
+      int physn = 0;
+      if constexpr (decltype(has_next)::value) physn = page_of(ap + NW);
+      __builtin_amdgcn_sched_barrier(0);         // the values are asked for before the keys are waited for
 
       f32x4 sc[4];
 #pragma unroll
@@ -104,14 +114,10 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(   // two work
         for (int ks = 0; ks < KS; ++ks)
           sc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[t][ks], qv[ks], sc[t], 0, 0, 0);
       }
-      const int apn = ap + 4;
-      if (apn < p_end) {                         // the keys of the wave's next page, while this one is mixed
-        int physn = min(max(table[apn % ring_pages], 0), n_pages - 1);
-        const bf16* kp = k_pages + physn * page_elems + (size_t)g * PAGE * HD;
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-          for (int ks = 0; ks < KS; ++ks) kreg[t][ks] = ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
+      if constexpr (decltype(has_next)::value) {
+        load_keys(physn);                        // they stay in flight while this page is mixed
+        phys = physn;
+        __builtin_amdgcn_sched_barrier(0);
       }
 
       const int base = ap * PAGE;
@@ -162,43 +168,51 @@ __global__ __launch_bounds__(256, 2) void attn_decode_mfma_kernel(   // two work
         for (int s = 0; s < 2; ++s)
           o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt][s], pb[s], o[dt], 0, 0, 0);
       }
-    }
+    };
+    for (; ap + NW < p_end; ap += NW) one_page(std::true_type{});
+    if (ap < p_end) one_page(std::false_type{});
   }
 
-  // the four lanes of a column hold parts of its sum; then the four waves merge
+  // the four lanes of a column hold parts of its sum; then the waves merge
   l += __shfl_xor(l, 16, WAVE);
   l += __shfl_xor(l, 32, WAVE);
   if (qd == 0) sm_m[wave][j] = m;
   __syncthreads();
-  float m_all = fmaxf(fmaxf(sm_m[0][j], sm_m[1][j]), fmaxf(sm_m[2][j], sm_m[3][j]));
+  float m_all = sm_m[0][j];
+#pragma unroll
+  for (int w = 1; w < NW; ++w) m_all = fmaxf(m_all, sm_m[w][j]);
   const float scale = __builtin_amdgcn_exp2f(m - m_all);
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) sm_o[wave][dt][lane] = o[dt] * scale;
   if (qd == 0) sm_l[wave][j] = l * scale;
   __syncthreads();
-  if (n_splits == 1) {                            // nothing to merge with: this is the result
-    if (j < G) {
+  if (j < G) {
+    float lt = sm_l[0][j];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) lt += sm_l[w][j];
+    if (n_splits == 1) {                          // nothing to merge with: this is the result
       bf16* orow = out + ((size_t)b * n_heads + g * G + j) * HD;
-      const float lt = sm_l[0][j] + sm_l[1][j] + sm_l[2][j] + sm_l[3][j];
       const float inv_l = lt > 0.f ? 1.0f / lt : 0.f;
-      for (int dt = wave; dt < DT; dt += 4) {
-        f32x4 v = sm_o[0][dt][lane] + sm_o[1][dt][lane] + sm_o[2][dt][lane] + sm_o[3][dt][lane];
+      for (int dt = wave; dt < DT; dt += NW) {
+        f32x4 v = sm_o[0][dt][lane];
+#pragma unroll
+        for (int w = 1; w < NW; ++w) v += sm_o[w][dt][lane];
 #pragma unroll
         for (int r = 0; r < 4; ++r) orow[dt * 16 + 4 * qd + r] = static_cast<bf16>(v[r] * inv_l);
       }
-    }
-    return;
-  }
-  if (j < G) {
-    float* part = partial + (((size_t)b * n_heads + g * G + j) * n_splits + split) * (HD + 2);
-    for (int dt = wave; dt < DT; dt += 4) {
-      f32x4 v = sm_o[0][dt][lane] + sm_o[1][dt][lane] + sm_o[2][dt][lane] + sm_o[3][dt][lane];
+    } else {
+      float* part = partial + (((size_t)b * n_heads + g * G + j) * n_splits + split) * (HD + 2);
+      for (int dt = wave; dt < DT; dt += NW) {
+        f32x4 v = sm_o[0][dt][lane];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) part[dt * 16 + 4 * qd + r] = v[r];
-    }
-    if (wave == 0 && qd == 0) {
-      part[HD] = m_all;
-      part[HD + 1] = sm_l[0][j] + sm_l[1][j] + sm_l[2][j] + sm_l[3][j];
+        for (int w = 1; w < NW; ++w) v += sm_o[w][dt][lane];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) part[dt * 16 + 4 * qd + r] = v[r];
+      }
+      if (wave == 0 && qd == 0) {
+        part[HD] = m_all;
+        part[HD + 1] = lt;
+      }
     }
   }
 }
@@ -444,17 +458,14 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
                                int n_splits, int n_pages, hipStream_t stream) {
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_heads / n_kv_heads > 16) return YALM_ERR_ARG;
   dim3 grid(n_splits, n_kv_heads, B);
-  if (head_dim == 128)
-    attn_decode_mfma_kernel<128><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages,
-                                                           (const bf16*)v_pages, block_table, table_stride,
-                                                           ring_pages, seq_slot, seq_len, partial,
-                                                           (bf16*)out, n_heads, n_kv_heads, window, n_splits,
-                                                           n_pages);
-  else
-    attn_decode_mfma_kernel<64><<<grid, 256, 0, stream>>>((const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages,
-                                                          block_table, table_stride, ring_pages, seq_slot, seq_len,
-                                                          partial, (bf16*)out, n_heads, n_kv_heads, window,
-                                                          n_splits, n_pages);
+#define YALM_DECODE(HD_, NW_)                                                                                       \
+  attn_decode_mfma_kernel<HD_, NW_><<<grid, NW_ * WAVE, 0, stream>>>(                                               \
+      (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot, \
+      seq_len, partial, (bf16*)out, n_heads, n_kv_heads, window, n_splits, n_pages)
+  // 4 waves a workgroup: 8 measured no faster with one split and slower with more (a CU draws about
+  // 33 GB/s whatever its number of waves, so a small batch needs its workgroups spread over all CUs)
+  if (head_dim == 128) YALM_DECODE(128, 4); else YALM_DECODE(64, 4);
+#undef YALM_DECODE
   int rc = launch_status();
   if (rc != YALM_OK || n_splits == 1) return rc;   // one split writes the result itself
   return yalm_attn_decode_combine_bf16(partial, out, B, n_heads, head_dim, n_splits, 1, stream);
