@@ -34,6 +34,11 @@ __device__ __forceinline__ bf16x8 zero_unless(bf16x8 v, bool ok) {
   return ok ? v : z;
 }
 
+template <int N_>
+__device__ __forceinline__ void skinny_wait_vmcnt() {   // vmcnt only: expcnt and lgkmcnt fields at their maxima
+  __builtin_amdgcn_s_waitcnt((N_ & 0xF) | ((N_ >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
 constexpr int EPI_F32 = 0, EPI_STORE = 1, EPI_ADD = 2, EPI_GATED = 3, EPI_ROPE = 4;
 
 struct RopeArgs {                                // epilogue of the fused q/k/v projection
@@ -66,7 +71,18 @@ struct ChainArgs {
 // A wave multiplies TW of the workgroup's NT tiles: with TW < NT the waves form NT / TW groups, each
 // with its own tiles and the chunks of K split over the waves of the group (less to keep in flight per
 // wave and more waves, at the price of one more load of the activations per group).
-template <int MT, int NT, int NWAVES, int EPI, int KS, bool PREFETCH = true, int TW = NT>
+//
+// DMA_S > 0 (one batch tile, K a multiple of 64): the operands go from global memory straight into
+// LDS (global_load_lds_dwordx4), every wave into a ring of DMA_S stages of its own, 64 k a stage, and
+// from there to the matrix cores.  A CU can only send so many requests a clock to the second-level
+// cache (measured: about 33 GB/s a CU with the 64-byte row pieces that the register path's lanes ask
+// for, 62 GB/s with whole 128-byte lines), and the activations' loads, though they hit that cache,
+// come out of the same budget.  Here every request is a whole line: 8 lanes read the 128 bytes of
+// one row, 8 rows an instruction; the 16-byte chunks of a row are XOR-swizzled by the row number in
+// the global address each lane asks for, so that the fragment reads of 8 rows fall on different
+// banks.  XR (8 or 16) rows of the activations are staged.  No wave waits for another before the
+// partial sums meet.
+template <int MT, int NT, int NWAVES, int EPI, int KS, bool PREFETCH = true, int TW = NT, int DMA_S = 0, int XR = 16>
 __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ X,
                                                                      const bf16* __restrict__ W,
                                                                      void* __restrict__ Cv, int M, int N, int K,
@@ -149,49 +165,122 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
     }
   };
 
-  bf16x8 wv[TW][KS], xv[MT][KS];
-  if (!PREFETCH) {
-    // few, large chunks: all loads of a chunk are in flight at once and the products
-    // start as the first arrive (K <= 512 * NWAVES is one round trip to memory)
-    bool first = true;
-    for (int c = kw; c < n_chunks; c += KW) {
-      load_chunk(c, wv, xv);
-      if (first) row_scales();
-      first = false;
+  if constexpr (DMA_S > 0) {
+    static_assert(MT == 1 && (XR == 8 || XR == 16) && DMA_S >= 2 && DMA_S <= 4, "one batch tile; 8 or 16 staged rows; 2..4 stages");
+    constexpr int KD = 64;                         // k a stage: one 128-byte line of every row
+    constexpr int XI = XR / 8;                     // DMA instructions a stage: 8 rows each
+    constexpr int L = 2 * TW + XI;
+    constexpr int STAGE_B = (16 * TW + XR) * 128;
+    extern __shared__ __attribute__((aligned(1024))) unsigned char dma_ring[];   // [NWAVES][DMA_S][STAGE_B]
+    unsigned char* ring = dma_ring + (size_t)wave * DMA_S * STAGE_B;
+    const int r8 = lane / 8, chunk = (lane % 8) ^ r8;          // this lane's row of an instruction and the chunk it asks for
+    const bf16* gw[2 * TW];
 #pragma unroll
-      for (int s = 0; s < KS; ++s)
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int t = 0; t < TW; ++t)
-            acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
+    for (int i = 0; i < 2 * TW; ++i) {
+      const int n = min(n0 + (grp * TW + i / 2) * 16 + (i % 2) * 8 + r8, N - 1);
+      gw[i] = W + (size_t)n * K + chunk * 8;
     }
-    if (first) row_scales();
-  } else {
-    int c = kw;
-    if (c < n_chunks) load_chunk(c, wv, xv);
+    const bf16* gx[XI];
+#pragma unroll
+    for (int i = 0; i < XI; ++i) gx[i] = X + (size_t)min(i * 8 + r8, M - 1) * K + chunk * 8;
+    const int nd = K / KD;                         // stages in all; this wave takes kw, kw + KW, ...
+    const int rotd = (int)((blockIdx.x * 5u) % (unsigned)nd);
+    const int mine = kw < nd ? (nd - kw + KW - 1) / KW : 0;
+    auto issue = [&](int i, int buf) {
+      int c = kw + i * KW + rotd;
+      if (c >= nd) c -= nd;
+      unsigned char* dst = ring + buf * STAGE_B;
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass drops a template that names this builtin, and its launch stub with it
+#pragma unroll
+      for (int u = 0; u < 2 * TW; ++u)
+        __builtin_amdgcn_global_load_lds(gw[u] + (size_t)c * KD, dst + u * 1024, 16, 0, 0);
+#pragma unroll
+      for (int u = 0; u < XI; ++u)
+        __builtin_amdgcn_global_load_lds(gx[u] + (size_t)c * KD, dst + (2 * TW + u) * 1024, 16, 0, 0);
+#endif
+    };
+#pragma unroll
+    for (int i = 0; i < DMA_S - 1; ++i)
+      if (i < mine) issue(i, i);
     row_scales();
-    for (; c < n_chunks; c += KW) {
-      bf16x8 wn[TW][KS], xn[MT][KS];
-      const bool more = c + KW < n_chunks;
-      if (more) load_chunk(c + KW, wn, xn);        // prefetch the wave's next chunk
+    // fragment reads: lane (q, j) of step s wants chunk 4 s + q of row j, which lies at (4 s + q) ^ (j & 7)
+    const int rd_w = j * 128, rd_x = (16 * TW + (j % XR)) * 128, swz = j & 7;
+    int buf = 0;
+    for (int i = 0; i < mine; ++i) {
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");       // the fragment reads of the buffer that is filled next are done
+      const int ahead = mine - 1 - i;              // stages behind this one that are (or now get) in flight
+      if (ahead >= DMA_S - 1) {
+        int nb = buf + DMA_S - 1;
+        if (nb >= DMA_S) nb -= DMA_S;
+        issue(i + DMA_S - 1, nb);
+        skinny_wait_vmcnt<(DMA_S - 1) * L>();
+      } else if (ahead == 2) {                     // the last stages: nothing more to ask for
+        skinny_wait_vmcnt<2 * L>();
+      } else if (ahead == 1) {
+        skinny_wait_vmcnt<L>();
+      } else {
+        skinny_wait_vmcnt<0>();
+      }
+      asm volatile("" ::: "memory");
+      const unsigned char* cur = ring + buf * STAGE_B;
 #pragma unroll
-      for (int s = 0; s < KS; ++s)
+      for (int s = 0; s < 2; ++s) {
+        const int off = ((4 * s + q) ^ swz) << 4;
+        const bf16x8 xf = *reinterpret_cast<const bf16x8*>(cur + rd_x + off);
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-          for (int t = 0; t < TW; ++t)
-            acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
-      if (more) {
-#pragma unroll
-        for (int s = 0; s < KS; ++s) {
-#pragma unroll
-          for (int t = 0; t < TW; ++t) wv[t][s] = wn[t][s];
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) xv[mt][s] = xn[mt][s];
+        for (int t = 0; t < TW; ++t) {
+          const bf16x8 wf = *reinterpret_cast<const bf16x8*>(cur + t * 2048 + rd_w + off);
+          acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf, wf, acc[0][t], 0, 0, 0);
+        }
+      }
+      if (++buf == DMA_S) buf = 0;
+    }
+  } else {
+    bf16x8 wv[TW][KS], xv[MT][KS];
+    if (!PREFETCH) {
+      // few, large chunks: all loads of a chunk are in flight at once and the products
+      // start as the first arrive (K <= 512 * NWAVES is one round trip to memory)
+      bool first = true;
+      for (int c = kw; c < n_chunks; c += KW) {
+        load_chunk(c, wv, xv);
+        if (first) row_scales();
+        first = false;
+  #pragma unroll
+        for (int s = 0; s < KS; ++s)
+  #pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+  #pragma unroll
+            for (int t = 0; t < TW; ++t)
+              acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
+      }
+      if (first) row_scales();
+    } else {
+      int c = kw;
+      if (c < n_chunks) load_chunk(c, wv, xv);
+      row_scales();
+      for (; c < n_chunks; c += KW) {
+        bf16x8 wn[TW][KS], xn[MT][KS];
+        const bool more = c + KW < n_chunks;
+        if (more) load_chunk(c + KW, wn, xn);        // prefetch the wave's next chunk
+  #pragma unroll
+        for (int s = 0; s < KS; ++s)
+  #pragma unroll
+          for (int mt = 0; mt < MT; ++mt)
+  #pragma unroll
+            for (int t = 0; t < TW; ++t)
+              acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xv[mt][s], wv[t][s], acc[mt][t], 0, 0, 0);
+        if (more) {
+  #pragma unroll
+          for (int s = 0; s < KS; ++s) {
+  #pragma unroll
+            for (int t = 0; t < TW; ++t) wv[t][s] = wn[t][s];
+  #pragma unroll
+            for (int mt = 0; mt < MT; ++mt) xv[mt][s] = xn[mt][s];
+          }
         }
       }
     }
+
   }
 
 #pragma unroll
@@ -311,19 +400,53 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
   }
 }
 
-// Up to 16 batch rows (measured at 4096..32000 weight rows, K 4096 and 14336): the gated
-// epilogue takes 32 rows and 4 waves a workgroup with all loads of a 256-wide chunk in flight
-// at once; other wide matrices 32 rows and 16 waves, a tile each for half of them (14.9 against
-// 17.0 us for the q/k/v projection of 6144 rows); a long K takes 16 rows, 8 waves and 512-wide
-// chunks; the small projections 16 rows, 8 waves and prefetched 128-wide chunks.  A producer
-// of the norm chain always owns 16 rows (one emitted part a workgroup).  More batch rows
-// (only when the split-K kernel refused the shape) keep 128-wide chunks for the registers.
+// Up to 16 batch rows.  K a multiple of 64 goes through LDS (DMA_S > 0): wide matrices (the gated
+// epilogue, or more than 4096 weight rows without a norm to prepare) in workgroups of 128, 64 or
+// 32 weight rows, as many as still make some 200 workgroups; the others 16 rows and 8 waves that
+// split K.  A producer of the norm chain always owns 16 rows (one emitted part a workgroup).
+// Other K keep the register path (measured at 4096..32000 weight rows, K 4096 and 14336): the
+// gated epilogue 32 rows and 4 waves with all loads of a 256-wide chunk in flight at once; other
+// wide matrices 32 rows and 16 waves, a tile each for half of them; a long K 16 rows, 8 waves and
+// 512-wide chunks; the small projections 16 rows, 8 waves and prefetched 128-wide chunks.  More
+// batch rows (only when the split-K kernel refused the shape) keep 128-wide chunks for the registers.
+// the LDS-DMA variant: its ring of stages is dynamic LDS, which has to be allowed once beyond 64 KB
+template <int NT, int NWAVES, int EPI, int TW, int S, int XR>
+int launch_dma(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, const ChainArgs& ca,
+               hipStream_t stream) {
+  constexpr size_t lds = (size_t)NWAVES * S * (16 * TW + XR) * 128;
+  static_assert(lds + NWAVES * TW * WAVE * 16 + 1024 <= 160 * 1024, "the ring and the partial sums fit the LDS of a CU");
+  auto kernel = &gemm_skinny_kernel<1, NT, NWAVES, EPI, 1, false, TW, S, XR>;
+  static bool allowed = false;
+  if (!allowed) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    allowed = true;
+  }
+  kernel<<<ceil_div(N, 16 * NT), NWAVES * WAVE, lds, stream>>>(X, W, C, M, N, K, H, ca);
+  return launch_status();
+}
+
 template <int MT, int EPI>
 int launch_mt(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, const ChainArgs& ca,
               hipStream_t stream) {
   constexpr int E = EPI == EPI_GATED ? EPI_F32 : EPI;   // the gated epilogue needs pairs of tiles
   const bool emit = ca.emit_nw != nullptr;
   if constexpr (MT == 1) {
+    if (K % 64 == 0) {                            // through LDS; measured at 8 rows against the register path:
+      const bool few = M <= 8;                     // gate/up 41.9 against 52.6 us, q/k/v 11.0 against 15.3,
+      if (EPI == EPI_GATED || (!emit && N > 4096 && K < 8192)) {   // down 21.3 against 25.2, o 7.0 against 8.3
+        if (N >= 200 * 128)                        // workgroups of 128 weight rows while they still fill the chip
+          return few ? launch_dma<8, 8, EPI, 2, 3, 8>(X, W, C, M, N, K, H, ca, stream)
+                     : launch_dma<8, 16, EPI, 1, 2, 16>(X, W, C, M, N, K, H, ca, stream);
+        if (N >= 200 * 64)
+          return few ? launch_dma<4, 16, EPI, 1, 2, 8>(X, W, C, M, N, K, H, ca, stream)
+                     : launch_dma<4, 16, EPI, 1, 2, 16>(X, W, C, M, N, K, H, ca, stream);
+        return few ? launch_dma<2, 16, EPI, 1, 2, 8>(X, W, C, M, N, K, H, ca, stream)
+                   : launch_dma<2, 16, EPI, 1, 2, 16>(X, W, C, M, N, K, H, ca, stream);
+      }
+      return few ? launch_dma<1, 8, E, 1, 3, 8>(X, W, C, M, N, K, H, ca, stream)
+                 : launch_dma<1, 8, E, 1, 3, 16>(X, W, C, M, N, K, H, ca, stream);
+    }
     if (EPI == EPI_GATED)
       gemm_skinny_kernel<1, 2, 4, EPI, 8, false><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
     else if (!emit && N > 4096 && K < 8192)
