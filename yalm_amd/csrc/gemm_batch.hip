@@ -164,6 +164,149 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_kernel(const bf16* _
   }
 }
 
+template <int N_>
+__device__ __forceinline__ void wait_vmcnt() {   // vmcnt only: expcnt and lgkmcnt fields at their maxima
+  __builtin_amdgcn_s_waitcnt((N_ & 0xF) | ((N_ >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+// The same product with both operands going from global memory straight into LDS
+// (global_load_lds_dwordx4), for K and K slices that are multiples of 64: a stage is 64 k, every wave
+// keeps a ring of S stages of its own weight rows, and the workgroup one ring of the activations, of
+// which every wave fetches 8 rows.  Every request to the second-level cache is a whole 128-byte line
+// (8 lanes a row), where the register path's lanes ask for 64-byte pieces and a CU's requests a clock
+// are what limits it; the 16-byte chunks of a row are XOR-swizzled by the row number in the global
+// address, so that the fragment reads of 8 rows fall on different banks.  One bare s_barrier a
+// stage: after it everyone's part of the stage's activations is there and everyone has read the
+// stage before.
+template <int MT, int NTW, int EPI, int S>
+__global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_dma_kernel(const bf16* __restrict__ X,
+                                                                        const bf16* __restrict__ W,
+                                                                        void* __restrict__ Cv,
+                                                                        float* __restrict__ partial, int M, int N,
+                                                                        int K, int H, int k_per_slice,
+                                                                        int always_partial) {
+  constexpr int KD = 64;
+  constexpr int WSTAGE = NTW * 2048;             // a wave's weight rows of a stage
+  constexpr int XSTAGE = NWAVES * 1024;          // 64 rows of the activations, 8 from every wave
+  constexpr int L = 2 * NTW + 1;                 // DMA instructions a wave and stage
+  static_assert(S >= 3 && S <= 4, "3 or 4 stages");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];   // [NWAVES][S][WSTAGE], then [S][XSTAGE]
+  const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
+  const int q = lane / 16, j = lane % 16;
+  unsigned char* wring = ring + (size_t)wave * S * WSTAGE;
+  unsigned char* xring = ring + (size_t)NWAVES * S * WSTAGE;
+  const int n0 = (blockIdx.x * NWAVES + wave) * 16 * NTW;
+  const int k_begin = blockIdx.y * k_per_slice, k_end = min(K, k_begin + k_per_slice);
+  const int n_st = max(0, k_end - k_begin) / KD;
+
+  const int r8 = lane / 8, chunk = (lane % 8) ^ r8;   // this lane's row of an instruction and the chunk it asks for
+  const bf16* gw[2 * NTW];
+#pragma unroll
+  for (int u = 0; u < 2 * NTW; ++u)
+    gw[u] = W + (size_t)min(n0 + (u / 2) * 16 + (u % 2) * 8 + r8, N - 1) * K + k_begin + chunk * 8;
+  const bf16* gx = X + (size_t)min(wave * 8 + r8, M - 1) * K + k_begin + chunk * 8;
+  auto issue = [&](int i, int buf) {
+#if defined(__HIP_DEVICE_COMPILE__)   // the host pass drops a template that names this builtin, and its launch stub with it
+#pragma unroll
+    for (int u = 0; u < 2 * NTW; ++u)
+      __builtin_amdgcn_global_load_lds(gw[u] + (size_t)i * KD, wring + buf * WSTAGE + u * 1024, 16, 0, 0);
+    __builtin_amdgcn_global_load_lds(gx + (size_t)i * KD, xring + buf * XSTAGE + wave * 1024, 16, 0, 0);
+#endif
+  };
+
+  f32x4 acc[MT][NTW];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int t = 0; t < NTW; ++t) acc[mt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int i = 0; i < S - 1; ++i)
+    if (i < n_st) issue(i, i);
+  // fragment reads: lane (q, j) of step s wants chunk 4 s + q of row j, which lies at (4 s + q) ^ (j & 7)
+  const int rd = j * 128, swz = j & 7;
+  int buf = 0;
+  for (int i = 0; i < n_st; ++i) {
+    const int ahead = n_st - 1 - i;               // stages behind this one that are in flight
+    if (ahead >= S - 2) wait_vmcnt<(S - 2) * L>();
+    else if (ahead == 1) wait_vmcnt<L>();
+    else wait_vmcnt<0>();
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (i + S - 1 < n_st) {
+      int nb = buf + S - 1;
+      if (nb >= S) nb -= S;
+      issue(i + S - 1, nb);                       // into the buffer that everyone read in the round before
+    }
+    const unsigned char* wcur = wring + buf * WSTAGE;
+    const unsigned char* xcur = xring + buf * XSTAGE;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int off = ((4 * s + q) ^ swz) << 4;
+      bf16x8 wf[NTW];
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) wf[t] = *reinterpret_cast<const bf16x8*>(wcur + t * 2048 + rd + off);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const bf16x8 xf = *reinterpret_cast<const bf16x8*>(xcur + mt * 2048 + rd + off);
+#pragma unroll
+        for (int t = 0; t < NTW; ++t)
+          acc[mt][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf, wf[t], acc[mt][t], 0, 0, 0);
+      }
+    }
+    if (++buf == S) buf = 0;
+  }
+
+  if (gridDim.y == 1 && !always_partial) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      if (EPI == 3) {
+        store_tile<3>(Cv, acc[mt][0], acc[mt][NTW - 1], mt * 16 + 4 * q, 0, n0 / 2 + j, M, N, H);
+      } else {
+#pragma unroll
+        for (int t = 0; t < NTW; ++t)
+          store_tile<EPI>(Cv, acc[mt][t], acc[mt][t], mt * 16 + 4 * q, n0 + t * 16 + j, 0, M, N, H);
+      }
+    }
+  } else {
+    float* part = partial + (size_t)blockIdx.y * M * N;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) {
+        int n = n0 + t * 16 + j;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          int m = mt * 16 + 4 * q + r;
+          if (m < M && n < N) part[(size_t)m * N + n] = acc[mt][t][r];
+        }
+      }
+  }
+}
+
+// launches one of the two kernels: the DMA one where K and the slices are multiples of 64
+template <int MT, int NTW, int EPI>
+int launch_kernel(dim3 grid, const bf16* X, const bf16* W, void* C, float* ws, int M, int N, int K, int H,
+                  int k_per_slice, int always_partial, hipStream_t stream) {
+  if (K % 64 == 0 && k_per_slice % 64 == 0) {
+    constexpr int S = NTW == 1 ? 4 : 3;
+    constexpr size_t lds = (size_t)NWAVES * S * NTW * 2048 + (size_t)S * NWAVES * 1024;
+    auto kernel = &gemm_batch_dma_kernel<MT, NTW, EPI, S>;
+    static bool allowed = false;                   // more than 64 KB of LDS has to be asked for once
+    if (!allowed) {
+      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (e != hipSuccess) return (int)e;
+      allowed = true;
+    }
+    kernel<<<grid, NWAVES * WAVE, lds, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice, always_partial);
+  } else {
+    gemm_batch_kernel<MT, NTW, EPI><<<grid, NWAVES * WAVE, 0, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice,
+                                                                        always_partial);
+  }
+  return launch_status();
+}
+
 // adds the K slices in order and applies the epilogue; a thread per (row, 4 columns)
 template <int EPI>
 __global__ void splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ Cv, int M, int N, int H,
@@ -228,8 +371,7 @@ int launch_mt(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, 
   const int k_per_slice = ceil_div(chunks, slices) * KC;
   slices = ceil_div(K, k_per_slice);
   dim3 grid(n_blocks, slices);
-  gemm_batch_kernel<MT, NTW, EPI><<<grid, NWAVES * WAVE, 0, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice, 0);
-  int rc = launch_status();
+  int rc = launch_kernel<MT, NTW, EPI>(grid, X, W, C, ws, M, N, K, H, k_per_slice, 0, stream);
   if (rc != YALM_OK || slices == 1) return rc;
   const long items = (long)M * (EPI == 3 ? (N / 2) / 4 : (N + 3) / 4);
   splitk_reduce_kernel<EPI><<<ceil_div(items, 256), 256, 0, stream>>>(ws, C, M, N, H, slices);
@@ -309,8 +451,7 @@ int launch_add_norm(const bf16* X, const bf16* W, float* C, float* ws, long ws_f
   const int k_per_slice = ceil_div(chunks, slices) * KC;
   slices = ceil_div(K, k_per_slice);
   dim3 grid(n_blocks, slices);
-  gemm_batch_kernel<MT, 1, 2><<<grid, NWAVES * WAVE, 0, stream>>>(X, W, C, ws, M, N, K, 0, k_per_slice, 1);
-  int rc = launch_status();
+  int rc = launch_kernel<MT, 1, 2>(grid, X, W, C, ws, M, N, K, 0, k_per_slice, 1, stream);
   if (rc != YALM_OK) return rc;
   reduce_add_norm_kernel<<<M, RN_THREADS, 0, stream>>>(ws, C, norm_w, eps, h, M, N, slices);
   return launch_status();
