@@ -178,8 +178,8 @@ __device__ __forceinline__ void wait_vmcnt() {   // vmcnt only: expcnt and lgkmc
 // address, so that the fragment reads of 8 rows fall on different banks.  One bare s_barrier a
 // stage: after it everyone's part of the stage's activations is there and everyone has read the
 // stage before.
-template <int MT, int NTW, int EPI, int S>
-__global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_dma_kernel(const bf16* __restrict__ X,
+template <int MT, int NTW, int EPI, int S, int NW>
+__global__ __launch_bounds__(NW * WAVE) void gemm_batch_dma_kernel(const bf16* __restrict__ X,
                                                                         const bf16* __restrict__ W,
                                                                         void* __restrict__ Cv,
                                                                         float* __restrict__ partial, int M, int N,
@@ -187,15 +187,16 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_dma_kernel(const bf1
                                                                         int always_partial) {
   constexpr int KD = 64;
   constexpr int WSTAGE = NTW * 2048;             // a wave's weight rows of a stage
-  constexpr int XSTAGE = NWAVES * 1024;          // 64 rows of the activations, 8 from every wave
-  constexpr int L = 2 * NTW + 1;                 // DMA instructions a wave and stage
+  constexpr int XSTAGE = 8 * 1024;               // 64 rows of the activations, 8 an instruction
+  constexpr int XI = 8 / NW;                     // of which every wave issues this many
+  constexpr int L = 2 * NTW + XI;                // DMA instructions a wave and stage
   static_assert(S >= 3 && S <= 4, "3 or 4 stages");
-  extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];   // [NWAVES][S][WSTAGE], then [S][XSTAGE]
+  extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];   // [NW][S][WSTAGE], then [S][XSTAGE]
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int q = lane / 16, j = lane % 16;
   unsigned char* wring = ring + (size_t)wave * S * WSTAGE;
-  unsigned char* xring = ring + (size_t)NWAVES * S * WSTAGE;
-  const int n0 = (blockIdx.x * NWAVES + wave) * 16 * NTW;
+  unsigned char* xring = ring + (size_t)NW * S * WSTAGE;
+  const int n0 = (blockIdx.x * NW + wave) * 16 * NTW;
   const int k_begin = blockIdx.y * k_per_slice, k_end = min(K, k_begin + k_per_slice);
   const int n_st = max(0, k_end - k_begin) / KD;
 
@@ -204,13 +205,17 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_dma_kernel(const bf1
 #pragma unroll
   for (int u = 0; u < 2 * NTW; ++u)
     gw[u] = W + (size_t)min(n0 + (u / 2) * 16 + (u % 2) * 8 + r8, N - 1) * K + k_begin + chunk * 8;
-  const bf16* gx = X + (size_t)min(wave * 8 + r8, M - 1) * K + k_begin + chunk * 8;
+  const bf16* gx[XI];
+#pragma unroll
+  for (int u = 0; u < XI; ++u) gx[u] = X + (size_t)min((wave * XI + u) * 8 + r8, M - 1) * K + k_begin + chunk * 8;
   auto issue = [&](int i, int buf) {
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass drops a template that names this builtin, and its launch stub with it
 #pragma unroll
     for (int u = 0; u < 2 * NTW; ++u)
       __builtin_amdgcn_global_load_lds(gw[u] + (size_t)i * KD, wring + buf * WSTAGE + u * 1024, 16, 0, 0);
-    __builtin_amdgcn_global_load_lds(gx + (size_t)i * KD, xring + buf * XSTAGE + wave * 1024, 16, 0, 0);
+#pragma unroll
+    for (int u = 0; u < XI; ++u)
+      __builtin_amdgcn_global_load_lds(gx[u] + (size_t)i * KD, xring + buf * XSTAGE + (wave * XI + u) * 1024, 16, 0, 0);
 #endif
   };
 
@@ -285,22 +290,23 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_dma_kernel(const bf1
   }
 }
 
-// launches one of the two kernels: the DMA one where K and the slices are multiples of 64
-template <int MT, int NTW, int EPI>
+// launches one of the two kernels: the DMA one (NW waves) where K and the slices are multiples of 64
+template <int MT, int NTW, int EPI, int NW>
 int launch_kernel(dim3 grid, const bf16* X, const bf16* W, void* C, float* ws, int M, int N, int K, int H,
                   int k_per_slice, int always_partial, hipStream_t stream) {
   if (K % 64 == 0 && k_per_slice % 64 == 0) {
-    constexpr int S = NTW == 1 ? 4 : 3;
-    constexpr size_t lds = (size_t)NWAVES * S * NTW * 2048 + (size_t)S * NWAVES * 1024;
-    auto kernel = &gemm_batch_dma_kernel<MT, NTW, EPI, S>;
+    constexpr int S = (NW * NTW <= 8) ? 4 : 3;
+    constexpr size_t lds = (size_t)NW * S * NTW * 2048 + (size_t)S * 8 * 1024;
+    auto kernel = &gemm_batch_dma_kernel<MT, NTW, EPI, S, NW>;
     static bool allowed = false;                   // more than 64 KB of LDS has to be asked for once
     if (!allowed) {
       hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
       if (e != hipSuccess) return (int)e;
       allowed = true;
     }
-    kernel<<<grid, NWAVES * WAVE, lds, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice, always_partial);
+    kernel<<<grid, NW * WAVE, lds, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice, always_partial);
   } else {
+    if (NW != NWAVES) return YALM_ERR_ARG;
     gemm_batch_kernel<MT, NTW, EPI><<<grid, NWAVES * WAVE, 0, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice,
                                                                         always_partial);
   }
@@ -355,27 +361,36 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, void* __
   }
 }
 
-template <int MT, int EPI>
-int launch_mt(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
+template <int MT, int EPI, int NW>
+int launch_nw(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
               hipStream_t stream) {
   constexpr int NTW = EPI == 3 ? 2 : 1;
-  const int rows_per_wg = NWAVES * 16 * NTW;
+  const int rows_per_wg = NW * 16 * NTW;
   const int n_blocks = ceil_div(N, rows_per_wg);
   const int chunks = ceil_div(K, KC);
   // slices: until every CU has a workgroup, while the partial sums stay small beside the weights
   // (slices * M * N * 4 bytes against N * K * 2) and a slice keeps at least 2 chunks
   int slices = 1;
-  while (n_blocks * slices < 256 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
+  while (n_blocks * slices < 200 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
     slices *= 2;
   if (ws == nullptr || (long)slices * M * N > ws_floats) slices = 1;
   const int k_per_slice = ceil_div(chunks, slices) * KC;
   slices = ceil_div(K, k_per_slice);
   dim3 grid(n_blocks, slices);
-  int rc = launch_kernel<MT, NTW, EPI>(grid, X, W, C, ws, M, N, K, H, k_per_slice, 0, stream);
+  int rc = launch_kernel<MT, NTW, EPI, NW>(grid, X, W, C, ws, M, N, K, H, k_per_slice, 0, stream);
   if (rc != YALM_OK || slices == 1) return rc;
   const long items = (long)M * (EPI == 3 ? (N / 2) / 4 : (N + 3) / 4);
   splitk_reduce_kernel<EPI><<<ceil_div(items, 256), 256, 0, stream>>>(ws, C, M, N, H, slices);
   return launch_status();
+}
+
+template <int MT, int EPI>
+int launch_mt(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
+              hipStream_t stream) {
+  // waves a workgroup of the DMA kernel (they share the activations' stage): measured at batch 64
+  // 8 waves 8120, 4 waves 8580, 2 waves 8410 tokens a second; at batch 32 5490, 5740 and 5870
+  if (K % 64 == 0) return launch_nw<MT, EPI, (MT <= 2 ? 2 : 4)>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+  return launch_nw<MT, EPI, 8>(X, W, C, ws, ws_floats, M, N, K, H, stream);
 }
 
 // The residual add that also does the NEXT RMSNorm: a workgroup per row adds the K slices to
@@ -438,23 +453,31 @@ __global__ __launch_bounds__(RN_THREADS) void reduce_add_norm_kernel(const float
   }
 }
 
-template <int MT>
-int launch_add_norm(const bf16* X, const bf16* W, float* C, float* ws, long ws_floats, int M, int N, int K,
-                    const float* norm_w, float eps, bf16* h, hipStream_t stream) {
-  const int n_blocks = ceil_div(N, NWAVES * 16);
+template <int MT, int NW>
+int launch_add_norm_nw(const bf16* X, const bf16* W, float* C, float* ws, long ws_floats, int M, int N, int K,
+                       const float* norm_w, float eps, bf16* h, hipStream_t stream) {
+  const int n_blocks = ceil_div(N, NW * 16);
   const int chunks = ceil_div(K, KC);
   int slices = 1;
-  while (n_blocks * slices < 256 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
+  while (n_blocks * slices < 200 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
     slices *= 2;
   while (slices > 1 && (long)slices * M * N > ws_floats) slices /= 2;
   if (ws == nullptr || (long)slices * M * N > ws_floats) return YALM_ERR_ARG;
   const int k_per_slice = ceil_div(chunks, slices) * KC;
   slices = ceil_div(K, k_per_slice);
   dim3 grid(n_blocks, slices);
-  int rc = launch_kernel<MT, 1, 2>(grid, X, W, C, ws, M, N, K, 0, k_per_slice, 1, stream);
+  int rc = launch_kernel<MT, 1, 2, NW>(grid, X, W, C, ws, M, N, K, 0, k_per_slice, 1, stream);
   if (rc != YALM_OK) return rc;
   reduce_add_norm_kernel<<<M, RN_THREADS, 0, stream>>>(ws, C, norm_w, eps, h, M, N, slices);
   return launch_status();
+}
+
+template <int MT>
+int launch_add_norm(const bf16* X, const bf16* W, float* C, float* ws, long ws_floats, int M, int N, int K,
+                    const float* norm_w, float eps, bf16* h, hipStream_t stream) {
+  if (K % 64 == 0 && MT > 2)
+    return launch_add_norm_nw<MT, 4>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream);
+  return launch_add_norm_nw<MT, NWAVES>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream);
 }
 
 template <int EPI>
