@@ -85,7 +85,10 @@ def test_rmsnorm(D, w_dtype, out_dtype):
 # more than 64 rows: K a multiple of 64 takes the kernel that loads straight into LDS (128x128 tiles,
 # or 256x256 where 160 of them exist), any other K the register-staged one
 GEMM_SHAPES = [(1, 16, 256), (3, 70, 96), (64, 130, 264), (65, 64, 80), (200, 333, 1000), (8, 4096 + 16, 136),
-               (130, 100, 50), (65, 64, 64), (200, 333, 1024), (300, 20480 + 8, 128), (513, 130, 192)]
+               (130, 100, 50), (65, 64, 64), (200, 333, 1024), (300, 20480 + 8, 128), (513, 130, 192),
+               # K a multiple of 64 (operands staged in LDS by DMA): few and odd rows, every row count of a stage
+               (5, 70, 192), (16, 4112, 128), (9, 100, 64), (12, 33, 320), (8, 26000, 64), (13, 13000, 128),
+               (3, 4096, 1024), (20, 70, 192), (33, 4112, 128), (50, 100, 64), (64, 333, 320)]
 
 
 @pytest.mark.parametrize("simple", [False, True])
@@ -115,7 +118,8 @@ def test_gemm_store_and_add(M, N, Kd, dtype, simple):
 @pytest.mark.parametrize("simple", [False, True])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,H,D", [(1, 16, 64), (5, 176, 64), (70, 100, 96), (64, 1000, 264), (3, 14336, 128),
-                                   (70, 100, 128), (300, 10300, 64), (260, 1000, 256)])
+                                   (70, 100, 128), (300, 10300, 64), (260, 1000, 256), (7, 100, 192), (13, 7000, 128),
+                                   (16, 13000, 64), (9, 3300, 320), (24, 100, 192), (61, 1000, 128)])
 def test_gemm_gated(M, H, D, dtype, simple):
     from yalm_amd.parts.swiglu import interleave_gate_up
     k = K()
@@ -585,7 +589,8 @@ def test_gemm_norm_qkv_rope(n_heads, n_kv, hd, rd, D):
     assert (vp.float().abs().sum(dim=(1, 2)) > 0).equal(touched)
 
 
-@pytest.mark.parametrize("M,N,Kd", [(1, 64, 256), (8, 4096, 1000), (33, 80, 96), (64, 4096, 264), (5, 16400, 64)])
+@pytest.mark.parametrize("M,N,Kd", [(1, 64, 256), (8, 4096, 1000), (33, 80, 96), (64, 4096, 264), (5, 16400, 64),
+                                    (11, 192, 192), (16, 4096, 128), (9, 1024, 64)])
 def test_gemm_chain_producer_and_consumer(M, N, Kd):
     """A residual-add GEMM that emits the next norm's activations and partial sums of squares,
     and a consumer that scales by them: together they equal rmsnorm(x_new) @ W2^T."""
