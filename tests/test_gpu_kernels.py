@@ -201,6 +201,44 @@ def test_rope_kv_write(n_heads, n_kv, hd, rd, dtype):
     assert (kp.float().abs().sum(dim=(1, 3)) > 0).equal(touched)
 
 
+@pytest.mark.parametrize("M,n_heads,n_kv,hd,D", [(17, 4, 2, 16, 4096), (40, 3, 1, 48, 1024), (64, 8, 2, 128, 264),
+                                                 (33, 2, 2, 64, 64)])
+def test_gemm_partial_and_rotation_that_adds_the_slices(M, n_heads, n_kv, hd, D):
+    """q/k/v projection of 17..64 rows whose K slices stay unadded, and the rotation kernel that adds them
+    while it reads: the same q and cache pages as the product, added first, gives."""
+    k = K()
+    PAGE = k.PAGE
+    Q, KV = n_heads * hd, n_kv * hd
+    N = Q + 2 * KV
+    h = rnd((M, D), 90, torch.bfloat16)
+    w = rnd((N, D), 91, torch.bfloat16, scale=1 / math.sqrt(D))
+    ws = torch.full((k.gemm_workspace_floats(M, N, D),), float("nan"), device=DEV)
+    slices = k.gemm_partial(h.to(DEV), w.to(DEV), ws)
+    assert 1 <= slices and slices * M * N <= ws.numel()
+    if D >= 1024:
+        assert slices > 1                                      # the case this test is for
+    qkv = ws[:slices * M * N].reshape(slices, M, N).sum(dim=0)
+    close(qkv, h.double() @ w.double().T, torch.float32, "sum of the slices")
+    # one sequence per row, at positions 61 + row (so that some cross a page)
+    table = make_table(200, hd, hd, 10000.0).to(DEV)
+    pos = [61 + m for m in range(M)]
+    bt = torch.arange(2 * M, dtype=torch.int32).reshape(M, 2).to(DEV)
+    outs = []
+    for source, n in ((qkv.contiguous(), 1), (ws, slices)):
+        kp = torch.zeros((2 * M, n_kv, PAGE, hd), dtype=torch.bfloat16, device=DEV)
+        vp = torch.zeros((2 * M, n_kv, hd, PAGE), dtype=torch.bfloat16, device=DEV)
+        q = torch.zeros((M, Q), dtype=torch.bfloat16, device=DEV)
+        k.rope_kv_write(source, q, None, None, None, kp, vp, bt, 2, i32(list(range(M))), i32(pos),
+                        i32(list(range(M))), i32([p + 1 for p in pos]), table, n_heads, n_kv, hd, hd, slices=n)
+        outs.append((q, kp, vp))
+    for a, b, what in zip(outs[0], outs[1], ("q", "k pages", "v pages")):
+        assert a.abs().sum() > 0
+        close(b, a.double().cpu(), torch.bfloat16, what)       # the slices are added in another order than torch's sum
+    with pytest.raises(ValueError):
+        k.rope_kv_write(ws[:M * N], outs[0][0], None, None, None, None, None, None, 0, i32(list(range(M))), i32(pos),
+                        i32(list(range(M))), i32([p + 1 for p in pos]), table, n_heads, n_kv, hd, hd, slices=2)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_heads,n_kv,hd,rd,lens,ring", [(4, 2, 16, 16, [5, 130, 64], 3), (3, 1, 48, 24, [200, 1], 2),
                                                           (8, 2, 128, 128, [70, 257], 8), (2, 2, 64, 64, [300], 3)])

@@ -91,7 +91,13 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
                                      const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                      const int* __restrict__ seq_slot, const int* __restrict__ seq_len,
                                      const float2* __restrict__ cos_sin, int n_positions, int n_heads,
-                                     int n_kv_heads, int hd, int rotary_dim, int n_pages) {
+                                     int n_kv_heads, int hd, int rotary_dim, int n_pages, int slices, long plane) {
+  // qkv may be `slices` partial products [slices][T][Q + 2 KV] of a GEMM that split K: added here, in order
+  auto rd = [&](const float* p) {
+    float v = p[0];
+    for (int s = 1; s < slices; ++s) v += p[(size_t)s * plane];
+    return v;
+  };
   int t = blockIdx.x;
   int job = blockIdx.y;
   int pos = tok_pos[t];
@@ -105,7 +111,7 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
     const float* src = row + job * hd;
     T* dst = q_out + (size_t)t * Q + job * hd;
     for (int p = threadIdx.x; p < hd / 2; p += WAVE) {
-      float x0 = src[2 * p], x1 = src[2 * p + 1];
+      float x0 = rd(src + 2 * p), x1 = rd(src + 2 * p + 1);
       if (rotate && p < half_rot) {
         float2 c = cs[p];
         float y0 = x0 * c.x - x1 * c.y;
@@ -151,7 +157,7 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
   if (is_k) {
     const float* src = row + Q + g * hd;
     for (int p = threadIdx.x; p < hd / 2; p += WAVE) {
-      float x0 = src[2 * p], x1 = src[2 * p + 1];
+      float x0 = rd(src + 2 * p), x1 = rd(src + 2 * p + 1);
       if (rotate && p < half_rot) {
         float2 c = cs[p];
         float y0 = x0 * c.x - x1 * c.y;
@@ -172,7 +178,7 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
   } else {
     const float* src = row + Q + KV + g * hd;
     for (int i = threadIdx.x; i < hd; i += WAVE) {
-      T a = from_f32<T>(src[i]);
+      T a = from_f32<T>(rd(src + i));
       if (vst) vst[(size_t)i * PAGE + r] = a;
       if (vpage) vpage[(size_t)i * PAGE + r] = a;      // values are kept transposed inside a page
     }
@@ -317,22 +323,24 @@ extern "C" int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_stage, 
                                   const int* seq_tile0, void* k_pages, void* v_pages, const int* block_table, int table_stride, int ring_pages,
                                   const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_len,
                                   const float* cos_sin, int n_positions, int T, int n_heads, int n_kv_heads,
-                                  int head_dim, int rotary_dim, int n_pages, int dtype, hipStream_t stream) {
+                                  int head_dim, int rotary_dim, int n_pages, int slices, int dtype,
+                                  hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (head_dim <= 0 || (head_dim & 1) || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > head_dim ||
-      n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0)
+      n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || slices < 1)
     return YALM_ERR_ARG;
+  const long plane = (long)T * (n_heads + 2 * n_kv_heads) * head_dim;
   dim3 grid(T, n_heads + 2 * n_kv_heads);
   if (dtype == YALM_F32)
     rope_kv_write_kernel<float><<<grid, WAVE, 0, stream>>>(
         qkv, (float*)q_out, (float*)k_stage, (float*)v_stage, seq_tile0, (float*)k_pages, (float*)v_pages, block_table,
         table_stride, ring_pages, tok_seq, tok_pos, seq_slot, seq_len, (const float2*)cos_sin, n_positions, n_heads,
-        n_kv_heads, head_dim, rotary_dim, n_pages);
+        n_kv_heads, head_dim, rotary_dim, n_pages, slices, plane);
   else if (dtype == YALM_BF16)
     rope_kv_write_kernel<bf16><<<grid, WAVE, 0, stream>>>(
         qkv, (bf16*)q_out, (bf16*)k_stage, (bf16*)v_stage, seq_tile0, (bf16*)k_pages, (bf16*)v_pages, block_table, table_stride,
         ring_pages, tok_seq, tok_pos, seq_slot, seq_len, (const float2*)cos_sin, n_positions, n_heads, n_kv_heads,
-        head_dim, rotary_dim, n_pages);
+        head_dim, rotary_dim, n_pages, slices, plane);
   else
     return YALM_ERR_DTYPE;
   return launch_status();

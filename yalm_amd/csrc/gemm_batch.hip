@@ -480,6 +480,32 @@ int launch_add_norm(const bf16* X, const bf16* W, float* C, float* ws, long ws_f
   return launch_add_norm_nw<MT, NWAVES>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream);
 }
 
+// the K slices only: [slices][M][N] in ws, for a consumer that adds them
+template <int MT, int NW>
+int launch_partial_nw(const bf16* X, const bf16* W, float* ws, long ws_floats, int M, int N, int K, int* slices_out,
+                      hipStream_t stream) {
+  const int n_blocks = ceil_div(N, NW * 16);
+  const int chunks = ceil_div(K, KC);
+  int slices = 1;
+  while (n_blocks * slices < 200 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
+    slices *= 2;
+  while (slices > 1 && (long)slices * M * N > ws_floats) slices /= 2;
+  if (ws == nullptr || (long)slices * M * N > ws_floats) return YALM_ERR_ARG;
+  const int k_per_slice = ceil_div(chunks, slices) * KC;
+  slices = ceil_div(K, k_per_slice);
+  *slices_out = slices;
+  dim3 grid(n_blocks, slices);
+  return launch_kernel<MT, 1, 0, NW>(grid, X, W, ws, ws, M, N, K, 0, k_per_slice, 1, stream);
+}
+
+template <int MT>
+int launch_partial(const bf16* X, const bf16* W, float* ws, long ws_floats, int M, int N, int K, int* slices_out,
+                   hipStream_t stream) {
+  if (K % 64 == 0)
+    return launch_partial_nw<MT, (MT <= 2 ? 2 : 4)>(X, W, ws, ws_floats, M, N, K, slices_out, stream);
+  return launch_partial_nw<MT, NWAVES>(X, W, ws, ws_floats, M, N, K, slices_out, stream);
+}
+
 template <int EPI>
 int dispatch(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
              hipStream_t stream) {
@@ -504,6 +530,20 @@ int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace
     case 1: return dispatch<1>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
     case 2: return dispatch<2>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
     case 3: return dispatch<3>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+  }
+  return YALM_ERR_ARG;
+}
+
+extern "C" int yalm_gemm_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N,
+                                 int K, int* slices, hipStream_t stream) {
+  if (M <= 16 || M > 64 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || slices == nullptr)
+    return YALM_ERR_ARG;
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  switch ((M + 15) / 16) {
+    case 2: return launch_partial<2>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
+    case 3: return launch_partial<3>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
+    case 4: return launch_partial<4>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
   }
   return YALM_ERR_ARG;
 }

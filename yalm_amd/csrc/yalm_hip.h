@@ -58,6 +58,11 @@ int yalm_gemm_norm_qkv_rope(const float* x, const float* norm_w, float eps, cons
 // Residual add and the next RMSNorm in one for 17..64 rows (bfloat16): C float32 [M,N] += A[M,K] * W[N,K]^T, then
 // h_out bfloat16 [M,N] = C_new * rsqrt(mean(C_new^2) + eps) * norm_w.  workspace: at least M * N floats (more lets
 // it split K).  Refuses (YALM_ERR_ARG) other shapes.
+// The K slices of A[M,K] * W[N,K]^T for 17..64 rows (bfloat16), left unadded: workspace [*slices][M][N] float32, for a
+// consumer that adds them itself (yalm_rope_kv_write).  Needs at least M * N floats; refuses (YALM_ERR_ARG) other shapes.
+int yalm_gemm_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N, int K,
+                      int* slices, hipStream_t stream);
+
 int yalm_gemm_add_norm(const void* A, const void* W, float* C, float* workspace, long workspace_floats, int M, int N,
                        int K, const float* norm_w, float eps, void* h_out, hipStream_t stream);
 
@@ -89,11 +94,13 @@ int yalm_gemm_chain_qkv_rope(const void* X, const float* ss_in, int n_parts_in, 
 //   block_table int32 [n_slots, table_stride]; page of position p: table[slot][(p / PAGE) % ring_pages]
 //   a token is written iff its page is among the last ring_pages pages of its sequence
 // reference: fused_rope_and_cache_update (src/infer.cu:660-705)
+// slices > 1: qkv holds that many partial products [slices][T][...] of a GEMM that split K (yalm_gemm_partial);
+// they are added in order while they are read.
 int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_stage, void* v_stage, const int* seq_tile0,
                        void* k_pages, void* v_pages, const int* block_table, int table_stride, int ring_pages, const int* tok_seq,
                        const int* tok_pos, const int* seq_slot, const int* seq_len, const float* cos_sin,
                        int n_positions, int T, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
-                       int n_pages, int dtype, hipStream_t stream);
+                       int n_pages, int slices, int dtype, hipStream_t stream);
 
 // The same for a step of whole prompts (every sequence from position 0; cu_seqlens [B + 1] token offsets,
 // n_tiles = seq_tile0[B]): whole page-shaped tiles at a time.  Needs a staging area; refuses

@@ -3,6 +3,8 @@ operands have the shapes, dtypes and layout its kernel and grid assume (a
 mismatch is an error here, never a wrong result or a fault on the device), then
 launches on torch's current stream.  Tensors must live on the GPU; there is no
 CPU path."""
+import ctypes
+
 import torch
 
 from . import library
@@ -214,6 +216,28 @@ def gemm_add_norm(a, w, x, norm_w, eps, h_out, workspace):
     return h_out
 
 
+def can_gemm_partial(M, K, dtype):
+    """True if gemm_partial takes the shape (17..64 rows of bfloat16)."""
+    return dtype == torch.bfloat16 and CHAIN_MAX_ROWS < M <= 64 and K % 8 == 0 and not FORCE_SIMPLE
+
+
+def gemm_partial(a, w, workspace):
+    """The K slices of a[M,K] @ w[N,K]^T, 17..64 rows of bfloat16, left unadded in `workspace`
+    ([slices][M][N] float32, flat; gemm_workspace_floats(M, N, K) elements let it split as it likes).
+    Returns the number of slices, for a consumer that adds them (rope_kv_write)."""
+    M, K = a.shape
+    N = w.shape[0]
+    p_a = _need(a, "a", torch.bfloat16, (M, K))
+    p_w = _need(w, "w", torch.bfloat16, (N, K))
+    p_ws = _need(workspace, "workspace", torch.float32, (None,))
+    if workspace.numel() < M * N:
+        raise ValueError("workspace holds %d floats, at least %d are needed" % (workspace.numel(), M * N))
+    slices = ctypes.c_int(0)
+    library.check(library.lib().yalm_gemm_partial(p_a, p_w, p_ws, workspace.numel(), M, N, K, ctypes.byref(slices),
+                                                  _stream()), "gemm_partial")
+    return slices.value
+
+
 def gemm_chain_parts(N):
     """Columns of the partial sums of squares that a producer with N output columns emits."""
     return library.lib().yalm_gemm_chain_parts(int(N))
@@ -298,15 +322,23 @@ def _check_heads(n_heads, n_kv_heads, head_dim):
 
 
 def rope_kv_write(qkv, q_out, k_stage, v_stage, seq_tile0, k_pages, v_pages, block_table, ring_pages, tok_seq, tok_pos,
-                  seq_slot, seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim):
+                  seq_slot, seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim, slices=1):
     """Rotates q and k by the angles of `cos_sin` at each token's position, writes q in
     q_out's dtype, k and v into the staging area (page format, tile seq_tile0[sequence] +
-    position // PAGE) if one is given, and into the pages of the cache if given."""
+    position // PAGE) if one is given, and into the pages of the cache if given.
+    slices > 1: qkv is the flat scratch of gemm_partial, [slices][T][q + 2 kv] float32, and the
+    slices are added while they are read."""
     _check_heads(n_heads, n_kv_heads, head_dim)
-    T = qkv.shape[0]
+    T = q_out.shape[0]
     Q, KV = n_heads * head_dim, n_kv_heads * head_dim
     dt = q_out.dtype
-    p_qkv = _need(qkv, "qkv", torch.float32, (T, Q + 2 * KV))
+    if slices == 1 and qkv.dim() == 2:
+        p_qkv = _need(qkv, "qkv", torch.float32, (T, Q + 2 * KV))
+    else:
+        p_qkv = _need(qkv, "qkv", torch.float32, (None,))
+        if slices < 1 or qkv.numel() < slices * T * (Q + 2 * KV):
+            raise ValueError("qkv holds %d floats, %d slices of %d rows need %d"
+                             % (qkv.numel(), slices, T, slices * T * (Q + 2 * KV)))
     p_q = _need(q_out, "q_out", dt, (T, Q))
     B = seq_slot.shape[0]
     p_ks = p_vs = p_t0 = None
@@ -341,7 +373,8 @@ def rope_kv_write(qkv, q_out, k_stage, v_stage, seq_tile0, k_pages, v_pages, blo
         rotary_dim = 0
     library.check(library.lib().yalm_rope_kv_write(
         p_qkv, p_q, p_ks, p_vs, p_t0, p_kp, p_vp, p_bt, stride, max(ring_pages, 1), p_ts, p_tp, p_ss, p_sl, p_cs,
-        n_pos, T, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, dtype_code(dt), _stream()), "rope_kv_write")
+        n_pos, T, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, int(slices), dtype_code(dt), _stream()),
+        "rope_kv_write")
 
 
 def rope_kv_write_tiles(qkv, q_out, k_stage, v_stage, cu_seqlens, seq_tile0, k_pages, v_pages, block_table, ring_pages,

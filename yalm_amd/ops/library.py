@@ -28,7 +28,8 @@ _SIGNATURES = {
     "yalm_gemm_chain_qkv_rope": (_I, [_P, _P, _I, _F, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I,
                                       _I, _I, _P]),
     "yalm_rope_kv_write": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
-                                _I, _I, _P]),
+                                _I, _I, _I, _P]),
+    "yalm_gemm_partial": (_I, [_P, _P, _P, ctypes.c_long, _I, _I, _I, _P, _P]),
     "yalm_gemm_bf16_dma_workspace": (ctypes.c_long, [_I, _I, _I]),
     "yalm_gemm_add_norm": (_I, [_P, _P, _P, _P, ctypes.c_long, _I, _I, _I, _P, _F, _P, _P]),
     "yalm_rope_kv_write_tiles": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I,
@@ -41,7 +42,7 @@ _SIGNATURES = {
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
 }
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 
 class KernelError(RuntimeError):

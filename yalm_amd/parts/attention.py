@@ -111,11 +111,18 @@ class GQAttention(Part):
             else:
                 h = ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
                 norm.forward(x, h, ctx)
-            qkv = ctx.ws.get("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
-            self._gemm(ctx, h, self.wqkv, qkv, kernels.EPI_STORE_F32)
+            n_qkv = self.q_dim + 2 * self.kv_dim
+            if kernels.can_gemm_partial(T, self.dim, h.dtype):
+                # the GEMM's K slices go to the rotation kernel as they are, which adds them: no kernel in between
+                qkv = ctx.ws.get("gemm.partial", (kernels.gemm_workspace_floats(T, n_qkv, self.dim),), torch.float32)
+                slices = kernels.gemm_partial(h, self.wqkv, qkv)
+            else:
+                qkv = ctx.ws.get("attn.qkv", (T, n_qkv), torch.float32)
+                self._gemm(ctx, h, self.wqkv, qkv, kernels.EPI_STORE_F32)
+                slices = 1
             kernels.rope_kv_write(qkv, q, None, None, None, k_pages, v_pages, group.table, group.ring_pages,
                                   ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads,
-                                  self.n_kv_heads, self.head_dim, pos.rotary_dim)
+                                  self.n_kv_heads, self.head_dim, pos.rotary_dim, slices=slices)
         o = ctx.ws.get("attn.o", (T, self.q_dim), self.wo.dtype)
         self._decode_attention(q, o, ctx, group, k_pages, v_pages)
         emit = self._emit_args(emit_for, ctx, T, self.dim)
