@@ -170,31 +170,53 @@ template <typename T, bool BASE2 = false>
 __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(const float* __restrict__ partial,
                                                                              T* __restrict__ out, int n_heads, int hd,
                                                                              int n_splits) {
-  // Every wave finds the maximum and the denominator for itself (lanes over splits);
-  // the four waves then share the splits of the weighted sum and add their parts in
-  // a fixed order, so that few loads wait on each other.
-  __shared__ float accs[COMBINE_THREADS / WAVE][MAX_HD];
+  // One trip to memory: every wave asks for the maxima and denominators of all splits (lanes over
+  // splits) and, before it waits for them, for the sums of its own first splits (waves share the
+  // splits of the weighted sum and add their parts in a fixed order).
+  constexpr int NWV = COMBINE_THREADS / WAVE;
+  constexpr int PRE = 4;                          // splits a wave asks for ahead
+  __shared__ float accs[NWV][MAX_HD];
   const int b = blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x & (WAVE - 1), g = threadIdx.x / WAVE;
   const int stride = hd + 2;
   const float* part = partial + ((size_t)b * n_heads + h) * n_splits * stride;
-  float m = -FLT_MAX;
-  for (int s = lane; s < n_splits; s += WAVE) m = fmaxf(m, part[(size_t)s * stride + hd]);
+  auto weight = [](float d) { return BASE2 ? exp2f(d) : expf(d); };
+  float pre[PRE][ACC];
+#pragma unroll
+  for (int u = 0; u < PRE; ++u) {
+    const int sp = min(g + u * NWV, n_splits - 1);
+#pragma unroll
+    for (int j = 0; j < ACC; ++j) {
+      pre[u][j] = part[(size_t)sp * stride + min(lane + j * WAVE, hd - 1)];   // elements beyond hd are never stored
+    }
+  }
+  const int s0 = min(lane, n_splits - 1);
+  const float m0 = part[(size_t)s0 * stride + hd], l0 = part[(size_t)s0 * stride + hd + 1];
+  float m = lane < n_splits ? m0 : -FLT_MAX;
+  for (int sp = lane + WAVE; sp < n_splits; sp += WAVE) m = fmaxf(m, part[(size_t)sp * stride + hd]);
   m = wave_max(m);
-  float l = 0.f;
-  for (int s = lane; s < n_splits; s += WAVE) {
-    const float* ps = part + (size_t)s * stride;
-    l += ps[hd + 1] * (BASE2 ? exp2f(ps[hd] - m) : expf(ps[hd] - m));
+  float l = lane < n_splits ? l0 * weight(m0 - m) : 0.f;
+  for (int sp = lane + WAVE; sp < n_splits; sp += WAVE) {
+    const float* ps = part + (size_t)sp * stride;
+    l += ps[hd + 1] * weight(ps[hd] - m);
   }
   l = wave_sum(l);
   const float inv_l = l > 0.f ? 1.0f / l : 0.f;
   float a[ACC];
 #pragma unroll
   for (int j = 0; j < ACC; ++j) a[j] = 0.f;
-#pragma unroll 4
-  for (int s = g; s < n_splits; s += COMBINE_THREADS / WAVE) {
-    const float* ps = part + (size_t)s * stride;
-    const float w = BASE2 ? exp2f(ps[hd] - m) : expf(ps[hd] - m);
+#pragma unroll
+  for (int u = 0; u < PRE; ++u) {
+    const int sp = g + u * NWV;
+    if (sp < n_splits) {
+      const float w = weight(part[(size_t)sp * stride + hd] - m);
+#pragma unroll
+      for (int j = 0; j < ACC; ++j) a[j] += pre[u][j] * w;
+    }
+  }
+  for (int sp = g + PRE * NWV; sp < n_splits; sp += NWV) {
+    const float* ps = part + (size_t)sp * stride;
+    const float w = weight(ps[hd] - m);
 #pragma unroll
     for (int j = 0; j < ACC; ++j) {
       const int d = lane + j * WAVE;
@@ -211,7 +233,7 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(co
       if (d >= hd) continue;
       float t = accs[0][d];
 #pragma unroll
-      for (int w = 1; w < COMBINE_THREADS / WAVE; ++w) t += accs[w][d];
+      for (int w = 1; w < NWV; ++w) t += accs[w][d];
       out[((size_t)b * n_heads + h) * hd + d] = from_f32<T>(t * inv_l);
     }
   }
