@@ -11,6 +11,9 @@
 #include "common.h"
 #include "yalm_hip.h"
 
+int yalm_gemm_bf16_dma_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N,
+                               int K, int* slices_out, hipStream_t stream);   // gemm_dma.hip
+
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -536,7 +539,8 @@ int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace
 
 extern "C" int yalm_gemm_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N,
                                  int K, int* slices, hipStream_t stream) {
-  if (M <= 16 || M > 64 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || slices == nullptr)
+  if (M > 64) return yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, slices, stream);
+  if (M <= 16 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || slices == nullptr)
     return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
@@ -553,9 +557,15 @@ extern "C" int yalm_gemm_partial(const void* A, const void* W, float* workspace,
 extern "C" int yalm_gemm_add_norm(const void* A, const void* W, float* C, float* workspace, long workspace_floats,
                                   int M, int N, int K, const float* norm_w, float eps, void* h_out,
                                   hipStream_t stream) {
-  if (M <= 16 || M > 64 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || norm_w == nullptr ||
-      h_out == nullptr)
-    return YALM_ERR_ARG;
+  if (norm_w == nullptr || h_out == nullptr) return YALM_ERR_ARG;
+  if (M > 64) {                                    // the tiled kernel's slices, then the same reduction
+    int slices = 0;
+    int rc = yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, &slices, stream);
+    if (rc != YALM_OK) return rc;
+    reduce_add_norm_kernel<<<M, RN_THREADS, 0, stream>>>(workspace, C, norm_w, eps, (bf16*)h_out, M, N, slices);
+    return launch_status();
+  }
+  if (M <= 16 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   switch ((M + 15) / 16) {

@@ -194,7 +194,7 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const 
 
 template <int EPI, int TM, int TN, int S, int NWM, int NWN, int MINW>
 int launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, float* partial, int slices,
-                 hipStream_t stream) {
+                 hipStream_t stream, bool add_slices = true) {
   const int tiles_per_slice = ceil_div(K / TK, slices);
   const dim3 grid(ceil_div(N, TN), ceil_div(M, TM), ceil_div(K / TK, tiles_per_slice));
   const size_t lds = (size_t)S * (TM + TN) * ROWB;
@@ -208,7 +208,7 @@ int launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int
   gemm_dma_kernel<EPI, TM, TN, S, NWM, NWN, MINW><<<grid, NWM * NWN * WAVE, lds, stream>>>(A, W, C, M, N, K, H, partial,
                                                                                        tiles_per_slice);
   int rc = launch_status();
-  if (rc != YALM_OK || grid.z == 1) return rc;
+  if (rc != YALM_OK || grid.z == 1 || !add_slices) return rc;
   return yalm_splitk_reduce(partial, C, M, N, H, (int)grid.z, EPI, stream);
 }
 
@@ -242,6 +242,26 @@ long yalm_gemm_bf16_dma_workspace(int M, int N, int K) {
   if (M <= 64 || K < TK || K % TK != 0 || (long)ceil_div(M, 256) * ceil_div(N, 256) >= 160) return 0;
   const int slices = slices_for(M, N, K, (long)1 << 40);
   return slices > 1 ? (long)slices * M * N : 0;
+}
+
+// The product's K slices, left unadded, as [*slices][M][N] float32 in the workspace (one slice: the product
+// itself), for a consumer that adds them.  More than 64 rows, K a multiple of 64, at least M * N floats.
+int yalm_gemm_bf16_dma_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N,
+                               int K, int* slices_out, hipStream_t stream) {
+  if (M <= 64 || K < TK || K % TK != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || workspace == nullptr ||
+      workspace_floats < (long)M * N || slices_out == nullptr)
+    return YALM_ERR_ARG;
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  if ((long)ceil_div(M, 256) * ceil_div(N, 256) >= 160) {
+    *slices_out = 1;
+    return launch_shape<0, 256, 256, 2, 4, 2, 1>(a, w, workspace, M, N, K, 0, nullptr, 1, stream);
+  }
+  int slices = slices_for(M, N, K, workspace_floats);
+  const int tiles_per_slice = ceil_div(K / TK, slices);
+  slices = ceil_div(K / TK, tiles_per_slice);          // what the launch makes of it
+  *slices_out = slices;
+  return launch_shape<0, 128, 128, 2, 2, 2, 2>(a, w, workspace, M, N, K, 0, workspace, slices, stream, false);
 }
 
 int yalm_gemm_bf16_dma(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,

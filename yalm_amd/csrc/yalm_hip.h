@@ -55,10 +55,10 @@ int yalm_gemm_norm_qkv_rope(const float* x, const float* norm_w, float eps, cons
                             int K, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, int n_pages,
                             hipStream_t stream);
 
-// Residual add and the next RMSNorm in one for 17..64 rows (bfloat16): C float32 [M,N] += A[M,K] * W[N,K]^T, then
+// Residual add and the next RMSNorm in one for 17..64 rows, or more with K a multiple of 64 (bfloat16): C float32 [M,N] += A[M,K] * W[N,K]^T, then
 // h_out bfloat16 [M,N] = C_new * rsqrt(mean(C_new^2) + eps) * norm_w.  workspace: at least M * N floats (more lets
 // it split K).  Refuses (YALM_ERR_ARG) other shapes.
-// The K slices of A[M,K] * W[N,K]^T for 17..64 rows (bfloat16), left unadded: workspace [*slices][M][N] float32, for a
+// The K slices of A[M,K] * W[N,K]^T for 17..64 rows, or more with K a multiple of 64 (bfloat16), left unadded: workspace [*slices][M][N] float32, for a
 // consumer that adds them itself (yalm_rope_kv_write).  Needs at least M * N floats; refuses (YALM_ERR_ARG) other shapes.
 int yalm_gemm_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N, int K,
                       int* slices, hipStream_t stream);

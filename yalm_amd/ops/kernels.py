@@ -194,7 +194,15 @@ def can_chain(M, K, dtype):
 
 def can_add_norm(M, K, dtype):
     """Whether gemm_add_norm takes this shape (the batches that gemm_chain leaves out)."""
-    return dtype == torch.bfloat16 and CHAIN_MAX_ROWS < M <= 64 and K % 8 == 0 and not FORCE_SIMPLE
+    if dtype != torch.bfloat16 or FORCE_SIMPLE or M <= CHAIN_MAX_ROWS:
+        return False
+    return K % 8 == 0 if M <= 64 else K % 64 == 0
+
+
+def fused_workspace_floats(M, N, K):
+    """Floats of scratch for gemm_add_norm and gemm_partial: what lets the GEMM split K as it likes,
+    and room for one whole product at least."""
+    return max(gemm_workspace_floats(M, N, K), M * N)
 
 
 def gemm_add_norm(a, w, x, norm_w, eps, h_out, workspace):
@@ -217,8 +225,8 @@ def gemm_add_norm(a, w, x, norm_w, eps, h_out, workspace):
 
 
 def can_gemm_partial(M, K, dtype):
-    """True if gemm_partial takes the shape (17..64 rows of bfloat16)."""
-    return dtype == torch.bfloat16 and CHAIN_MAX_ROWS < M <= 64 and K % 8 == 0 and not FORCE_SIMPLE
+    """True if gemm_partial takes the shape (more than 16 rows of bfloat16; more than 64: K a multiple of 64)."""
+    return can_add_norm(M, K, dtype)
 
 
 def gemm_partial(a, w, workspace):

@@ -114,7 +114,7 @@ class GQAttention(Part):
             n_qkv = self.q_dim + 2 * self.kv_dim
             if kernels.can_gemm_partial(T, self.dim, h.dtype):
                 # the GEMM's K slices go to the rotation kernel as they are, which adds them: no kernel in between
-                qkv = ctx.ws.get("gemm.partial", (kernels.gemm_workspace_floats(T, n_qkv, self.dim),), torch.float32)
+                qkv = ctx.ws.get("gemm.partial", (kernels.fused_workspace_floats(T, n_qkv, self.dim),), torch.float32)
                 slices = kernels.gemm_partial(h, self.wqkv, qkv)
             else:
                 qkv = ctx.ws.get("attn.qkv", (T, n_qkv), torch.float32)
@@ -126,7 +126,7 @@ class GQAttention(Part):
         o = ctx.ws.get("attn.o", (T, self.q_dim), self.wo.dtype)
         self._decode_attention(q, o, ctx, group, k_pages, v_pages)
         emit = self._emit_args(emit_for, ctx, T, self.dim)
-        ready = self._add_norm_args(emit_for, ctx, T, self.dim) if emit is None else None
+        ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.q_dim) if emit is None else None
         if emit is not None and kernels.can_chain(T, self.q_dim, o.dtype):
             nw2, xn2, ss2, eps2 = emit
             kernels.gemm_chain(o, self.wo, x, kernels.EPI_ADD_F32, emit=(nw2, xn2, ss2))

@@ -109,18 +109,18 @@ class Part:
         ss = ctx.ws.get("chain.ss", (T, kernels.gemm_chain_parts(width)), torch.float32)
         return nw, xn, ss, eps
 
-    def _add_norm_args(self, emit_for, ctx, T, width):
-        """Operands for a residual-add GEMM of 17..64 rows that also does the norm `emit_for` (the next
-        one on the residual stream) and leaves its activations ready, or None."""
+    def _add_norm_args(self, emit_for, ctx, T, width, K):
+        """Operands for a residual-add GEMM [T, K] x [width, K] of more than 16 rows that also does the norm
+        `emit_for` (the next one on the residual stream) and leaves its activations ready, or None."""
         from ..ops import kernels
         if emit_for is None or not hasattr(emit_for, "fused") or ctx.mode != "decode":
             return None
-        if not kernels.can_add_norm(T, width, ctx.act_dtype):
+        if not kernels.can_add_norm(T, K, ctx.act_dtype):
             return None
         import torch
         nw, eps = emit_for.fused()
         h = ctx.ws.get("chain.h", (T, width), torch.bfloat16)          # read by the consumer before the next is written
-        ws = ctx.ws.get("gemm.partial", (kernels.gemm_workspace_floats(T, width, width),), torch.float32)
+        ws = ctx.ws.get("gemm.partial", (kernels.fused_workspace_floats(T, width, K),), torch.float32)
         return nw, eps, h, ws
 
     def fuses_norm(self, norm, x, ctx):

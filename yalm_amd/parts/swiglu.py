@@ -72,7 +72,7 @@ class SwiGLU(Part):
             norm.forward(x, h, ctx)
             self._gemm(ctx, h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
         emit = self._emit_args(emit_for, ctx, T, self.dim)
-        ready = self._add_norm_args(emit_for, ctx, T, self.dim) if emit is None else None
+        ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.hidden) if emit is None else None
         if emit is not None and kernels.can_chain(T, self.hidden, mid.dtype):
             nw2, xn2, ss2, eps2 = emit
             kernels.gemm_chain(mid, self.w_down, x, kernels.EPI_ADD_F32, emit=(nw2, xn2, ss2))
