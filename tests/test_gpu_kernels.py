@@ -59,7 +59,7 @@ def test_embed(dtype):
 
 @pytest.mark.parametrize("out_dtype", DTYPES)
 @pytest.mark.parametrize("w_dtype", DTYPES)
-@pytest.mark.parametrize("D", [50, 1000, 4100])
+@pytest.mark.parametrize("D", [50, 1000, 4100, 4096, 8192, 8196, 2050])
 def test_rmsnorm(D, w_dtype, out_dtype):
     x = rnd((7, D), 2, scale=3.0)
     w = (1 + 0.1 * rnd((D,), 3)).to(w_dtype)
