@@ -119,7 +119,8 @@ def test_gemm_store_and_add(M, N, Kd, dtype, simple):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,H,D", [(1, 16, 64), (5, 176, 64), (70, 100, 96), (64, 1000, 264), (3, 14336, 128),
                                    (70, 100, 128), (300, 10300, 64), (260, 1000, 256), (7, 100, 192), (13, 7000, 128),
-                                   (16, 13000, 64), (9, 3300, 320), (24, 100, 192), (61, 1000, 128)])
+                                   (16, 13000, 64), (9, 3300, 320), (24, 100, 192), (61, 1000, 128),
+                                   (513, 12820, 64), (2048, 14336, 64)])   # whole rounds of 256x256 tiles + a launch of 256x128
 def test_gemm_gated(M, H, D, dtype, simple):
     from yalm_amd.parts.swiglu import interleave_gate_up
     k = K()

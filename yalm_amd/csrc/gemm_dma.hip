@@ -47,7 +47,7 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const 
                                                                          const bf16* __restrict__ W,
                                                                          void* __restrict__ Cv, int M, int N, int K,
                                                                          int H, float* __restrict__ partial,
-                                                                         int tiles_per_slice) {
+                                                                         int tiles_per_slice, int n_tile0) {
   constexpr int NW = NWM * NWN;
   constexpr int ROWS = TM + TN;                    // A rows, then W rows
   constexpr int STAGE_B = ROWS * ROWB;
@@ -59,7 +59,7 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const 
   extern __shared__ __attribute__((aligned(1024))) unsigned char stages[];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
   const int wm = wave / NWN, wn = wave % NWN;
-  const int m0 = blockIdx.y * TM, n0 = blockIdx.x * TN;
+  const int m0 = blockIdx.y * TM, n0 = (blockIdx.x + n_tile0) * TN;   // a launch may own a range of the columns
   const int li = lane % 32, lh = lane / 32;
 
   // instruction i of this wave fills rows (i * NW + wave) * RPI ... of a stage; the lane's
@@ -194,9 +194,10 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const 
 
 template <int EPI, int TM, int TN, int S, int NWM, int NWN, int MINW>
 int launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, float* partial, int slices,
-                 hipStream_t stream, bool add_slices = true) {
+                 hipStream_t stream, bool add_slices = true, int n_tile0 = 0, int n_tiles = -1) {
   const int tiles_per_slice = ceil_div(K / TK, slices);
-  const dim3 grid(ceil_div(N, TN), ceil_div(M, TM), ceil_div(K / TK, tiles_per_slice));
+  if (n_tiles < 0) n_tiles = ceil_div(N, TN) - n_tile0;     // column tiles n_tile0 ... of this launch
+  const dim3 grid(n_tiles, ceil_div(M, TM), ceil_div(K / TK, tiles_per_slice));
   const size_t lds = (size_t)S * (TM + TN) * ROWB;
   static bool allowed = false;                     // more than 64 KB of LDS has to be asked for once
   if (!allowed) {
@@ -206,7 +207,7 @@ int launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int
     allowed = true;
   }
   gemm_dma_kernel<EPI, TM, TN, S, NWM, NWN, MINW><<<grid, NWM * NWN * WAVE, lds, stream>>>(A, W, C, M, N, K, H, partial,
-                                                                                       tiles_per_slice);
+                                                                                       tiles_per_slice, n_tile0);
   int rc = launch_status();
   if (rc != YALM_OK || grid.z == 1 || !add_slices) return rc;
   return yalm_splitk_reduce(partial, C, M, N, H, (int)grid.z, EPI, stream);
@@ -238,6 +239,17 @@ int launch(const bf16* A, const bf16* W, void* C, float* ws, long ws_floats, int
       auto filled = [](long tiles) { return (double)tiles / (double)(ceil_div(tiles, 256L) * 256L); };
       if (filled(t192) * 0.93 > filled(t256))
         return launch_shape<EPI, 256, 192, 2, 4, 2, 1>(A, W, C, M, N, K, H, nullptr, 1, stream);
+    }
+    // A last round of workgroups that is at most half full: its columns go to a second launch of
+    // 256x128 tiles, which fills the chip with them (2,048 x 28,672: 3 rounds + 1 of half-wide tiles
+    // instead of 3.5 that cost 4).
+    const int mt = ceil_div(M, 256), nt = ceil_div(N, 256);
+    const long rounds = t256 / 256, rest = t256 % 256;
+    const int nt_main = (int)(rounds * 256 / mt);
+    if (rounds >= 1 && rest > 0 && rest <= 128 && nt_main > 0 && nt_main < nt) {
+      int rc = launch_shape<EPI, 256, 256, 2, 4, 2, 1>(A, W, C, M, N, K, H, nullptr, 1, stream, true, 0, nt_main);
+      if (rc != YALM_OK) return rc;
+      return launch_shape<EPI, 256, 128, 2, 4, 2, 1>(A, W, C, M, N, K, H, nullptr, 1, stream, true, 2 * nt_main);
     }
     return launch_shape<EPI, 256, 256, 2, 4, 2, 1>(A, W, C, M, N, K, H, nullptr, 1, stream);
   }
