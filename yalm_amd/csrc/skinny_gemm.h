@@ -1,10 +1,12 @@
 // The decode GEMM (at most 64 rows) on the matrix cores, shared by gemm_mfma.hip and
 // gemm_fused.hip:  C = epilogue(row_scale * (X[M,K] * W[N,K]^T)), bfloat16 operands,
 // float32 accumulation.  It is bound by the one pass over the weights.  A workgroup owns
-// 16 * NT weight rows and all of K; its waves split K in chunks of 32 * KS, every lane
-// streaming 16 bytes of a weight row per load (the four lane groups of a row read 64
-// contiguous bytes); the batch is the other MFMA operand (16 rows a tile, MT tiles);
-// partial sums of the waves meet in LDS, then the epilogue runs once.
+// 16 * NT weight rows and all of K and its waves split K; the batch is the other MFMA
+// operand (16 rows a tile, MT tiles); partial sums of the waves meet in LDS, then the
+// epilogue runs once.  Two ways from memory to the matrix cores: with K a multiple of 64
+// and one batch tile, through LDS by DMA in whole 128-byte lines (see DMA_S below); else
+// straight into registers, chunks of 32 * KS, every lane 16 bytes of a weight row per load
+// (the four lane groups of a row read 64 contiguous bytes).
 //
 // Chaining norms through the GEMMs of a decode step: a producer with the residual-add
 // epilogue can also emit, for the NEXT RMSNorm, the activations bfloat16(x * w_norm) and
@@ -75,8 +77,8 @@ struct ChainArgs {
 // DMA_S > 0 (one batch tile, K a multiple of 64): the operands go from global memory straight into
 // LDS (global_load_lds_dwordx4), every wave into a ring of DMA_S stages of its own, 64 k a stage, and
 // from there to the matrix cores.  A CU can only send so many requests a clock to the second-level
-// cache (measured: about 33 GB/s a CU with the 64-byte row pieces that the register path's lanes ask
-// for, 62 GB/s with whole 128-byte lines), and the activations' loads, though they hit that cache,
+// cache (measured from memory: about 37 GB/s a CU with the 64-byte row pieces that the register path's
+// lanes ask for, 90 GB/s with whole 128-byte lines), and the activations' loads, though they hit that cache,
 // come out of the same budget.  Here every request is a whole line: 8 lanes read the 128 bytes of
 // one row, 8 rows an instruction; the 16-byte chunks of a row are XOR-swizzled by the row number in
 // the global address each lane asks for, so that the fragment reads of 8 rows fall on different
