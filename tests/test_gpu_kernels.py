@@ -115,6 +115,52 @@ def test_gemm_store_and_add(M, N, Kd, dtype, simple):
         k.FORCE_SIMPLE = False
 
 
+def _random_gemm_shapes(n, seed):
+    """Row counts on both sides of every kernel's limits (16, 64, 128, 256), widths from tiny to several
+    workgroups' worth, K with and without the factors (8, 64) that choose the path."""
+    rng = np.random.default_rng(seed)
+    rows = [1, 2, 7, 8, 9, 15, 16, 17, 31, 32, 33, 48, 63, 64, 65, 100, 127, 128, 129, 200, 255, 256, 257, 300]
+    shapes = []
+    for _ in range(n):
+        M = int(rng.choice(rows))
+        N = int(rng.choice([1, 15, 16, 17, 100, 255, 256, 300, 1000, 2050, 4096, 6200]))
+        K = int(rng.choice([8, 24, 64, 72, 128, 192, 200, 320, 1024, 1032]))
+        shapes.append((M, N, K))
+    return shapes
+
+
+@pytest.mark.parametrize("with_workspace", [False, True])
+def test_gemm_random_shapes(with_workspace):
+    """Every dispatch branch of the bfloat16 GEMM at shapes nobody tuned for, all epilogues."""
+    from yalm_amd.parts.swiglu import interleave_gate_up
+    k = K()
+    for idx, (M, N, Kd) in enumerate(_random_gemm_shapes(40, 7 if with_workspace else 8)):
+        a = rnd((M, Kd), 1000 + idx, torch.bfloat16)
+        w = rnd((N, Kd), 2000 + idx, torch.bfloat16, scale=1 / math.sqrt(Kd))
+        want = a.double() @ w.double().T
+        ad, wd = a.to(DEV), w.to(DEV)
+        ws = None
+        if with_workspace:
+            n = k.gemm_workspace_floats(M, max(N, 32 * ((N + 15) // 16)), Kd)
+            ws = torch.full((n,), float("nan"), device=DEV) if n else None
+        tag = "M %d N %d K %d" % (M, N, Kd)
+        out = torch.empty((M, N), device=DEV)
+        k.gemm(ad, wd, out, k.EPI_STORE_F32, workspace=ws)
+        close(out, want, torch.float32, tag + " f32")
+        out2 = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+        k.gemm(ad, wd, out2, k.EPI_STORE, workspace=ws)
+        close(out2, want, torch.bfloat16, tag + " bf16")
+        res = rnd((M, N), 3000 + idx)
+        acc = res.to(DEV).clone()
+        k.gemm(ad, wd, acc, k.EPI_ADD_F32, workspace=ws)
+        close(acc, want + res.double(), torch.float32, tag + " add")
+        wu = rnd((N, Kd), 4000 + idx, torch.bfloat16, scale=1 / math.sqrt(Kd))
+        gated = R.silu(want) * (a.double() @ wu.double().T)
+        outg = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+        k.gemm(ad, interleave_gate_up(w, wu).to(DEV), outg, k.EPI_GATED, hidden=N, workspace=ws)
+        close(outg, gated, torch.bfloat16, tag + " gated", factor=2.0)
+
+
 @pytest.mark.parametrize("simple", [False, True])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("M,H,D", [(1, 16, 64), (5, 176, 64), (70, 100, 96), (64, 1000, 264), (3, 14336, 128),
