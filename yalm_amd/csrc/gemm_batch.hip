@@ -190,8 +190,9 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_batch_dma_kernel(const bf16* _
                                                                         int always_partial) {
   constexpr int KD = 64;
   constexpr int WSTAGE = NTW * 2048;             // a wave's weight rows of a stage
-  constexpr int XSTAGE = 8 * 1024;               // 64 rows of the activations, 8 an instruction
-  constexpr int XI = 8 / NW;                     // of which every wave issues this many
+  constexpr int XG = MT <= 4 ? 8 : 16;           // DMA instructions for the activations: 8 rows each, 64 or 128 rows
+  constexpr int XSTAGE = XG * 1024;
+  constexpr int XI = XG / NW;                    // of which every wave issues this many
   constexpr int L = 2 * NTW + XI;                // DMA instructions a wave and stage
   static_assert(S >= 3 && S <= 4, "3 or 4 stages");
   extern __shared__ __attribute__((aligned(1024))) unsigned char ring[];   // [NW][S][WSTAGE], then [S][XSTAGE]
@@ -293,13 +294,16 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_batch_dma_kernel(const bf16* _
   }
 }
 
-// launches one of the two kernels: the DMA one (NW waves) where K and the slices are multiples of 64
+// launches one of the two kernels: the DMA one (NW waves; up to 128 rows) where K and the slices are
+// multiples of 64, else the register one (8 waves; up to 64 rows)
 template <int MT, int NTW, int EPI, int NW>
 int launch_kernel(dim3 grid, const bf16* X, const bf16* W, void* C, float* ws, int M, int N, int K, int H,
                   int k_per_slice, int always_partial, hipStream_t stream) {
   if (K % 64 == 0 && k_per_slice % 64 == 0) {
-    constexpr int S = (NW * NTW <= 8) ? 4 : 3;
-    constexpr size_t lds = (size_t)NW * S * NTW * 2048 + (size_t)S * 8 * 1024;
+    constexpr int XG = MT <= 4 ? 8 : 16;
+    constexpr int S = (NW * NTW <= 8 && XG == 8) || (NW * NTW <= 4) ? 4 : 3;
+    constexpr size_t lds = (size_t)NW * S * NTW * 2048 + (size_t)S * XG * 1024;
+    static_assert(lds <= 128 * 1024, "the rings fit the LDS of a CU");
     auto kernel = &gemm_batch_dma_kernel<MT, NTW, EPI, S, NW>;
     static bool allowed = false;                   // more than 64 KB of LDS has to be asked for once
     if (!allowed) {
@@ -308,12 +312,14 @@ int launch_kernel(dim3 grid, const bf16* X, const bf16* W, void* C, float* ws, i
       allowed = true;
     }
     kernel<<<grid, NW * WAVE, lds, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice, always_partial);
-  } else {
-    if (NW != NWAVES) return YALM_ERR_ARG;
+    return launch_status();
+  }
+  if constexpr (MT <= 4 && NW == NWAVES) {
     gemm_batch_kernel<MT, NTW, EPI><<<grid, NWAVES * WAVE, 0, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice,
                                                                         always_partial);
+    return launch_status();
   }
-  return launch_status();
+  return YALM_ERR_ARG;
 }
 
 // adds the K slices in order and applies the epilogue; a thread per (row, 4 columns)
@@ -393,7 +399,8 @@ int launch_mt(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, 
   // waves a workgroup of the DMA kernel (they share the activations' stage): measured at batch 64
   // 8 waves 8120, 4 waves 8580, 2 waves 8410 tokens a second; at batch 32 5490, 5740 and 5870
   if (K % 64 == 0) return launch_nw<MT, EPI, (MT <= 2 ? 2 : 4)>(X, W, C, ws, ws_floats, M, N, K, H, stream);
-  return launch_nw<MT, EPI, 8>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+  if constexpr (MT > 4) return YALM_ERR_ARG;
+  else return launch_nw<MT, EPI, 8>(X, W, C, ws, ws_floats, M, N, K, H, stream);
 }
 
 // The residual add that also does the NEXT RMSNorm: a workgroup per row adds the K slices to
@@ -480,7 +487,8 @@ int launch_add_norm(const bf16* X, const bf16* W, float* C, float* ws, long ws_f
                     const float* norm_w, float eps, bf16* h, hipStream_t stream) {
   if (K % 64 == 0 && MT > 2)
     return launch_add_norm_nw<MT, 4>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream);
-  return launch_add_norm_nw<MT, NWAVES>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream);
+  if constexpr (MT > 4) return YALM_ERR_ARG;
+  else return launch_add_norm_nw<MT, NWAVES>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream);
 }
 
 // the K slices only: [slices][M][N] in ws, for a consumer that adds them
@@ -506,7 +514,8 @@ int launch_partial(const bf16* X, const bf16* W, float* ws, long ws_floats, int 
                    hipStream_t stream) {
   if (K % 64 == 0)
     return launch_partial_nw<MT, (MT <= 2 ? 2 : 4)>(X, W, ws, ws_floats, M, N, K, slices_out, stream);
-  return launch_partial_nw<MT, NWAVES>(X, W, ws, ws_floats, M, N, K, slices_out, stream);
+  if constexpr (MT > 4) return YALM_ERR_ARG;
+  else return launch_partial_nw<MT, NWAVES>(X, W, ws, ws_floats, M, N, K, slices_out, stream);
 }
 
 template <int EPI>
@@ -516,16 +525,21 @@ int dispatch(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, i
     case 2: return launch_mt<2, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
     case 3: return launch_mt<3, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
     case 4: return launch_mt<4, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+    case 5: return launch_mt<5, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+    case 6: return launch_mt<6, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+    case 7: return launch_mt<7, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+    case 8: return launch_mt<8, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
   }
   return YALM_ERR_ARG;
 }
 }  // namespace
 
-// 17..64 rows; workspace: float32 scratch for the K slices (may be null: one slice then).
-// Refuses (YALM_ERR_ARG) what it does not take.
+// 17..64 rows, and up to 128 with K a multiple of 64; workspace: float32 scratch for the K slices (may be
+// null: one slice then).  Refuses (YALM_ERR_ARG) what it does not take.
 int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
                          int K, int epilogue, int H, hipStream_t stream) {
-  if (M <= 16 || M > 64 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
+  if (M <= 16 || M > (K % 64 == 0 ? 128 : 64) || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15))
+    return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   switch (epilogue) {
@@ -539,7 +553,8 @@ int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace
 
 extern "C" int yalm_gemm_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N,
                                  int K, int* slices, hipStream_t stream) {
-  if (M > 64) return yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, slices, stream);
+  if (M > 128 || (M > 64 && K % 64 != 0))
+    return yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, slices, stream);
   if (M <= 16 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || slices == nullptr)
     return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
@@ -548,6 +563,10 @@ extern "C" int yalm_gemm_partial(const void* A, const void* W, float* workspace,
     case 2: return launch_partial<2>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
     case 3: return launch_partial<3>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
     case 4: return launch_partial<4>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
+    case 5: return launch_partial<5>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
+    case 6: return launch_partial<6>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
+    case 7: return launch_partial<7>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
+    case 8: return launch_partial<8>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
   }
   return YALM_ERR_ARG;
 }
@@ -558,7 +577,7 @@ extern "C" int yalm_gemm_add_norm(const void* A, const void* W, float* C, float*
                                   int M, int N, int K, const float* norm_w, float eps, void* h_out,
                                   hipStream_t stream) {
   if (norm_w == nullptr || h_out == nullptr) return YALM_ERR_ARG;
-  if (M > 64) {                                    // the tiled kernel's slices, then the same reduction
+  if (M > 128 || (M > 64 && K % 64 != 0)) {        // the tiled kernel's slices, then the same reduction
     int slices = 0;
     int rc = yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, &slices, stream);
     if (rc != YALM_OK) return rc;
@@ -572,6 +591,10 @@ extern "C" int yalm_gemm_add_norm(const void* A, const void* W, float* C, float*
     case 2: return launch_add_norm<2>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
     case 3: return launch_add_norm<3>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
     case 4: return launch_add_norm<4>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
+    case 5: return launch_add_norm<5>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
+    case 6: return launch_add_norm<6>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
+    case 7: return launch_add_norm<7>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
+    case 8: return launch_add_norm<8>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
   }
   return YALM_ERR_ARG;
 }

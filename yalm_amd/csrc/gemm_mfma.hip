@@ -198,7 +198,7 @@ int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, float* workspace,
   if (K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
-  if (M > 16 && M <= 64) {
+  if (M > 16 && M <= 128) {                        // (more than 64 rows: only with K a multiple of 64)
     int rc = yalm_gemm_bf16_batch(A, W, C, workspace, workspace_floats, M, N, K, epilogue, H, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }

@@ -84,7 +84,7 @@ GEMM_SPLIT_MAX = 16          # most K slices a GEMM uses, given the workspace
 def gemm_workspace_floats(M, N, K):
     """Floats of scratch with which a bfloat16 gemm splits K across workgroups: 17..64 rows, and
     more rows than that while the output's tiles alone would leave most of the chip idle."""
-    if 16 < M <= 64:
+    if 16 < M <= 64 or (M <= 128 and K % 64 == 0):
         return GEMM_SPLIT_MAX * M * N
     if M > 64:
         return int(library.lib().yalm_gemm_bf16_dma_workspace(M, N, K))
