@@ -60,6 +60,7 @@ class Engine:
         model.prepare(n_positions)
         self.ws = Workspace(self.device)
         self.use_graphs = use_graphs
+        self._graph_safe = model.graph_safe()          # the parts are fixed from here on: asked once, not every step
         self._graphs = {}
         self._meta_host = None
 
@@ -110,11 +111,17 @@ class Engine:
                 raise StepError("slot %r is not held by a live sequence" % (s,))
             starts.append(self.cache.seq_len[s])
         V = self.model.vocab_size
-        for t in tokens:
-            ids = np.asarray(t, dtype=np.int64)
-            if ids.ndim != 1 or ids.min() < 0 or ids.max() >= V:
-                bad = [tok for tok in t if not 0 <= tok < V]
-                raise StepError("token id %r is outside the vocabulary of %d" % (bad[0] if bad else t, V))
+        if max(n_tok) == 1:                               # a decode step: one comparison pair for the batch
+            firsts = [t[0] for t in tokens]
+            if not (0 <= min(firsts) and max(firsts) < V):
+                bad = [tok for tok in firsts if not 0 <= tok < V]
+                raise StepError("token id %r is outside the vocabulary of %d" % (bad[0] if bad else firsts, V))
+        else:
+            for t in tokens:
+                ids = np.asarray(t, dtype=np.int64)
+                if ids.ndim != 1 or ids.min() < 0 or ids.max() >= V:
+                    bad = [tok for tok in t if not 0 <= tok < V]
+                    raise StepError("token id %r is outside the vocabulary of %d" % (bad[0] if bad else t, V))
         if want is None:
             want = [[n - 1] for n in n_tok]
         for w, n in zip(want, n_tok):
@@ -179,7 +186,7 @@ class Engine:
 
     def _decode(self, slots, tokens, want, starts, new_lens):
         B = len(slots)
-        use_graph = self.use_graphs and self.model.graph_safe()
+        use_graph = self.use_graphs and self._graph_safe
         Bk = self._bucket(B) if use_graph else B
         # launch shapes may depend on the longest sequence only through this bucket (a power of
         # two of pages), so that a captured graph stays valid until a sequence outgrows it
