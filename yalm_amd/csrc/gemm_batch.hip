@@ -1,13 +1,15 @@
-// Decode GEMM for 17..64 rows, bfloat16: C = epilogue(X[M,K] * W[N,K]^T).
+// Decode GEMM for 17..64 rows (to 128 with K a multiple of 64), bfloat16: C = epilogue(X[M,K] * W[N,K]^T).
 //
 // With more than 16 rows the activations outweigh a workgroup's share of the weights,
-// so reading them once per 16 weight rows (as gemm_skinny does) makes L1, not HBM, the
-// limit.  Here K is split across workgroups and N across the 8 waves of a workgroup:
-// every wave owns 16 (32 for the gated epilogue) weight rows, the workgroup's chunk
-// of the activations [M x 128] goes through LDS once and all waves read it from there,
-// the weights go straight to registers, prefetched one chunk ahead.  Each K slice writes
-// its float32 partial product; a second kernel adds the slices in a fixed order and
-// applies the epilogue (one slice: the first kernel applies it itself).
+// so reading them once per 16 weight rows (as gemm_skinny does) makes the first-level cache,
+// not HBM, the limit.  Here K is split across workgroups and N across the waves of a
+// workgroup: every wave owns 16 (32 for the gated epilogue) weight rows, and the workgroup's
+// chunk of the activations goes through LDS once and all waves read it from there.  Two
+// kernels: with K a multiple of 64 both operands are staged in LDS by DMA (2 or 4 waves, see
+// gemm_batch_dma_kernel); else the activations go through registers into LDS and the weights
+// straight to registers, prefetched one chunk ahead (8 waves).  Each K slice writes its
+// float32 partial product; a second kernel adds the slices in a fixed order and applies the
+// epilogue (one slice: the first kernel applies it itself).
 #include "common.h"
 #include "yalm_hip.h"
 
@@ -571,7 +573,7 @@ extern "C" int yalm_gemm_partial(const void* A, const void* W, float* workspace,
   return YALM_ERR_ARG;
 }
 
-// C (float32 residual stream) += A * W^T for 17..64 rows, and h = RMSNorm(C_new) * norm_w in bfloat16
+// C (float32 residual stream) += A * W^T for more than 16 rows, and h = RMSNorm(C_new) * norm_w in bfloat16
 // for the next consumer.  Needs scratch for at least M * N floats; refuses (YALM_ERR_ARG) other shapes.
 extern "C" int yalm_gemm_add_norm(const void* A, const void* W, float* C, float* workspace, long workspace_floats,
                                   int M, int N, int K, const float* norm_w, float eps, void* h_out,

@@ -82,7 +82,7 @@ GEMM_SPLIT_MAX = 16          # most K slices a GEMM uses, given the workspace
 
 
 def gemm_workspace_floats(M, N, K):
-    """Floats of scratch with which a bfloat16 gemm splits K across workgroups: 17..64 rows, and
+    """Floats of scratch with which a bfloat16 gemm splits K across workgroups: 17..64 rows (to 128 with K a multiple of 64), and
     more rows than that while the output's tiles alone would leave most of the chip idle."""
     if 16 < M <= 64 or (M <= 128 and K % 64 == 0):
         return GEMM_SPLIT_MAX * M * N
@@ -206,8 +206,8 @@ def fused_workspace_floats(M, N, K):
 
 
 def gemm_add_norm(a, w, x, norm_w, eps, h_out, workspace):
-    """x float32 [M, N] += a[M, K] @ w[N, K]^T for 17..64 bfloat16 rows, and h_out bfloat16 [M, N] =
-    RMSNorm(x_new) with the weights norm_w (float32 [N]): the residual add and the next norm in one.
+    """x float32 [M, N] += a[M, K] @ w[N, K]^T for more than 16 bfloat16 rows (more than 64: K a multiple
+    of 64), and h_out bfloat16 [M, N] = RMSNorm(x_new) with the weights norm_w (float32 [N]): the residual add and the next norm in one.
     workspace: float32 scratch of gemm_workspace_floats(M, N, K) elements."""
     M, K = a.shape
     N = w.shape[0]
@@ -230,7 +230,8 @@ def can_gemm_partial(M, K, dtype):
 
 
 def gemm_partial(a, w, workspace):
-    """The K slices of a[M,K] @ w[N,K]^T, 17..64 rows of bfloat16, left unadded in `workspace`
+    """The K slices of a[M,K] @ w[N,K]^T, more than 16 rows of bfloat16 (more than 64: K a multiple of
+    64), left unadded in `workspace`
     ([slices][M][N] float32, flat; gemm_workspace_floats(M, N, K) elements let it split as it likes).
     Returns the number of slices, for a consumer that adds them (rope_kv_write)."""
     M, K = a.shape

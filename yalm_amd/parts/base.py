@@ -18,7 +18,7 @@ product: fuses_norm(norm, x, ctx) says so for a step, and forward_prenorm(x, nor
 ..., emit_for=next_norm) then replaces norm.forward + forward.  With emit_for it may
 also leave, in ctx.normed[id(next_norm)], either (xn, ss, eps): the activations already
 multiplied by that norm's weights and the partial sums of squares (its residual-add GEMM
-writes them; up to 16 rows), or (h, None, None): the norm's finished output (17..64 rows),
+writes them; up to 16 rows), or (h, None, None): the norm's finished output (more than 16 rows),
 which the next consumer takes instead of reading the residual stream.
 
 All of them: param_specs() -> [ParamSpec], load(get, compute_dtype, device),
