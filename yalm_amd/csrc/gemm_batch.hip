@@ -192,7 +192,9 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_batch_dma_kernel(const bf16* _
                                                                         int always_partial) {
   constexpr int KD = 64;
   constexpr int WSTAGE = NTW * 2048;             // a wave's weight rows of a stage
-  constexpr int XG = MT <= 4 ? 8 : 16;           // DMA instructions for the activations: 8 rows each, 64 or 128 rows
+  constexpr int XG0 = MT <= 2 ? 4 : (MT <= 4 ? 8 : 16);  // DMA instructions for the activations: 8 rows each, 32, 64 or
+  constexpr int XG = XG0 < NW ? NW : XG0;        // 128 rows (and at least one instruction a wave)
+  static_assert(XG % NW == 0, "the activations' instructions divide over the waves");
   constexpr int XSTAGE = XG * 1024;
   constexpr int XI = XG / NW;                    // of which every wave issues this many
   constexpr int L = 2 * NTW + XI;                // DMA instructions a wave and stage
@@ -302,8 +304,9 @@ template <int MT, int NTW, int EPI, int NW>
 int launch_kernel(dim3 grid, const bf16* X, const bf16* W, void* C, float* ws, int M, int N, int K, int H,
                   int k_per_slice, int always_partial, hipStream_t stream) {
   if (K % 64 == 0 && k_per_slice % 64 == 0) {
-    constexpr int XG = MT <= 4 ? 8 : 16;
-    constexpr int S = (NW * NTW <= 8 && XG == 8) || (NW * NTW <= 4) ? 4 : 3;
+    constexpr int XG0 = MT <= 2 ? 4 : (MT <= 4 ? 8 : 16);
+    constexpr int XG = XG0 < NW ? NW : XG0;
+    constexpr int S = (NW * NTW <= 8 && XG <= 8) || (NW * NTW <= 4) ? 4 : 3;
     constexpr size_t lds = (size_t)NW * S * NTW * 2048 + (size_t)S * XG * 1024;
     static_assert(lds <= 128 * 1024, "the rings fit the LDS of a CU");
     auto kernel = &gemm_batch_dma_kernel<MT, NTW, EPI, S, NW>;
