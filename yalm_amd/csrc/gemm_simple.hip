@@ -1,8 +1,8 @@
 // C = A[M,K] * W[N,K]^T, float32 arithmetic for every storage type: the kernels of the
 // true 32-bit path and the fallback of the bfloat16 path for shapes the MFMA kernels
 // refuse.  gemm_simple: 64x64 tile, 16-deep k steps through LDS, 256 threads with a 4x4
-// register tile each; any M, N, K.  gemm_rows_f32: at most 16 rows of float32, one pass
-// over the weights (below).
+// register tile each; any M, N, K.  gemm_rows_f32: at most 64 rows of float32, a pass over
+// the weights for every 16 of them (below).
 #include "common.h"
 #include "yalm_hip.h"
 
@@ -199,14 +199,23 @@ int launch_rows_f32(const float* A, const float* W, void* C, int M, int N, int K
   return launch_status();
 }
 
-// float32, at most 16 rows, K a multiple of 4 and 16-byte aligned operands; YALM_ERR_ARG: not taken
+// float32, at most 64 rows (16 a pass over the weights: up to four passes still beat the tiles, which
+// are mostly padding then), K a multiple of 4 and 16-byte aligned operands; YALM_ERR_ARG: not taken
 int gemm_rows_f32(const void* A, const void* W, void* C, int M, int N, int K, int epilogue, int H, hipStream_t stream) {
-  if (M > 16 || K % 4 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
-  const float* a = (const float*)A;
+  if (M > 64 || K % 4 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
   const float* w = (const float*)W;
-  if (M <= 4) return launch_rows_f32<4>(a, w, C, M, N, K, epilogue, H, stream);
-  if (M <= 8) return launch_rows_f32<8>(a, w, C, M, N, K, epilogue, H, stream);
-  return launch_rows_f32<16>(a, w, C, M, N, K, epilogue, H, stream);
+  const int out_cols = epilogue == 3 ? H : N;
+  for (int m0 = 0; m0 < M; m0 += 16) {
+    const float* a = (const float*)A + (size_t)m0 * K;
+    float* c = (float*)C + (size_t)m0 * out_cols;
+    const int rows = min(16, M - m0);
+    int rc;
+    if (rows <= 4) rc = launch_rows_f32<4>(a, w, c, rows, N, K, epilogue, H, stream);
+    else if (rows <= 8) rc = launch_rows_f32<8>(a, w, c, rows, N, K, epilogue, H, stream);
+    else rc = launch_rows_f32<16>(a, w, c, rows, N, K, epilogue, H, stream);
+    if (rc != YALM_OK) return rc;
+  }
+  return YALM_OK;
 }
 
 template <typename T>
