@@ -484,3 +484,28 @@ def test_command_line_options_have_the_references_meanings():
         with pytest.raises(SystemExit) as e:
             parse_args(bad)
         assert e.value.code == 1
+
+
+def test_prefill_tile_order_names_every_second_tile_once_the_longest_first():
+    from yalm_amd.ops import kernels
+    PAGE = kernels.PAGE
+
+    def check(lens):
+        order = kernels.prefill_tile_order(lens)
+        assert order.dtype == np.int32
+        tiles = [(n + PAGE - 1) // PAGE for n in lens]
+        first = np.concatenate([[0], np.cumsum(tiles)])
+        want = sorted(int(first[b]) + t for b, n in enumerate(tiles) for t in range(0, n, 2))
+        assert sorted(order.tolist()) == want
+        seqs = [int(np.searchsorted(first, g, side="right")) - 1 for g in order.tolist()]
+        work = [min(g - int(first[b]) + 2, tiles[b]) for g, b in zip(order.tolist(), seqs)]
+        return seqs, work, tiles
+
+    seqs, work, tiles = check([130, 1, 64, 700, 65])              # short: by the keys a tile sees
+    assert work == sorted(work, reverse=True)
+    seqs, work, tiles = check([130, 1, 3000, 64, 2500, 65])        # long: sequence by sequence
+    runs = [b for i, b in enumerate(seqs) if i == 0 or seqs[i - 1] != b]
+    assert len(runs) == len(set(runs)) and [tiles[b] for b in runs] == sorted(tiles, reverse=True)
+    for b in runs:
+        w = [x for x, s in zip(work, seqs) if s == b]
+        assert w == sorted(w, reverse=True)

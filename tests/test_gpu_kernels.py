@@ -405,6 +405,32 @@ def test_attn_prefill(n_heads, n_kv, hd, window, lens, dtype, simple):
     close(out, packed_attention_reference(q, kk, v, lens, n_heads, n_kv, hd, window), dtype, "prefill attention")
 
 
+@pytest.mark.parametrize("n_heads,n_kv,hd,window,lens", [
+    (8, 2, 128, 0, [200]), (5, 5, 64, 0, [129, 1, 640]), (4, 1, 64, 70, [300, 64, 1]), (40, 8, 128, 0, [700]),
+    (24, 8, 64, 100, [1100, 90]), (8, 2, 128, 0, [2200, 90, 2100])])
+def test_attn_prefill_in_a_given_tile_order(n_heads, n_kv, hd, window, lens):
+    """The order of the tiles (with more workgroups than compute units it is folded) changes no
+    bit of the result, and every position is still written."""
+    k = K()
+    dtype = torch.bfloat16
+    T = sum(lens)
+    q = rnd((T, n_heads * hd), 23, dtype).to(DEV)
+    kk = rnd((T, n_kv * hd), 24, dtype)
+    v = rnd((T, n_kv * hd), 25, dtype)
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    seq = np.repeat(np.arange(len(lens)), lens)
+    pos = np.concatenate([np.arange(n) for n in lens])
+    ks, vs, tile0 = stage(kk, v, lens, n_kv, hd, dtype, poison=False)
+    ks, vs = ks.to(DEV), vs.to(DEV)
+    outs = []
+    for order in (None, i32(k.prefill_tile_order(lens))):
+        out = torch.full((T, n_heads * hd), float("nan"), dtype=dtype, device=DEV)
+        k.attn_prefill(q, ks, vs, out, i32(cu), i32(tile0), i32(seq), i32(pos), n_heads, n_kv, hd, window, order)
+        outs.append(out.cpu())
+    assert not torch.isnan(outs[1].float()).any()
+    assert torch.equal(outs[0], outs[1])
+
+
 def paged_case(lens, n_kv, hd, window, dtype, seed, poison=True):
     """Random keys/values of sequences of the given lengths laid out in pages the way
     the cache does (ring for a window), the rest of the pool poisoned with NaN."""

@@ -225,13 +225,16 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 // measured no faster at 2,048 tokens and slower beyond) the workgroup of every second tile of
 // a sequence works.  The heads of a tile are neighbours in the launch order, so that the
 // workgroups running together cost the same and the heads of a group share their keys in the
-// cache; a prompt's last tiles, which see the most keys, start first.
+// cache; the tiles that see the most keys start first.  With tile_order (the working tiles,
+// those that see the most keys first) only these are launched, and from workgroup fold_at on
+// the order is turned round: when every compute unit gets two workgroups, the second of the
+// one that began with the longest is the shortest.
 // ---------------------------------------------------------------------------
 template <int HD, int NC>
 __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_stage, const bf16* __restrict__ v_stage,
-    bf16* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_tile0, int B, int n_heads,
-    int n_kv_heads, int window) {
+    bf16* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_tile0,
+    const int* __restrict__ tile_order, int fold_at, int B, int n_heads, int n_kv_heads, int window) {
   constexpr int KS = HD / 32, DT = HD / 16;
   constexpr int KROW = HD + 8;                    // LDS row strides (elements): 16 bytes of padding
   constexpr int VROW = PAGE + 8;
@@ -242,7 +245,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
 
   // heads run fastest and tiles from the last to the first: within a sequence the last tiles see
   // the most keys, and workgroups that start first should be the long ones
-  const int h = blockIdx.x, gt = (int)gridDim.y - 1 - (int)blockIdx.y;
+  int h = blockIdx.x, gt = (int)gridDim.y - 1 - (int)blockIdx.y;
+  if (tile_order) {
+    int lin = (int)blockIdx.y * n_heads + h;
+    const int total = (int)gridDim.y * n_heads;
+    if (lin >= fold_at) lin = total - 1 - (lin - fold_at);
+    h = lin % n_heads;
+    gt = tile_order[lin / n_heads];
+    if ((unsigned)gt >= (unsigned)seq_tile0[B]) return;
+  }
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE, qd = lane / 16, j = lane % 16;
   int b = 0;
   {
@@ -431,24 +442,44 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_mfma_kernel(
   }
 }
 
+// compute units of the current device (asked once: this library drives one device a process)
+int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0)
+      v = 256;
+    n = v;
+  }
+  return n;
+}
+
 bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
   return (head_dim == 64 || head_dim == 128) && n_kv_heads > 0 && n_heads % n_kv_heads == 0;
 }
 }  // namespace
 
 int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out,
-                                const int* cu_seqlens, const int* seq_tile0, int T, int B, int n_tiles, int n_heads,
-                                int n_kv_heads, int head_dim, int window, hipStream_t stream) {
+                                const int* cu_seqlens, const int* seq_tile0, const int* tile_order, int n_order,
+                                int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
+                                hipStream_t stream) {
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_tiles > 65535) return YALM_ERR_ARG;
-  dim3 grid(n_heads, n_tiles);
+  if (tile_order && (n_order <= 0 || n_order > n_tiles)) return YALM_ERR_ARG;
+  dim3 grid(n_heads, tile_order ? n_order : n_tiles);
+  // two workgroups fit a compute unit: with more than one and at most two each, the second
+  // half of the launch runs from the shortest workgroup up
+  const long total = (long)grid.x * grid.y;
+  const int cus = compute_units();
+  const int fold_at = total > cus && total <= 2 * cus ? cus : (int)total;
   const size_t lds = 2 * ((size_t)PAGE * (head_dim + 8) + (size_t)head_dim * (PAGE + 8)) * sizeof(bf16);
   const bf16 *qp = (const bf16*)q, *kp = (const bf16*)k_stage, *vp = (const bf16*)v_stage;
   if (head_dim == 128)
-    attn_prefill_mfma_kernel<128, 2><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, cu_seqlens, seq_tile0, B,
-                                                                n_heads, n_kv_heads, window);
+    attn_prefill_mfma_kernel<128, 2><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, cu_seqlens, seq_tile0, tile_order,
+                                                                fold_at, B, n_heads, n_kv_heads, window);
   else
-    attn_prefill_mfma_kernel<64, 2><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, cu_seqlens, seq_tile0, B,
-                                                               n_heads, n_kv_heads, window);
+    attn_prefill_mfma_kernel<64, 2><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, cu_seqlens, seq_tile0, tile_order,
+                                                               fold_at, B, n_heads, n_kv_heads, window);
   return launch_status();
 }
 

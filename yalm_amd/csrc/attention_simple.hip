@@ -7,8 +7,9 @@
 #include "yalm_hip.h"
 
 int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out,
-                                const int* cu_seqlens, const int* seq_tile0, int T, int B, int n_tiles, int n_heads,
-                                int n_kv_heads, int head_dim, int window, hipStream_t stream);
+                                const int* cu_seqlens, const int* seq_tile0, const int* tile_order, int n_order,
+                                int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
+                                hipStream_t stream);
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
@@ -246,8 +247,9 @@ bool bad_heads(int n_heads, int n_kv_heads, int hd) {
 
 extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void* v_stage, void* out,
                                  const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
-                                 int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
-                                 int dtype, int force_simple, hipStream_t stream) {
+                                 const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads,
+                                 int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
+                                 hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_tiles <= 0) return YALM_ERR_ARG;
   dim3 grid(T, n_heads);
@@ -260,8 +262,8 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
   }
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
   if (!force_simple) {
-    int rc = yalm_attn_prefill_bf16_mfma(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, T, B, n_tiles, n_heads,
-                                         n_kv_heads, head_dim, window, stream);
+    int rc = yalm_attn_prefill_bf16_mfma(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tile_order, n_order, T, B,
+                                         n_tiles, n_heads, n_kv_heads, head_dim, window, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   attn_prefill_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,

@@ -11,4 +11,4 @@ extern "C" const char* yalm_error_string(int code) {
   }
 }
 
-extern "C" int yalm_abi_version(void) { return 11; }
+extern "C" int yalm_abi_version(void) { return 12; }

@@ -115,11 +115,14 @@ int yalm_rope_kv_write_tiles(const float* qkv, void* q_out, void* k_stage, void*
 // start at position 0), packed without padding.  window 0 = all keys.
 //   q, out [T, n_heads, hd]; k_stage, v_stage: the staging area rope_kv_write filled
 //   (key j of sequence b: tile seq_tile0[b] + j / PAGE, row j % PAGE), all `dtype`
+//   tile_order (may be null): n_order tiles of the staging area, every second tile of each
+//   sequence from its first, those that see the most keys first; it changes the order of the
+//   work and no result
 // reference: attn_dot + attn_softmax + att_mix (src/infer.cu:339-523) for every position
 int yalm_attn_prefill(const void* q, const void* k_stage, const void* v_stage, void* out, const int* cu_seqlens,
-                      const int* seq_tile0, const int* tok_seq, const int* tok_pos, int T, int B, int n_tiles,
-                      int n_heads, int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
-                      hipStream_t stream);
+                      const int* seq_tile0, const int* tok_seq, const int* tok_pos, const int* tile_order, int n_order,
+                      int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window, int dtype,
+                      int force_simple, hipStream_t stream);
 
 // One query per sequence over the pages of the cache (the new key is already written).
 //   q, out [B, n_heads, hd]; seq_len[b] = keys of sequence b including the new one;

@@ -47,7 +47,8 @@ class StepContext:
     or 'decode' (one token per sequence).  Device tensors, all int32:
       tokens[T], tok_seq[T] (row of the batch), tok_pos[T] (position in its sequence),
       seq_slot[B] (-1: padding row), seq_len[B] (length after this step), cu_seqlens[B+1],
-      seq_tile0[B+1] (prefill: first 64-token tile of each sequence in the staging area; n_tiles in all).
+      seq_tile0[B+1] (prefill: first 64-token tile of each sequence in the staging area; n_tiles in all),
+      tile_order (prefill, may be None: the order in which attention should take the tiles).
     max_position: the largest position in the step (host value, for table checks).
     pages_bucket: decode only; an upper bound (a power of two) of the pages of the step's
     longest sequence, the only way launch shapes may depend on lengths."""
@@ -60,6 +61,7 @@ class StepContext:
         self.shared_lines = set(shared_lines)
         self.tokens = self.tok_seq = self.tok_pos = self.seq_slot = self.seq_len = self.cu_seqlens = None
         self.seq_tile0 = None
+        self.tile_order = None
         self.n_tiles = 0
         self.normed = {}                  # id(norm part) -> (xn, ss, eps): activations a producer emitted for it
         self.pages_bucket = 1 << 30       # decode: no sequence of the step has more pages than this

@@ -17,7 +17,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import PAGE, CacheError, CacheManager
-from ..ops import library
+from ..ops import kernels, library
 from .context import StepContext, Workspace
 
 DECODE_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024)
@@ -157,7 +157,8 @@ class Engine:
         R = len(rows)
         tile0 = np.zeros(B + 1, dtype=np.int32)
         np.cumsum([(n + PAGE - 1) // PAGE for n in n_tok], out=tile0[1:])
-        n_meta = 3 * T + 4 * B + 2 + R
+        order = kernels.prefill_tile_order(n_tok)
+        n_meta = 3 * T + 4 * B + 2 + R + len(order)
         host = np.empty(n_meta, dtype=np.int32)
         host[0:T] = np.concatenate([np.asarray(t, dtype=np.int32) for t in tokens])
         host[T:2 * T] = np.repeat(np.arange(B, dtype=np.int32), n_tok)
@@ -167,15 +168,17 @@ class Engine:
         host[o + B:o + 2 * B] = new_lens
         host[o + 2 * B:o + 3 * B + 1] = cu
         host[o + 3 * B + 1:o + 4 * B + 2] = tile0
-        host[o + 4 * B + 2:] = rows
+        host[o + 4 * B + 2:o + 4 * B + 2 + R] = rows
+        host[o + 4 * B + 2 + R:] = order
         meta = self.ws.get("meta", (n_meta,), torch.int32)
         meta.copy_(torch.from_numpy(host))
         ctx = self._context("prefill", self.ws, meta, T, B, max(n_tok) - 1)
         ctx.seq_tile0 = meta[o + 3 * B + 1:o + 4 * B + 2]
+        ctx.tile_order = meta[o + 4 * B + 2 + R:]
         ctx.n_tiles = int(tile0[-1])
         ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), list(n_tok), [0] * B
         logits = self.ws.get("logits", (R, self.model.vocab_size), torch.float32) if R else None
-        self.model.forward(ctx, meta[o + 4 * B + 2:] if R else None, logits)
+        self.model.forward(ctx, meta[o + 4 * B + 2:o + 4 * B + 2 + R] if R else None, logits)
         return logits if R else torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
 
     def _bucket(self, B):

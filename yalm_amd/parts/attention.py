@@ -184,7 +184,7 @@ class GQAttention(Part):
         o = ws.get("attn.o", (T, self.q_dim), act)
         if prefill:
             kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, ctx.seq_tile0, ctx.tok_seq, ctx.tok_pos,
-                                 self.n_heads, self.n_kv_heads, self.head_dim, self.window)
+                                 self.n_heads, self.n_kv_heads, self.head_dim, self.window, ctx.tile_order)
         else:
             self._decode_attention(q, o, ctx, group, k_pages, v_pages)
         self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)
