@@ -1,9 +1,11 @@
 #!/usr/bin/env python3
 """Measures the library on one MI355X: decode tokens/s at batch 8 (the value),
 at batch 1 and 64 (points), and the prefill of a 2,048-token prompt, for a
-Mistral-7B-shaped model with random weights and random token ids.
+Mistral-7B-shaped model with random weights and random token ids (--shape: the
+Llama-3.2-3B shape with prompts of 512 tokens at context 8,192, or the Mistral-7B-v0.1
+shape with its window of 4,096 positions and prompts of 6,000 tokens).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--dtype bf16|fp32]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--dtype bf16|fp32] [--shape NAME]
 
 A step is one decode step as generation does it: the step function for a batch
 of sequences (one token each, from the cache), greedy sampling on the device
@@ -25,8 +27,24 @@ MISTRAL_7B = {
     "vocab_size": 32000, "max_position_embeddings": 32768, "rope_theta": 1000000.0, "rms_norm_eps": 1e-5,
     "hidden_act": "silu", "tie_word_embeddings": False, "bos_token_id": 1, "eos_token_id": 2,
 }
-CONTEXT = 4096
-PROMPT = 2048
+# BASELINE.json configs[3]: Llama-3.2-3B shape (llama3 rope scaling, tied head, a vocabulary that is no power of two)
+LLAMA_3B = {
+    "architectures": ["LlamaForCausalLM"], "hidden_size": 3072, "intermediate_size": 8192,
+    "num_hidden_layers": 28, "num_attention_heads": 24, "num_key_value_heads": 8, "head_dim": 128,
+    "vocab_size": 128256, "max_position_embeddings": 131072, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "hidden_act": "silu", "tie_word_embeddings": True, "bos_token_id": 128000, "eos_token_id": 128001,
+}
+# BASELINE.json configs[4]: Mistral-7B-v0.1 shape (a window of 4,096 positions: ring cache)
+MISTRAL_7B_V01 = dict(MISTRAL_7B, rope_theta=10000.0, sliding_window=4096)
+# shape -> (config, name, context, prompt length of the decode runs)
+SHAPES = {
+    "mistral-7b-v0.2": (MISTRAL_7B, "Mistral-7B-v0.2 shape", 4096, 2048),
+    "llama-3.2-3b": (LLAMA_3B, "Llama-3.2-3B shape", 8192, 512),
+    "mistral-7b-v0.1": (MISTRAL_7B_V01, "Mistral-7B-v0.1 shape", 8192, 6000),
+}
+PREFILL = 2048                   # tokens of the timed prompt
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 BASELINE_TOK_S = 63.8            # the reference's published batch-1 figure (RTX 4090), README.md:14
@@ -52,6 +70,8 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--points", default="1,64", help="further batch sizes to measure")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--shape", default="mistral-7b-v0.2", choices=sorted(SHAPES),
+                    help="the layer sizes: BASELINE.json's configs[2] (default), [3] or [4]")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not measured" % args.gpus, flush=True)
@@ -62,16 +82,17 @@ def main():
     from yalm_amd.cache import PAGE
 
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
-    n_layers = args.layers or MISTRAL_7B["num_hidden_layers"]
+    CFG, shape_name, CONTEXT, PROMPT = SHAPES[args.shape]
+    n_layers = args.layers or CFG["num_hidden_layers"]
     dev = "cuda:0"
     t0 = time.time()
-    model = Model.random(MISTRAL_7B, seed=0, dtype=dtype, device=dev, n_layers=n_layers)
+    model = Model.random(CFG, seed=0, dtype=dtype, device=dev, n_layers=n_layers)
     torch.cuda.synchronize()
     sys.stderr.write("[bench] %d layers of random weights in %.1f s\n" % (n_layers, time.time() - t0))
     batches = sorted({args.batch} | {int(b) for b in args.points.split(",") if b})
     engine = Engine(model, max_tokens=max(batches) * CONTEXT, max_batch=max(batches))
     sampler = Sampler(0)
-    V = MISTRAL_7B["vocab_size"]
+    V = CFG["vocab_size"]
     gen = torch.Generator().manual_seed(1)
 
     def sync():
@@ -80,7 +101,7 @@ def main():
     # ---------------------------------------------------------------- prefill of one 2,048-token prompt
     prefill = None
     if not args.no_prefill:
-        prompt = torch.randint(0, V, (PROMPT,), generator=gen).tolist()
+        prompt = torch.randint(0, V, (PREFILL,), generator=gen).tolist()
         times = []
         for i in range(3):
             slots = engine.start(1)
@@ -92,8 +113,8 @@ def main():
             times.append(time.perf_counter() - t)
             engine.release(slots)
         sec = min(times[1:])
-        fl = prefill_flops(MISTRAL_7B, n_layers, PROMPT)
-        prefill = {"value": round(PROMPT / sec, 1), "tokens": PROMPT, "ms": round(sec * 1e3, 3),
+        fl = prefill_flops(CFG, n_layers, PREFILL)
+        prefill = {"value": round(PREFILL / sec, 1), "tokens": PREFILL, "ms": round(sec * 1e3, 3),
                    "frac": round(fl / sec / FLOP_PEAK[args.dtype], 4)}
         sys.stderr.write("[bench] prefill %s\n" % prefill)
 
@@ -121,7 +142,8 @@ def main():
         end_len = engine.length(slots[0])
         engine.release(slots)
         mean_ctx = (start_len + 1 + end_len) / 2.0
-        kv_bytes = sum(g.bytes_per_token() for g in engine.cache.kv_groups) * mean_ctx * B
+        kv_bytes = sum(g.bytes_per_token() * (min(mean_ctx, g.window) if g.window else mean_ctx)
+                       for g in engine.cache.kv_groups) * B          # a windowed group reads its window only
         step_bytes = model.weight_bytes() + (B - 1) * model.embedding.weight_bytes() + kv_bytes
         return {"tok_s": B * steps / sec, "ms": sec / steps * 1e3, "bytes": step_bytes, "ctx": mean_ctx}
 
@@ -135,16 +157,18 @@ def main():
     main_r = results[args.batch]
     achieved = main_r["bytes"] / (main_r["ms"] * 1e-3) / 1e9
     line = {
-        "metric": "decode tok/s @ batch %d, Mistral-7B shape, context %d" % (args.batch, CONTEXT),
+        "metric": "decode tok/s @ batch %d, %s, context %d" % (args.batch, shape_name.replace("-v0.2", ""), CONTEXT),
         "value": round(main_r["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(main_r["ms"], 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": round(results[1]["tok_s"] / BASELINE_TOK_S, 2) if 1 in results else None,
         "dtype": args.dtype, "data": "synthetic: seeded random weights and token ids",
         "config": {
-            "model": "Mistral-7B-v0.2 shape", "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
-            "layers": n_layers, "layers_of_config": MISTRAL_7B["num_hidden_layers"], "dim": 4096, "hidden_dim": 14336,
-            "n_heads": 32, "n_kv_heads": 8, "head_dim": 128, "vocab_size": 32000, "rope_theta": 1e6,
-            "norm_eps": 1e-5, "tied": False, "window": 0, "prompt_len": PROMPT,
+            "model": shape_name, "global_batch": args.batch, "seq_len": CONTEXT, "parallelism": "none",
+            "layers": n_layers, "layers_of_config": CFG["num_hidden_layers"], "dim": CFG["hidden_size"],
+            "hidden_dim": CFG["intermediate_size"], "n_heads": CFG["num_attention_heads"],
+            "n_kv_heads": CFG["num_key_value_heads"], "head_dim": CFG["head_dim"], "vocab_size": V,
+            "rope_theta": CFG["rope_theta"], "norm_eps": CFG["rms_norm_eps"], "tied": CFG["tie_word_embeddings"],
+            "window": CFG.get("sliding_window") or 0, "prompt_len": PROMPT,
             "decode_mean_context": round(main_r["ctx"], 1), "kv_dtype": args.dtype, "page_tokens": PAGE,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",

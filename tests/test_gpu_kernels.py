@@ -630,6 +630,43 @@ def test_argmax_and_sample():
     assert torch.allclose(prob.cpu().double(), torch.tensor(want, dtype=torch.float64), rtol=1e-4, atol=1e-9)
 
 
+@pytest.mark.parametrize("V", [4, 7, 255, 1029, 32003, 128256])
+def test_sampling_at_vocabularies_of_any_size(V):
+    """Rows that do not start on a 16-byte boundary (odd V), fewer entries than a wave's tile, and
+    vocabularies that give every wave several tiles: the first maximum, the walk of the running sum
+    and the probability of a token against the plain functions."""
+    k = K()
+    g = torch.Generator().manual_seed(41 + V)
+    n = 5
+    logits = torch.randn((n, V), generator=g) * 3
+    logits[0, 0] = logits[0, V - 1] = 40.0                   # ties at both ends: the first wins
+    logits[1, V - 1] = 41.0                                  # the last entry (the scalar tail)
+    logits[2, min(V - 1, 2)] = logits[2, V // 2] = 42.0
+    dl = logits.to(DEV)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    k.argmax(dl, out)
+    assert out.cpu().tolist() == [R.sample_argmax(l) for l in logits]
+    flat = torch.randn((n, V), generator=g)                  # flat rows: the walk ends deep inside the row
+    for rows, temp in ((logits, 1.0), (flat, 0.7), (flat, 3.0)):
+        d = rows.to(DEV)
+        for us in ([0.0, 0.999999, 0.5, 0.25, 0.9], [0.1, 0.33, 0.66, 0.75, 1.0]):
+            u = torch.tensor(us)
+            k.sample(d, u.to(DEV), temp, out)
+            got = out.cpu().tolist()
+            for r in range(n):
+                assert 0 <= got[r] < V
+                p = torch.softmax(rows[r].double() / temp, 0)
+                c = torch.cumsum(p, 0)
+                want = R.sample_temperature(rows[r], temp, float(u[r]))
+                lo = float(c[got[r]] - p[got[r]])
+                assert got[r] == want or (lo - 1e-5 <= float(u[r]) <= float(c[got[r]]) + 1e-5), (V, temp, r, got[r], want)
+    idx = [0, V - 1, V // 2, min(V - 1, 3), V // 3]
+    prob = torch.empty(n, device=DEV)
+    k.token_prob(dl, i32(idx), prob)
+    want = [R.sample_prob(logits[r], i) for r, i in enumerate(idx)]
+    assert torch.allclose(prob.cpu().double(), torch.tensor(want, dtype=torch.float64), rtol=1e-4, atol=1e-9)
+
+
 # ------------------------------------------------------------------ fused decode GEMMs
 
 @pytest.mark.parametrize("M,N,Kd", [(1, 64, 256), (8, 4096 + 32, 136), (7, 100, 96), (3, 17000, 64), (2, 4096, 4096), (8, 48, 4096)])
