@@ -194,12 +194,24 @@ FULL_WIDTH = {"architectures": ["MistralForCausalLM"], "hidden_size": 4096, "int
               "hidden_act": "silu", "tie_word_embeddings": False, "bos_token_id": 1, "eos_token_id": 2}
 
 
-def test_one_layer_at_the_width_of_the_big_models(tmp_path_factory):
-    """One layer with the sizes of Mistral-7B (a small vocabulary): the kernels take their big-shape paths
-    (256x256 and 128x128 GEMM tiles in the prompt step, 256 parts in the norm chain, split-K for 20 rows,
-    matrix-core attention with 4 heads a group), and the logits still follow the plain implementation."""
+# the widths of Llama-3.2-3B: 24 heads in groups of 3, outputs of 3,072 (192 workgroups of 16 rows), llama3
+# rope scaling, and the head shared with the embedding at a vocabulary that is no power of two
+WIDTH_3B = {"architectures": ["LlamaForCausalLM"], "hidden_size": 3072, "intermediate_size": 8192,
+            "num_hidden_layers": 1, "num_attention_heads": 24, "num_key_value_heads": 8, "head_dim": 128,
+            "vocab_size": 5003, "max_position_embeddings": 4096, "rope_theta": 500000.0, "rms_norm_eps": 1e-5,
+            "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                             "original_max_position_embeddings": 64},
+            "hidden_act": "silu", "tie_word_embeddings": True, "bos_token_id": 1, "eos_token_id": 2}
+
+
+@pytest.mark.parametrize("name,FULL_WIDTH", [("mistral_7b", FULL_WIDTH), ("llama_3b", WIDTH_3B)])
+def test_one_layer_at_the_width_of_the_big_models(tmp_path_factory, name, FULL_WIDTH):
+    """One layer with the sizes of Mistral-7B or Llama-3.2-3B (a small vocabulary): the kernels take their
+    big-shape paths (256x256 and 128x128 GEMM tiles in the prompt step, 256 parts in the norm chain, split-K
+    for 20 rows, matrix-core attention with 4 or 3 heads a group), and the logits still follow the plain
+    implementation."""
     from yalm_amd.engine import Engine, Model
-    folder = helpers.make_folder(tmp_path_factory.mktemp("wide"), "full_width", FULL_WIDTH, seed=1,
+    folder = helpers.make_folder(tmp_path_factory.mktemp("wide"), "full_width_" + name, FULL_WIDTH, seed=1,
                                  stored=torch.bfloat16)
     model = Model.from_folder(folder, dtype=torch.bfloat16, device="cuda:0")
     engine = Engine(model, max_tokens=4096)
