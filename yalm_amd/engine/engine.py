@@ -20,7 +20,7 @@ from ..cache.manager import PAGE, CacheError, CacheManager
 from ..ops import kernels, library
 from .context import StepContext, Workspace
 
-DECODE_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 1024)
+DECODE_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 96, 128, 192, 256, 512, 1024)
 
 
 class StepError(ValueError):

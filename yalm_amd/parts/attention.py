@@ -20,6 +20,7 @@ from .base import Part, build_part, part
 
 # decode attention is split over pages so that about this many workgroups run
 TARGET_WORKGROUPS = 256
+RESIDENT_WORKGROUPS = 512       # decode-attention workgroups that the chip holds at once (two a compute unit)
 
 
 @part("mixer", "gqa_attention")
@@ -68,6 +69,8 @@ class GQAttention(Part):
         mfma = self.head_dim in (64, 128) and self.n_heads // self.n_kv_heads <= 16 and not kernels.FORCE_SIMPLE
         if mfma:         # a workgroup of 4 waves per (split, KV head, sequence), a page per wave at a time
             per = max(1, B * self.n_kv_heads)
+            if per > RESIDENT_WORKGROUPS:         # more than run at once: in quarters the last round is short
+                return max(1, min((max_pages + 3) // 4, 4))
             return max(1, min((max_pages + 3) // 4, TARGET_WORKGROUPS // per))
         return max(1, min(max_pages, TARGET_WORKGROUPS // max(1, B * self.n_heads)))
 
