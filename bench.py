@@ -6,6 +6,7 @@ Llama-3.2-3B shape with prompts of 512 tokens at context 8,192, or the Mistral-7
 shape with its window of 4,096 positions and prompts of 6,000 tokens).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--dtype bf16|fp32] [--shape NAME]
+                    [--prompt-len N] [--prefill-len N] [--batch B] [--points B,B] [--no-prefill]
 
 A step is one decode step as generation does it: the step function for a batch
 of sequences (one token each, from the cache), greedy sampling on the device
@@ -70,6 +71,8 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--points", default="1,64", help="further batch sizes to measure")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--prompt-len", type=int, default=0, help="tokens every sequence holds before decoding (0: the shape's)")
+    ap.add_argument("--prefill-len", type=int, default=PREFILL, help="tokens of the timed prompt")
     ap.add_argument("--shape", default="mistral-7b-v0.2", choices=sorted(SHAPES),
                     help="the layer sizes: BASELINE.json's configs[2] (default), [3] or [4]")
     args = ap.parse_args()
@@ -83,6 +86,10 @@ def main():
 
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
     CFG, shape_name, CONTEXT, PROMPT = SHAPES[args.shape]
+    if args.prompt_len:
+        PROMPT = args.prompt_len
+        CONTEXT = max(CONTEXT, PROMPT + args.steps + args.warmup + 64)
+    PREFILL_LEN = args.prefill_len
     n_layers = args.layers or CFG["num_hidden_layers"]
     dev = "cuda:0"
     t0 = time.time()
@@ -101,7 +108,7 @@ def main():
     # ---------------------------------------------------------------- prefill of one 2,048-token prompt
     prefill = None
     if not args.no_prefill:
-        prompt = torch.randint(0, V, (PREFILL,), generator=gen).tolist()
+        prompt = torch.randint(0, V, (PREFILL_LEN,), generator=gen).tolist()
         times = []
         for i in range(3):
             slots = engine.start(1)
@@ -113,8 +120,8 @@ def main():
             times.append(time.perf_counter() - t)
             engine.release(slots)
         sec = min(times[1:])
-        fl = prefill_flops(CFG, n_layers, PREFILL)
-        prefill = {"value": round(PREFILL / sec, 1), "tokens": PREFILL, "ms": round(sec * 1e3, 3),
+        fl = prefill_flops(CFG, n_layers, PREFILL_LEN)
+        prefill = {"value": round(PREFILL_LEN / sec, 1), "tokens": PREFILL_LEN, "ms": round(sec * 1e3, 3),
                    "frac": round(fl / sec / FLOP_PEAK[args.dtype], 4)}
         sys.stderr.write("[bench] prefill %s\n" % prefill)
 
@@ -125,9 +132,10 @@ def main():
         ids = list(range(B))
         # prompts in chunks of sequences, so that the prefill workspace stays small
         tokens = []
-        for i in range(0, B, 8):
-            logits = engine.step(slots[i:i + 8], prompts[i:i + 8])
-            tokens += sampler.sample(logits, 0.0, ids[i:i + 8], [0] * len(slots[i:i + 8]))
+        n = max(1, min(8, 48000 // PROMPT))
+        for i in range(0, B, n):
+            logits = engine.step(slots[i:i + n], prompts[i:i + n])
+            tokens += sampler.sample(logits, 0.0, ids[i:i + n], [0] * len(slots[i:i + n]))
         for _ in range(warmup):
             logits = engine.step(slots, [[t] for t in tokens])
             tokens = sampler.sample(logits, 0.0, ids, [0] * B)
