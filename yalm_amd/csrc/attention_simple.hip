@@ -3,6 +3,7 @@
 // (query, head); keys are taken 64 at a time, a lane per key for the scores
 // and a lane per output element for the mix; softmax state in float32.
 #include <float.h>
+#include <mutex>
 #include "common.h"
 #include "yalm_hip.h"
 
@@ -314,4 +315,54 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
       seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
   attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
   return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// yalm_attn_decode for callers that cannot allocate: the partial results of the splits go to a
+// fixed array in device memory instead of a workspace of the caller's.  Every GPU that the library
+// runs on holds its own copy of the array, at its own address, until the process ends.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) float scratch[YALM_ATTN_DECODE_STATIC_BYTES / sizeof(float)];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex scratch_mutex;
+float* scratch_of_device[MAX_DEVICES];      // the array's address on each device, asked for once
+
+// The address of `scratch` on the current device (in host code the array's name is no device address).
+int scratch_pointer(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= MAX_DEVICES) return YALM_ERR_ARG;
+  std::lock_guard<std::mutex> hold(scratch_mutex);
+  if (scratch_of_device[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (p == nullptr) return YALM_ERR_ARG;
+    scratch_of_device[dev] = (float*)p;
+  }
+  *ptr = scratch_of_device[dev];
+  return YALM_OK;
+}
+}  // namespace
+
+extern "C" int yalm_attn_decode_static(const void* q, const void* k_pages, const void* v_pages,
+                                       const int* block_table, int table_stride, int ring_pages,
+                                       const int* seq_slot, const int* seq_len, void* out, int B, int n_heads,
+                                       int n_kv_heads, int head_dim, int window, int n_splits, int n_pages, int dtype,
+                                       int force_simple, hipStream_t stream) {
+  if (B <= 0) return YALM_OK;
+  if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0)
+    return YALM_ERR_ARG;
+  if (yalm_attn_decode_workspace(B, n_heads, head_dim, n_splits) > (long)YALM_ATTN_DECODE_STATIC_BYTES)
+    return YALM_ERR_SCRATCH;
+  float* partial = nullptr;
+  int rc = scratch_pointer(&partial);
+  if (rc != YALM_OK) return rc;
+  // nothing in the array has to start at zero: every split of every (sequence, head) writes its
+  // sums, maximum and denominator before the merge reads them, also for padding rows
+  return yalm_attn_decode(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, partial,
+                          B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, dtype, force_simple, stream);
 }

@@ -7,6 +7,7 @@
 #define YALM_OK 0
 #define YALM_ERR_ARG 1001          // an argument the kernel family refuses
 #define YALM_ERR_DTYPE 1002        // unknown dtype code
+#define YALM_ERR_SCRATCH 1003      // the sizes need more scratch than the fixed array of the entry point holds
 
 // dtype codes shared with the Python side
 #define YALM_F32 0

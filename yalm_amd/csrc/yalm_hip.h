@@ -134,6 +134,22 @@ int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, co
                      int n_pages, int dtype, int force_simple, hipStream_t stream);
 long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits);
 
+// yalm_attn_decode without a workspace argument, for callers that cannot allocate device memory
+// (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+// counterpart in the reference.  The partial results of the splits go to a fixed array of
+// YALM_ATTN_DECODE_STATIC_BYTES in device memory that belongs to the library; every GPU it runs on
+// holds its own copy until the process ends.  The call allocates and frees nothing.  Sizes with
+// yalm_attn_decode_workspace(B, n_heads, head_dim, n_splits) > YALM_ATTN_DECODE_STATIC_BYTES are
+// refused with YALM_ERR_SCRATCH (1003).  All calls on one GPU share that GPU's array, which keeps
+// the last call's contents (nothing in it has to be cleared between calls): calls that overlap on
+// one GPU, on different streams or from different threads, race.  The first call on a device looks
+// the array's address up and should not run under stream capture.
+#define YALM_ATTN_DECODE_STATIC_BYTES (8l << 20)
+int yalm_attn_decode_static(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                            int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
+                            int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits, int n_pages,
+                            int dtype, int force_simple, hipStream_t stream);
+
 // out[r] = index of the maximum of logits[r, :], lowest index on ties (src/sampler.cpp:27-38)
 int yalm_argmax(const float* logits, int* out, int R, int V, hipStream_t stream);
 // out[r] = first index whose running sum of exp((l - max)/T) reaches u[r] * total, else V-1
