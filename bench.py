@@ -21,14 +21,14 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# BASELINE.json configs[2]: Mistral-7B-v0.2 shape
+# Mistral-7B-v0.2 shape
 MISTRAL_7B = {
     "architectures": ["MistralForCausalLM"], "hidden_size": 4096, "intermediate_size": 14336,
     "num_hidden_layers": 32, "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 128,
     "vocab_size": 32000, "max_position_embeddings": 32768, "rope_theta": 1000000.0, "rms_norm_eps": 1e-5,
     "hidden_act": "silu", "tie_word_embeddings": False, "bos_token_id": 1, "eos_token_id": 2,
 }
-# BASELINE.json configs[3]: Llama-3.2-3B shape (llama3 rope scaling, tied head, a vocabulary that is no power of two)
+# Llama-3.2-3B shape (llama3 rope scaling, tied head, a vocabulary that is no power of two)
 LLAMA_3B = {
     "architectures": ["LlamaForCausalLM"], "hidden_size": 3072, "intermediate_size": 8192,
     "num_hidden_layers": 28, "num_attention_heads": 24, "num_key_value_heads": 8, "head_dim": 128,
@@ -37,7 +37,7 @@ LLAMA_3B = {
                      "original_max_position_embeddings": 8192},
     "hidden_act": "silu", "tie_word_embeddings": True, "bos_token_id": 128000, "eos_token_id": 128001,
 }
-# BASELINE.json configs[4]: Mistral-7B-v0.1 shape (a window of 4,096 positions: ring cache)
+# Mistral-7B-v0.1 shape (a window of 4,096 positions: ring cache)
 MISTRAL_7B_V01 = dict(MISTRAL_7B, rope_theta=10000.0, sliding_window=4096)
 # shape -> (config, name, context, prompt length of the decode runs)
 SHAPES = {
@@ -74,7 +74,7 @@ def main():
     ap.add_argument("--prompt-len", type=int, default=0, help="tokens every sequence holds before decoding (0: the shape's)")
     ap.add_argument("--prefill-len", type=int, default=PREFILL, help="tokens of the timed prompt")
     ap.add_argument("--shape", default="mistral-7b-v0.2", choices=sorted(SHAPES),
-                    help="the layer sizes: BASELINE.json's configs[2] (default), [3] or [4]")
+                    help="the layer sizes: the Mistral-7B-v0.2 shape (default), Llama-3.2-3B or Mistral-7B-v0.1")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not measured" % args.gpus, flush=True)
@@ -98,6 +98,11 @@ def main():
     sys.stderr.write("[bench] %d layers of random weights in %.1f s\n" % (n_layers, time.time() - t0))
     batches = sorted({args.batch} | {int(b) for b in args.points.split(",") if b})
     engine = Engine(model, max_tokens=max(batches) * CONTEXT, max_batch=max(batches))
+    t0 = time.time()
+    n_graphs = engine.warmup(batches, min_len=PROMPT + 1, max_len=PROMPT + args.steps + args.warmup + 1)
+    torch.cuda.synchronize()
+    sys.stderr.write("[bench] %d decode graphs captured ahead in %.2f s; their shared buffers hold %.1f MB\n"
+                     % (n_graphs, time.time() - t0, engine.graph_bytes() / 1e6))
     sampler = Sampler(0)
     V = CFG["vocab_size"]
     gen = torch.Generator().manual_seed(1)
@@ -162,6 +167,8 @@ def main():
             B, results[B]["tok_s"], results[B]["ms"], results[B]["bytes"] / 1e9,
             results[B]["bytes"] / results[B]["ms"] / 1e6))
 
+    sys.stderr.write("[bench] %d graphs captured in all; graph buffers %.1f MB, other step buffers %.1f MB\n"
+                     % (engine.graphs_captured, engine.graph_bytes() / 1e6, engine.ws.bytes() / 1e6))
     main_r = results[args.batch]
     achieved = main_r["bytes"] / (main_r["ms"] * 1e-3) / 1e9
     line = {

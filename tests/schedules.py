@@ -64,6 +64,30 @@ def batches(requests, groups, prompt_lens):
     return steps
 
 
+def interleaved(requests, groups, prompt_lens, start_at):
+    """Batches that overlap in time: group g's first step is step number start_at[g] of the merged
+    trace at the earliest, and from then on the live groups take turns, a step each.  Every step
+    still belongs to one batch (its requests all start or all go on by one token); a later batch
+    starts while sequences of earlier ones are still live, and takes the slots and pages that
+    their leavers gave back."""
+    per_group = [batches(requests, [g], prompt_lens) for g in groups]
+    cursor = [0] * len(groups)
+    steps = []
+    while any(c < len(p) for c, p in zip(cursor, per_group)):
+        progressed = False
+        for g, plan in enumerate(per_group):
+            if cursor[g] < len(plan) and len(steps) >= start_at[g]:
+                s = dict(plan[cursor[g]], step=len(steps))
+                steps.append(s)
+                cursor[g] += 1
+                progressed = True
+        if not progressed:                    # nothing live yet and the next group starts later: it starts now
+            g = min((g for g in range(len(groups)) if cursor[g] < len(per_group[g])), key=lambda g: start_at[g])
+            start_at = list(start_at)
+            start_at[g] = len(steps)
+    return steps
+
+
 def max_tokens_needed(steps):
     """The most tokens live requests hold at any time, each rounded up to 64."""
     held, worst = {}, 0

@@ -155,6 +155,31 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     assert "input_layernorm.weight: expected a floating-point tensor" in msg
 
 
+def test_tensors_the_model_does_not_use_are_passed_over(tmp_path, capsys):
+    """What convert.py:127-207 does with a real folder's extras: rotary_emb.inv_freq buffers of older
+    exports and an lm_head.weight stored next to a tied embedding are read past, not refused."""
+    from yalm_amd.engine.model import Model
+    folder = write_random_model(str(tmp_path / "m"), tiny_configs.TINY_LLAMA, seed=1)          # tied
+    src = TensorSource(folder)
+    t = {n: src.get(n).clone() for n in src.names()}
+    assert "lm_head.weight" not in t
+    t["lm_head.weight"] = t["model.embed_tokens.weight"].clone()
+    for l in range(tiny_configs.TINY_LLAMA["num_hidden_layers"]):
+        t["model.layers.%d.self_attn.rotary_emb.inv_freq" % l] = torch.ones(8)
+    extra = str(tmp_path / "extra")
+    os.makedirs(extra)
+    write_file(os.path.join(extra, "model.safetensors"), t)
+    with open(os.path.join(extra, "config.json"), "w") as f:
+        json.dump(tiny_configs.TINY_LLAMA, f)
+    model = Model.from_folder(extra, dtype=torch.float32, device="cpu")
+    assert model.head.weight is model.embedding.table
+    warned = capsys.readouterr().err
+    assert "3 tensors" in warned and "lm_head.weight" in warned and "rotary_emb.inv_freq" in warned
+    with pytest.raises(WeightsError) as e:
+        Model.from_folder(extra, dtype=torch.float32, device="cpu", strict=True)
+    assert "unexpected (3)" in str(e.value) and "missing" not in str(e.value)
+
+
 def test_container_errors(tmp_path):
     def write(header, data=b"", name="x.safetensors"):
         blob = json.dumps(header).encode()

@@ -38,7 +38,7 @@ def plain_greedy(folder, prompt, n_new, stop=()):
 
 @pytest.mark.parametrize("name", ["tiny_llama", "tiny_mistral", "tiny_wide_heads"])
 def test_greedy_generation_matches_the_plain_implementation(folders, name):
-    """BASELINE configs[0]: prompts of 5, 17 and 1 tokens, then 8 greedy steps (float32); also
+    """The tiny Llama workload: prompts of 5, 17 and 1 tokens, then 8 greedy steps (float32); also
     with untied heads, where the next token is not simply the last one again."""
     from yalm_amd import Engine, Model, generate
     model = Model.from_folder(folders[name], dtype=torch.float32, device="cuda:0")
@@ -54,7 +54,7 @@ def test_greedy_generation_matches_the_plain_implementation(folders, name):
 
 
 def test_temperature_sampling_with_a_fixed_seed(folders):
-    """BASELINE configs[1]: prompts of 2, 30, 9, 23 tokens, 20 steps past the window at
+    """The tiny Mistral workload: prompts of 2, 30, 9, 23 tokens, 20 steps past the window at
     temperature 0.8.  A request's tokens depend on the seed and its id, not on its batch,
     and equal the plain sampler's pick given the same uniform numbers."""
     from yalm_amd import Engine, Model, generate
@@ -196,6 +196,11 @@ def test_step_refuses_what_it_cannot_do(folders):
         Engine(on_cpu, max_tokens=64)
 
 
+def generated(stdout):
+    """The token ids a completion printed: what stands between the first line and the statistics."""
+    return stdout.split("\n\n")[0].split("\n", 1)[1].split()
+
+
 def test_command_line(folders):
     """python -m yalm_amd <folder> in the reference's manner: completion with token ids,
     greedy; and perplexity of a token sequence against the plain implementation."""
@@ -205,16 +210,17 @@ def test_command_line(folders):
                         "-n", "6", "-t", "0", "--dtype", "float32"], cwd=ROOT, stdout=subprocess.PIPE,
                        stderr=subprocess.PIPE, text=True, timeout=300)
     assert p.returncode == 0, p.stderr[-3000:]
-    first = p.stdout.split("\n\n")[0].split()
+    assert p.stdout.startswith("Model active bytes with full context window: ")
+    first = generated(p.stdout)
     want = plain_greedy(folder, prompt, 6, stop=(2,))
     assert [int(t) for t in first] == want
-    assert "Generation stats:" in p.stdout and "throughput:" in p.stdout
+    assert "Generation stats:" in p.stdout and "throughput:" in p.stdout and "bandwidth:" in p.stdout
     # the same model made from its configuration and seed alone, without a folder
     p = subprocess.run([sys.executable, "-m", "yalm_amd", "--random", os.path.join(folder, "config.json"),
                         "--weight-seed", "6", "--tokens", ",".join(map(str, prompt)), "-n", "6", "-t", "0", "--dtype",
                         "float32"], cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
     assert p.returncode == 0, p.stderr[-3000:]
-    assert [int(t) for t in p.stdout.split("\n\n")[0].split()] == want
+    assert [int(t) for t in generated(p.stdout)] == want
     toks = helpers.random_requests(tiny_configs.TINY_LLAMA, [30], seed=7)["r0"]
     p = subprocess.run([sys.executable, "-m", "yalm_amd", folder, "-m", "perp", "--tokens", " ".join(map(str, toks)),
                         "--dtype", "float32"], cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
@@ -265,7 +271,8 @@ def test_command_line_with_a_tokenizer(folders, tmp_path):
     prompt = tok.encode(text, True)
     assert prompt[:6] == [1, 3 + ord("T"), 3 + ord("h"), 3 + ord("e"), 260, 261]     # no space is put before the text
     want = plain_greedy(folder, prompt, 5, stop=(cfg["eos_token_id"],))
-    assert p.stdout.startswith(printed(want, prompt[-1])), (p.stdout[:80], printed(want, prompt[-1]))
+    shown = p.stdout.split(b"\n", 1)[1]                    # behind the line about the model's active bytes
+    assert shown.startswith(printed(want, prompt[-1])), (shown[:80], printed(want, prompt[-1]))
 
     p = subprocess.run([sys.executable, "-m", "yalm_amd", folder, "-m", "passkey", "-n", "2", "-l", "1", "--seed", "4",
                         "--dtype", "float32"], cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=300)

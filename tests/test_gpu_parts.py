@@ -229,7 +229,27 @@ def define_toy_parts():
                 state[slot] = sums[-1]
                 o += n
 
+    class RunningMeanMixerOnDevice(RunningMeanMixer):
+        """The same mixer with a decode step that a graph can hold: the rows' slots and positions are
+        read on the device, the state is advanced by device operations, and padding rows (slot -1)
+        change nothing.  Whole prompts (never captured) take the host-driven way."""
+        graph_safe = True
+
+        def forward(self, h, x, ctx, line, writes_cache=True):
+            if ctx.mode != "decode":
+                return super().forward(h, x, ctx, line, writes_cache)
+            from yalm_amd.ops import kernels
+            state = ctx.cache.group_of(line).line_state(line)          # [n_slots, dim]
+            slot = ctx.seq_slot.long()
+            live = (slot >= 0)[:, None]
+            index = slot.clamp(min=0)
+            state.index_add_(0, index, h.float() * live)               # a padding row adds zeros
+            counts = (ctx.tok_pos + 1).float()[:, None]
+            mean = (state.index_select(0, index) / counts * live).contiguous()
+            kernels.gemm(mean, self.w, x, kernels.EPI_ADD_F32)
+
     register_part("mixer", "toy_running_mean", RunningMeanMixer, replace=True)
+    register_part("mixer", "toy_running_mean_on_device", RunningMeanMixerOnDevice, replace=True)
     return RunningMeanMixer
 
 
@@ -254,7 +274,7 @@ class ToyConfig:
         norm = {"eps": d["eps"]}
         pos = PartSpec("rope", {"head_dim": 16, "rotary_dim": 16, "theta": 100.0, "scaling": None,
                                 "weight_rows": "interleaved"})
-        mixers = [PartSpec("toy_running_mean", {}, prefix="mean."),
+        mixers = [PartSpec(d.get("mean_mixer", "toy_running_mean"), {}, prefix="mean."),
                   PartSpec("gqa_attention", {"n_heads": 2, "n_kv_heads": 1, "head_dim": 16, "window": 0,
                                              "position": pos}, prefix="attn.")]
         layers = [LayerSpec("prenorm_residual", m, PartSpec("swiglu", {"hidden": d["hidden"]}, prefix="ff."),
@@ -291,7 +311,11 @@ def toy_plain_forward(w, d, tokens):
     return R.rmsnorm(x, w["toy.norm.weight"], d["eps"]) @ w["toy.emb.weight"].double().T
 
 
-def test_toy_mixer_and_architecture_from_outside(tmp_path):
+@pytest.mark.parametrize("mixer", ["toy_running_mean", "toy_running_mean_on_device"])
+def test_toy_mixer_and_architecture_from_outside(tmp_path, mixer):
+    """Layer 0 carries state of its own.  With the host-driven mixer only that layer runs kernel by
+    kernel in a decode step and the layers around it are replayed from graphs; with the device-driven
+    one the whole step is one graph and the state is advanced inside it, once a step."""
     from yalm_amd import Engine, Model, register_architecture, write_random_model
     from yalm_amd.cache import StateGroup
     from yalm_amd.config import unregister_architecture
@@ -300,26 +324,34 @@ def test_toy_mixer_and_architecture_from_outside(tmp_path):
     register_architecture("ToyForCausalLM", ToyConfig, replace=True)
     try:
         d = {"architectures": ["ToyForCausalLM"], "width": 40, "hidden": 48, "vocab": 61, "positions": 200,
-             "eps": 1e-5}
+             "eps": 1e-5, "mean_mixer": mixer}
         folder = write_random_model(str(tmp_path / "toy"), d, seed=2)
         model = Model.from_folder(folder, dtype=torch.float32, device=DEV)
-        assert not model.graph_safe()
         engine = Engine(model, max_tokens=1024)
+        if mixer == "toy_running_mean":
+            assert not model.graph_safe()
+            assert engine._segments == [(True, 0, 1), (False, 1, 2), (True, 2, 5)]
+        else:
+            assert model.graph_safe() and engine._segments == [(True, 0, 5)]
         assert len(engine.cache.state_groups) == 1 and isinstance(engine.cache.group_of(0), StateGroup)
         assert engine.cache.group_of(1) is engine.cache.group_of(2)          # the layer that runs twice: two lines
         cfg, w = R.read_folder(folder)
         requests = {"a": [5, 9, 60, 3, 3, 17, 44, 8, 0, 31], "b": [7, 7, 2], "c": list(range(40, 61)) + list(range(30)),
                     "d": [60, 0, 1, 59, 2, 58]}
         for steps in (schedules.whole(requests), schedules.tail_one_by_one(requests, 4),
-                      schedules.batches(requests, [["a", "b"], ["c", "d"]], {"a": 4, "b": 1, "c": 33, "d": 2})):
+                      schedules.batches(requests, [["a", "b"], ["c", "d"]], {"a": 4, "b": 1, "c": 33, "d": 2}),
+                      schedules.interleaved(requests, [["a", "b"], ["c", "d"]], {"a": 4, "b": 1, "c": 33, "d": 2},
+                                            [0, 2])):
             out = schedules.replay_in_process(engine, steps)
             got = schedules.per_request(steps, out, requests)
             for rid, toks in requests.items():
                 want = toy_plain_forward(w, d, toks).float().numpy()
                 helpers.check_logits(got[rid], want, "float32", "toy %s" % rid)
+        assert engine.graphs_captured > 0 and engine._graphs        # the decode steps above were replayed
     finally:
         unregister_architecture("ToyForCausalLM")
         unregister_part("mixer", "toy_running_mean")
+        unregister_part("mixer", "toy_running_mean_on_device")
 
 
 # ---------------------------------------------------------------------------

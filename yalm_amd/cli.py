@@ -5,7 +5,10 @@
       -h                 this text
       -d [hip,cuda]      device; there is no CPU path here (default - hip)
       -m [completion,passkey,perplexity]   mode, may be abbreviated (default - completion)
-      -T <int>           sliding window context length (0 - max)
+      -T <int>           sliding window context length (0 - max): every layer attends to the last <int>
+                         positions only, so a text may be longer than the model's context.  Unlike the
+                         reference, whose -T also keeps the first two positions as attention sinks and
+                         re-rotates them every step, this is a plain window.
       -i <string>        input prompt           } completion and perplexity:
       -f <filepath>      input file with prompt } exactly one of -i, -f, --tokens
       -t <float>         temperature (default - 1.0; 0 = greedy)
@@ -189,6 +192,16 @@ def run_completion(a):
             sys.stdout.flush()
         last[i] = t
 
+    print("Model active bytes with full context window: %d" % (
+        model.weight_bytes() + sum(g.bytes_per_token() * (g.window or engine.n_positions) for g in engine.cache.kv_groups)))
+    # graphs for the decode steps to come are captured before the clock starts (main.cpp:81-85 warms up too)
+    shortest, longest = min(len(p) for p in prompts), min(max_len, max(len(p) for p in prompts) + steps)
+    sizes = list(range(1, min(len(prompts), engine.cache.n_slots) + 1))
+    from .engine import StepError
+    try:
+        engine.warmup(sizes, min_len=shortest + 1, max_len=longest)
+    except StepError:                                   # more bucket pairs than the engine keeps: the full batch only
+        engine.warmup(sizes[-1:], min_len=shortest + 1, max_len=min(longest, 2 * shortest + 64))
     t0 = time.perf_counter()
     out = generate(engine, prompts, max_new_tokens=steps, temperature=a["temperature"], seed=seed, stop_ids=stop,
                    on_token=on_token, stats=stats)
@@ -200,8 +213,8 @@ def run_completion(a):
             print("[%d] %s" % (i, text))
     total = stats.prompt_tokens + stats.new_tokens
     print("\n\nGeneration stats:\n  %d tokens\n  throughput: %.5gtok/s\n  latency: %.5gs/tok\n  hydrate: %.5gs\n"
-          "  prefill: %.5gtok/s\n  decode: %.5gtok/s\n  total: %.5gs\n"
-          % (total, total / elapsed, elapsed / max(total, 1), stats.prefill_seconds,
+          "  bandwidth: %.5gGB/s\n  prefill: %.5gtok/s\n  decode: %.5gtok/s\n  total: %.5gs\n"
+          % (total, total / elapsed, elapsed / max(total, 1), stats.prefill_seconds, stats.bytes_read / 1e9 / elapsed,
              stats.prefill_tokens_per_second, stats.decode_tokens_per_second, elapsed))
     return out
 
@@ -209,19 +222,19 @@ def run_completion(a):
 def run_perplexity(a):
     """src/main.cpp:150-235: logits at every position, log-probability of the next
     token; ppl = exp(-sum/N), error = ppl * sqrt((ss - sum^2/N)/N/N), N = len - 1."""
-    from .sampling import Sampler
     model = _load(a)
     prompts, _ = _prompts(a, model)
-    engine = _engine(a, model, sum(len(p) + 64 for p in prompts))
-    sampler = Sampler(0)
+    engine = _engine(a, model, max(len(p) + 64 for p in prompts))
     results = []
     for p in prompts:
         if len(p) < 2:
             error_usage("perplexity needs at least two tokens")
+        if len(p) > engine.n_positions:
+            error_usage("the text has %d tokens, the context holds %d: give a window with -T" % (len(p), engine.n_positions))
         t0 = time.perf_counter()
         slots = engine.start(1)
-        logits = engine.step(slots, [p], [list(range(len(p) - 1))])
-        probs = sampler.prob(logits, p[1:])
+        # the probability of each next token; the logits are made a block of rows at a time
+        probs = engine.step(slots, [p], [list(range(len(p) - 1))], targets=[p[1:]]).tolist()
         engine.release(slots)
         elapsed = time.perf_counter() - t0
         N = len(p) - 1

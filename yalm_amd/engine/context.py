@@ -5,14 +5,21 @@ import torch
 
 class Workspace:
     """Named device buffers that are reused from step to step and grow on demand.
-    A buffer is a flat allocation; `get` returns a view of the asked shape."""
+    A buffer is a flat allocation; `get` returns a view of the asked shape.
+
+    While `frozen` a buffer may not grow (a graph is being captured).  Once `pinned`
+    (captured graphs hold the buffers' addresses) a buffer that has to grow is
+    replaced for later users, and the old one is kept for the graphs that still use
+    it until `drop_retired`."""
 
     def __init__(self, device):
         self.device = device
         self._flat = {}
-        self.frozen = False           # set while a graph that uses these buffers exists
+        self._retired = []
+        self.frozen = False           # set while a graph is captured on these buffers
+        self.pinned = False           # set once a captured graph uses these buffers
 
-    def get(self, name, shape, dtype):
+    def _buffer(self, name, shape, dtype, zeroed):
         n = 1
         for s in shape:
             n *= int(s)
@@ -21,25 +28,27 @@ class Workspace:
         if buf is None or buf.numel() < n:
             if self.frozen:
                 raise RuntimeError("workspace buffer %r would have to grow inside a captured graph" % (name,))
-            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            if buf is not None and self.pinned:
+                self._retired.append(buf)
+            make = torch.zeros if zeroed else torch.empty
+            buf = make(max(n, 1), dtype=dtype, device=self.device)
             self._flat[key] = buf
         return buf[:n].view(*shape)
 
+    def get(self, name, shape, dtype):
+        return self._buffer(name, shape, dtype, False)
+
     def get_zeroed(self, name, shape, dtype):
         """Like get, but the buffer is zero when it is first made (users keep it so)."""
-        n = 1
-        for s in shape:
-            n *= int(s)
-        key = (name, dtype)
-        buf = self._flat.get(key)
-        if buf is None or buf.numel() < n:
-            if self.frozen:
-                raise RuntimeError("workspace buffer %r would have to grow inside a captured graph" % (name,))
-            self._flat[key] = torch.zeros(max(n, 1), dtype=dtype, device=self.device)
-        return self._flat[key][:n].view(*shape)
+        return self._buffer(name, shape, dtype, True)
+
+    def drop_retired(self):
+        """Frees the replaced buffers; only when no graph that used them is left."""
+        self._retired.clear()
+        self.pinned = False
 
     def bytes(self):
-        return sum(b.numel() * b.element_size() for b in self._flat.values())
+        return sum(b.numel() * b.element_size() for b in list(self._flat.values()) + self._retired)
 
 
 class StepContext:
@@ -50,6 +59,8 @@ class StepContext:
       seq_tile0[B+1] (prefill: first 64-token tile of each sequence in the staging area; n_tiles in all),
       tile_order (prefill, may be None: the order in which attention should take the tiles).
     max_position: the largest position in the step (host value, for table checks).
+    host_slots, host_n_tokens, host_start: the step's real sequences as host lists (a decode step's
+    padding rows, seq_slot -1, are not in them), for parts whose launches depend on host values.
     pages_bucket: decode only; an upper bound (a power of two) of the pages of the step's
     longest sequence, the only way launch shapes may depend on lengths."""
 
@@ -63,6 +74,7 @@ class StepContext:
         self.seq_tile0 = None
         self.tile_order = None
         self.n_tiles = 0
+        self.x = None                     # the residual stream of the step, float32 [T, dim]
         self.normed = {}                  # id(norm part) -> (xn, ss, eps): activations a producer emitted for it
         self.pages_bucket = 1 << 30       # decode: no sequence of the step has more pages than this
         self.max_position = 0

@@ -13,6 +13,8 @@ read positions, lengths, slots and block tables from device memory, so the
 graph needs no patching from step to step (the reference patches kernel nodes
 every step, src/infer.cu:1225-1247).  Rows that pad a batch to its bucket
 carry slot -1 and change no result."""
+from collections import OrderedDict
+
 import numpy as np
 import torch
 
@@ -27,23 +29,52 @@ class StepError(ValueError):
     pass
 
 
-class _DecodeGraph:
-    """A captured decode step for one bucket size, with its own buffers."""
+class _BucketBuffers:
+    """The step metadata of one batch-size bucket: a pinned host copy and the device tensor
+    that every graph of the bucket reads."""
 
     def __init__(self, engine, bucket):
         self.bucket = bucket
-        self.ws = Workspace(engine.device)
         n_meta = 6 * bucket + 1
         self.meta_host = torch.empty(n_meta, dtype=torch.int32, pin_memory=True)
         self.meta = torch.zeros(n_meta, dtype=torch.int32, device=engine.device)
-        self.logits = torch.empty((bucket, engine.model.vocab_size), dtype=torch.float32, device=engine.device)
-        self.graph = None
-        self.ctx = engine._context("decode", self.ws, self.meta, bucket, bucket, 0)
         self.copied = None            # event after the last upload of meta_host
+
+    def host(self):
+        if self.copied is not None:
+            self.copied.synchronize()                    # the last upload has read the pinned buffer
+        return self.meta_host.numpy()
+
+    def upload(self):
+        self.meta.copy_(self.meta_host, non_blocking=True)
+        if self.copied is None:
+            self.copied = torch.cuda.Event()
+        self.copied.record()
+
+
+class _DecodeGraph:
+    """A decode step for one (batch bucket, pages bucket): the model's graph-safe runs of units as
+    captured graphs, the others as (None, first, end) to be run kernel by kernel in between."""
+
+    def __init__(self, engine, bufs, pages_bucket):
+        B = bufs.bucket
+        self.bufs = bufs
+        self.ctx = engine._context("decode", engine.graph_ws, bufs.meta, B, B, 0)
+        self.ctx.pages_bucket = pages_bucket
+        self.eager_ctx = engine._context("decode", engine.ws, bufs.meta, B, B, 0)
+        self.eager_ctx.pages_bucket = pages_bucket
+        self.segments = []
+        self.x = None
+        self.logits = None
 
 
 class Engine:
-    def __init__(self, model, max_tokens, max_batch=None, use_graphs=True):
+    """max_tokens: the most tokens live sequences hold at any time (each rounded up to a page);
+    max_batch: the most sequences alive at once; use_graphs: replay decode steps from captured
+    graphs; max_graphs: the most (batch bucket, pages bucket) graphs kept (the least recently
+    used one goes first)."""
+
+    def __init__(self, model, max_tokens, max_batch=None, use_graphs=True, max_graphs=24):
         if model.device is None:
             raise StepError("the model has no weights yet")
         if model.device.type != "cuda":
@@ -57,12 +88,17 @@ class Engine:
         n_positions = model.spec.max_positions if self.cache.unbounded else \
             min(model.spec.max_positions, self.cache.max_seq_len)
         self.n_positions = n_positions
-        model.prepare(n_positions)
-        self.ws = Workspace(self.device)
+        model.prepare(n_positions)                      # tables only ever grow: other engines of the model keep theirs
+        self._tables_version = model.tables_version
+        self.ws = Workspace(self.device)                # steps that run kernel by kernel
+        self.graph_ws = Workspace(self.device)          # shared by all captured graphs (they never run together)
         self.use_graphs = use_graphs
-        self._graph_safe = model.graph_safe()          # the parts are fixed from here on: asked once, not every step
-        self._graphs = {}
-        self._meta_host = None
+        self.max_graphs = max(1, int(max_graphs))
+        self._segments = model.decode_segments()        # the parts are fixed from here on: asked once, not every step
+        self._any_graph = any(safe for safe, _, _ in self._segments)
+        self._graphs = OrderedDict()                    # (batch bucket, pages bucket) -> _DecodeGraph, least recently used first
+        self._buckets = {}
+        self.graphs_captured = 0
 
     # ------------------------------------------------------------------ sequences
     def start(self, n):
@@ -75,6 +111,19 @@ class Engine:
 
     def length(self, slot):
         return self.cache.seq_len[slot]
+
+    def step_bytes(self, slots):
+        """Bytes a step over these sequences has to read: every weight once, an embedding row each,
+        and the keys and values the sequences hold (a window's worth where a line keeps a window).
+        The reference's Config::active_bytes (src/model.cpp:71-96) for a batch, with the head at
+        its stored width."""
+        total = self.model.weight_bytes() + (len(slots) - 1) * self.model.embedding.weight_bytes()
+        for g in self.cache.kv_groups:
+            per_token = g.bytes_per_token()
+            for s in slots:
+                n = self.cache.seq_len[s]
+                total += per_token * (min(n, g.window) if g.window else n)
+        return total
 
     # ------------------------------------------------------------------ the step
     def _context(self, mode, ws, meta, T, B, max_position):
@@ -89,12 +138,17 @@ class Engine:
         ctx.max_position = max_position
         return ctx
 
-    def step(self, slots, tokens, want=None):
+    def step(self, slots, tokens, want=None, targets=None):
         """slots: the sequences of the batch that take part in this step;
         tokens[i]: the next tokens of slots[i]; want[i]: indices into tokens[i] whose
         logits are asked for (default: the last).  Returns float32 [n_wanted, vocab]
         on the device, in the order of the slots and of want; the tensor is valid
-        until the next step."""
+        until the next step.
+
+        targets[i][k] (optional): a token id for the k-th wanted place of slots[i].  The step then
+        returns float32 [n_wanted], the probability softmax(logits)[target] at each wanted place
+        (src/sampler.cpp:11-25), and the logits are made and used a block of rows at a time: what a
+        text's perplexity needs, in memory that does not grow with the text."""
         B = len(slots)
         if B == 0:
             raise StepError("a step needs at least one sequence")
@@ -128,6 +182,11 @@ class Engine:
             for j in w:
                 if not 0 <= j < n:
                     raise StepError("wanted place %r is outside the %d tokens of its sequence" % (j, n))
+        if targets is not None:
+            if len(targets) != B or any(len(t) != len(w) for t, w in zip(targets, want)):
+                raise StepError("targets must name one token for every wanted place")
+            if any(not 0 <= tok < V for t in targets for tok in t):
+                raise StepError("a target token is outside the vocabulary of %d" % V)
         if all(s == 0 for s in starts):
             mode = "prefill"
         elif all(n == 1 for n in n_tok):
@@ -144,10 +203,16 @@ class Engine:
         except CacheError as e:
             raise StepError(str(e)) from None
         if mode == "decode":
-            return self._decode(slots, tokens, want, starts, new_lens)
-        return self._prefill(slots, tokens, want, n_tok, new_lens)
+            logits = self._decode(slots, tokens, want, starts, new_lens)
+            if targets is None:
+                return logits
+            flat = torch.tensor([tok for t in targets for tok in t], dtype=torch.int32, device=self.device)
+            return kernels.token_prob(logits, flat, torch.empty(flat.shape[0], dtype=torch.float32, device=self.device))
+        return self._prefill(slots, tokens, want, n_tok, new_lens, targets)
 
-    def _prefill(self, slots, tokens, want, n_tok, new_lens):
+    HEAD_ROWS = 1024        # rows of logits made at a time when only token probabilities are asked for
+
+    def _prefill(self, slots, tokens, want, n_tok, new_lens, targets=None):
         B, T = len(slots), sum(n_tok)
         rows = []
         cu = np.zeros(B + 1, dtype=np.int32)
@@ -177,9 +242,22 @@ class Engine:
         ctx.tile_order = meta[o + 4 * B + 2 + R:]
         ctx.n_tiles = int(tile0[-1])
         ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), list(n_tok), [0] * B
-        logits = self.ws.get("logits", (R, self.model.vocab_size), torch.float32) if R else None
-        self.model.forward(ctx, meta[o + 4 * B + 2:o + 4 * B + 2 + R] if R else None, logits)
-        return logits if R else torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
+        V = self.model.vocab_size
+        want_rows = meta[o + 4 * B + 2:o + 4 * B + 2 + R]
+        if targets is not None:
+            probs = torch.empty(R, dtype=torch.float32, device=self.device)
+            flat = torch.tensor([tok for t in targets for tok in t], dtype=torch.int32, device=self.device)
+            n_units = self.model.n_units()
+            self.model.run_units(ctx, 0, n_units - 1)
+            for r0 in range(0, R, self.HEAD_ROWS):
+                r1 = min(R, r0 + self.HEAD_ROWS)
+                block = self.ws.get("logits", (r1 - r0, V), torch.float32)
+                self.model.run_units(ctx, n_units - 1, n_units, want_rows[r0:r1], block)
+                kernels.token_prob(block, flat[r0:r1], probs[r0:r1])
+            return probs
+        logits = self.ws.get("logits", (R, V), torch.float32) if R else None
+        self.model.forward(ctx, want_rows if R else None, logits)
+        return logits if R else torch.empty((0, V), dtype=torch.float32, device=self.device)
 
     def _bucket(self, B):
         for b in DECODE_BUCKETS:
@@ -187,28 +265,13 @@ class Engine:
                 return b
         return B
 
-    def _decode(self, slots, tokens, want, starts, new_lens):
+    @staticmethod
+    def _fill_decode_meta(host, Bk, tokens, starts, slots, new_lens):
+        """The metadata of a decode step of len(slots) sequences in Bk rows; the rows behind
+        them are padding (token -1, slot -1, length 0)."""
         B = len(slots)
-        use_graph = self.use_graphs and self._graph_safe
-        Bk = self._bucket(B) if use_graph else B
-        # launch shapes may depend on the longest sequence only through this bucket (a power of
-        # two of pages), so that a captured graph stays valid until a sequence outgrows it
-        pages_bucket = 1
-        while pages_bucket * PAGE < max(new_lens):
-            pages_bucket *= 2
-        g = self._graphs.get((Bk, pages_bucket)) if use_graph else None
-        if use_graph and g is None:
-            g = _DecodeGraph(self, Bk)
-            g.ctx.pages_bucket = pages_bucket
-            self._graphs[(Bk, pages_bucket)] = g
-        if g is not None:
-            if g.copied is not None:
-                g.copied.synchronize()                   # the last upload has read the pinned buffer
-            host = g.meta_host.numpy()
-        else:
-            host = np.empty(6 * Bk + 1, dtype=np.int32)
         host[0:Bk] = -1
-        host[0:B] = [t[0] for t in tokens]
+        host[0:B] = tokens
         host[Bk:2 * Bk] = np.arange(Bk, dtype=np.int32)
         host[2 * Bk:3 * Bk] = 0
         host[2 * Bk:2 * Bk + B] = starts
@@ -217,8 +280,26 @@ class Engine:
         host[4 * Bk:5 * Bk] = 0
         host[4 * Bk:4 * Bk + B] = new_lens
         host[5 * Bk:6 * Bk + 1] = np.arange(Bk + 1, dtype=np.int32)
+
+    @staticmethod
+    def _pages_bucket(n_tokens):
+        """Launch shapes may depend on the longest sequence only through this bucket (a power of
+        two of pages), so that a captured graph stays valid until a sequence outgrows it."""
+        pages_bucket = 1
+        while pages_bucket * PAGE < n_tokens:
+            pages_bucket *= 2
+        return pages_bucket
+
+    def _decode(self, slots, tokens, want, starts, new_lens):
+        B = len(slots)
+        use_graph = self.use_graphs and self._any_graph
+        Bk = self._bucket(B) if use_graph else B
+        pages_bucket = self._pages_bucket(max(new_lens))
+        firsts = [t[0] for t in tokens]
         rows = [i for i, w in enumerate(want) if len(w) > 0]
-        if g is None:
+        if not use_graph:
+            host = np.empty(6 * Bk + 1, dtype=np.int32)
+            self._fill_decode_meta(host, Bk, firsts, starts, slots, new_lens)
             meta = self.ws.get("meta", (6 * Bk + 1,), torch.int32)
             meta.copy_(torch.from_numpy(host))
             ctx = self._context("decode", self.ws, meta, Bk, Bk, max(starts))
@@ -227,14 +308,18 @@ class Engine:
             logits = self.ws.get("logits", (Bk, self.model.vocab_size), torch.float32)
             self.model.forward(ctx, None, logits)                     # every row
         else:
-            g.meta.copy_(g.meta_host, non_blocking=True)
-            if g.copied is None:
-                g.copied = torch.cuda.Event()
-            g.copied.record()
-            g.ctx.max_position = max(starts)
-            if g.graph is None:
-                self._capture(g)
-            g.graph.replay()
+            g = self._graph(Bk, pages_bucket)
+            self._fill_decode_meta(g.bufs.host(), Bk, firsts, starts, slots, new_lens)
+            g.bufs.upload()
+            for graph, lo, hi in g.segments:
+                if graph is not None:
+                    graph.replay()
+                else:                                                 # a run of units that no graph can hold
+                    ctx = g.eager_ctx
+                    ctx.x = g.x
+                    ctx.max_position = max(starts)
+                    ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), [1] * B, list(starts)
+                    self.model.run_units(ctx, lo, hi, None, g.logits)
             logits = g.logits
         if rows == list(range(B)):
             return logits[:B]
@@ -242,16 +327,93 @@ class Engine:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         return logits[torch.tensor(rows, device=self.device)]
 
-    def _capture(self, g):
-        """Runs the step once eagerly on the graph's buffers (every buffer gets its
-        size), then captures it."""
-        self.model.forward(g.ctx, None, g.logits)
+    # ------------------------------------------------------------------ captured decode steps
+    def _graph(self, Bk, pages_bucket):
+        """The captured step for the bucket pair, made now if there is none (most recently used last)."""
+        if self.model.tables_version != self._tables_version:       # a table the graphs point to was replaced
+            self.drop_graphs()
+            self._tables_version = self.model.tables_version
+        key = (Bk, pages_bucket)
+        g = self._graphs.get(key)
+        if g is None:
+            while len(self._graphs) >= self.max_graphs:
+                self._graphs.popitem(last=False)
+            if not self._graphs:
+                self.graph_ws.drop_retired()
+            g = self._capture(Bk, pages_bucket)
+            self._graphs[key] = g
+        else:
+            self._graphs.move_to_end(key)
+        return g
+
+    def _capture(self, Bk, pages_bucket):
+        """Captures the decode step of a bucket pair on rows of padding only: nothing that a live
+        sequence holds (cache pages, per-sequence state) is read or written, so capturing in the
+        middle of a request changes nothing for it.  The step runs once kernel by kernel first
+        (every buffer gets its size), then under capture."""
+        bufs = self._buckets.get(Bk)
+        if bufs is None:
+            bufs = self._buckets[Bk] = _BucketBuffers(self, Bk)
+        self._fill_decode_meta(bufs.host(), Bk, [], [], [], [])
+        bufs.upload()
+        g = _DecodeGraph(self, bufs, pages_bucket)
+        ws, ctx = self.graph_ws, g.ctx
+        ctx.max_position = 0
+        ctx.x = g.x = ws.get("x", (Bk, self.model.dim), torch.float32)
+        g.logits = ws.get("logits", (Bk, self.model.vocab_size), torch.float32)
+        for safe, lo, hi in self._segments:
+            if safe:
+                self.model.run_units(ctx, lo, hi, None, g.logits)
         torch.cuda.synchronize(self.device)
-        g.ws.frozen = True
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            self.model.forward(g.ctx, None, g.logits)
-        g.graph = graph
+        ws.frozen = True
+        try:
+            for safe, lo, hi in self._segments:
+                graph = None
+                if safe:
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.graph(graph):
+                        self.model.run_units(ctx, lo, hi, None, g.logits)
+                g.segments.append((graph, lo, hi))
+        finally:
+            ws.frozen = False
+        ws.pinned = True
+        self.graphs_captured += 1
+        return g
+
+    def warmup(self, batch_sizes=(1,), max_len=None, min_len=1):
+        """Captures the decode graphs for batches of the given sizes and for sequences of min_len to
+        max_len tokens (default: the longest the engine holds) ahead of the first request, so that no
+        live step pays for a capture.  It runs on padding rows: no slot or page is taken and live
+        sequences are left alone (the reference runs one forward before it measures,
+        src/main.cpp:81-85, which overwrites a cache row).  Returns the number of graphs captured."""
+        if not (self.use_graphs and self._any_graph):
+            return 0
+        longest = self.n_positions if self.cache.unbounded else min(self.n_positions, self.cache.max_seq_len)
+        max_len = longest if max_len is None else min(int(max_len), longest)
+        min_len = max(1, min(int(min_len), max_len))
+        pairs = []
+        for Bk in sorted({self._bucket(int(b)) for b in batch_sizes if int(b) > 0}):
+            pb = self._pages_bucket(min_len)
+            while True:
+                pairs.append((Bk, pb))
+                if pb * PAGE >= max_len:
+                    break
+                pb *= 2
+        if len(pairs) > self.max_graphs:
+            raise StepError("warmup asks for %d graphs, the engine keeps %d (max_graphs)" % (len(pairs), self.max_graphs))
+        before = self.graphs_captured
+        for Bk, pb in pairs:
+            self._graph(Bk, pb)
+        return self.graphs_captured - before
+
+    def drop_graphs(self):
+        """Forgets every captured graph and the buffers only they used."""
+        self._graphs.clear()
+        self.graph_ws.drop_retired()
+
+    def graph_bytes(self):
+        """Device bytes of the buffers that the captured graphs share."""
+        return self.graph_ws.bytes() + sum(b.meta.numel() * 4 for b in self._buckets.values())
 
     def synchronize(self):
         torch.cuda.synchronize(self.device)

@@ -46,6 +46,7 @@ class Model:
         self.shared_lines = set(readers)
         self.compute_dtype = None
         self.device = None
+        self.tables_version = 0
 
     # ------------------------------------------------------------------ weights
     def top_parts(self):
@@ -73,15 +74,16 @@ class Model:
         return self
 
     @classmethod
-    def from_folder(cls, path, dtype=torch.bfloat16, device="cuda:0", window=None):
+    def from_folder(cls, path, dtype=torch.bfloat16, device="cuda:0", window=None, strict=False):
         """The model of a folder with config.json and *.safetensors; the class of the
-        configuration is chosen by config.json's architecture."""
+        configuration is chosen by config.json's architecture.  strict: tensors in the
+        folder that the model does not use are an error (else a warning)."""
         cfg = config_from_folder(path)
         if window:
             cfg = cfg.with_window(window)
         model = cls(cfg.to_spec(), cfg)
         source = TensorSource(path)
-        source.check(model.param_specs())
+        source.check(model.param_specs(), strict=strict)
         return model.load(source.get, dtype, device)
 
     @classmethod
@@ -114,15 +116,49 @@ class Model:
         return out
 
     def prepare(self, n_positions):
-        """Lets position encodings build their tables for positions < n_positions."""
+        """Lets position encodings build their tables for positions < n_positions.  A table that
+        already reaches that far stays as it is (engines that share the model keep using it);
+        `tables_version` counts the times a table was replaced, for whoever holds its address."""
         for p in self.all_parts():
             if hasattr(p, "prepare"):
+                before = getattr(p, "table", None)
+                if before is not None and getattr(p, "n_positions", 0) >= n_positions:
+                    continue
                 p.prepare(n_positions, self.device)
+                if before is not None:
+                    self.tables_version += 1
+
+    # ------------------------------------------------------------------ the step as a row of units
+    # unit 0 is the embedding, units 1..n the schedule's entries, unit n + 1 the final norm and the head
+    def n_units(self):
+        return len(self.schedule) + 2
+
+    def unit_parts(self, u):
+        if u == 0:
+            return list(_walk(self.embedding))
+        if u == len(self.schedule) + 1:
+            return list(_walk(self.final_norm)) + list(_walk(self.head))
+        return list(_walk(self.blocks[self.schedule[u - 1].layer]))
+
+    def unit_graph_safe(self, u):
+        """True if the unit launches only kernels whose arguments stay valid from step to step
+        (a part that does not says so with `graph_safe = False`)."""
+        return all(getattr(p, "graph_safe", True) for p in self.unit_parts(u))
 
     def graph_safe(self):
-        """True if every part launches only kernels whose arguments stay valid from
-        step to step (a part that is not says so with `graph_safe = False`)."""
-        return all(getattr(p, "graph_safe", True) for p in self.all_parts())
+        return all(self.unit_graph_safe(u) for u in range(self.n_units()))
+
+    def decode_segments(self):
+        """The units of a decode step in runs of equal kind: [(graph_safe, first unit, end unit)].
+        A run that is graph-safe can be captured and replayed; the others run kernel by kernel."""
+        out = []
+        for u in range(self.n_units()):
+            safe = self.unit_graph_safe(u)
+            if out and out[-1][0] == safe:
+                out[-1] = (safe, out[-1][1], u + 1)
+            else:
+                out.append((safe, u, u + 1))
+        return out
 
     def weight_bytes(self):
         """Bytes of weights a step reads: every weight once, one embedding row."""
@@ -136,27 +172,40 @@ class Model:
         """Runs the step's tokens through the layers (the cache is read and written
         through ctx) and writes logits for the rows want_rows (int32 device tensor;
         None: every row, in order)."""
-        T = ctx.tokens.shape[0]
-        x = ctx.ws.get("x", (T, self.dim), torch.float32)
-        self.embedding.forward(ctx.tokens, x, ctx)
-        ctx.normed.clear()
+        return self.run_units(ctx, 0, self.n_units(), want_rows, logits)
+
+    def run_units(self, ctx, lo, hi, want_rows=None, logits=None):
+        """Units lo..hi-1 of the step.  The residual stream stays in ctx.x between calls; nothing
+        else is handed from one call to the next (the last entry of a run prepares no norm for
+        whoever comes after it)."""
         n = len(self.schedule)
-        for i, e in enumerate(self.schedule):
-            block = self.blocks[e.layer]
-            if self._takes_next_norm[e.layer]:
-                nxt = self.blocks[self.schedule[i + 1].layer] if i + 1 < n else None
-                next_norm = getattr(nxt, "mixer_norm", None) if nxt is not None else self.final_norm
-                block.forward(x, ctx, e.cache, e.writes_cache, next_norm=next_norm)
-            else:
-                block.forward(x, ctx, e.cache, e.writes_cache)
-        if logits is not None and logits.shape[0] > 0:
-            R = logits.shape[0]
-            if want_rows is None and R == T and self.head.fuses_norm(self.final_norm, x, ctx):
-                self.head.forward_prenorm(x, self.final_norm, logits, ctx)
-            else:
-                h = ctx.ws.get("head.h", (R, self.dim), ctx.act_dtype)
-                self.final_norm.forward(x, h, ctx, row_index=want_rows)
-                self.head.forward(h, logits, ctx)
+        ctx.normed.clear()
+        for u in range(lo, hi):
+            if u == 0:
+                T = ctx.tokens.shape[0]
+                ctx.x = ctx.ws.get("x", (T, self.dim), torch.float32)
+                self.embedding.forward(ctx.tokens, ctx.x, ctx)
+            elif u <= n:
+                e = self.schedule[u - 1]
+                block = self.blocks[e.layer]
+                if self._takes_next_norm[e.layer]:
+                    next_norm = None
+                    if u + 1 < hi:                    # the consumer runs in this call
+                        nxt = self.blocks[self.schedule[u].layer] if u < n else None
+                        next_norm = self.final_norm if nxt is None else getattr(nxt, "first_norm", lambda: None)()
+                    block.forward(ctx.x, ctx, e.cache, e.writes_cache, next_norm=next_norm)
+                else:
+                    block.forward(ctx.x, ctx, e.cache, e.writes_cache)
+            elif logits is not None and logits.shape[0] > 0:
+                x = ctx.x
+                R, T = logits.shape[0], x.shape[0]
+                if want_rows is None and R == T and self.head.fuses_norm(self.final_norm, x, ctx):
+                    self.head.forward_prenorm(x, self.final_norm, logits, ctx)
+                else:
+                    h = ctx.ws.get("head.h", (R, self.dim), ctx.act_dtype)
+                    self.final_norm.forward(x, h, ctx, row_index=want_rows)
+                    self.head.forward(h, logits, ctx)
+        ctx.normed.clear()
         return logits
 
 

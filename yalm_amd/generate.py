@@ -22,6 +22,7 @@ class GenerationStats:
     batches: int = 0
     batch_sizes: List[int] = field(default_factory=list)
     batches_first_tokens: int = 0          # tokens sampled from prefill logits (not decode steps)
+    bytes_read: int = 0                    # what the steps had to read: weights once a step, live keys and values
 
     @property
     def prefill_tokens_per_second(self):
@@ -72,6 +73,7 @@ def generate(engine, prompts, max_new_tokens=256, temperature=0.0, seed=0, stop_
     stop = set(stop_ids)
     ids = list(request_ids) if request_ids is not None else list(range(len(prompts)))
     max_len = engine.n_positions
+    step_bytes = getattr(engine, "step_bytes", lambda slots: 0)
     results = [[] for _ in prompts]
     if max_new_tokens <= 0 or not prompts:
         return results
@@ -86,6 +88,7 @@ def generate(engine, prompts, max_new_tokens=256, temperature=0.0, seed=0, stop_
         try:
             t0 = time.perf_counter()
             logits = engine.step(slots, [prompts[i] for i in batch])
+            stats.bytes_read += step_bytes(slots)
             tokens = sampler.sample(logits, temperature, [ids[i] for i, _ in live], [0] * len(live))
             stats.prefill_seconds += time.perf_counter() - t0
             stats.prompt_tokens += sum(len(prompts[i]) for i in batch)
@@ -111,6 +114,7 @@ def generate(engine, prompts, max_new_tokens=256, temperature=0.0, seed=0, stop_
                 if not live:
                     break
                 logits = engine.step([s for _, s in live], [[results[i][-1]] for i, _ in live])
+                stats.bytes_read += step_bytes([s for _, s in live])
                 tokens = sampler.sample(logits, temperature, [ids[i] for i, _ in live],
                                         [len(results[i]) for i, _ in live])
                 stats.decode_steps += 1

@@ -9,7 +9,9 @@ it is in.  Kinds of parts and the methods each must have:
   mixer          cache_request() -> KVRequest | StateRequest | None
                  forward(h[T, dim], x_f32[T, dim], ctx, line, writes_cache): adds its output to x
   feed_forward   forward(h[T, dim], x_f32[T, dim], ctx): adds its output to x
-  block          forward(x_f32[T, dim], ctx, line, writes_cache): one layer on the residual stream
+  block          forward(x_f32[T, dim], ctx, line, writes_cache): one layer on the residual stream;
+                 optional: a `next_norm` argument (the norm that reads the stream after this layer, whose
+                 activations the layer may prepare) and first_norm() (the norm it applies first)
   embedding      forward(tokens_i32[T], x_f32[T, dim], ctx)
   head           forward(h[R, dim], logits_f32[R, vocab], ctx)
 
@@ -20,6 +22,12 @@ also leave, in ctx.normed[id(next_norm)], either (xn, ss, eps): the activations 
 multiplied by that norm's weights and the partial sums of squares (its residual-add GEMM
 writes them; up to 16 rows), or (h, None, None): the norm's finished output (more than 16 rows),
 which the next consumer takes instead of reading the residual stream.
+
+A part whose launches in a decode step depend on host values (it reads ctx.host_*, or sizes that
+change from step to step) says so with the class attribute `graph_safe = False`; the layers around
+it are still replayed from captured graphs.  A graph-safe part reads positions, lengths and slots
+from the step's device tensors only, and leaves rows with seq_slot -1 (padding) without effect on
+the cache or on per-sequence state.
 
 All of them: param_specs() -> [ParamSpec], load(get, compute_dtype, device),
 weight_bytes().  `h` is in the compute dtype (bfloat16 or float32); the

@@ -19,6 +19,11 @@ class PreNormResidualBlock(Part):
     def children(self):
         return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
 
+    def first_norm(self):
+        """The norm that reads the residual stream first when this layer runs (the layer before
+        may prepare its activations), or None."""
+        return self.mixer_norm
+
     def forward(self, x, ctx, line, writes_cache=True, next_norm=None):
         if self.mixer.fuses_norm(self.mixer_norm, x, ctx):
             self.mixer.forward_prenorm(x, self.mixer_norm, ctx, line, writes_cache,

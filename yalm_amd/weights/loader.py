@@ -2,13 +2,20 @@
 loader opens every *.safetensors of a model folder (convert.py:229-230), checks
 the declared set against the files in one pass, and fails with ONE error that
 lists missing tensors, unexpected tensors and wrong shapes (the reference's
-get_tensor / check_tensor, src/model.cpp:98-126, stop at the first).
+get_tensor / check_tensor, src/model.cpp:98-126, stop at the first).  Tensors
+that no part declared are not an error by themselves: the reference's converter
+picks what it needs by name and passes over the rest (convert.py:127-207), and
+real folders carry such extras (`...rotary_emb.inv_freq` buffers, an
+`lm_head.weight` stored next to a tied embedding); they are named in a warning,
+and in the error if there is one, where a misspelt name shows as a missing and
+an unexpected tensor side by side.
 
 Precision on the device: with compute dtype float32 every floating tensor
 becomes float32; with bfloat16, matrices become bfloat16 while a vector that is
 stored in 32-bit stays so (norm weights, model.cpp:156-161); integer tables
 become int32."""
 import os
+import sys
 from dataclasses import dataclass
 from typing import Optional, Tuple
 
@@ -69,8 +76,10 @@ class TensorSource:
     def get(self, name):
         return self.where[name].tensor(name)
 
-    def check(self, specs):
-        """Compares the declared tensors with the files; one error for everything."""
+    def check(self, specs, strict=False):
+        """Compares the declared tensors with the files; one error for everything.  Tensors that
+        nobody declared are an error only with strict=True; else they are passed over with a
+        warning.  Returns their names."""
         want = {}
         for s in specs:
             want[s.name] = s
@@ -83,7 +92,7 @@ class TensorSource:
                     wrong.append("%s: expected %s, found %s" % (n, list(s.shape), list(self.shape(n))))
                 elif not self.dtype(n).is_floating_point and s.init != "table":
                     wrong.append("%s: expected a floating-point tensor, found %s" % (n, self.dtype(n)))
-        if missing or unexpected or wrong:
+        if missing or wrong or (unexpected and strict):
             lines = ["the tensors in %s do not match the model:" % self.folder]
             if missing:
                 lines.append("  missing (%d): %s" % (len(missing), ", ".join(sorted(missing))))
@@ -92,6 +101,11 @@ class TensorSource:
             if wrong:
                 lines.append("  wrong shape or dtype (%d): %s" % (len(wrong), "; ".join(sorted(wrong))))
             raise WeightsError("\n".join(lines))
+        if unexpected:
+            shown = ", ".join(unexpected[:8]) + (", ..." if len(unexpected) > 8 else "")
+            sys.stderr.write("[yalm_amd] %d tensors in %s are not used by the model and are passed over: %s\n"
+                             % (len(unexpected), self.folder, shown))
+        return unexpected
 
 
 def device_dtype(stored_dtype, ndim, compute_dtype):
