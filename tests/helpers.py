@@ -19,20 +19,29 @@ BF16_MAX_TOL = 6e-2
 BF16_RMS_TOL = 2e-2
 
 
-def make_folder(tmp, name, cfg, seed=0, stored=torch.float32):
+def make_folder(tmp, name, cfg, seed=0, stored=torch.float32, device="cpu"):
     from yalm_amd.weights import write_random_model
     folder = os.path.join(str(tmp), "%s_%d_%s" % (name, seed, str(stored).split(".")[-1]))
     if not os.path.exists(os.path.join(folder, "model.safetensors")):
-        write_random_model(folder, cfg, seed=seed, dtype=stored)
+        write_random_model(folder, cfg, seed=seed, dtype=stored, device=device)
     return folder
 
 
 @functools.lru_cache(maxsize=None)
 def _folder_weights(folder, rounded):
-    cfg, w = R.read_folder(folder)
+    """The folder's tensors for the plain implementation, which widens each to float64 where it
+    uses it (layer by layer: a model of billions of elements never stands in float64 as a whole).
+    rounded: the values the engine's bfloat16 path stores."""
     if rounded:
-        w = {k: v.to(torch.bfloat16).to(torch.float64) for k, v in w.items()}
-    return cfg, w
+        cfg, w = _folder_weights(folder, False)           # tensors stored in bfloat16 are shared, not read again
+        return cfg, {k: v if v.dtype == torch.bfloat16 else v.to(torch.bfloat16) for k, v in w.items()}
+    return R.read_folder(folder)
+
+
+def forget_plain_results():
+    """Drops the cached weights and logits of the plain implementation (after a test with a big model)."""
+    plain_logits.cache_clear()
+    _folder_weights.cache_clear()
 
 
 @functools.lru_cache(maxsize=None)

@@ -227,3 +227,38 @@ def test_one_layer_at_the_width_of_the_big_models(tmp_path_factory, name, FULL_W
             want = helpers.plain_logits(folder, tuple(toks), "bfloat16")
             helpers.check_logits(got[rid], want, "bfloat16", "full width, request %s (%d tokens)" % (rid, len(toks)))
     assert not engine.cache.slots.held
+
+
+# the Mistral-7B-v0.2 shape at its real layer sizes and vocabulary, all 32 layers
+WHOLE_7B = dict(FULL_WIDTH, vocab_size=32000, num_hidden_layers=32, max_position_embeddings=32768)
+
+
+@pytest.fixture(scope="module")
+def folder_7b(tmp_path_factory):
+    folder = helpers.make_folder(tmp_path_factory.mktemp("layers_7b"), "layers_7b", WHOLE_7B, seed=21,
+                                 stored=torch.bfloat16, device="cuda:0")
+    yield folder
+    helpers.forget_plain_results()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_whole_mistral_7b_shape(folder_7b, dtype):
+    """All 32 layers of 4096 x 14336 with 32/8 heads of 128 and the head of 32000 x 4096: three requests of at
+    most 48 tokens, each alone and whole, with its last 32 tokens one by one, and as a batch of unequal
+    lengths, in the true 32-bit path and in bfloat16, against the plain implementation on the same
+    (bfloat16-stored) weights."""
+    from yalm_amd.engine import Engine, Model
+    model = Model.from_folder(folder_7b, dtype=helpers.torch_dtype(dtype), device="cuda:0")
+    engine = Engine(model, max_tokens=1024)
+    requests = helpers.random_requests(WHOLE_7B, [48, 33, 17], seed=22)
+    first = {"r0": 20, "r1": 33 - 5, "r2": 1}
+    for what, steps in (("whole", schedules.whole(requests)),
+                        ("last 32 one by one", schedules.tail_one_by_one(requests, 32)),
+                        ("a batch of unequal lengths", schedules.batches(requests, [list(requests)], first))):
+        got = schedules.per_request(steps, schedules.replay_in_process(engine, steps), requests)
+        for rid, toks in requests.items():
+            want = helpers.plain_logits(folder_7b, tuple(toks), dtype)
+            helpers.check_logits(got[rid], want, dtype, "7B sizes, 32 layers, %s, %s, request %s" % (dtype, what, rid))
+    assert not engine.cache.slots.held
+    del engine, model
+    torch.cuda.empty_cache()

@@ -79,10 +79,11 @@ def random_values(name, shape, init, fan_in, seed, device="cpu"):
     return out.reshape(shape)
 
 
-def write_random_model(folder, config, seed, dtype=torch.float32):
+def write_random_model(folder, config, seed, dtype=torch.float32, device="cpu"):
     """Writes config.json and model.safetensors for `config` (a config.json
     dictionary or a typed configuration) with weights drawn from `seed`, stored
-    in `dtype`.  Returns the folder."""
+    in `dtype`.  device: where the values are drawn (a GPU makes billions of them
+    in seconds).  Returns the folder."""
     from ..config import config_from_dict
     from ..engine.model import param_specs_of
     cfg = config_from_dict(config) if isinstance(config, dict) else config
@@ -91,7 +92,8 @@ def write_random_model(folder, config, seed, dtype=torch.float32):
     for spec in param_specs_of(cfg.to_spec()):
         if spec.optional:
             continue
-        tensors[spec.name] = random_values(spec.name, spec.shape, spec.init, spec.fan_in, seed).to(dtype)
+        tensors[spec.name] = random_values(spec.name, spec.shape, spec.init, spec.fan_in, seed,
+                                           device=device).to(dtype).cpu()
     write_file(os.path.join(folder, "model.safetensors"), tensors, {"format": "pt", "seed": seed})
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(cfg.to_dict(), f, indent=1)
