@@ -88,7 +88,10 @@ GEMM_SHAPES = [(1, 16, 256), (3, 70, 96), (64, 130, 264), (65, 64, 80), (200, 33
                (130, 100, 50), (65, 64, 64), (200, 333, 1024), (300, 20480 + 8, 128), (513, 130, 192),
                # K a multiple of 64 (operands staged in LDS by DMA): few and odd rows, every row count of a stage
                (5, 70, 192), (16, 4112, 128), (9, 100, 64), (12, 33, 320), (8, 26000, 64), (13, 13000, 128),
-               (3, 4096, 1024), (20, 70, 192), (33, 4112, 128), (50, 100, 64), (64, 333, 320)]
+               (3, 4096, 1024), (20, 70, 192), (33, 4112, 128), (50, 100, 64), (64, 333, 320),
+               # widths of the big models' projections and rows that end inside a tile
+               (8, 3072, 128), (5, 6144, 64), (16, 5120, 192), (3, 2048, 64), (7, 1000, 64), (9, 6010, 128),
+               (1, 3080, 256), (12, 4100, 64)]
 
 
 @pytest.mark.parametrize("simple", [False, True])
@@ -738,8 +741,61 @@ def test_gemm_norm_qkv_rope(n_heads, n_kv, hd, rd, D):
     assert (vp.float().abs().sum(dim=(1, 2)) > 0).equal(touched)
 
 
+@pytest.mark.parametrize("M", [1, 5, 16])
+@pytest.mark.parametrize("n_heads,n_kv,hd,rd,D", [(4, 2, 16, 16, 64), (3, 1, 48, 48, 80), (6, 3, 32, 16, 192),
+                                                   (32, 8, 128, 128, 128), (24, 8, 128, 128, 64), (10, 5, 64, 64, 256)])
+def test_gemm_chain_qkv_rope(n_heads, n_kv, hd, rd, D, M):
+    """The q/k/v projection of a decode step from activations a producer emitted (already multiplied by the
+    norm's weights, with partial sums of squares), with rotation and cache write in its epilogue; among the
+    shapes the 6144 and 5120 weight rows of the big models' projections."""
+    k = K()
+    PAGE = k.PAGE
+    rng = np.random.default_rng(M)
+    pos = [int(p) for p in rng.integers(0, 190, size=M)]
+    slots = [int(s) for s in rng.permutation(M + 2)[:M]]
+    if M > 2:
+        slots[2] = -1                                  # a padding row
+    Q, KV = n_heads * hd, n_kv * hd
+    x = rnd((M, D), 57, scale=2.0)
+    nw = 1 + 0.1 * rnd((D,), 58)
+    w = rnd((Q + 2 * KV, D), 59, torch.bfloat16, scale=1 / math.sqrt(D))
+    xn = (x * nw).to(torch.bfloat16)
+    parts = 3
+    ss = torch.zeros((M, parts))
+    for p_, cols in enumerate(np.array_split(np.arange(D), parts)):
+        ss[:, p_] = (x[:, cols].double() ** 2).sum(dim=1).float()
+    table = make_table(200, hd, rd, 10000.0)
+    ring, n_pages = 3, 64
+    bt = torch.tensor(rng.permutation(n_pages)[: (M + 2) * ring].reshape(M + 2, ring), dtype=torch.int32)
+    kp = torch.zeros((n_pages, n_kv, PAGE, hd), dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros((n_pages, n_kv, hd, PAGE), dtype=torch.bfloat16, device=DEV)
+    q_out = torch.zeros((M, Q), dtype=torch.bfloat16, device=DEV)
+    k.gemm_chain_qkv_rope(xn.to(DEV), (ss.to(DEV), 1e-5), w.to(DEV), q_out, kp, vp, bt.to(DEV), ring, i32(pos),
+                          i32(slots), table.to(DEV), n_heads, n_kv, hd, rd)
+    scale = 1.0 / torch.sqrt((x.double() ** 2).mean(dim=1, keepdim=True) + 1e-5)
+    qkv = (xn.double() @ w.double().T) * scale
+    f = R.rope_inv_freq(hd, rd, 10000.0)
+    p = torch.tensor(pos)
+    q_want = R.rope_interleaved(qkv[:, :Q].reshape(M, n_heads, hd), p, f).reshape(M, Q)
+    k_want = R.rope_interleaved(qkv[:, Q:Q + KV].reshape(M, n_kv, hd), p, f)
+    v_want = qkv[:, Q + KV:].reshape(M, n_kv, hd)
+    close(q_out, q_want, torch.bfloat16, "q", factor=1.5)
+    kp, vp = kp.cpu(), vp.cpu()
+    touched = torch.zeros((n_pages, PAGE), dtype=torch.bool)
+    for m in range(M):
+        if slots[m] < 0:
+            continue
+        page, r = int(bt[slots[m], (pos[m] // PAGE) % ring]), pos[m] % PAGE
+        close(kp[page, :, r, :], k_want[m], torch.bfloat16, "k row %d" % m, factor=1.5)
+        close(vp[page, :, :, r], v_want[m], torch.bfloat16, "v row %d" % m, factor=1.5)
+        touched[page, r] = True
+    assert (kp.float().abs().sum(dim=(1, 3)) > 0).equal(touched)
+    assert (vp.float().abs().sum(dim=(1, 2)) > 0).equal(touched)
+
+
 @pytest.mark.parametrize("M,N,Kd", [(1, 64, 256), (8, 4096, 1000), (33, 80, 96), (64, 4096, 264), (5, 16400, 64),
-                                    (11, 192, 192), (16, 4096, 128), (9, 1024, 64)])
+                                    (11, 192, 192), (16, 4096, 128), (9, 1024, 64), (8, 3072, 128), (3, 3000, 64),
+                                    (20, 3072, 64)])
 def test_gemm_chain_producer_and_consumer(M, N, Kd):
     """A residual-add GEMM that emits the next norm's activations and partial sums of squares,
     and a consumer that scales by them: together they equal rmsnorm(x_new) @ W2^T."""
