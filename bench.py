@@ -10,7 +10,11 @@ shape with its window of 4,096 positions and prompts of 6,000 tokens).
 
 A step is one decode step as generation does it: the step function for a batch
 of sequences (one token each, from the cache), greedy sampling on the device
-and the read-back of the tokens.  One JSON line is printed.  Peaks are MI355X's
+and the read-back of the tokens.  The shape's workload decodes over a range of
+positions (2,048 to 4,096 for the default shape); a run of K steps takes the K
+positions in the middle of that range, so that its mean context is the whole
+range's (K = 2,048 is the range itself), by prefilling that many random tokens.
+One JSON line is printed.  Peaks are MI355X's
 published ones: HBM 8 TB/s; dense MFMA bf16/fp16 2.5 PFLOP/s, fp32 157.3 TFLOP/s."""
 import argparse
 import json
@@ -39,11 +43,11 @@ LLAMA_3B = {
 }
 # Mistral-7B-v0.1 shape (a window of 4,096 positions: ring cache)
 MISTRAL_7B_V01 = dict(MISTRAL_7B, rope_theta=10000.0, sliding_window=4096)
-# shape -> (config, name, context, prompt length of the decode runs)
+# shape -> (config, name, context, first and last position of the workload's decoding)
 SHAPES = {
-    "mistral-7b-v0.2": (MISTRAL_7B, "Mistral-7B-v0.2 shape", 4096, 2048),
-    "llama-3.2-3b": (LLAMA_3B, "Llama-3.2-3B shape", 8192, 512),
-    "mistral-7b-v0.1": (MISTRAL_7B_V01, "Mistral-7B-v0.1 shape", 8192, 6000),
+    "mistral-7b-v0.2": (MISTRAL_7B, "Mistral-7B-v0.2 shape", 4096, (2048, 4096)),
+    "llama-3.2-3b": (LLAMA_3B, "Llama-3.2-3B shape", 8192, (512, 8192)),
+    "mistral-7b-v0.1": (MISTRAL_7B_V01, "Mistral-7B-v0.1 shape", 8192, (6000, 7024)),
 }
 PREFILL = 2048                   # tokens of the timed prompt
 HBM_PEAK = 8.0e12
@@ -71,7 +75,9 @@ def main():
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--points", default="1,64", help="further batch sizes to measure")
     ap.add_argument("--no-prefill", action="store_true")
-    ap.add_argument("--prompt-len", type=int, default=0, help="tokens every sequence holds before decoding (0: the shape's)")
+    ap.add_argument("--prompt-len", type=int, default=0,
+                    help="tokens every sequence holds before decoding (0: so that the run lies in the middle of the "
+                         "shape's range of positions)")
     ap.add_argument("--prefill-len", type=int, default=PREFILL, help="tokens of the timed prompt")
     ap.add_argument("--shape", default="mistral-7b-v0.2", choices=sorted(SHAPES),
                     help="the layer sizes: the Mistral-7B-v0.2 shape (default), Llama-3.2-3B or Mistral-7B-v0.1")
@@ -85,10 +91,13 @@ def main():
     from yalm_amd.cache import PAGE
 
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
-    CFG, shape_name, CONTEXT, PROMPT = SHAPES[args.shape]
+    CFG, shape_name, CONTEXT, (first, last) = SHAPES[args.shape]
+    # the timed steps' positions lie in the middle of the workload's range (all of it if they are as many)
+    run = args.steps + args.warmup
+    PROMPT = max(first, min((first + last - args.steps) // 2 - args.warmup, last - run))
     if args.prompt_len:
         PROMPT = args.prompt_len
-        CONTEXT = max(CONTEXT, PROMPT + args.steps + args.warmup + 64)
+    CONTEXT = max(CONTEXT, PROMPT + run + 64)
     PREFILL_LEN = args.prefill_len
     n_layers = args.layers or CFG["num_hidden_layers"]
     dev = "cuda:0"
