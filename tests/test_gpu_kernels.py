@@ -408,6 +408,54 @@ def test_attn_prefill(n_heads, n_kv, hd, window, lens, dtype, simple):
     close(out, packed_attention_reference(q, kk, v, lens, n_heads, n_kv, hd, window), dtype, "prefill attention")
 
 
+def masked_attention_float64(q, k, v, n_heads, n_kv, hd, window):
+    """softmax(q k^T / sqrt(hd) + mask) v for one sequence, all positions at once (float64)."""
+    n = q.shape[0]
+    qh = q.double().reshape(n, n_heads, hd).transpose(0, 1)
+    kh = k.double().reshape(n, n_kv, hd).transpose(0, 1).repeat_interleave(n_heads // n_kv, dim=0)
+    vh = v.double().reshape(n, n_kv, hd).transpose(0, 1).repeat_interleave(n_heads // n_kv, dim=0)
+    i = torch.arange(n)[:, None]
+    j = torch.arange(n)[None, :]
+    visible = (j <= i) & ((i - j < window) if window else torch.ones((n, n), dtype=torch.bool))
+    out = torch.empty((n_heads, n, hd), dtype=torch.float64)
+    for h in range(n_heads):                          # a head at a time: [n, n] scores
+        s = (qh[h] @ kh[h].T) / math.sqrt(hd)
+        s = s.masked_fill(~visible, float("-inf"))
+        out[h] = torch.softmax(s, dim=-1) @ vh[h]
+    return out.transpose(0, 1).reshape(n, n_heads * hd)
+
+
+@pytest.mark.parametrize("n_heads,n_kv,hd,window,lens", [(40, 8, 64, 0, [1700]), (40, 8, 128, 300, [1500, 260]),
+                                                         (32, 8, 128, 0, [2048])])
+def test_attn_prefill_with_many_and_with_few_workgroups(n_heads, n_kv, hd, window, lens):
+    """The matrix-core prefill kernel has two forms: workgroups of eight waves that take a tile's keys in two
+    halves (launches of at most two workgroups a compute unit, the third case) and of four waves (more, the
+    first two).  Both against a float64 masked softmax, itself checked against the plain implementation."""
+    k = K()
+    dtype = torch.bfloat16
+    small = [rnd((70, 2 * 16), 31), rnd((70, 16), 32), rnd((70, 16), 33)]
+    assert torch.allclose(masked_attention_float64(*small, 2, 1, 16, 9),
+                          R.attention(small[0].reshape(70, 2, 16), small[1].reshape(70, 1, 16),
+                                      small[2].reshape(70, 1, 16), 9).reshape(70, 32), atol=1e-12)
+    T = sum(lens)
+    q = rnd((T, n_heads * hd), 13, dtype)
+    kk = rnd((T, n_kv * hd), 14, dtype)
+    v = rnd((T, n_kv * hd), 15, dtype)
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    seq = np.repeat(np.arange(len(lens)), lens)
+    pos = np.concatenate([np.arange(n) for n in lens])
+    ks, vs, tile0 = stage(kk, v, lens, n_kv, hd, dtype)
+    out = torch.empty((T, n_heads * hd), dtype=dtype, device=DEV)
+    order = i32(k.prefill_tile_order(lens))
+    k.attn_prefill(q.to(DEV), ks.to(DEV), vs.to(DEV), out, i32(cu), i32(tile0), i32(seq), i32(pos), n_heads, n_kv, hd,
+                   window, order)
+    want, o = [], 0
+    for n in lens:
+        want.append(masked_attention_float64(q[o:o + n], kk[o:o + n], v[o:o + n], n_heads, n_kv, hd, window))
+        o += n
+    close(out, torch.cat(want), dtype, "prefill attention")
+
+
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens", [
     (8, 2, 128, 0, [200]), (5, 5, 64, 0, [129, 1, 640]), (4, 1, 64, 70, [300, 64, 1]), (40, 8, 128, 0, [700]),
     (24, 8, 64, 100, [1100, 90]), (8, 2, 128, 0, [2200, 90, 2100])])

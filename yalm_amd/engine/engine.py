@@ -13,6 +13,7 @@ read positions, lengths, slots and block tables from device memory, so the
 graph needs no patching from step to step (the reference patches kernel nodes
 every step, src/infer.cu:1225-1247).  Rows that pad a batch to its bucket
 carry slot -1 and change no result."""
+import sys
 from collections import OrderedDict
 
 import numpy as np
@@ -96,6 +97,8 @@ class Engine:
         self.max_graphs = max(1, int(max_graphs))
         self._segments = model.decode_segments()        # the parts are fixed from here on: asked once, not every step
         self._any_graph = any(safe for safe, _, _ in self._segments)
+        for text in model.describe()[1]:                # a slow fallback is said once, not hidden
+            sys.stderr.write("[yalm_amd] %s\n" % text)
         self._graphs = OrderedDict()                    # (batch bucket, pages bucket) -> _DecodeGraph, least recently used first
         self._buckets = {}
         self.graphs_captured = 0

@@ -160,6 +160,20 @@ class Model:
                 out.append((safe, u, u + 1))
         return out
 
+    def describe(self):
+        """({line on the kernels that serve a part: the schedule entries it stands for}, the lines that
+        name a slow fallback), at the model's compute dtype."""
+        lines, slow = {}, []
+        for i, e in enumerate(self.schedule):
+            for p in _walk(self.blocks[e.layer]):
+                text, is_slow = p.describe(self.compute_dtype)
+                entries = lines.setdefault(text, [])
+                if i not in entries:
+                    entries.append(i)
+                if is_slow and text not in slow:
+                    slow.append(text)
+        return lines, slow
+
     def weight_bytes(self):
         """Bytes of weights a step reads: every weight once, one embedding row."""
         total = self.embedding.weight_bytes() + self.final_norm.weight_bytes() + self.head.weight_bytes()

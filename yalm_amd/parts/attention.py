@@ -65,6 +65,18 @@ class GQAttention(Part):
     def cache_request(self):
         return KVRequest(self.n_kv_heads, self.head_dim, self.window)
 
+    def describe(self, compute_dtype):
+        what = "attention, %d heads in %d groups of head size %d%s" % (
+            self.n_heads, self.n_kv_heads, self.head_dim, ", window %d" % self.window if self.window else "")
+        if compute_dtype != torch.bfloat16:
+            return what + ": float32-arithmetic kernels", False
+        group = self.n_heads // self.n_kv_heads
+        if self.head_dim in (64, 128) and group <= 16:
+            return what + ": matrix-core kernels", False
+        why = "head size %d" % self.head_dim if self.head_dim not in (64, 128) else "%d heads a group" % group
+        return what + ": float32-arithmetic kernels on bfloat16 storage (the matrix-core kernels take head sizes " \
+                      "64 and 128 and up to 16 heads a group, not %s): correct, several times slower" % why, True
+
     def decode_splits(self, B, max_pages):
         mfma = self.head_dim in (64, 128) and self.n_heads // self.n_kv_heads <= 16 and not kernels.FORCE_SIMPLE
         if mfma:         # a workgroup of 4 waves per (split, KV head, sequence), a page per wave at a time

@@ -92,6 +92,11 @@ class Part:
     def children(self):
         return []
 
+    def describe(self, compute_dtype):
+        """(one line on which kernels serve this part at the compute dtype, True if that is a slow
+        fallback the user should know of)."""
+        return type(self).__name__, False
+
     @staticmethod
     def _gemm(ctx, a, w, out, epilogue, hidden=0):
         """kernels.gemm with the scratch that lets small batches split K."""
