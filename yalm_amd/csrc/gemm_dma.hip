@@ -1,21 +1,24 @@
-// Prefill GEMM whose k tiles go from global memory straight into LDS:
-// C = epilogue(A[M,K] * W[N,K]^T), bfloat16 operands, float32 accumulation, more than 64 rows.
+// GEMMs of more than 64 rows whose k tiles go from global memory straight into LDS:
+// C = epilogue(A[M,K] * W[N,K]^T), bfloat16 operands, float32 accumulation.
 //
-// A workgroup owns a TM x TN tile of C.  Its waves issue global_load_lds_dwordx4 (16 bytes a
-// lane, a wave's 64 lanes land as 1 KB contiguous in LDS) for k tile kt + S - 1 into a ring
-// of S stages while they multiply k tile kt; no register or LDS write instruction stands
-// between memory and the matrix cores.  Rows are kept unpadded (128 bytes for 64 k) and the
-// 16-byte chunks of a row are XOR-swizzled by the row number, which every lane applies to
-// the GLOBAL address it asks for, so that the b128 fragment reads of 16 consecutive rows
-// fall on different banks.  The compiler does not know that these loads write LDS: the
-// kernel waits for them itself (s_waitcnt vmcnt) and uses the bare s_barrier, because
-// __syncthreads() carries a fence that would wait for the loads of all stages.
+// A workgroup owns a tile of C.  Its waves issue global_load_lds_dwordx4 (16 bytes a lane, a
+// wave's 64 lanes land as 1 KB contiguous in LDS) for later k tiles while they multiply the
+// current one; no register or LDS write instruction stands between memory and the matrix
+// cores.  Rows are kept unpadded (128 bytes for 64 k) and the 16-byte chunks of a row are
+// XOR-swizzled by the row number, which every lane applies to the GLOBAL address it asks
+// for, so that the b128 fragment reads of 16 consecutive rows fall on different banks.  The
+// compiler does not know that these loads write LDS: the kernels wait for them themselves
+// (s_waitcnt vmcnt) and use the bare s_barrier, because __syncthreads() carries a fence that
+// would wait for the loads of all stages.
 //
-// With few tiles (a decode batch of more than 64 rows) K is split over grid z as well: every slice
-// writes its float32 partial product and yalm_splitk_reduce adds them in order and applies the epilogue.
+// Two kernels.  gemm_dma_kernel (128x128 tiles, two stages, two workgroups a CU) serves decode batches
+// of more than 64 rows: with few tiles K is split over grid z as well, every slice writes its float32
+// partial product and yalm_splitk_reduce adds them in order and applies the epilogue.  gemm_ring_kernel
+// (256-row tiles, five slots in turn, loads issued between the products) serves prompt steps.
 //
 // Takes any M and N and K % 64 == 0; other shapes are refused (YALM_ERR_ARG) and the
-// caller runs the kernel of gemm_mfma.hip.  Sums are in a fixed order for a given shape.
+// caller runs the kernel of gemm_mfma.hip.  Sums are in a fixed order for a given shape, and the
+// same order in both kernels.
 #include "common.h"
 #include "yalm_hip.h"
 
@@ -213,6 +216,242 @@ int launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int
   return yalm_splitk_reduce(partial, C, M, N, H, (int)grid.z, EPI, stream);
 }
 
+// ---------------------------------------------------------------------------
+// The kernel for many tiles: 256 x TN tiles, 8 waves, and a ring of five 32 KB slots that holds the k tiles of
+// W and of A in turn (W0 A0 W1 A1 W2 ...; tile t has W in slot 2t mod 5 and A in slot (2t + 1) mod 5), so that
+// two and a half k tiles are in flight or in use.  What it does differently from the kernel above, each measured:
+//  * a vector memory instruction holds its wave for tens of clocks, more while the memory system is busy; issued
+//    as a burst behind the barrier they stall every wave at once and the matrix cores idle.  Here a wave issues
+//    one DMA instruction in every few products, all through the iteration, and each has a k step or more to land;
+//  * the barrier stands between k steps 2 and 3 of a tile: the fragments of the last k step are in registers by
+//    then, so nobody reads the tile's slots any more and they are refilled at once, and the first fragments
+//    of the next tile are read while the last products of this one run;
+//  * the fragments of a k step are read during the products of the one before (two register sets);
+//  * the DMA takes its base from scalar registers and a 32-bit offset a lane (inline asm: the compiler would
+//    add a 64-bit pair a lane for every instruction).
+// The order of statements in the loop is the order of the instructions: a scheduling fence follows each.
+// ---------------------------------------------------------------------------
+constexpr int RING_SLOT = 32768, RING_SLOTS = 5, RING_TM = 256;
+
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0x3F | (0x7 << 4) | (0x0 << 8) | (0x3 << 14)); }
+
+// the product index of a k step (of n_products) behind which DMA instruction d of n_dma is issued
+__host__ __device__ constexpr int dma_place(int d, int n_dma, int n_products) { return (d + 1) * n_products / (n_dma + 1) - 1 < 0 ? 0 : (d + 1) * n_products / (n_dma + 1) - 1; }
+
+template <int EPI, int TN, int MAP>
+__global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                           void* __restrict__ Cv, int M, int N, int K, int H, int n_tile0,
+                                                           int n_tiles) {
+  constexpr int TM = RING_TM, NW = 8, NWM = 4, NWN = 2, WM = TM / NWM, WN = TN / NWN, FA = WM / 32, FB = WN / 32;
+  constexpr int KS = TK / 16;
+  constexpr int DA = (TM / 8) / NW, DW = (TN / 8) / NW;     // DMA instructions (8 rows each) a wave and slot
+  constexpr int DA1 = DA / 2, DW1 = (DW + 1) / 2;           // of them in the first of the two k steps that issue them
+  constexpr int NMF = FA * FB;                              // products a k step
+  static_assert(TM % (8 * NW) == 0 && TN % (8 * NW) == 0 && DA % 2 == 0, "the rows of a slot must divide over the waves");
+  static_assert(FA + FB <= NMF, "a fragment read follows a product");
+  static_assert(EPI != 3 || FB % 2 == 0, "the gated epilogue pairs column tiles");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char stages[];
+  const int tid = threadIdx.x, lane = tid % WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  const int wm = wave / NWN, wn = wave % NWN;
+  const int li = lane % 32, lh = lane / 32;
+  int tile_m, tile_n;
+  if (MAP == 0) {
+    tile_m = blockIdx.y;
+    tile_n = blockIdx.x + n_tile0;
+  } else {
+    // Workgroup L runs on XCD L mod 8.  Every XCD takes a run of the tile sequence (groups of MAP tile columns;
+    // in a group the rows fastest, then the columns), so that the tiles it works on at a time share rows and
+    // columns in its second-level cache.
+    const int mt = (M + TM - 1) / TM, T = mt * n_tiles, chunk = (T + 7) / 8;
+    const int L = blockIdx.x, t = (L % 8) * chunk + L / 8;
+    if (t >= T || L / 8 >= chunk) return;
+    const int per_group = mt * MAP, g = t / per_group, r = t % per_group;
+    const int width = min(MAP, n_tiles - g * MAP);        // the last group may be narrower
+    tile_n = n_tile0 + g * MAP + r % width;
+    tile_m = r / width;
+  }
+  const int m0 = tile_m * TM, n0 = tile_n * TN;
+  const int nk = K / TK;
+
+  // DMA instruction i of a wave fills rows (i * 8 + wave) * 8 ... + 7 of a slot; a lane's place there is (row,
+  // 16-byte slot of the row), and it asks memory for the chunk that belongs there (rows past the edge repeat the
+  // last one and are never stored)
+  unsigned off_a[DA], off_w[DW];
+  const char* a_base = (const char*)(A + (size_t)m0 * K);
+  const char* w_base = (const char*)(W + (size_t)n0 * K);
+#pragma unroll
+  for (int i = 0; i < DA; ++i) {
+    const int row = (i * NW + wave) * RPI + lane / CPR;
+    off_a[i] = (unsigned)(((size_t)min(row, M - 1 - m0) * K + ((lane % CPR) ^ swizzle_of(row)) * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < DW; ++i) {
+    const int row = (i * NW + wave) * RPI + lane / CPR;
+    off_w[i] = (unsigned)(((size_t)min(row, N - 1 - n0) * K + ((lane % CPR) ^ swizzle_of(row)) * 8) * 2);
+  }
+  auto dma = [&](const char* base, unsigned off, int slot, int i) {
+    const unsigned lds_addr = (unsigned)(uintptr_t)(stages + slot * RING_SLOT + (i * NW + wave) * 1024);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(off), "s"(base) : "memory");
+  };
+
+  f32x16 acc[FA][FB];
+#pragma unroll
+  for (int a = 0; a < FA; ++a)
+#pragma unroll
+    for (int b = 0; b < FB; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+
+  // fragments: A rows of the wave's row tiles; W rows of its column tiles, where for the gated epilogue even tiles
+  // are the gate rows and odd tiles the up rows of two 16-row blocks.  Address in a slot: row * 128 + ((2 ks + lh)
+  // ^ swizzle) * 16; tiles 32 (16, 64) rows apart share the swizzle.
+  const int a_row = wm * WM + li;
+  const int w_row = (EPI == 3) ? wn * WN + (li / 16) * 32 + (li % 16) : wn * WN + li;
+  int a_at[KS], w_at[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    a_at[ks] = a_row * ROWB + (((2 * ks + lh) ^ swizzle_of(a_row)) << 4);
+    w_at[ks] = w_row * ROWB + (((2 * ks + lh) ^ swizzle_of(w_row)) << 4);
+  }
+  auto frag_a = [&](int slot, int ks, int a) {
+    return *reinterpret_cast<const bf16x8*>(stages + slot * RING_SLOT + a_at[ks] + a * 32 * ROWB);
+  };
+  auto frag_w = [&](int slot, int ks, int b) {
+    const int rows = (EPI == 3) ? (b / 2) * 64 + (b % 2) * 16 : b * 32;
+    return *reinterpret_cast<const bf16x8*>(stages + slot * RING_SLOT + w_at[ks] + rows * ROWB);
+  };
+
+  // before the loop: W0 A0 W1 and the first half of A1 (what iterations -2 and -1 would have issued)
+#pragma unroll
+  for (int i = 0; i < DW; ++i) dma(w_base, off_w[i], 0, i);
+#pragma unroll
+  for (int i = 0; i < DA; ++i) dma(a_base, off_a[i], 1, i);
+  if (nk > 1) {
+#pragma unroll
+    for (int i = 0; i < DW; ++i) dma(w_base + ROWB, off_w[i], 2, i);
+#pragma unroll
+    for (int i = 0; i < DA1; ++i) dma(a_base + ROWB, off_a[i], 3, i);
+    wait_vmcnt<DW + DA1>();
+  } else {
+    wait_vmcnt<0>();
+  }
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  bf16x8 fa[2][FA], fw[2][FB];
+#pragma unroll
+  for (int a = 0; a < FA; ++a) fa[0][a] = frag_a(1, 0, a);
+#pragma unroll
+  for (int b = 0; b < FB; ++b) fw[0][b] = frag_w(0, 0, b);
+
+  int ws = 0, as = 1;                              // slots of the tile that is multiplied
+  for (int kt = 0; kt < nk; ++kt) {
+    const int ws1 = ws + 2 >= RING_SLOTS ? ws + 2 - RING_SLOTS : ws + 2;          // of tile kt + 1
+    const int as1 = as + 2 >= RING_SLOTS ? as + 2 - RING_SLOTS : as + 2;
+    const int ws2 = ws1 + 2 >= RING_SLOTS ? ws1 + 2 - RING_SLOTS : ws1 + 2;       // of tile kt + 2
+    const int as2 = as1 + 2 >= RING_SLOTS ? as1 + 2 - RING_SLOTS : as1 + 2;
+    const bool t1 = kt + 1 < nk, t2 = kt + 2 < nk;
+    const char* a1 = a_base + (size_t)(kt + 1) * ROWB;
+    const char* a2 = a_base + (size_t)(kt + 2) * ROWB;
+    const char* w2 = w_base + (size_t)(kt + 2) * ROWB;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int c = ks & 1, n = c ^ 1;
+      if (ks == KS - 1) {
+        // The last fragments of tile kt are in registers; this wave's share of tile kt + 1 has landed (the second
+        // half of A(kt + 1) from k step 0, and everything older; W(kt + 2) may still be on its way).  Behind the
+        // barrier that holds for all waves: tile kt + 1 can be read and the slots of tile kt written.
+        wait_lgkmcnt0();
+        if (t2) wait_vmcnt<DW>(); else wait_vmcnt<0>();
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int j = 0; j < NMF; ++j) {
+        const int a = j % FA, b = j / FA;
+        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[c][a], fw[c][b], acc[a][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (ks < KS - 1) {                           // a fragment of k step ks + 1 of this tile
+          if (j < FA) fa[n][j] = frag_a(as, ks + 1, j);
+          else if (j < FA + FB) fw[n][j - FA] = frag_w(ws, ks + 1, j - FA);
+        } else {                                     // of k step 0 of the next tile (behind the last tile: read, never used)
+          if (j < FA) fa[n][j] = frag_a(as1, 0, j);
+          else if (j < FA + FB) fw[n][j - FA] = frag_w(ws1, 0, j - FA);
+        }
+        // k step 0: the second half of A(kt + 1); 1 and 2: W(kt + 2); 3, behind the barrier: the first half of A(kt + 2)
+        if (ks == 0) {
+#pragma unroll
+          for (int d = 0; d < DA - DA1; ++d)
+            if (j == dma_place(d, DA - DA1, NMF) && t1) dma(a1, off_a[DA1 + d], as1, DA1 + d);
+        } else if (ks == 1) {
+#pragma unroll
+          for (int d = 0; d < DW1; ++d)
+            if (j == dma_place(d, DW1, NMF) && t2) dma(w2, off_w[d], ws2, d);
+        } else if (ks == 2) {
+#pragma unroll
+          for (int d = 0; d < DW - DW1; ++d)
+            if (j == dma_place(d, DW - DW1, NMF) && t2) dma(w2, off_w[DW1 + d], ws2, DW1 + d);
+        } else {
+#pragma unroll
+          for (int d = 0; d < DA1; ++d)
+            if (j == dma_place(d, DA1, NMF) && t2) dma(a2, off_a[d], as2, d);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    ws = ws1;
+    as = as1;
+  }
+  wait_vmcnt<0>();                                 // nothing of this workgroup is on its way into LDS when it ends
+
+#pragma unroll
+  for (int a = 0; a < FA; ++a) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int m = m0 + wm * WM + a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+      if (m >= M) continue;
+      if (EPI == 3) {
+#pragma unroll
+        for (int pp = 0; pp < FB / 2; ++pp) {
+          const int hcol = (n0 + wn * WN + pp * 64) / 2 + li;
+          if (hcol < H)
+            ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
+        }
+      } else {
+#pragma unroll
+        for (int b = 0; b < FB; ++b) {
+          const int nn = n0 + wn * WN + b * 32 + li;
+          if (nn >= N) continue;
+          const size_t o = (size_t)m * N + nn;
+          if (EPI == 0) ((float*)Cv)[o] = acc[a][b][r];
+          if (EPI == 1) ((bf16*)Cv)[o] = static_cast<bf16>(acc[a][b][r]);
+          if (EPI == 2) ((float*)Cv)[o] += acc[a][b][r];
+        }
+      }
+    }
+  }
+}
+
+// column tiles n_tile0 ... n_tile0 + n_tiles - 1 (n_tiles < 0: to the last) of a 256 x TN tiling
+template <int EPI, int TN, int MAP>
+int launch_ring(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream, int n_tile0 = 0,
+                int n_tiles = -1) {
+  if (n_tiles < 0) n_tiles = ceil_div(N, TN) - n_tile0;
+  const int mt = ceil_div(M, RING_TM);
+  const dim3 grid = MAP == 0 ? dim3(n_tiles, mt, 1) : dim3(8 * ceil_div(mt * n_tiles, 8), 1, 1);
+  const size_t lds = (size_t)RING_SLOTS * RING_SLOT;
+  static bool allowed = false;                     // more than 64 KB of LDS has to be asked for once
+  if (!allowed) {
+    hipError_t e = hipFuncSetAttribute((const void*)&gemm_ring_kernel<EPI, TN, MAP>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return (int)e;
+    allowed = true;
+  }
+  gemm_ring_kernel<EPI, TN, MAP><<<grid, 512, lds, stream>>>(A, W, C, M, N, K, H, n_tile0, n_tiles);
+  return launch_status();
+}
+
 // slices of K for the 128x128 tiles: with few rows (a big decode batch) the tiles alone leave most CUs
 // without work and the weights would stream through a few of them
 int slices_for(int M, int N, int K, long workspace_floats) {
@@ -224,35 +463,47 @@ int slices_for(int M, int N, int K, long workspace_floats) {
   return slices;
 }
 
-// 256x256 tiles (8 waves, two stages of 64 KB, one workgroup a CU) ask the caches for the
-// fewest bytes per product; 128x128 tiles (4 waves, two workgroups a CU) where those would
-// leave CUs without work.
+// Which kernel takes a shape.  Prompt steps (384 rows and more) go to the ring kernel; fewer rows (decode batches
+// of more than 64 rows) to 128x128 tiles with K split over workgroups.
+bool takes_ring(int M) { return M >= 384; }
+
+// Time of a ring launch, in rounds of 256x256 tiles: a tile of 192 (128) columns costs 0.81 (0.63) of one of 256
+// (measured at 8,192 x 4,096 x 14,336: 350, 283 and 221 us a round), and a last round that fills the fraction f
+// of the CUs costs 0.45 + 0.55 f of a full one (the chip clocks higher with fewer CUs at work).
+double ring_cost(long tiles, double tile_cost) {
+  const long rounds = tiles / 256, rest = tiles % 256;
+  return ((double)rounds + (rest ? 0.45 + 0.55 * (double)rest / 256.0 : 0.0)) * tile_cost;
+}
+
+// 256-row tiles of 256, 192 or 128 columns, or whole rounds of 256x256 tiles and the remaining columns in a second
+// launch of 256x128 tiles: whichever the cost model puts first (2,048 x 6,144: 192 columns, 256 tiles for 256 CUs;
+// 2,048 x 4,096: 128 columns; 2,048 x 28,672: three rounds of 256x256 and one of 256x128).
+template <int EPI>
+int launch_ring_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
+  const int mt = ceil_div(M, 256), nt = ceil_div(N, 256);
+  const double c256 = ring_cost((long)mt * nt, 1.0);
+  const double c192 = EPI == 3 ? 1e30 : ring_cost((long)mt * ceil_div(N, 192), 0.81);
+  const double c128 = ring_cost((long)mt * ceil_div(N, 128), 0.63);
+  const int nt_main = (int)(((long)mt * nt / 256) * 256 / mt);
+  double c_two = 1e30;
+  if (nt_main > 0 && nt_main < nt)
+    c_two = ring_cost((long)mt * nt_main, 1.0) + ring_cost((long)mt * (ceil_div(N, 128) - 2 * nt_main), 0.63) + 0.03;
+  if (c_two < c256 && c_two < c192 && c_two < c128) {
+    int rc = launch_ring<EPI, 256, 4>(A, W, C, M, N, K, H, stream, 0, nt_main);
+    if (rc != YALM_OK) return rc;
+    return launch_ring<EPI, 128, 4>(A, W, C, M, N, K, H, stream, 2 * nt_main);
+  }
+  if (c192 < c256 && c192 < c128) {
+    if constexpr (EPI != 3) return launch_ring<EPI, 192, 0>(A, W, C, M, N, K, H, stream);
+  }
+  if (c128 < c256) return launch_ring<EPI, 128, 4>(A, W, C, M, N, K, H, stream);
+  return launch_ring<EPI, 256, 4>(A, W, C, M, N, K, H, stream);
+}
+
 template <int EPI>
 int launch(const bf16* A, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
            hipStream_t stream) {
-  const long t256 = (long)ceil_div(M, 256) * ceil_div(N, 256);
-  if (t256 >= 160) {
-    // 256x192 tiles where they fill the last round of workgroups so much better that it outweighs their
-    // fewer products per byte (2,048 x 6,144: 256 tiles for 256 CUs instead of 192; 100 against 123 us)
-    if (EPI != 3) {
-      const long t192 = (long)ceil_div(M, 256) * ceil_div(N, 192);
-      auto filled = [](long tiles) { return (double)tiles / (double)(ceil_div(tiles, 256L) * 256L); };
-      if (filled(t192) * 0.93 > filled(t256))
-        return launch_shape<EPI, 256, 192, 2, 4, 2, 1>(A, W, C, M, N, K, H, nullptr, 1, stream);
-    }
-    // A last round of workgroups that is at most half full: its columns go to a second launch of
-    // 256x128 tiles, which fills the chip with them (2,048 x 28,672: 3 rounds + 1 of half-wide tiles
-    // instead of 3.5 that cost 4).
-    const int mt = ceil_div(M, 256), nt = ceil_div(N, 256);
-    const long rounds = t256 / 256, rest = t256 % 256;
-    const int nt_main = (int)(rounds * 256 / mt);
-    if (rounds >= 1 && rest > 0 && rest <= 128 && nt_main > 0 && nt_main < nt) {
-      int rc = launch_shape<EPI, 256, 256, 2, 4, 2, 1>(A, W, C, M, N, K, H, nullptr, 1, stream, true, 0, nt_main);
-      if (rc != YALM_OK) return rc;
-      return launch_shape<EPI, 256, 128, 2, 4, 2, 1>(A, W, C, M, N, K, H, nullptr, 1, stream, true, 2 * nt_main);
-    }
-    return launch_shape<EPI, 256, 256, 2, 4, 2, 1>(A, W, C, M, N, K, H, nullptr, 1, stream);
-  }
+  if (takes_ring(M)) return launch_ring_shape<EPI>(A, W, C, M, N, K, H, stream);
   const int slices = ws != nullptr ? slices_for(M, N, K, ws_floats) : 1;
   return launch_shape<EPI, 128, 128, 2, 2, 2, 2>(A, W, C, M, N, K, H, ws, slices, stream);
 }
@@ -261,7 +512,7 @@ int launch(const bf16* A, const bf16* W, void* C, float* ws, long ws_floats, int
 
 // floats of scratch with which yalm_gemm_bf16_dma would split K (0: it would not)
 long yalm_gemm_bf16_dma_workspace(int M, int N, int K) {
-  if (M <= 64 || K < TK || K % TK != 0 || (long)ceil_div(M, 256) * ceil_div(N, 256) >= 160) return 0;
+  if (M <= 64 || K < TK || K % TK != 0 || takes_ring(M)) return 0;
   const int slices = slices_for(M, N, K, (long)1 << 40);
   return slices > 1 ? (long)slices * M * N : 0;
 }
@@ -275,9 +526,9 @@ int yalm_gemm_bf16_dma_partial(const void* A, const void* W, float* workspace, l
     return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
-  if ((long)ceil_div(M, 256) * ceil_div(N, 256) >= 160) {
+  if (takes_ring(M)) {
     *slices_out = 1;
-    return launch_shape<0, 256, 256, 2, 4, 2, 1>(a, w, workspace, M, N, K, 0, nullptr, 1, stream);
+    return launch_ring_shape<0>(a, w, workspace, M, N, K, 0, stream);
   }
   int slices = slices_for(M, N, K, workspace_floats);
   const int tiles_per_slice = ceil_div(K / TK, slices);
