@@ -241,7 +241,8 @@ __host__ __device__ constexpr int dma_place(int d, int n_dma, int n_products) { 
 template <int EPI, int TN, int MAP>
 __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
                                                            void* __restrict__ Cv, int M, int N, int K, int H, int n_tile0,
-                                                           int n_tiles) {
+                                                           int n_tiles, float* __restrict__ partial,
+                                                           int tiles_per_slice) {
   constexpr int TM = RING_TM, NW = 8, NWM = 4, NWN = 2, WM = TM / NWM, WN = TN / NWN, FA = WM / 32, FB = WN / 32;
   constexpr int KS = TK / 16;
   constexpr int DA = (TM / 8) / NW, DW = (TN / 8) / NW;     // DMA instructions (8 rows each) a wave and slot
@@ -272,14 +273,17 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
     tile_m = r / width;
   }
   const int m0 = tile_m * TM, n0 = tile_n * TN;
-  const int nk = K / TK;
+  // slices of K (grid z without the XCD mapping, grid y with it): each writes its float32 partial product
+  const int slice = MAP == 0 ? blockIdx.z : blockIdx.y, n_slices = MAP == 0 ? gridDim.z : gridDim.y;
+  const int kt0 = slice * tiles_per_slice;
+  const int nk = min(K / TK - kt0, tiles_per_slice);
 
   // DMA instruction i of a wave fills rows (i * 8 + wave) * 8 ... + 7 of a slot; a lane's place there is (row,
   // 16-byte slot of the row), and it asks memory for the chunk that belongs there (rows past the edge repeat the
   // last one and are never stored)
   unsigned off_a[DA], off_w[DW];
-  const char* a_base = (const char*)(A + (size_t)m0 * K);
-  const char* w_base = (const char*)(W + (size_t)n0 * K);
+  const char* a_base = (const char*)(A + (size_t)m0 * K + (size_t)kt0 * TK);
+  const char* w_base = (const char*)(W + (size_t)n0 * K + (size_t)kt0 * TK);
 #pragma unroll
   for (int i = 0; i < DA; ++i) {
     const int row = (i * NW + wave) * RPI + lane / CPR;
@@ -405,6 +409,22 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   }
   wait_vmcnt<0>();                                 // nothing of this workgroup is on its way into LDS when it ends
 
+  if (n_slices > 1) {                              // a slice of K: the plain sums, column n = weight row n
+    float* plane = partial + (size_t)slice * M * N;
+#pragma unroll
+    for (int a = 0; a < FA; ++a)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int m = m0 + wm * WM + a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
+        if (m >= M) continue;
+#pragma unroll
+        for (int b = 0; b < FB; ++b) {
+          const int wr = (EPI == 3) ? wn * WN + (b / 2) * 64 + (li / 16) * 32 + (b % 2) * 16 + (li % 16) : wn * WN + b * 32 + li;
+          if (n0 + wr < N) plane[(size_t)m * N + n0 + wr] = acc[a][b][r];
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int a = 0; a < FA; ++a) {
 #pragma unroll
@@ -434,12 +454,15 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
 }
 
 // column tiles n_tile0 ... n_tile0 + n_tiles - 1 (n_tiles < 0: to the last) of a 256 x TN tiling
+// (slices > 1: the slices of K go to `partial` as [slices][M][N], unadded)
 template <int EPI, int TN, int MAP>
 int launch_ring(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream, int n_tile0 = 0,
-                int n_tiles = -1) {
+                int n_tiles = -1, float* partial = nullptr, int slices = 1) {
   if (n_tiles < 0) n_tiles = ceil_div(N, TN) - n_tile0;
   const int mt = ceil_div(M, RING_TM);
-  const dim3 grid = MAP == 0 ? dim3(n_tiles, mt, 1) : dim3(8 * ceil_div(mt * n_tiles, 8), 1, 1);
+  const int tiles_per_slice = ceil_div(K / TK, slices);
+  slices = ceil_div(K / TK, tiles_per_slice);
+  const dim3 grid = MAP == 0 ? dim3(n_tiles, mt, slices) : dim3(8 * ceil_div(mt * n_tiles, 8), slices, 1);
   const size_t lds = (size_t)RING_SLOTS * RING_SLOT;
   static bool allowed = false;                     // more than 64 KB of LDS has to be asked for once
   if (!allowed) {
@@ -448,7 +471,8 @@ int launch_ring(const bf16* A, const bf16* W, void* C, int M, int N, int K, int 
     if (e != hipSuccess) return (int)e;
     allowed = true;
   }
-  gemm_ring_kernel<EPI, TN, MAP><<<grid, 512, lds, stream>>>(A, W, C, M, N, K, H, n_tile0, n_tiles);
+  gemm_ring_kernel<EPI, TN, MAP><<<grid, 512, lds, stream>>>(A, W, C, M, N, K, H, n_tile0, n_tiles, partial,
+                                                             tiles_per_slice);
   return launch_status();
 }
 
@@ -467,43 +491,85 @@ int slices_for(int M, int N, int K, long workspace_floats) {
 // of more than 64 rows) to 128x128 tiles with K split over workgroups.
 bool takes_ring(int M) { return M >= 384; }
 
-// Time of a ring launch, in rounds of 256x256 tiles: a tile of 192 (128) columns costs 0.81 (0.63) of one of 256
-// (measured at 8,192 x 4,096 x 14,336: 350, 283 and 221 us a round), and a last round that fills the fraction f
-// of the CUs costs 0.45 + 0.55 f of a full one (the chip clocks higher with fewer CUs at work).
-double ring_cost(long tiles, double tile_cost) {
+// What a prompt step's GEMM is launched as: the tile width, the slices of K, and whether whole rounds of 256x256
+// tiles are followed by a second launch of 256x128 tiles for the remaining columns.
+struct RingPlan {
+  int tn = 256, slices = 1, nt_main = 0;         // nt_main > 0: two launches, the first over nt_main tile columns
+};
+
+// Estimated time in us of `tiles` workgroups of `iters` k tiles each.  An iteration of a 256x256 tile takes about
+// 1.66 us with all CUs at work (8,192 x 28,672 x 4,096: 14 rounds in 1,493 us); a tile of 192 (128) columns costs
+// 0.81 (0.63) of that (8,192 x 4,096 x 14,336: 350, 283 and 221 us a round); a last round on the fraction f of the CUs
+// costs about 0.55 + 0.45 f of a full one (the chip clocks higher with fewer CUs at work); a workgroup's first loads
+// and its epilogue take some 6 us.
+double ring_time(long tiles, int iters, int tn) {
+  const double per_iter = 1.66 * (tn == 256 ? 1.0 : (tn == 192 ? 0.81 : 0.63));
   const long rounds = tiles / 256, rest = tiles % 256;
-  return ((double)rounds + (rest ? 0.45 + 0.55 * (double)rest / 256.0 : 0.0)) * tile_cost;
+  const double f = (double)rest / 256.0;
+  return ((double)rounds + (rest ? 0.55 + 0.45 * f : 0.0)) * iters * per_iter + 6.0;
 }
 
-// 256-row tiles of 256, 192 or 128 columns, or whole rounds of 256x256 tiles and the remaining columns in a second
-// launch of 256x128 tiles: whichever the cost model puts first (2,048 x 6,144: 192 columns, 256 tiles for 256 CUs;
-// 2,048 x 4,096: 128 columns; 2,048 x 28,672: three rounds of 256x256 and one of 256x128).
-template <int EPI>
-int launch_ring_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int H, hipStream_t stream) {
-  const int mt = ceil_div(M, 256), nt = ceil_div(N, 256);
-  const double c256 = ring_cost((long)mt * nt, 1.0);
-  const double c192 = EPI == 3 ? 1e30 : ring_cost((long)mt * ceil_div(N, 192), 0.81);
-  const double c128 = ring_cost((long)mt * ceil_div(N, 128), 0.63);
+// Splits K where the tiles alone leave most CUs without work (short prompts, narrow outputs): a second kernel then
+// adds the slices (about (slices + 2) * M * N * 4 bytes at 4 TB/s).
+RingPlan ring_plan(int M, int N, int K, bool gated, long workspace_floats) {
+  const int mt = ceil_div(M, 256), nk = K / TK;
+  RingPlan best;
+  double best_t = 1e30;
+  for (int tn : {256, 192, 128}) {
+    if (gated && tn == 192) continue;
+    const long tiles = (long)mt * ceil_div(N, tn);
+    for (int s = 1; s <= 8; s *= 2) {
+      if (s > 1 && (tiles * s > 256 || nk / s < 8 || (long)s * M * N > workspace_floats)) break;
+      const int iters = ceil_div(nk, s);
+      const double t = ring_time(tiles * s, iters, tn) + (s > 1 ? 3.0 + (double)(s + 2) * M * N * 4.0 / 4.0e6 : 0.0);
+      if (t < best_t) { best_t = t; best.tn = tn; best.slices = s; best.nt_main = 0; }
+    }
+  }
+  const int nt = ceil_div(N, 256);
   const int nt_main = (int)(((long)mt * nt / 256) * 256 / mt);
-  double c_two = 1e30;
-  if (nt_main > 0 && nt_main < nt)
-    c_two = ring_cost((long)mt * nt_main, 1.0) + ring_cost((long)mt * (ceil_div(N, 128) - 2 * nt_main), 0.63) + 0.03;
-  if (c_two < c256 && c_two < c192 && c_two < c128) {
-    int rc = launch_ring<EPI, 256, 4>(A, W, C, M, N, K, H, stream, 0, nt_main);
+  if (nt_main > 0 && nt_main < nt) {
+    const double t = ring_time((long)mt * nt_main, nk, 256) + ring_time((long)mt * (ceil_div(N, 128) - 2 * nt_main), nk, 128);
+    if (t < best_t) { best_t = t; best.tn = 256; best.slices = 1; best.nt_main = nt_main; }
+  }
+  return best;
+}
+
+// partial: scratch for the slices of K (the plan was made with its size); with always_partial the product's slices
+// stay there unadded (one slice: the product itself), *slices_out says how many
+template <int EPI>
+int launch_ring_shape(const bf16* A, const bf16* W, void* C, float* partial, long partial_floats, int M, int N, int K,
+                      int H, hipStream_t stream, int* slices_out = nullptr) {
+  const bool keep = slices_out != nullptr;
+  const RingPlan p = ring_plan(M, N, K, EPI == 3, partial != nullptr ? partial_floats : 0);
+  if (p.nt_main > 0) {
+    if (keep) *slices_out = 1;
+    int rc = launch_ring<EPI, 256, 4>(A, W, C, M, N, K, H, stream, 0, p.nt_main);
     if (rc != YALM_OK) return rc;
-    return launch_ring<EPI, 128, 4>(A, W, C, M, N, K, H, stream, 2 * nt_main);
+    return launch_ring<EPI, 128, 4>(A, W, C, M, N, K, H, stream, 2 * p.nt_main);
   }
-  if (c192 < c256 && c192 < c128) {
-    if constexpr (EPI != 3) return launch_ring<EPI, 192, 0>(A, W, C, M, N, K, H, stream);
+  int slices = p.slices;
+  if (slices > 1) {                                // what the launch makes of it
+    const int per = ceil_div(K / TK, slices);
+    slices = ceil_div(K / TK, per);
   }
-  if (c128 < c256) return launch_ring<EPI, 128, 4>(A, W, C, M, N, K, H, stream);
-  return launch_ring<EPI, 256, 4>(A, W, C, M, N, K, H, stream);
+  if (keep) *slices_out = slices;
+  int rc;
+  if (p.tn == 192) {
+    if constexpr (EPI != 3) rc = launch_ring<EPI, 192, 0>(A, W, C, M, N, K, H, stream, 0, -1, partial, slices);
+    else rc = YALM_ERR_ARG;
+  } else if (p.tn == 128) {
+    rc = launch_ring<EPI, 128, 4>(A, W, C, M, N, K, H, stream, 0, -1, partial, slices);
+  } else {
+    rc = launch_ring<EPI, 256, 4>(A, W, C, M, N, K, H, stream, 0, -1, partial, slices);
+  }
+  if (rc != YALM_OK || slices == 1 || keep) return rc;
+  return yalm_splitk_reduce(partial, C, M, N, H, slices, EPI, stream);
 }
 
 template <int EPI>
 int launch(const bf16* A, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
            hipStream_t stream) {
-  if (takes_ring(M)) return launch_ring_shape<EPI>(A, W, C, M, N, K, H, stream);
+  if (takes_ring(M)) return launch_ring_shape<EPI>(A, W, C, ws, ws_floats, M, N, K, H, stream);
   const int slices = ws != nullptr ? slices_for(M, N, K, ws_floats) : 1;
   return launch_shape<EPI, 128, 128, 2, 2, 2, 2>(A, W, C, M, N, K, H, ws, slices, stream);
 }
@@ -512,7 +578,11 @@ int launch(const bf16* A, const bf16* W, void* C, float* ws, long ws_floats, int
 
 // floats of scratch with which yalm_gemm_bf16_dma would split K (0: it would not)
 long yalm_gemm_bf16_dma_workspace(int M, int N, int K) {
-  if (M <= 64 || K < TK || K % TK != 0 || takes_ring(M)) return 0;
+  if (M <= 64 || K < TK || K % TK != 0) return 0;
+  if (takes_ring(M)) {
+    const int s = ring_plan(M, N, K, false, (long)1 << 40).slices;     // (a gated product of the same shape splits no further)
+    return s > 1 ? (long)s * M * N : 0;
+  }
   const int slices = slices_for(M, N, K, (long)1 << 40);
   return slices > 1 ? (long)slices * M * N : 0;
 }
@@ -526,9 +596,13 @@ int yalm_gemm_bf16_dma_partial(const void* A, const void* W, float* workspace, l
     return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
-  if (takes_ring(M)) {
-    *slices_out = 1;
-    return launch_ring_shape<0>(a, w, workspace, M, N, K, 0, stream);
+  if (takes_ring(M)) {              // one slice: the ring kernel stores the product itself, to the workspace
+    const RingPlan p = ring_plan(M, N, K, false, workspace_floats);
+    if (p.slices == 1) {
+      *slices_out = 1;
+      return launch_ring_shape<0>(a, w, workspace, nullptr, 0, M, N, K, 0, stream);
+    }
+    return launch_ring_shape<0>(a, w, nullptr, workspace, workspace_floats, M, N, K, 0, stream, slices_out);
   }
   int slices = slices_for(M, N, K, workspace_floats);
   const int tiles_per_slice = ceil_div(K / TK, slices);
