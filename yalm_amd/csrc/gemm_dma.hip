@@ -14,7 +14,8 @@
 // Two kernels.  gemm_dma_kernel (128x128 tiles, two stages, two workgroups a CU) serves decode batches
 // of more than 64 rows: with few tiles K is split over grid z as well, every slice writes its float32
 // partial product and yalm_splitk_reduce adds them in order and applies the epilogue.  gemm_ring_kernel
-// (256-row tiles, five slots in turn, loads issued between the products) serves prompt steps.
+// (256-row tiles, five slots in turn, loads issued between the products; K split the same way for short
+// prompts) serves prompt steps and the biggest decode batches.
 //
 // Takes any M and N and K % 64 == 0; other shapes are refused (YALM_ERR_ARG) and the
 // caller runs the kernel of gemm_mfma.hip.  Sums are in a fixed order for a given shape, and the
@@ -487,9 +488,10 @@ int slices_for(int M, int N, int K, long workspace_floats) {
   return slices;
 }
 
-// Which kernel takes a shape.  Prompt steps (384 rows and more) go to the ring kernel; fewer rows (decode batches
-// of more than 64 rows) to 128x128 tiles with K split over workgroups.
-bool takes_ring(int M) { return M >= 384; }
+// Which kernel takes a shape.  160 rows and more (prompt steps, big decode batches) go to the ring kernel; fewer
+// to 128x128 tiles with K split over workgroups (a layer's four products at 160 / 256 / 383 rows: 161 / 170 /
+// 250 us against 182 / 180 / 259).
+bool takes_ring(int M) { return M >= 160; }
 
 // What a prompt step's GEMM is launched as: the tile width, the slices of K, and whether whole rounds of 256x256
 // tiles are followed by a second launch of 256x128 tiles for the remaining columns.
