@@ -82,8 +82,8 @@ def test_rmsnorm(D, w_dtype, out_dtype):
 
 # ------------------------------------------------------------------ GEMM
 
-# more than 64 rows: K a multiple of 64 takes the kernel that loads straight into LDS (128x128 tiles,
-# or 256x256 where 160 of them exist), any other K the register-staged one
+# more than 64 rows: K a multiple of 64 takes the kernels that load straight into LDS (128x128 tiles up to 159 rows,
+# 256-row tiles in a ring of LDS slots from 160), any other K the register-staged one
 GEMM_SHAPES = [(1, 16, 256), (3, 70, 96), (64, 130, 264), (65, 64, 80), (200, 333, 1000), (8, 4096 + 16, 136),
                (130, 100, 50), (65, 64, 64), (200, 333, 1024), (300, 20480 + 8, 128), (513, 130, 192),
                # K a multiple of 64 (operands staged in LDS by DMA): few and odd rows, every row count of a stage
@@ -116,6 +116,75 @@ def test_gemm_store_and_add(M, N, Kd, dtype, simple):
         close(acc, want + res.double(), torch.float32, "gemm add", factor=4 if dtype == torch.float32 else 1)
     finally:
         k.FORCE_SIMPLE = False
+
+
+# (rows, columns or hidden width, K, epilogue): prompt-step shapes, one for every way the launcher of the 256-row
+# tiles goes: tiles of 256, 192 and 128 columns, whole rounds of 256x256 followed by 256x128 tiles for the remaining
+# columns (28,672 columns at 2,048 rows), K split over workgroups (few tiles), one, two and three k tiles (the
+# start and the end of the ring of LDS slots), rows and columns that end inside a tile, many row tiles.
+PROMPT_GEMMS = [(2048, 6144, 192, "f32"), (2048, 4096, 256, "add"), (1000, 4100, 320, "bf16"),
+                (2048, 14336, 128, "gated"), (2048, 28672, 128, "f32"), (512, 4096, 4096, "add"),
+                (384, 1000, 2048, "gated"), (160, 4096, 2048, "f32"), (8192, 512, 64, "f32"), (300, 700, 128, "add"),
+                (257, 513, 192, "bf16"), (161, 96, 704, "gated"), (4096, 8192, 64, "bf16"), (700, 24000, 256, "add")]
+
+
+@pytest.mark.parametrize("with_workspace", [True, False])
+@pytest.mark.parametrize("M,N,Kd,epi", PROMPT_GEMMS)
+def test_gemm_of_prompt_steps(M, N, Kd, epi, with_workspace):
+    k = K()
+    from yalm_amd.parts.swiglu import interleave_gate_up
+    a = rnd((M, Kd), 91, torch.bfloat16).to(DEV)
+    if epi == "gated":
+        H = N
+        wg = rnd((H, Kd), 92, torch.bfloat16, scale=1 / math.sqrt(Kd))
+        wu = rnd((H, Kd), 93, torch.bfloat16, scale=1 / math.sqrt(Kd))
+        w = interleave_gate_up(wg, wu).to(DEV)
+        rows = w.shape[0]
+        ad = a.double()
+        want = (R.silu(ad @ wg.to(DEV).double().T) * (ad @ wu.to(DEV).double().T)).cpu()
+    else:
+        w = rnd((N, Kd), 92, torch.bfloat16, scale=1 / math.sqrt(Kd)).to(DEV)
+        rows = N
+        want = (a.double() @ w.double().T).cpu()
+    floats = k.gemm_workspace_floats(M, rows, Kd) if with_workspace else 0
+    ws = torch.full((floats,), float("nan"), device=DEV) if floats else None
+    if epi == "gated":
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+        k.gemm(a, w, out, k.EPI_GATED, hidden=N, workspace=ws)
+        close(out, want, torch.bfloat16, "gated", factor=2.0)
+    elif epi == "f32":
+        out = torch.full((M, N), float("nan"), device=DEV)
+        k.gemm(a, w, out, k.EPI_STORE_F32, workspace=ws)
+        close(out, want, torch.float32, "float32 out")
+    elif epi == "bf16":
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+        k.gemm(a, w, out, k.EPI_STORE, workspace=ws)
+        close(out, want, torch.bfloat16, "bfloat16 out")
+    else:
+        res = rnd((M, N), 94)
+        out = res.to(DEV).clone()
+        k.gemm(a, w, out, k.EPI_ADD_F32, workspace=ws)
+        close(out, want + res.double(), torch.float32, "residual add")
+
+
+def test_gemm_of_a_prompt_step_is_the_same_with_and_without_k_slices():
+    """The 128x128 kernel, the 256-row kernel and their K slices sum k in one order: equal bits."""
+    k = K()
+    M, N, Kd = 512, 4096, 4096
+    a = rnd((M, Kd), 95, torch.bfloat16).to(DEV)
+    w = rnd((N, Kd), 96, torch.bfloat16, scale=1 / 64).to(DEV)
+    floats = k.gemm_workspace_floats(M, N, Kd)
+    assert floats >= 2 * M * N                                   # few tiles: the launcher would split K
+    outs = []
+    for ws in (torch.empty((floats,), device=DEV), None):
+        out = torch.empty((M, N), device=DEV)
+        k.gemm(a, w, out, k.EPI_STORE_F32, workspace=ws)
+        outs.append(out)
+    # slices are added in order, but ((a + b) + (c + d)) is another rounding than (((a + b) + c) + d)
+    close(outs[0], outs[1].double().cpu(), torch.float32, "sliced against whole")
+    out = torch.empty((M, N), device=DEV)
+    k.gemm(a, w, out, k.EPI_STORE_F32, workspace=None)
+    assert torch.equal(out, outs[1])                             # and a launch repeats itself bit for bit
 
 
 def _random_gemm_shapes(n, seed):

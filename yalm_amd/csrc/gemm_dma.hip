@@ -374,7 +374,7 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
       }
 #pragma unroll
       for (int j = 0; j < NMF; ++j) {
-        const int a = j % FA, b = j / FA;
+        const int a = j / FB, b = j % FB;
         acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[c][a], fw[c][b], acc[a][b], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);
         if (ks < KS - 1) {                           // a fragment of k step ks + 1 of this tile
