@@ -297,7 +297,7 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   }
   auto dma = [&](const char* base, unsigned off, int slot, int i) {
     const unsigned lds_addr = (unsigned)(uintptr_t)(stages + slot * RING_SLOT + (i * NW + wave) * 1024);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(off), "s"(base) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(lds_addr), "v"(off), "s"(base) : "memory", "m0");
   };
 
   f32x16 acc[FA][FB];
