@@ -237,7 +237,11 @@ constexpr int RING_SLOT = 32768, RING_SLOTS = 5, RING_TM = 256;
 __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0x3F | (0x7 << 4) | (0x0 << 8) | (0x3 << 14)); }
 
 // the product index of a k step (of n_products) behind which DMA instruction d of n_dma is issued
-__host__ __device__ constexpr int dma_place(int d, int n_dma, int n_products) { return (d + 1) * n_products / (n_dma + 1) - 1 < 0 ? 0 : (d + 1) * n_products / (n_dma + 1) - 1; }
+// (evenly spread: 2 of 8 go behind products 1 and 4)
+__host__ __device__ constexpr int dma_place(int d, int n_dma, int n_products) {
+  const int at = (d + 1) * n_products / (n_dma + 1) - 1;
+  return at < 0 ? 0 : at;
+}
 
 template <int EPI, int TN, int MAP>
 __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
