@@ -22,6 +22,7 @@
 // same order in both kernels.
 #include "common.h"
 #include "yalm_hip.h"
+#include <type_traits>
 
 int yalm_splitk_reduce(const float* partial, void* C, int M, int N, int H, int slices, int epilogue,
                        hipStream_t stream);                                  // gemm_batch.hip
@@ -30,6 +31,7 @@ namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int TK = 64;
 constexpr int ROWB = TK * 2;                     // bytes a row of a stage
@@ -458,6 +460,230 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same ring with v_mfma_f32_16x16x32_bf16, for tiles of 256 and 192 columns.  The chip is power-bound under
+// this loop (the shader clock falls to 1.5-1.8 GHz), and on random operands the 16x16x32 instruction does about a
+// sixth more products for the same power than 32x32x16 (2.16 against 1.83 PFLOP/s out of registers: it moves a
+// quarter of the accumulator registers per product); the whole GEMM gains 5-10 %.  (Tiles of 128 columns, 64x64 a
+// wave, are 2-9 % slower this way and stay with the kernel above.)
+// A wave owns 64 rows x TN/2 columns: 4 x FB tiles of 16x16.  A tile's 64 k are two k steps of 32; a k step is FB
+// groups of four products that share one W fragment.  The W fragments come from LDS through a ring of four, three
+// groups ahead of their use; the A fragments of a k step are read during the one before.  The barrier stands in
+// front of the group behind which no fragment of the tile is read any more (the ring holds the last three); behind
+// it the first fragments of the next tile are read.
+// ---------------------------------------------------------------------------
+template <int EPI, int TN, int MAP>
+__global__ __launch_bounds__(512, 1) void gemm_ring16_kernel(const bf16* __restrict__ A, const bf16* __restrict__ W,
+                                                             void* __restrict__ Cv, int M, int N, int K, int H,
+                                                             int n_tile0, int n_tiles, float* __restrict__ partial,
+                                                             int tiles_per_slice) {
+  constexpr int TM = RING_TM, NW = 8, NWM = 4, NWN = 2, WM = TM / NWM, WN = TN / NWN, FA = WM / 16, FB = WN / 16;
+  constexpr int DA = (TM / 8) / NW, DW = (TN / 8) / NW;     // DMA instructions (8 rows each) a wave and slot
+  constexpr int DA1 = DA / 2, DW1 = (DW + 1) / 2;           // of them in the first of the two quarters that issue them
+  constexpr int RB = 4;                                     // the ring of W fragments
+  constexpr int NG = 2 * FB;                                // groups a tile
+  constexpr int GB = NG - (RB - 1);                         // the barrier stands in front of this group
+  constexpr int QG = NG / 4;                                // groups a quarter of the tile (the DMA's timetable)
+  constexpr int G3 = GB > 3 * QG ? GB : 3 * QG;             // the first group of the last quarter behind the barrier
+  static_assert(FA == 4 && NG % RB == 0 && NG % 4 == 0, "64 rows a wave; the ring goes round whole times a tile");
+  static_assert(2 * QG <= GB && NG - G3 >= 1, "W(kt + 2) is issued in front of the barrier, half of A(kt + 2) behind it");
+  static_assert(EPI != 3 || FB % 2 == 0, "the gated epilogue pairs column tiles");
+  extern __shared__ __attribute__((aligned(1024))) unsigned char stages[];
+  const int tid = threadIdx.x, lane = tid % WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
+  const int wm = wave / NWN, wn = wave % NWN;
+  const int l16 = lane % 16, lq = lane / 16;
+  int tile_m, tile_n;
+  if (MAP == 0) {
+    tile_m = blockIdx.y;
+    tile_n = blockIdx.x + n_tile0;
+  } else {                                                  // blocks of tiles for every XCD, as in gemm_ring_kernel
+    const int mt = (M + TM - 1) / TM, T = mt * n_tiles, chunk = (T + 7) / 8;
+    const int L = blockIdx.x, t = (L % 8) * chunk + L / 8;
+    if (t >= T || L / 8 >= chunk) return;
+    const int per_group = mt * MAP, g = t / per_group, r = t % per_group;
+    const int width = min(MAP, n_tiles - g * MAP);
+    tile_n = n_tile0 + g * MAP + r % width;
+    tile_m = r / width;
+  }
+  const int m0 = tile_m * TM, n0 = tile_n * TN;
+  const int slice = MAP == 0 ? blockIdx.z : blockIdx.y, n_slices = MAP == 0 ? gridDim.z : gridDim.y;
+  const int kt0 = slice * tiles_per_slice;
+  const int nk = min(K / TK - kt0, tiles_per_slice);
+
+  unsigned off_a[DA], off_w[DW];
+  const char* a_base = (const char*)(A + (size_t)m0 * K + (size_t)kt0 * TK);
+  const char* w_base = (const char*)(W + (size_t)n0 * K + (size_t)kt0 * TK);
+#pragma unroll
+  for (int i = 0; i < DA; ++i) {
+    const int row = (i * NW + wave) * RPI + lane / CPR;
+    off_a[i] = (unsigned)(((size_t)min(row, M - 1 - m0) * K + ((lane % CPR) ^ swizzle_of(row)) * 8) * 2);
+  }
+#pragma unroll
+  for (int i = 0; i < DW; ++i) {
+    const int row = (i * NW + wave) * RPI + lane / CPR;
+    off_w[i] = (unsigned)(((size_t)min(row, N - 1 - n0) * K + ((lane % CPR) ^ swizzle_of(row)) * 8) * 2);
+  }
+  // the LDS address of this wave's first row block of a slot (scalar); instruction i lies i * 8 KB further
+  const unsigned lds0 = (unsigned)(uintptr_t)stages + (unsigned)(wave * 1024);
+  auto slot_addr = [&](int slot) { return lds0 + (unsigned)slot * RING_SLOT; };
+  auto dma = [&](const char* base, unsigned off, unsigned lds_slot, int i) {
+    const unsigned add = (unsigned)(i * NW * 1024);
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 : : "s"(lds_slot), "v"(off), "s"(base), "s"(add) : "memory", "m0", "scc");
+  };
+
+  f32x4 acc[FA][FB];
+#pragma unroll
+  for (int a = 0; a < FA; ++a)
+#pragma unroll
+    for (int b = 0; b < FB; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  // fragments (operand rows = lane % 16, 8 k at k offset 8 * (lane / 16)): address in a slot row * 128 +
+  // ((4 s + lq) ^ swizzle) * 16 for k step s; tiles 16 rows apart share the swizzle
+  const int a_row = wm * WM + l16, w_row = wn * WN + l16;
+  int a_at[2], w_at[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) {
+    a_at[s] = a_row * ROWB + (((4 * s + lq) ^ swizzle_of(a_row)) << 4);
+    w_at[s] = w_row * ROWB + (((4 * s + lq) ^ swizzle_of(w_row)) << 4);
+  }
+  auto frag_a = [&](int slot, int s, int a) {
+    return *reinterpret_cast<const bf16x8*>(stages + slot * RING_SLOT + a_at[s] + a * 16 * ROWB);
+  };
+  auto frag_w = [&](int slot, int s, int b) {
+    return *reinterpret_cast<const bf16x8*>(stages + slot * RING_SLOT + w_at[s] + b * 16 * ROWB);
+  };
+
+  // before the loop: W0 A0 W1 and the first half of A1 (what iterations -2 and -1 would have issued)
+#pragma unroll
+  for (int i = 0; i < DW; ++i) dma(w_base, off_w[i], slot_addr(0), i);
+#pragma unroll
+  for (int i = 0; i < DA; ++i) dma(a_base, off_a[i], slot_addr(1), i);
+  if (nk > 1) {
+#pragma unroll
+    for (int i = 0; i < DW; ++i) dma(w_base + ROWB, off_w[i], slot_addr(2), i);
+#pragma unroll
+    for (int i = 0; i < DA1; ++i) dma(a_base + ROWB, off_a[i], slot_addr(3), i);
+    wait_vmcnt<DW + DA1>();
+  } else {
+    wait_vmcnt<0>();
+  }
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  bf16x8 fa[2][FA], fb[RB];
+#pragma unroll
+  for (int a = 0; a < FA; ++a) fa[0][a] = frag_a(1, 0, a);
+#pragma unroll
+  for (int g = 0; g < RB - 1; ++g) fb[g] = frag_w(0, g / FB, g % FB);
+
+  int ws = 0, as = 1;                              // slots of the tile that is multiplied
+  // one k tile; T1 / T2: tiles kt + 1 / kt + 2 exist (the loop's last two iterations stand apart, so that the
+  // others carry no branch)
+  auto iteration = [&](int kt, auto t1_, auto t2_) {
+    constexpr bool T1 = decltype(t1_)::value, T2 = decltype(t2_)::value;
+    const int ws1 = ws + 2 >= RING_SLOTS ? ws + 2 - RING_SLOTS : ws + 2;          // of tile kt + 1
+    const int as1 = as + 2 >= RING_SLOTS ? as + 2 - RING_SLOTS : as + 2;
+    const int ws2 = ws1 + 2 >= RING_SLOTS ? ws1 + 2 - RING_SLOTS : ws1 + 2;       // of tile kt + 2
+    const int as2 = as1 + 2 >= RING_SLOTS ? as1 + 2 - RING_SLOTS : as1 + 2;
+    const unsigned l_as1 = slot_addr(as1), l_ws2 = slot_addr(ws2), l_as2 = slot_addr(as2);
+    const char* a1 = a_base + (size_t)(kt + 1) * ROWB;
+    const char* a2 = a_base + (size_t)(kt + 2) * ROWB;
+    const char* w2 = w_base + (size_t)(kt + 2) * ROWB;
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {                 // group g: W fragment b of k step s against the four A fragments
+      const int s = g / FB, b = g % FB;
+      if (g == GB) {
+        // No fragment of tile kt is read from here on; this wave's share of tile kt + 1 has landed (W(kt + 2) may
+        // still be on its way).  Behind the barrier that holds for all waves.
+        wait_lgkmcnt0();
+        if (T2) wait_vmcnt<DW>(); else wait_vmcnt<0>();
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+#pragma unroll
+      for (int a = 0; a < FA; ++a) {
+        acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[s][a], fb[g % RB], acc[a][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (a == 0) {                                // the W fragment RB - 1 groups ahead (behind the barrier: of the next tile;
+          const int gn = g + RB - 1;                 // behind the last tile: read, never used)
+          if (gn < NG) fb[gn % RB] = frag_w(ws, gn / FB, gn % FB);
+          else fb[gn % RB] = frag_w(ws1, (gn - NG) / FB, (gn - NG) % FB);
+        }
+        if (a == 2 && s == 0 && b >= FB - FA)        // the A fragments of k step 1, in the last four groups of k step 0
+          fa[1][b - (FB - FA)] = frag_a(as, 1, b - (FB - FA));
+        if (a >= 2 && g >= GB && (g - GB) * 2 + (a - 2) < FA)      // those of the next tile behind the barrier, two a group
+          fa[0][(g - GB) * 2 + (a - 2)] = frag_a(as1, 0, (g - GB) * 2 + (a - 2));
+        // DMA by quarters of the tile: the second half of A(kt + 1); W(kt + 2) in two halves; behind the barrier the
+        // first half of A(kt + 2); behind the second and the fourth product of a group
+        if (a == 1 || a == 3) {
+          const int q = g / QG, d = (g % QG) * 2 + (a == 3);
+          if (q == 0) { if (T1 && d < DA - DA1) dma(a1, off_a[DA1 + d], l_as1, DA1 + d); }
+          else if (q == 1) { if (T2 && d < DW1) dma(w2, off_w[d], l_ws2, d); }
+          else if (q == 2) { if (T2 && d < DW - DW1) dma(w2, off_w[DW1 + d], l_ws2, DW1 + d); }
+          if (g >= G3) {
+            const int d2 = (g - G3) * 2 + (a == 3);
+            if (T2 && d2 < DA1) dma(a2, off_a[d2], l_as2, d2);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    ws = ws1;
+    as = as1;
+  };
+  int kt = 0;
+  for (; kt + 2 < nk; ++kt) iteration(kt, std::true_type{}, std::true_type{});
+  if (kt + 1 < nk) { iteration(kt, std::true_type{}, std::false_type{}); ++kt; }
+  if (kt < nk) iteration(kt, std::false_type{}, std::false_type{});
+  wait_vmcnt<0>();                                 // nothing of this workgroup is on its way into LDS when it ends
+
+  // C: lane (lq, l16) holds rows 4 lq .. 4 lq + 3 of column l16 of every tile
+  if (n_slices > 1) {                              // a slice of K: the plain sums, column n = weight row n
+    float* plane = partial + (size_t)slice * M * N;
+#pragma unroll
+    for (int a = 0; a < FA; ++a)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int m = m0 + wm * WM + a * 16 + 4 * lq + r;
+        if (m >= M) continue;
+#pragma unroll
+        for (int b = 0; b < FB; ++b) {
+          const int nn = n0 + wn * WN + b * 16 + l16;
+          if (nn < N) plane[(size_t)m * N + nn] = acc[a][b][r];
+        }
+      }
+    return;
+  }
+#pragma unroll
+  for (int a = 0; a < FA; ++a) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int m = m0 + wm * WM + a * 16 + 4 * lq + r;
+      if (m >= M) continue;
+      if (EPI == 3) {                              // weight rows: 16 gate rows, 16 up rows, ...: even tiles gate, odd tiles up
+#pragma unroll
+        for (int pp = 0; pp < FB / 2; ++pp) {
+          const int hcol = (n0 + wn * WN) / 2 + pp * 16 + l16;
+          if (hcol < H)
+            ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
+        }
+      } else {
+#pragma unroll
+        for (int b = 0; b < FB; ++b) {
+          const int nn = n0 + wn * WN + b * 16 + l16;
+          if (nn >= N) continue;
+          const size_t o = (size_t)m * N + nn;
+          if (EPI == 0) ((float*)Cv)[o] = acc[a][b][r];
+          if (EPI == 1) ((bf16*)Cv)[o] = static_cast<bf16>(acc[a][b][r]);
+          if (EPI == 2) ((float*)Cv)[o] += acc[a][b][r];
+        }
+      }
+    }
+  }
+}
+
 // column tiles n_tile0 ... n_tile0 + n_tiles - 1 (n_tiles < 0: to the last) of a 256 x TN tiling
 // (slices > 1: the slices of K go to `partial` as [slices][M][N], unadded)
 template <int EPI, int TN, int MAP>
@@ -469,15 +695,17 @@ int launch_ring(const bf16* A, const bf16* W, void* C, int M, int N, int K, int 
   slices = ceil_div(K / TK, tiles_per_slice);
   const dim3 grid = MAP == 0 ? dim3(n_tiles, mt, slices) : dim3(8 * ceil_div(mt * n_tiles, 8), slices, 1);
   const size_t lds = (size_t)RING_SLOTS * RING_SLOT;
+  // tiles of 256 and 192 columns: the kernel with the 16x16x32 products; of 128: the one with 32x32x16
+  void (*kernel)(const bf16*, const bf16*, void*, int, int, int, int, int, int, float*, int);
+  if constexpr (TN == 128) kernel = &gemm_ring_kernel<EPI, TN, MAP>;
+  else kernel = &gemm_ring16_kernel<EPI, TN, MAP>;
   static bool allowed = false;                     // more than 64 KB of LDS has to be asked for once
   if (!allowed) {
-    hipError_t e = hipFuncSetAttribute((const void*)&gemm_ring_kernel<EPI, TN, MAP>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
     allowed = true;
   }
-  gemm_ring_kernel<EPI, TN, MAP><<<grid, 512, lds, stream>>>(A, W, C, M, N, K, H, n_tile0, n_tiles, partial,
-                                                             tiles_per_slice);
+  kernel<<<grid, 512, lds, stream>>>(A, W, C, M, N, K, H, n_tile0, n_tiles, partial, tiles_per_slice);
   return launch_status();
 }
 
@@ -504,12 +732,12 @@ struct RingPlan {
 };
 
 // Estimated time in us of `tiles` workgroups of `iters` k tiles each.  An iteration of a 256x256 tile takes about
-// 1.66 us with all CUs at work (8,192 x 28,672 x 4,096: 14 rounds in 1,493 us); a tile of 192 (128) columns costs
-// 0.81 (0.63) of that (8,192 x 4,096 x 14,336: 350, 283 and 221 us a round); a last round on the fraction f of the CUs
+// 1.53 us with all CUs at work, of a tile of 192 columns 1.24 and of 128 columns 1.05 (8,192 x 4,096 x 14,336: 325,
+// 265 and 221 us a round of 224 iterations); a last round on the fraction f of the CUs
 // costs about 0.55 + 0.45 f of a full one (the chip clocks higher with fewer CUs at work); a workgroup's first loads
 // and its epilogue take some 6 us.
 double ring_time(long tiles, int iters, int tn) {
-  const double per_iter = 1.66 * (tn == 256 ? 1.0 : (tn == 192 ? 0.81 : 0.63));
+  const double per_iter = tn == 256 ? 1.53 : (tn == 192 ? 1.24 : 1.05);
   const long rounds = tiles / 256, rest = tiles % 256;
   const double f = (double)rest / 256.0;
   return ((double)rounds + (rest ? 0.55 + 0.45 * f : 0.0)) * iters * per_iter + 6.0;
@@ -517,12 +745,11 @@ double ring_time(long tiles, int iters, int tn) {
 
 // Splits K where the tiles alone leave most CUs without work (short prompts, narrow outputs): a second kernel then
 // adds the slices (about (slices + 2) * M * N * 4 bytes at 4 TB/s).
-RingPlan ring_plan(int M, int N, int K, bool gated, long workspace_floats) {
+RingPlan ring_plan(int M, int N, int K, long workspace_floats) {
   const int mt = ceil_div(M, 256), nk = K / TK;
   RingPlan best;
   double best_t = 1e30;
   for (int tn : {256, 192, 128}) {
-    if (gated && tn == 192) continue;
     const long tiles = (long)mt * ceil_div(N, tn);
     for (int s = 1; s <= 8; s *= 2) {
       if (s > 1 && (tiles * s > 256 || nk / s < 8 || (long)s * M * N > workspace_floats)) break;
@@ -546,7 +773,7 @@ template <int EPI>
 int launch_ring_shape(const bf16* A, const bf16* W, void* C, float* partial, long partial_floats, int M, int N, int K,
                       int H, hipStream_t stream, int* slices_out = nullptr) {
   const bool keep = slices_out != nullptr;
-  const RingPlan p = ring_plan(M, N, K, EPI == 3, partial != nullptr ? partial_floats : 0);
+  const RingPlan p = ring_plan(M, N, K, partial != nullptr ? partial_floats : 0);
   if (p.nt_main > 0) {
     if (keep) *slices_out = 1;
     int rc = launch_ring<EPI, 256, 4>(A, W, C, M, N, K, H, stream, 0, p.nt_main);
@@ -561,8 +788,7 @@ int launch_ring_shape(const bf16* A, const bf16* W, void* C, float* partial, lon
   if (keep) *slices_out = slices;
   int rc;
   if (p.tn == 192) {
-    if constexpr (EPI != 3) rc = launch_ring<EPI, 192, 0>(A, W, C, M, N, K, H, stream, 0, -1, partial, slices);
-    else rc = YALM_ERR_ARG;
+    rc = launch_ring<EPI, 192, 0>(A, W, C, M, N, K, H, stream, 0, -1, partial, slices);
   } else if (p.tn == 128) {
     rc = launch_ring<EPI, 128, 4>(A, W, C, M, N, K, H, stream, 0, -1, partial, slices);
   } else {
@@ -586,7 +812,7 @@ int launch(const bf16* A, const bf16* W, void* C, float* ws, long ws_floats, int
 long yalm_gemm_bf16_dma_workspace(int M, int N, int K) {
   if (M <= 64 || K < TK || K % TK != 0) return 0;
   if (takes_ring(M)) {
-    const int s = ring_plan(M, N, K, false, (long)1 << 40).slices;     // (a gated product of the same shape splits no further)
+    const int s = ring_plan(M, N, K, (long)1 << 40).slices;
     return s > 1 ? (long)s * M * N : 0;
   }
   const int slices = slices_for(M, N, K, (long)1 << 40);
@@ -603,7 +829,7 @@ int yalm_gemm_bf16_dma_partial(const void* A, const void* W, float* workspace, l
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   if (takes_ring(M)) {              // one slice: the ring kernel stores the product itself, to the workspace
-    const RingPlan p = ring_plan(M, N, K, false, workspace_floats);
+    const RingPlan p = ring_plan(M, N, K, workspace_floats);
     if (p.slices == 1) {
       *slices_out = 1;
       return launch_ring_shape<0>(a, w, workspace, nullptr, 0, M, N, K, 0, stream);
