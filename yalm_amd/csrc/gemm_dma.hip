@@ -732,12 +732,12 @@ struct RingPlan {
 };
 
 // Estimated time in us of `tiles` workgroups of `iters` k tiles each.  An iteration of a 256x256 tile takes about
-// 1.53 us with all CUs at work, of a tile of 192 columns 1.24 and of 128 columns 1.05 (8,192 x 4,096 x 14,336: 325,
-// 265 and 221 us a round of 224 iterations); a last round on the fraction f of the CUs
+// 1.47 us with all CUs at work, of a tile of 192 columns 1.30 and of 128 columns 1.00 (8,192 x 4,096 x 14,336: 329,
+// 291 and 225 us a round of 224 iterations); a last round on the fraction f of the CUs
 // costs about 0.55 + 0.45 f of a full one (the chip clocks higher with fewer CUs at work); a workgroup's first loads
 // and its epilogue take some 6 us.
 double ring_time(long tiles, int iters, int tn) {
-  const double per_iter = tn == 256 ? 1.53 : (tn == 192 ? 1.24 : 1.05);
+  const double per_iter = tn == 256 ? 1.47 : (tn == 192 ? 1.30 : 1.00);
   const long rounds = tiles / 256, rest = tiles % 256;
   const double f = (double)rest / 256.0;
   return ((double)rounds + (rest ? 0.55 + 0.45 * f : 0.0)) * iters * per_iter + 6.0;
