@@ -168,7 +168,8 @@ def test_gemm_of_prompt_steps(M, N, Kd, epi, with_workspace):
 
 
 def test_gemm_of_a_prompt_step_is_the_same_with_and_without_k_slices():
-    """The 128x128 kernel, the 256-row kernel and their K slices sum k in one order: equal bits."""
+    """A product in K slices agrees with the whole one within float32 rounding, and a launch repeats itself bit
+    for bit."""
     k = K()
     M, N, Kd = 512, 4096, 4096
     a = rnd((M, Kd), 95, torch.bfloat16).to(DEV)

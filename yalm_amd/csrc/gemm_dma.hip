@@ -11,15 +11,14 @@
 // (s_waitcnt vmcnt) and use the bare s_barrier, because __syncthreads() carries a fence that
 // would wait for the loads of all stages.
 //
-// Two kernels.  gemm_dma_kernel (128x128 tiles, two stages, two workgroups a CU) serves decode batches
-// of more than 64 rows: with few tiles K is split over grid z as well, every slice writes its float32
-// partial product and yalm_splitk_reduce adds them in order and applies the epilogue.  gemm_ring_kernel
+// gemm_dma_kernel (128x128 tiles, two stages, two workgroups a CU) serves decode batches of 65 to 159
+// rows: with few tiles K is split over grid z as well, every slice writes its float32 partial product and
+// yalm_splitk_reduce adds them in order and applies the epilogue.  gemm_ring_kernel and gemm_ring16_kernel
 // (256-row tiles, five slots in turn, loads issued between the products; K split the same way for short
-// prompts) serves prompt steps and the biggest decode batches.
+// prompts) serve prompt steps and the biggest decode batches.
 //
 // Takes any M and N and K % 64 == 0; other shapes are refused (YALM_ERR_ARG) and the
-// caller runs the kernel of gemm_mfma.hip.  Sums are in a fixed order for a given shape, and the
-// same order in both kernels.
+// caller runs the kernel of gemm_mfma.hip.  Sums are in a fixed order for a given shape.
 #include "common.h"
 #include "yalm_hip.h"
 #include <type_traits>
