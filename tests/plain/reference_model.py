@@ -132,24 +132,73 @@ def attention_probs_one_query(qh, K, head_dim):
     return e / e.sum()
 
 
-def attention(q, k, v, window=0):
+def attention(q, k, v, window=0, sinks=0, inv_freq=None):
     """src/infer.cpp:218-250 and 321-330 for every query position of a whole
     sequence.  q: [T, n_heads, hd]; k, v: [T, n_kv_heads, hd].  Query head h
     reads KV head h // (n_heads // n_kv_heads).  The reference sees only the
     cache rows [0, kv_len); for a whole sequence that is: key j is visible to
     query i iff j <= i and (window == 0 or i - j < window), the last
-    `window` positions including the current one (src/infer.cpp:486-488)."""
+    `window` positions including the current one (src/infer.cpp:486-488).
+
+    sinks (src/infer.cpp:305-319, 484-488 in closed form; `attention_context_ring`
+    below is the same a step at a time): the first `sinks` positions stay
+    visible behind the window.  The reference's cache of n = window + sinks rows
+    keeps them from position n on and turns their keys one position further at
+    every such step, i - n + 1 times up to query i; rotations add up, so the
+    sink keys are the rotated keys turned by max(0, i - n + 1) positions more."""
     T, n_heads, hd = q.shape
     n_kv = k.shape[1]
     group = n_heads // n_kv
     out = torch.zeros(T, n_heads, hd, dtype=F64)
+    k = k.to(F64)
     v = v.to(F64)
     for i in range(T):
         lo = 0 if window == 0 else max(0, i - window + 1)
+        K, V = k[lo:i + 1], v[lo:i + 1]
+        n_behind = min(sinks, lo)                       # sinks the window no longer covers
+        if n_behind > 0:
+            turn = max(0, i - (window + sinks) + 1)
+            ks = k[:n_behind]
+            if turn > 0:
+                ks = rope_interleaved(ks, torch.full((n_behind,), turn), inv_freq)
+            K = torch.cat([ks, K], dim=0)
+            V = torch.cat([v[:n_behind], V], dim=0)
         for h in range(n_heads):
             g = h // group
-            p = attention_probs_one_query(q[i, h], k[lo:i + 1, g], hd)
-            out[i, h] = p @ v[lo:i + 1, g]
+            p = attention_probs_one_query(q[i, h], K[:, g], hd)
+            out[i, h] = p @ V[:, g]
+    return out
+
+
+KV_SINKS = 2                                            # src/model.h:12
+
+
+def attention_context_ring(q, k, v, context, inv_freq):
+    """The reference's cache of `context` rows a token at a time, as written
+    (src/infer.cpp:484-488: kv_sink, kv_pos, kv_len; 298-303: the new key and
+    value go to row kv_pos; 305-319: each kept sink key is turned by one
+    position; 321-330: attention over rows [0, kv_len)).  q, k: rotated at
+    their positions.  Pins the closed form of `attention` with
+    window = context - KV_SINKS and sinks = KV_SINKS."""
+    T, n_heads, hd = q.shape
+    n_kv = k.shape[1]
+    group = n_heads // n_kv
+    kb = torch.zeros(context, n_kv, hd, dtype=F64)
+    vb = torch.zeros(context, n_kv, hd, dtype=F64)
+    out = torch.zeros(T, n_heads, hd, dtype=F64)
+    one = torch.ones(1)
+    for pos in range(T):
+        kv_sink = KV_SINKS if pos >= context else 0
+        kv_pos = kv_sink + (pos - kv_sink) % (context - kv_sink)
+        kv_len = context if pos >= context else pos + 1
+        kb[kv_pos] = k[pos].to(F64)
+        vb[kv_pos] = v[pos].to(F64)
+        for r in range(kv_sink):
+            kb[r] = rope_interleaved(kb[r:r + 1], one, inv_freq)[0]
+        for h in range(n_heads):
+            g = h // group
+            p = attention_probs_one_query(q[pos, h], kb[:kv_len, g], hd)
+            out[pos, h] = p @ vb[:kv_len, g]
     return out
 
 
@@ -178,7 +227,7 @@ def embedding(table, tokens):
 # ----------------------------------------------------------------------------
 
 def read_config(cfg):
-    """convert.py:22-54 with the additions `rope_scaling` and `sliding_window`."""
+    """convert.py:22-54 with the additions `rope_scaling`, `sliding_window` and `attention_sinks`."""
     arch = cfg["architectures"][0]
     assert arch in ("LlamaForCausalLM", "MistralForCausalLM"), arch
     c = {}
@@ -193,6 +242,7 @@ def read_config(cfg):
     c["rotary_dim"] = int(c["head_dim"] * cfg.get("partial_rotary_factor", 1))
     c["norm_eps"] = cfg["rms_norm_eps"]
     c["window"] = cfg.get("sliding_window") or 0
+    c["sinks"] = cfg.get("attention_sinks") or 0
     c["tied"] = cfg.get("tie_word_embeddings", None) is not False   # convert.py:200-204, 241
     c["rope_scaling"] = cfg.get("rope_scaling")
     assert cfg.get("hidden_act", "silu") == "silu"
@@ -214,7 +264,7 @@ def model_inv_freq(c):
 # whole model
 # ----------------------------------------------------------------------------
 
-def forward(weights, cfg, tokens, window_override=None, position_offset=0):
+def forward(weights, cfg, tokens, window_override=None, position_offset=0, sinks_override=None):
     """src/infer.cpp:477-521 and 256-386 for every position of one sequence.
 
     weights: tensors under Hugging Face names; cfg: the config.json dict;
@@ -224,6 +274,7 @@ def forward(weights, cfg, tokens, window_override=None, position_offset=0):
     and the classifier (the embedding table when tied, model.cpp:389-398)."""
     c = read_config(cfg)
     window = c["window"] if window_override is None else window_override
+    sinks = c["sinks"] if sinks_override is None else sinks_override
     T = len(tokens)
     tok = torch.tensor(tokens, dtype=torch.long)
     pos = torch.arange(T) + position_offset
@@ -242,7 +293,7 @@ def forward(weights, cfg, tokens, window_override=None, position_offset=0):
         v = (xb @ wv.T).reshape(T, KV, hd)
         q = rope_interleaved(q, pos, inv_freq)
         k = rope_interleaved(k, pos, inv_freq)
-        a = attention(q, k, v, window).reshape(T, H * hd)
+        a = attention(q, k, v, window, sinks, inv_freq).reshape(T, H * hd)
         x = x + a @ weights[p + "self_attn.o_proj.weight"].to(F64).T
         xb = rmsnorm(x, weights[p + "post_attention_layernorm.weight"], c["norm_eps"])
         x = x + swiglu_ffn(xb, weights[p + "mlp.gate_proj.weight"], weights[p + "mlp.down_proj.weight"],

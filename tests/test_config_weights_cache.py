@@ -44,6 +44,24 @@ def test_config_reads_the_architectures_own_keys():
     assert c3.rope_scaling.factor == 8.0 and config_from_dict(c3.to_dict()) == c3
 
 
+def test_a_context_is_two_sinks_and_a_window():
+    """The reference's -T n (src/infer.cpp:484-488, src/model.h:12): 2 sinks beside the last n - 2."""
+    c = config_from_dict(tiny_configs.TINY_LLAMA)
+    assert c.with_context(0) is c and c.attention_sinks == 0
+    t = c.with_context(40)
+    assert (t.sliding_window, t.attention_sinks) == (38, 2)
+    assert all(l.mixer.params["window"] == 38 and l.mixer.params["sinks"] == 2 for l in t.to_spec().layers)
+    assert config_from_dict(t.to_dict()) == t                  # the folder of such a model keeps both
+    assert c.with_window(16).attention_sinks == 0 and c.with_window(16, 3).attention_sinks == 3
+    for n in (1, 2):
+        with pytest.raises(ConfigError, match="sinks"):
+            c.with_context(n)
+    with pytest.raises(ConfigError, match="attention_sinks"):
+        config_from_dict(dict(tiny_configs.TINY_LLAMA, attention_sinks=2))        # sinks without a window
+    s = config_from_dict(tiny_configs.TINY_SINKS)
+    assert (s.sliding_window, s.attention_sinks, s.rotary_dim) == (37, 3, 24)
+
+
 @pytest.mark.parametrize("change,text", [
     ({"architectures": ["GPT2LMHeadModel"]}, "not supported"),
     ({"num_key_value_heads": 3}, "multiple"),
@@ -274,6 +292,13 @@ def test_cache_groups_and_page_accounting():
     assert c.group_of(1) is full and full.lines == [0, 1] and ring.lines == [2]
     assert full.ring_pages == 8 and ring.ring_pages == 3            # ceil(100/64) + 1
     assert full.k_pages.shape == (2, 10, 2, 64, 16) and full.v_pages.shape == (2, 10, 2, 16, 64)
+    assert full.sinks == 0 and full.sink_k is None and ring.sinks == 0
+    # lines that keep sinks beside the window are a group of their own, with a place for them per slot
+    reqs = {0: KVRequest(2, 16, 100), 1: KVRequest(2, 16, 100, 3), 2: KVRequest(2, 16, 100, 3)}
+    s = CacheManager(reqs, 640, 512, torch.float32, "cpu", n_slots=4)
+    assert len(s.kv_groups) == 2 and s.group_of(1) is s.group_of(2) and s.group_of(0).sinks == 0
+    k, v = s.group_of(2).line_sinks(2)
+    assert k.shape == v.shape == (4, 2, 3, 16) and k.is_contiguous() and s.group_of(1).ring_pages == 3
     s = c.acquire(2)
     assert c.extend(s, [70, 1]) == [70, 1]
     assert full.pool.n_free == 10 - 3 and ring.pool.n_free == 10 - 3

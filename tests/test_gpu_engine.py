@@ -44,6 +44,8 @@ OVERLAPPING = {
                    [[30, 2, 64], [65, 1], [3, 64, 9]], [0, 4, 30]),
     "tiny_mistral": ([30, 64, 12, 50, 41, 64], [[0, 1], [2, 3, 4], [5]], [[17, 40], [1, 33, 16], [2]], [0, 3, 45]),
     "small_windowed": ([300, 90, 200, 130, 64], [[0, 1], [2, 3], [4, 1]], [[260, 64], [97, 100], [1, 80]], [0, 5, 70]),
+    # sinks beside the window: a slot that is taken again still holds its last sequence's sinks
+    "tiny_sinks": ([150, 60, 200, 130, 64], [[0, 1], [2, 3], [4, 1]], [[120, 2], [97, 100], [1, 50]], [0, 5, 70]),
 }
 
 

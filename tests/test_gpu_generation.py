@@ -236,6 +236,41 @@ def test_command_line(folders):
     assert bad.returncode == 1 and "no CPU path" in bad.stderr
 
 
+def test_a_context_shorter_than_the_text(folders):
+    """The reference's -T <n>: the first two positions stay as sinks beside the last n - 2.  Greedy
+    generation far past a context of 24 through the Python entry point and through the command line,
+    against the plain implementation with the same sinks and window."""
+    from yalm_amd import Engine, Model, generate
+    folder = folders["tiny_wide_heads"]          # an untied head: the next token is not simply the last one again
+    cfg, w = R.read_folder(folder)
+    prompt = [1, 17, 200, 33, 5]
+    n_new, context = 90, 24
+
+    def plain(seq):
+        return R.forward(w, cfg, seq, window_override=context - 2, sinks_override=2)
+
+    want = []
+    seq = list(prompt)
+    for _ in range(n_new):
+        want.append(R.sample_argmax(plain(seq)[-1]))
+        seq.append(want[-1])
+    unlimited = plain_greedy(folder, prompt, n_new)
+    assert want[:context - len(prompt)] == unlimited[:context - len(prompt)] and want != unlimited
+    model = Model.from_folder(folder, dtype=torch.float32, device="cuda:0", context=context)
+    engine = Engine(model, max_tokens=512)
+    assert generate(engine, [prompt], max_new_tokens=n_new, temperature=0.0, stop_ids=[])[0] == want
+    # a prompt that is itself longer than the context, with company
+    long_prompt = prompt + want[:50]
+    out = generate(engine, [long_prompt, prompt], max_new_tokens=n_new - 50, temperature=0.0, stop_ids=[])
+    assert out[0] == want[50:] and out[1] == want[:n_new - 50]
+    p = subprocess.run([sys.executable, "-m", "yalm_amd", folder, "--tokens", ",".join(map(str, prompt)), "-n",
+                        str(n_new), "-t", "0", "-T", str(context), "--dtype", "float32"], cwd=ROOT,
+                       stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-3000:]
+    stop_at = want.index(2) + 1 if 2 in want else len(want)          # the command line stops at the end token
+    assert [int(t) for t in generated(p.stdout)] == want[:stop_at]
+
+
 def test_command_line_with_a_tokenizer(folders, tmp_path):
     """Text prompts and the passkey mode (src/main.cpp:237-332) need tokenizer.json: a byte-level one with a
     few words is written next to the random model; what the program prints is the plain implementation's

@@ -714,6 +714,165 @@ def test_attn_vector_of_the_reference():
     assert torch.allclose(got[1, :3], torch.tensor([0., 0, 1]), atol=1e-4)
 
 
+# ------------------------------------------------------------------ attention sinks
+
+def window_lse_float64(q, k, window):
+    """Logarithm of the sum of exp(score) over the keys a window shows, [T, n_heads]."""
+    T, n_heads, hd = q.shape
+    group = n_heads // k.shape[1]
+    out = torch.zeros((T, n_heads), dtype=torch.float64)
+    for i in range(T):
+        lo = max(0, i - window + 1) if window else 0
+        for h in range(n_heads):
+            out[i, h] = torch.logsumexp((k[lo:i + 1, h // group].double() @ q[i, h].double()) / math.sqrt(hd), 0)
+    return out
+
+
+@pytest.mark.parametrize("simple", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,rd,window,sinks,lens", [
+    (4, 2, 16, 16, 5, 2, [30, 3, 1, 8]), (6, 3, 48, 24, 37, 3, [150, 41]), (8, 2, 128, 128, 94, 2, [300, 96, 97]),
+    (4, 1, 64, 32, 70, 4, [200, 64]), (2, 2, 32, 0, 9, 1, [40])])
+def test_attn_prefill_with_sinks(n_heads, n_kv, hd, rd, window, sinks, lens, dtype, simple):
+    """Sinks stored from the staging area, the attention kernel's log-sum-exp, and the sinks behind the
+    window mixed in with their keys turned, against the plain implementation's closed form."""
+    k = K()
+    T, B = sum(lens), len(lens)
+    q = rnd((T, n_heads * hd), 33, dtype)
+    kk = rnd((T, n_kv * hd), 34, dtype)
+    v = rnd((T, n_kv * hd), 35, dtype)
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    seq = np.repeat(np.arange(B), lens)
+    pos = np.concatenate([np.arange(n) for n in lens])
+    ks, vs, tile0 = stage(kk, v, lens, n_kv, hd, dtype)
+    n_slots = B + 3
+    slots = [int(x) for x in np.random.default_rng(5).permutation(n_slots)[:B]]
+    sink_k = torch.full((n_slots, n_kv, sinks, hd), 7.0, dtype=dtype, device=DEV)
+    sink_v = torch.full((n_slots, n_kv, sinks, hd), 7.0, dtype=dtype, device=DEV)
+    table = make_table(max(lens) + 1, hd, rd, 80.0).to(DEV) if rd else None
+    out = torch.empty((T, n_heads * hd), dtype=dtype, device=DEV)
+    lse = torch.empty((T, n_heads), dtype=torch.float32, device=DEV)
+    qd, ksd, vsd = q.to(DEV), ks.to(DEV), vs.to(DEV)
+    k.FORCE_SIMPLE = simple
+    try:
+        k.sink_store(ksd, vsd, i32(tile0), i32(slots), i32(lens), sink_k, sink_v, False)
+        k.attn_prefill(qd, ksd, vsd, out, i32(cu), i32(tile0), i32(seq), i32(pos), n_heads, n_kv, hd, window, lse=lse)
+        plain_window = out.clone()
+        k.attn_sink_mix(qd, out, lse, sink_k, sink_v, i32(seq), i32(pos), i32(slots), table, n_heads, rd, window)
+    finally:
+        k.FORCE_SIMPLE = False
+    inv = R.rope_inv_freq(hd, rd, 80.0)
+    o = 0
+    for b, n in enumerate(lens):
+        qb, kb, vb = (t[o:o + n].reshape(n, -1, hd) for t in (q, kk, v))
+        have = min(n, sinks)
+        assert torch.equal(sink_k[slots[b], :, :have].cpu(), kb[:have].transpose(0, 1)), "stored sink keys"
+        assert torch.equal(sink_v[slots[b], :, :have].cpu(), vb[:have].transpose(0, 1)), "stored sink values"
+        assert (sink_k[slots[b], :, have:] == 7.0).all(), "sinks that the sequence does not have yet stay untouched"
+        close(lse[o:o + n], window_lse_float64(qb, kb, window), torch.float32, "log-sum-exp of sequence %d" % b)
+        want = R.attention(qb, kb, vb, window, sinks, inv).reshape(n, -1)
+        close(out[o:o + n], want, dtype, "prefill attention with sinks, sequence %d" % b)
+        if n > window + 1:         # the sinks matter: without them the result is another
+            assert (plain_window[o:o + n].double().cpu() - want).abs().max() > 1e-2
+        o += n
+    unused = [s for s in range(n_slots) if s not in slots]
+    assert (sink_k[unused] == 7.0).all() and (sink_v[unused] == 7.0).all()
+
+
+@pytest.mark.parametrize("simple", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,rd,window,sinks,lens,splits", [
+    (4, 2, 16, 16, 5, 2, [30, 7, 6, 1, 2], 1), (6, 3, 48, 24, 37, 3, [150, 41, 40, 39, 3], 2),
+    (8, 2, 128, 128, 94, 2, [300, 96, 97, 95], 1), (32, 8, 128, 128, 94, 2, [700, 200], 3),
+    (4, 1, 64, 32, 70, 4, [200, 73, 74, 2], 2)])
+def test_attn_decode_with_sinks(n_heads, n_kv, hd, rd, window, sinks, lens, splits, dtype, simple):
+    """A decode step's sinks: the sequences still at their first positions store the key they just wrote;
+    the others have theirs from before; every query mixes in the sinks its window no longer covers."""
+    k = K()
+    B = len(lens)
+    kp, vp, bt, slots, ring, keys, vals = paged_case(lens, n_kv, hd, window, dtype, 40)
+    n_slots = bt.shape[0]
+    q = rnd((B, n_heads * hd), 36, dtype)
+    sink_k = torch.full((n_slots, n_kv, sinks, hd), float("nan"), dtype=dtype)
+    sink_v = torch.full((n_slots, n_kv, sinks, hd), float("nan"), dtype=dtype)
+    for b, n in enumerate(lens):          # what earlier steps stored; the newest position is this step's to store
+        have = min(sinks, n - 1)
+        sink_k[slots[b], :, :have] = keys[b][:have].transpose(0, 1)
+        sink_v[slots[b], :, :have] = vals[b][:have].transpose(0, 1)
+    sink_k, sink_v = sink_k.to(DEV), sink_v.to(DEV)
+    table = make_table(max(lens) + 1, hd, rd, 80.0).to(DEV)
+    qd = torch.cat([q, torch.zeros((1, n_heads * hd), dtype=dtype)]).to(DEV)
+    out = torch.full((B + 1, n_heads * hd), 5.0, dtype=dtype, device=DEV)
+    lse = torch.empty((B + 1, n_heads), dtype=torch.float32, device=DEV)
+    partial = torch.empty(k.attn_decode_workspace_floats(B + 1, n_heads, hd, splits), device=DEV)
+    seq_slot, seq_len = i32(slots + [-1]), i32(lens + [0])
+    kpd, vpd, btd = kp.to(DEV), vp.to(DEV), bt.to(DEV)
+    k.FORCE_SIMPLE = simple
+    try:
+        k.sink_store(kpd, vpd, btd, seq_slot, seq_len, sink_k, sink_v, True)
+        k.attn_decode(qd, kpd, vpd, btd, ring, seq_slot, seq_len, out, partial, n_heads, n_kv, hd, window, splits,
+                      lse=lse)
+        k.attn_sink_mix(qd, out, lse, sink_k, sink_v, i32(list(range(B + 1))), i32([n - 1 for n in lens] + [0]),
+                        seq_slot, table, n_heads, rd, window)
+    finally:
+        k.FORCE_SIMPLE = False
+    inv = R.rope_inv_freq(hd, rd, 80.0)
+    for b, n in enumerate(lens):
+        have = min(sinks, n)
+        assert torch.equal(sink_k[slots[b], :, :have].cpu(), keys[b][:have].transpose(0, 1)), "sink keys of row %d" % b
+        assert torch.equal(sink_v[slots[b], :, :have].cpu(), vals[b][:have].transpose(0, 1)), "sink values of row %d" % b
+        qf = torch.zeros((n, n_heads, hd), dtype=torch.float64)
+        qf[-1] = q[b].double().reshape(n_heads, hd)
+        want = R.attention(qf, keys[b], vals[b], window, sinks, inv)[-1].reshape(-1)
+        close(out[b], want, dtype, "decode attention with sinks, row %d (%d keys)" % (b, n))
+        close(lse[b], window_lse_float64(qf, keys[b], window)[-1], torch.float32, "log-sum-exp of row %d" % b)
+    assert (out[B] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_sink_far_behind_the_window_decides(dtype):
+    """One sink key is made so that, turned by the number of positions the sinks have been pushed on at
+    this query (position - window - sinks + 1), it is the query itself, at a position many windows on:
+    the result is that sink's value if and only if the key is turned by exactly that much."""
+    k = K()
+    hd, window, sinks, n = 64, 20, 2, 333
+    table = make_table(n, hd, hd, 4.0)
+    inv = R.rope_inv_freq(hd, hd, 4.0)
+    base = torch.zeros(hd, dtype=torch.float64)
+    base[0::2] = 6.0                                   # every pair along its first axis
+    pos = n - 1
+    turn = pos - window - sinks + 1
+    qrot = R.rope_interleaved(base.reshape(1, 1, hd), torch.tensor([pos]), inv).reshape(1, hd)
+    kj = R.rope_interleaved(base.reshape(1, 1, hd), torch.tensor([pos - turn]), inv).reshape(hd)
+    sink_k = torch.zeros((1, 1, sinks, hd), dtype=dtype)
+    sink_v = torch.zeros((1, 1, sinks, hd), dtype=dtype)
+    sink_k[0, 0, 1] = kj.to(dtype)
+    sink_v[0, 0, 0, 0] = 1.0
+    sink_v[0, 0, 1, 1] = 1.0
+    out = torch.zeros((1, hd), dtype=dtype, device=DEV)
+    out[0, 2] = 1.0                                    # what the window gave
+    lse = torch.full((1, 1), 100.0, dtype=torch.float32, device=DEV)
+    k.attn_sink_mix(qrot.to(dtype).to(DEV), out, lse, sink_k.to(DEV), sink_v.to(DEV), i32([0]), i32([pos]), i32([0]),
+                    table.to(DEV), 1, hd, window)
+    got = out.cpu().double()[0]
+    # turned right, the sink scores |base|^2 / sqrt(hd) = 144 against 100 for the window; one position off
+    # it would score 120 (the plain rotation says so) and still win, hence the second run below
+    assert got[1] > 0.999 and got[0] < 1e-3 and got[2] < 1e-3, got[:3]
+    right = R.rope_interleaved(kj.reshape(1, 1, hd), torch.tensor([turn]), inv).reshape(hd)
+    assert abs(float(right @ qrot[0]) / math.sqrt(hd) - 144.0) < 1e-6
+    for wrong in (turn - 1, turn + 1, 0):
+        off = R.rope_interleaved(kj.reshape(1, 1, hd), torch.tensor([wrong]), inv).reshape(hd)
+        assert float(off @ qrot[0]) / math.sqrt(hd) < 121.0
+    # with the window at 132 a sink turned one position off (120) would lose; the right one (144) wins
+    out2 = torch.zeros((1, hd), dtype=dtype, device=DEV)
+    out2[0, 2] = 1.0
+    lse.fill_(132.0)
+    k.attn_sink_mix(qrot.to(dtype).to(DEV), out2, lse, sink_k.to(DEV), sink_v.to(DEV), i32([0]), i32([pos]), i32([0]),
+                    table.to(DEV), 1, hd, window)
+    got2 = out2.cpu().double()[0]
+    assert got2[1] > 0.999 and got2[2] < 1e-3, got2[:3]
+
+
 # ------------------------------------------------------------------ sampling
 
 def test_argmax_and_sample():

@@ -2,7 +2,7 @@
 requests into steps: each request alone and whole; with the last 32 tokens one
 by one; in batches of unequal lengths whose shorter requests end earlier, one
 batch after another so that slots and pages are used again (the cache is
-poisoned with NaN between batches).  float32 and bfloat16, five tiny
+poisoned with NaN between batches).  float32 and bfloat16, eight tiny
 configurations."""
 import numpy as np
 import pytest
@@ -21,6 +21,8 @@ LENGTHS = {
     "tiny_wide_heads": [150, 33, 260, 64, 65],
     "tiny_long": [700, 64, 129],
     "small_windowed": [300, 97, 64, 200, 31],
+    "small_sinks": [300, 97, 130, 200, 31],
+    "tiny_sinks": [150, 33, 260, 64, 41, 3],
 }
 # batches: (request indices, first-step lengths)
 GROUPS = {
@@ -30,6 +32,9 @@ GROUPS = {
     "tiny_wide_heads": [([0, 1, 2], [120, 3, 101]), ([3, 4], [63, 64]), ([1, 0], [32, 100])],
     "tiny_long": [([0, 1, 2], [500, 1, 100]), ([2, 1], [128, 63])],
     "small_windowed": [([0, 1, 2], [250, 96, 1]), ([3, 4, 1], [97, 30, 60])],
+    # a request that starts with one token writes its sinks in decode steps and passes the window later
+    "small_sinks": [([0, 1, 2], [250, 96, 1]), ([3, 4, 1], [97, 30, 60])],
+    "tiny_sinks": [([0, 1, 2], [120, 3, 101]), ([3, 4, 5], [1, 40, 2]), ([1, 0], [32, 100])],
 }
 
 _engines = {}

@@ -323,3 +323,56 @@ def test_perplexity_of_uniform_logits_is_the_vocabulary():
     V = 17
     ppl, err = R.perplexity(torch.zeros(5, V), [1, 2, 3, 4, 5])
     assert abs(ppl - V) < 1e-9 and err < 1e-6
+
+
+# ---------------------------------------------------------------- attention sinks
+
+def _rotated_qkv(seed, T, H, KV, hd, rotary_dim, theta):
+    g = torch.Generator().manual_seed(seed)
+    inv = R.rope_inv_freq(hd, rotary_dim, theta)
+    pos = torch.arange(T)
+    q = R.rope_interleaved(torch.randn(T, H, hd, generator=g, dtype=F64), pos, inv)
+    k = R.rope_interleaved(torch.randn(T, KV, hd, generator=g, dtype=F64), pos, inv)
+    v = torch.randn(T, KV, hd, generator=g, dtype=F64)
+    return q, k, v, inv
+
+
+@pytest.mark.parametrize("context,T,rotary_dim", [(5, 23, 8), (9, 30, 4), (3, 11, 8), (16, 16, 8)])
+def test_sinks_in_closed_form_equal_the_reference_ring_step_by_step(context, T, rotary_dim):
+    """`attention` with a window of context - 2 and 2 sinks against the reference's cache of
+    `context` rows filled and turned a token at a time (src/infer.cpp:484-488, 298-330)."""
+    q, k, v, inv = _rotated_qkv(context, T, 4, 2, 8, rotary_dim, 50.0)
+    ring = R.attention_context_ring(q, k, v, context, inv)
+    closed = R.attention(q, k, v, window=context - R.KV_SINKS, sinks=R.KV_SINKS, inv_freq=inv)
+    assert torch.allclose(ring, closed, rtol=0, atol=1e-12)
+    # what plausible mistakes give is different: sinks left as they were stored, sinks turned by one
+    # position too few, and no sinks at all
+    if T > context + 1:
+        still = R.attention(q, k, v, window=context - 2, sinks=2, inv_freq=torch.zeros_like(inv))
+        assert (still - ring).abs().max() > 1e-3
+        assert (R.attention(q, k, v, window=context - 2) - ring).abs().max() > 1e-3
+
+
+def test_sinks_reduce_to_the_window_and_to_all_keys():
+    q, k, v, inv = _rotated_qkv(7, 40, 6, 3, 8, 8, 100.0)
+    # no sinks: the window alone; a window that covers everything: all keys, whatever the sinks
+    assert torch.equal(R.attention(q, k, v, window=9, sinks=0, inv_freq=inv), R.attention(q, k, v, window=9))
+    assert torch.allclose(R.attention(q, k, v, window=40, sinks=3, inv_freq=inv), R.attention(q, k, v))
+    # up to position window + sinks - 1 every key is visible and none is turned
+    some = R.attention(q, k, v, window=9, sinks=3, inv_freq=inv)
+    assert torch.allclose(some[:12], R.attention(q, k, v)[:12])
+    assert (some[12] - R.attention(q, k, v)[12]).abs().max() > 1e-6
+    # a sink behind the window lies window + sinks - 1 - j behind the query wherever the query is: with keys
+    # and queries that are the same vector at every position (before rotation) and values that name
+    # their position, the weights of the sinks are the same at every position past the context
+    T, hd = 40, 8
+    base_q, base_k = torch.randn(1, 1, hd, dtype=F64), torch.randn(1, 1, hd, dtype=F64)
+    pos = torch.arange(T)
+    qq = R.rope_interleaved(base_q.expand(T, 1, hd).clone(), pos, inv)
+    kk = R.rope_interleaved(base_k.expand(T, 1, hd).clone(), pos, inv)
+    vv = torch.zeros(T, 1, hd, dtype=F64)
+    vv[0, 0, 0] = 1.0                       # element 0 of the output = weight of sink 0
+    vv[1, 0, 1] = 1.0                       # element 1 = weight of sink 1
+    out = R.attention(qq, kk, vv, window=6, sinks=2, inv_freq=inv)
+    assert torch.allclose(out[8:, 0, :2], out[8, 0, :2].expand(T - 8, 2), rtol=0, atol=1e-12)
+    assert out[8, 0, 0] > 0 and out[8, 0, 1] > 0

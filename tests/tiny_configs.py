@@ -102,8 +102,28 @@ SMALL_WINDOWED.update({
     "rms_norm_eps": 1e-5,
 })
 
+# attention sinks beside a window (what the reference's -T makes of a model): three sinks and a
+# window of 37 keys, which prompts and decoding pass several times over; half of each head rotated
+TINY_SINKS = copy.deepcopy(TINY_WIDE_HEADS)
+TINY_SINKS.update({
+    "sliding_window": 37,
+    "attention_sinks": 3,
+    "partial_rotary_factor": 0.5,
+    "rope_theta": 300.0,
+})
+
+# the same at the head size of the matrix-core kernels, a context of 96 = 2 sinks + 94
+SMALL_SINKS = copy.deepcopy(SMALL_WINDOWED)
+SMALL_SINKS.update({
+    "sliding_window": 94,
+    "attention_sinks": 2,
+    "rope_theta": 10000.0,
+})
+
 ALL = {
     "small_windowed": SMALL_WINDOWED,
+    "small_sinks": SMALL_SINKS,
+    "tiny_sinks": TINY_SINKS,
     "tiny_llama": TINY_LLAMA,
     "tiny_mistral": TINY_MISTRAL,
     "tiny_llama3": TINY_LLAMA3,

@@ -7,7 +7,9 @@ the group's block table names the pages that hold its positions.  Cache lines
 and share page numbers: groups that keep all keys and groups that keep a window
 have pools and tables of their own.  A windowed group keeps, per sequence, a ring
 of ceil(window / PAGE) + 1 pages: position p lives in table column (p // PAGE)
-% ring_pages.  Beside the pages there is per-sequence state of fixed size
+% ring_pages; if it also keeps attention sinks (the first positions of a
+sequence, visible behind the window), their keys and values have a place of
+their own per slot, because the ring overwrites their pages.  Beside the pages there is per-sequence state of fixed size
 (StateGroup) for mixers that carry one; it is cleared when a slot is acquired,
 because unlike keys behind the length, stale state is not harmless.
 
@@ -38,6 +40,7 @@ class KVRequest:
     n_kv_heads: int
     head_dim: int
     window: int = 0            # 0: all keys
+    sinks: int = 0             # with a window: the first `sinks` positions are kept beside it
 
 
 @dataclass(frozen=True)
@@ -135,10 +138,22 @@ class KVGroup:
         self.table_host = np.full((n_slots, self.ring_pages), -1, dtype=np.int32)
         self.table = torch.full((n_slots, self.ring_pages), -1, dtype=torch.int32, device=device)
         self._dirty = set()
+        self.sinks = request.sinks if self.window > 0 else 0
+        # A slot's sinks need no clearing when the slot is taken again: a sink is read only once its
+        # position lies behind the window, and by then the slot's present sequence has written it.
+        self.sink_k = self.sink_v = None
+        if self.sinks:
+            self.sink_k = torch.zeros((n, n_slots, H, self.sinks, hd), dtype=dtype, device=device)
+            self.sink_v = torch.zeros((n, n_slots, H, self.sinks, hd), dtype=dtype, device=device)
 
     def line_pages(self, line):
         i = self.line_index[line]
         return self.k_pages[i], self.v_pages[i]
+
+    def line_sinks(self, line):
+        """The line's sink keys and values, [slot, head, sink, element] each."""
+        i = self.line_index[line]
+        return self.sink_k[i], self.sink_v[i]
 
     def pages_needed(self, old_len, new_len):
         """Pages to take so that positions < new_len of a sequence of old_len have a place."""

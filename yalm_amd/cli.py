@@ -5,10 +5,9 @@
       -h                 this text
       -d [hip,cuda]      device; there is no CPU path here (default - hip)
       -m [completion,passkey,perplexity]   mode, may be abbreviated (default - completion)
-      -T <int>           sliding window context length (0 - max): every layer attends to the last <int>
-                         positions only, so a text may be longer than the model's context.  Unlike the
-                         reference, whose -T also keeps the first two positions as attention sinks and
-                         re-rotates them every step, this is a plain window.
+      -T <int>           sliding window context length (0 - max): past <int> positions every layer attends
+                         to the first two positions (attention sinks, placed as if they lay just behind
+                         the window) and to the last <int> - 2, so a text may be longer than <int>
       -i <string>        input prompt           } completion and perplexity:
       -f <filepath>      input file with prompt } exactly one of -i, -f, --tokens
       -t <float>         temperature (default - 1.0; 0 = greedy)
@@ -114,9 +113,9 @@ def _load(a):
         with open(a["random"]) as f:
             cfg = config_from_dict(json.load(f))
         if a["context"]:
-            cfg = cfg.with_window(a["context"])
+            cfg = cfg.with_context(a["context"])
         return Model.random(cfg, a["weight_seed"], dtype=dtype, device="cuda:0")
-    model = Model.from_folder(a["checkpoint"], dtype=dtype, device="cuda:0", window=a["context"])
+    model = Model.from_folder(a["checkpoint"], dtype=dtype, device="cuda:0", context=a["context"])
     return model
 
 

@@ -7,6 +7,9 @@ from typing import List, Optional
 from .spec import LayerSpec, ModelSpec, PartSpec
 
 
+KV_SINKS = 2          # positions kept as attention sinks under a shortened context (src/model.h:12)
+
+
 class ConfigError(ValueError):
     pass
 
@@ -58,6 +61,7 @@ class LlamaConfig:
     partial_rotary_factor: float = 1.0
     rope_scaling: Optional[RopeScaling] = None
     sliding_window: int = 0                   # 0: every key is visible
+    attention_sinks: int = 0                  # with a window: the first positions stay visible beside it
     tie_word_embeddings: bool = True
     hidden_act: str = "silu"
     bos_token_id: Optional[int] = None
@@ -98,6 +102,7 @@ class LlamaConfig:
             partial_rotary_factor=float(d.get("partial_rotary_factor", 1.0)),
             rope_scaling=RopeScaling.from_dict(rs) if rs else None,
             sliding_window=int(window) if window else 0,
+            attention_sinks=int(d.get("attention_sinks") or 0),
             # convert.py:241, 200-204: the head is a tensor of its own only if the key is exactly false
             tie_word_embeddings=d.get("tie_word_embeddings", None) is not False,
             hidden_act=d.get("hidden_act", "silu"),
@@ -126,15 +131,33 @@ class LlamaConfig:
                               % (self.partial_rotary_factor, self.rotary_dim, self.head_dim))
         if self.sliding_window < 0:
             raise ConfigError("sliding_window must not be negative")
+        if self.attention_sinks < 0 or (self.attention_sinks and not self.sliding_window):
+            raise ConfigError("attention_sinks (%d) must not be negative and needs a sliding_window"
+                              % self.attention_sinks)
 
     @property
     def rotary_dim(self):
         return int(self.head_dim * self.partial_rotary_factor)                           # convert.py:43
 
-    def with_window(self, window):
-        """The reference's `-T <n>`: attend over the last n positions only."""
+    def with_window(self, window, sinks=0):
+        """Attend over the last `window` positions only, and over the first `sinks` beside them."""
         import dataclasses
-        return dataclasses.replace(self, sliding_window=int(window)) if window else self
+        if not window:
+            return self
+        cfg = dataclasses.replace(self, sliding_window=int(window), attention_sinks=int(sinks))
+        cfg.validate()
+        return cfg
+
+    def with_context(self, n):
+        """The reference's `-T <n>` (src/main.cpp:437-439, src/infer.cpp:484-488): a context of n
+        positions.  Up to position n - 1 every key is visible; from there on the first KV_SINKS
+        positions and the last n - KV_SINKS."""
+        if not n:
+            return self
+        if int(n) <= KV_SINKS:
+            raise ConfigError("a context of %d positions leaves no window beside the %d attention sinks"
+                              % (int(n), KV_SINKS))
+        return self.with_window(int(n) - KV_SINKS, KV_SINKS)
 
     # ------------------------------------------------------------------ writing
     def to_dict(self):
@@ -153,6 +176,8 @@ class LlamaConfig:
             d["rope_scaling"] = self.rope_scaling.to_dict()
         if self.sliding_window:
             d["sliding_window"] = self.sliding_window
+        if self.attention_sinks:
+            d["attention_sinks"] = self.attention_sinks
         if self.bos_token_id is not None:
             d["bos_token_id"] = self.bos_token_id
         if self.eos_token_ids:
@@ -177,7 +202,8 @@ class LlamaConfig:
                 block="prenorm_residual",
                 mixer=PartSpec("gqa_attention", {
                     "n_heads": self.num_attention_heads, "n_kv_heads": self.num_key_value_heads,
-                    "head_dim": self.head_dim, "window": self.sliding_window, "position": pos,
+                    "head_dim": self.head_dim, "window": self.sliding_window, "sinks": self.attention_sinks,
+                    "position": pos,
                 }, prefix="self_attn."),
                 feed_forward=PartSpec("swiglu", {"hidden": self.intermediate_size}, prefix="mlp."),
                 mixer_norm=PartSpec("rmsnorm", norm, prefix="input_layernorm."),

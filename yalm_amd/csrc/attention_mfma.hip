@@ -19,13 +19,14 @@
 #include "yalm_hip.h"
 
 // attention_simple.hip; base2: the partial results' maxima are exponents of 2, not of e
-int yalm_attn_decode_combine_bf16(const float* partial, void* out, int B, int n_heads, int head_dim, int n_splits,
-                                  int base2, hipStream_t stream);
+int yalm_attn_decode_combine_bf16(const float* partial, void* out, float* lse, int B, int n_heads, int head_dim,
+                                  int n_splits, int base2, hipStream_t stream);
 
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+constexpr float LN2 = 0.6931471805599453f;      // the kernels' maxima are exponents of 2
 
 __device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x8 zero8() { return (bf16x8){0, 0, 0, 0, 0, 0, 0, 0}; }
@@ -43,7 +44,7 @@ template <int HD, int NW>
 __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_kernel(   // 2 waves a SIMD: head size 128 needs their registers
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
-    const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out,
+    const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out, float* __restrict__ lse,
     int n_heads, int n_kv_heads, int window, int n_splits, int n_pages) {
   constexpr int KS = HD / 32, DT = HD / 16;
   __shared__ float sm_m[NW][16];
@@ -200,6 +201,8 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 #pragma unroll
         for (int r = 0; r < 4; ++r) orow[dt * 16 + 4 * qd + r] = static_cast<bf16>(v[r] * inv_l);
       }
+      if (lse != nullptr && wave == 0 && qd == 0)  // natural logarithm of the sum of exp(score): for a later mix with further keys
+        lse[(size_t)b * n_heads + g * G + j] = lt > 0.f ? m_all * LN2 + logf(lt) : -FLT_MAX;
     } else {
       float* part = partial + (((size_t)b * n_heads + g * G + j) * n_splits + split) * (HD + 2);
       for (int dt = wave; dt < DT; dt += NW) {
@@ -239,8 +242,9 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 template <int HD, int NC, int KSPL>
 __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_stage, const bf16* __restrict__ v_stage,
-    bf16* __restrict__ out, const int* __restrict__ cu_seqlens, const int* __restrict__ seq_tile0,
-    const int* __restrict__ tile_order, int fold_at, int B, int n_heads, int n_kv_heads, int window) {
+    bf16* __restrict__ out, float* __restrict__ lse, const int* __restrict__ cu_seqlens,
+    const int* __restrict__ seq_tile0, const int* __restrict__ tile_order, int fold_at, int B, int n_heads,
+    int n_kv_heads, int window) {
   constexpr int KS = HD / 32, DT = HD / 16;
   constexpr int KROW = HD + 8;                    // LDS row strides (elements): 16 bytes of padding
   constexpr int VROW = PAGE + 8;
@@ -460,6 +464,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
       const float m_new = fmaxf(m[c], m2);
       const float f1 = __builtin_amdgcn_exp2f(m[c] - m_new), f2 = __builtin_amdgcn_exp2f(m2 - m_new);
       l[c] = l[c] * f1 + l2 * f2;
+      m[c] = m_new;
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) o[c][dt] = o[c][dt] * f1 + mo[(c * DT + dt) * 256 + tid] * f2;
     }
@@ -476,6 +481,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) orow[dt * 16 + 4 * qd + r] = static_cast<bf16>(o[c][dt][r] * inv_l);
+      if (lse != nullptr && qd == 0) lse[(size_t)(start + pos_q[c]) * n_heads + h] = m[c] * LN2 + logf(lt);
     }
   }
 }
@@ -498,7 +504,7 @@ bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
 }
 }  // namespace
 
-int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out,
+int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out, float* lse,
                                 const int* cu_seqlens, const int* seq_tile0, const int* tile_order, int n_order,
                                 int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
                                 hipStream_t stream) {
@@ -528,10 +534,10 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
       allowed = true;
     }
     if (head_dim == 128)
-      k128<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
+      k128<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
                                        n_kv_heads, window);
     else
-      k64<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
+      k64<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
                                       n_kv_heads, window);
     return launch_status();
   }
@@ -541,29 +547,29 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
   const int fold_at = total > cus && total <= 2 * cus ? cus : (int)total;
   const size_t lds = 2 * tile_bytes;
   if (head_dim == 128)
-    attn_prefill_mfma_kernel<128, 2, 1><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, cu_seqlens, seq_tile0, tile_order,
+    attn_prefill_mfma_kernel<128, 2, 1><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, tile_order,
                                                                    fold_at, B, n_heads, n_kv_heads, window);
   else
-    attn_prefill_mfma_kernel<64, 2, 1><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, cu_seqlens, seq_tile0, tile_order,
+    attn_prefill_mfma_kernel<64, 2, 1><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, tile_order,
                                                                   fold_at, B, n_heads, n_kv_heads, window);
   return launch_status();
 }
 
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
-                               float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
+                               float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                                int n_splits, int n_pages, hipStream_t stream) {
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_heads / n_kv_heads > 16) return YALM_ERR_ARG;
   dim3 grid(n_splits, n_kv_heads, B);
 #define YALM_DECODE(HD_, NW_)                                                                                       \
   attn_decode_mfma_kernel<HD_, NW_><<<grid, NW_ * WAVE, 0, stream>>>(                                               \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot, \
-      seq_len, partial, (bf16*)out, n_heads, n_kv_heads, window, n_splits, n_pages)
+      seq_len, partial, (bf16*)out, lse, n_heads, n_kv_heads, window, n_splits, n_pages)
   // 4 waves a workgroup: 8 measured no faster with one split and slower with more (a CU draws about
   // 33 GB/s whatever its number of waves, so a small batch needs its workgroups spread over all CUs)
   if (head_dim == 128) YALM_DECODE(128, 4); else YALM_DECODE(64, 4);
 #undef YALM_DECODE
   int rc = launch_status();
   if (rc != YALM_OK || n_splits == 1) return rc;   // one split writes the result itself
-  return yalm_attn_decode_combine_bf16(partial, out, B, n_heads, head_dim, n_splits, 1, stream);
+  return yalm_attn_decode_combine_bf16(partial, out, lse, B, n_heads, head_dim, n_splits, 1, stream);
 }

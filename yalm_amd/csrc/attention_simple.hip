@@ -7,13 +7,13 @@
 #include "common.h"
 #include "yalm_hip.h"
 
-int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out,
+int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out, float* lse,
                                 const int* cu_seqlens, const int* seq_tile0, const int* tile_order, int n_order,
                                 int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
                                 hipStream_t stream);
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
-                               float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
+                               float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                                int n_splits, int n_pages, hipStream_t stream);
 
 namespace {
@@ -27,7 +27,7 @@ constexpr int COMBINE_THREADS = 256;
 template <typename T>
 __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
     const T* __restrict__ q, const T* __restrict__ k_stage, const T* __restrict__ v_stage, T* __restrict__ out,
-    const int* __restrict__ seq_tile0, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_heads,
+    float* __restrict__ lse, const int* __restrict__ seq_tile0, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_heads,
     int n_kv_heads, int hd, int window) {
   __shared__ float qs[MAX_HD];
   __shared__ float ps[WAVE];
@@ -85,6 +85,8 @@ __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
     int d = lane + a * WAVE;
     if (d < hd) out[((size_t)t * n_heads + h) * hd + d] = from_f32<T>(acc[a] / l);
   }
+  // natural logarithm of the sum of exp(score) over the keys seen: for a later mix with further keys
+  if (lse != nullptr && lane == 0) lse[(size_t)t * n_heads + h] = m + logf(l);
 }
 
 // ---------------------------------------------------------------------------
@@ -170,8 +172,9 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
 // BASE2: the maxima of the partial results are exponents of 2 (the matrix-core kernel's), else of e
 template <typename T, bool BASE2 = false>
 __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(const float* __restrict__ partial,
-                                                                             T* __restrict__ out, int n_heads, int hd,
-                                                                             int n_splits) {
+                                                                             T* __restrict__ out,
+                                                                             float* __restrict__ lse, int n_heads,
+                                                                             int hd, int n_splits) {
   // One trip to memory: every wave asks for the maxima and denominators of all splits (lanes over
   // splits) and, before it waits for them, for the sums of its own first splits (waves share the
   // splits of the weighted sum and add their parts in a fixed order).
@@ -204,6 +207,8 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(co
   }
   l = wave_sum(l);
   const float inv_l = l > 0.f ? 1.0f / l : 0.f;
+  if (lse != nullptr && threadIdx.x == 0)
+    lse[(size_t)b * n_heads + h] = l > 0.f ? (BASE2 ? m * 0.6931471805599453f : m) + logf(l) : -FLT_MAX;
   float a[ACC];
 #pragma unroll
   for (int j = 0; j < ACC; ++j) a[j] = 0.f;
@@ -246,8 +251,8 @@ bool bad_heads(int n_heads, int n_kv_heads, int hd) {
 }
 }  // namespace
 
-extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void* v_stage, void* out,
-                                 const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
+extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* lse,
+                                     const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                                  const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads,
                                  int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
                                  hipStream_t stream) {
@@ -256,31 +261,41 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32) {
     attn_prefill_simple_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)q, (const float*)k_stage,
-                                                                 (const float*)v_stage, (float*)out, seq_tile0,
+                                                                 (const float*)v_stage, (float*)out, lse, seq_tile0,
                                                                  tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
                                                                  window);
     return launch_status();
   }
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
   if (!force_simple) {
-    int rc = yalm_attn_prefill_bf16_mfma(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tile_order, n_order, T, B,
+    int rc = yalm_attn_prefill_bf16_mfma(q, k_stage, v_stage, out, lse, cu_seqlens, seq_tile0, tile_order, n_order, T, B,
                                          n_tiles, n_heads, n_kv_heads, head_dim, window, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   attn_prefill_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,
-                                                              (const bf16*)v_stage, (bf16*)out, seq_tile0, tok_seq,
+                                                              (const bf16*)v_stage, (bf16*)out, lse, seq_tile0, tok_seq,
                                                               tok_pos, n_heads, n_kv_heads, head_dim, window);
   return launch_status();
 }
 
+extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void* v_stage, void* out,
+                                 const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
+                                 const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads,
+                                 int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
+                                 hipStream_t stream) {
+  return yalm_attn_prefill_lse(q, k_stage, v_stage, out, nullptr, cu_seqlens, seq_tile0, tok_seq, tok_pos, tile_order,
+                               n_order, T, B, n_tiles, n_heads, n_kv_heads, head_dim, window, dtype, force_simple,
+                               stream);
+}
+
 // merges the partial results of the splits (also used by the MFMA kernel)
-int yalm_attn_decode_combine_bf16(const float* partial, void* out, int B, int n_heads, int head_dim, int n_splits,
-                                  int base2, hipStream_t stream) {
+int yalm_attn_decode_combine_bf16(const float* partial, void* out, float* lse, int B, int n_heads, int head_dim,
+                                  int n_splits, int base2, hipStream_t stream) {
   dim3 cgrid(B, n_heads);
   if (base2)
-    attn_decode_combine_kernel<bf16, true><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
+    attn_decode_combine_kernel<bf16, true><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim, n_splits);
   else
-    attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
+    attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim, n_splits);
   return launch_status();
 }
 
@@ -288,10 +303,11 @@ extern "C" long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int
   return (long)B * n_heads * n_splits * (head_dim + 2) * (long)sizeof(float);
 }
 
-extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
-                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
-                                float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
-                                int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream) {
+extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                                    int table_stride, int ring_pages, const int* seq_slot, const int* seq_len,
+                                    void* out, float* lse, float* partial, int B, int n_heads, int n_kv_heads,
+                                    int head_dim, int window, int n_splits, int n_pages, int dtype, int force_simple,
+                                    hipStream_t stream) {
   if (B <= 0) return YALM_OK;
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0)
     return YALM_ERR_ARG;
@@ -300,21 +316,30 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
     attn_decode_simple_kernel<float><<<grid, WAVE, 0, stream>>>(
         (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
         seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
-    attn_decode_combine_kernel<float><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (float*)out, n_heads, head_dim, n_splits);
+    attn_decode_combine_kernel<float><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (float*)out, lse, n_heads, head_dim, n_splits);
     return launch_status();
   }
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
   if (!force_simple) {
     int rc = yalm_attn_decode_bf16_mfma(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len,
-                                        out, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages,
-                                        stream);
+                                        out, lse, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits,
+                                        n_pages, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   attn_decode_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
       seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
-  attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, n_heads, head_dim, n_splits);
+  attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim, n_splits);
   return launch_status();
+}
+
+extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
+                                float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
+                                int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream) {
+  return yalm_attn_decode_lse(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out,
+                              nullptr, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, dtype,
+                              force_simple, stream);
 }
 
 // ---------------------------------------------------------------------------

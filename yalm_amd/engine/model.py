@@ -74,13 +74,17 @@ class Model:
         return self
 
     @classmethod
-    def from_folder(cls, path, dtype=torch.bfloat16, device="cuda:0", window=None, strict=False):
+    def from_folder(cls, path, dtype=torch.bfloat16, device="cuda:0", window=None, strict=False, context=None):
         """The model of a folder with config.json and *.safetensors; the class of the
         configuration is chosen by config.json's architecture.  strict: tensors in the
-        folder that the model does not use are an error (else a warning)."""
+        folder that the model does not use are an error (else a warning).  window: attend over
+        the last `window` positions only; context: the reference's -T (attention sinks and a window
+        that fill a context of that many positions)."""
         cfg = config_from_folder(path)
         if window:
             cfg = cfg.with_window(window)
+        if context:
+            cfg = cfg.with_context(context)
         model = cls(cfg.to_spec(), cfg)
         source = TensorSource(path)
         source.check(model.param_specs(), strict=strict)

@@ -457,10 +457,11 @@ def prefill_tile_order(n_tokens):
 
 
 def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
-                 window, tile_order=None):
+                 window, tile_order=None, lse=None):
     """Causal (and windowed) attention of packed sequences that start at position 0, over
     the keys and values that rope_kv_write staged for this step.  tile_order (device int32,
-    from prefill_tile_order) only changes the order of the work."""
+    from prefill_tile_order) only changes the order of the work.  lse (float32 [T, n_heads], optional)
+    receives the logarithm of every query's sum of exp(score), for attn_sink_mix."""
     _check_heads(n_heads, n_kv_heads, head_dim)
     T = q.shape[0]
     dt = q.dtype
@@ -478,9 +479,10 @@ def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_p
     if tile_order is not None:
         n_order = tile_order.shape[0]
         p_or = _need(tile_order, "tile_order", torch.int32, (n_order,))
-    library.check(library.lib().yalm_attn_prefill(p_q, p_k, p_v, p_o, p_cu, p_t0, p_ts, p_tp, p_or, n_order, T, B,
-                                                  n_tiles, n_heads, n_kv_heads, head_dim, int(window),
-                                                  dtype_code(dt), 1 if FORCE_SIMPLE else 0, _stream()),
+    p_lse = None if lse is None else _need(lse, "lse", torch.float32, (T, n_heads))
+    library.check(library.lib().yalm_attn_prefill_lse(p_q, p_k, p_v, p_o, p_lse, p_cu, p_t0, p_ts, p_tp, p_or, n_order,
+                                                      T, B, n_tiles, n_heads, n_kv_heads, head_dim, int(window),
+                                                      dtype_code(dt), 1 if FORCE_SIMPLE else 0, _stream()),
                   "attn_prefill")
     return out
 
@@ -490,8 +492,8 @@ def attn_decode_workspace_floats(B, n_heads, head_dim, n_splits):
 
 
 def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len, out, partial, n_heads, n_kv_heads,
-                head_dim, window, n_splits):
-    """One query per sequence over the cache pages; seq_len counts the new key."""
+                head_dim, window, n_splits, lse=None):
+    """One query per sequence over the cache pages; seq_len counts the new key.  lse as in attn_prefill."""
     _check_heads(n_heads, n_kv_heads, head_dim)
     B = q.shape[0]
     dt = q.dtype
@@ -510,9 +512,64 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
     p_w = _need(partial, "partial", torch.float32)
     if partial.numel() < need:
         raise ValueError("attn_decode workspace too small: %d floats, %d needed" % (partial.numel(), need))
-    library.check(library.lib().yalm_attn_decode(
-        p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_w, B, n_heads, n_kv_heads, head_dim,
+    p_lse = None if lse is None else _need(lse, "lse", torch.float32, (B, n_heads))
+    library.check(library.lib().yalm_attn_decode_lse(
+        p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_lse, p_w, B, n_heads, n_kv_heads, head_dim,
         int(window), int(n_splits), n_pages, dtype_code(dt), 1 if FORCE_SIMPLE else 0, _stream()), "attn_decode")
+    return out
+
+
+MAX_SINKS = 16
+
+
+def sink_store(k_src, v_src, page0, seq_slot, seq_len, sink_k, sink_v, decode):
+    """Copies the keys and values of positions < n_sinks that this step wrote from their page into the
+    per-slot store sink_k, sink_v [slots, n_kv_heads, n_sinks, head_dim].  k_src, v_src: pages in the
+    cache's format.  decode: page0 is the block table (the page of positions 0..63 of slot s is
+    page0[s, 0]) and the step wrote position seq_len - 1; else page0[b] is sequence b's first tile of
+    the staging area and the step wrote positions 0 .. seq_len - 1."""
+    n_slots, n_kv_heads, n_sinks, head_dim = sink_k.shape
+    dt = sink_k.dtype
+    n_src = k_src.shape[0]
+    B = seq_slot.shape[0]
+    p_k = _need(k_src, "k_src", dt, (n_src, n_kv_heads, PAGE, head_dim))
+    p_v = _need(v_src, "v_src", dt, (n_src, n_kv_heads, head_dim, PAGE))
+    if decode:
+        p_p0 = _need(page0, "page0", torch.int32, (None, None))
+        if page0.shape[0] < n_slots:
+            raise ValueError("the block table has %d rows for %d slots" % (page0.shape[0], n_slots))
+        stride = page0.shape[1]
+    else:
+        p_p0 = _need(page0, "page0", torch.int32, (B + 1,))
+        stride = 0
+    library.check(library.lib().yalm_sink_store(
+        p_k, p_v, p_p0, stride, _need(seq_slot, "seq_slot", torch.int32, (B,)),
+        _need(seq_len, "seq_len", torch.int32, (B,)), _need(sink_k, "sink_k", dt),
+        _need(sink_v, "sink_v", dt, (n_slots, n_kv_heads, n_sinks, head_dim)), 1 if decode else 0, B, n_src, n_slots,
+        n_kv_heads, head_dim, n_sinks, dtype_code(dt), _stream()), "sink_store")
+
+
+def attn_sink_mix(q, out, lse, sink_k, sink_v, tok_seq, tok_pos, seq_slot, cos_sin, n_heads, rotary_dim, window):
+    """Adds the attention sinks that the window no longer covers to the attention result `out`
+    (in place): for the token at position p the sinks j < min(n_sinks, p - window + 1), their keys
+    turned by max(0, p - window - n_sinks + 1) positions with the table cos_sin (None: not turned).
+    lse is what attn_prefill / attn_decode left for these queries."""
+    n_slots, n_kv_heads, n_sinks, head_dim = sink_k.shape
+    _check_heads(n_heads, n_kv_heads, head_dim)
+    T = q.shape[0]
+    dt = q.dtype
+    B = seq_slot.shape[0]
+    n_pos, p_cs = 0, None
+    if cos_sin is not None and rotary_dim > 0:
+        n_pos = cos_sin.shape[0]
+        p_cs = _need(cos_sin, "cos_sin", torch.float32, (n_pos, rotary_dim // 2, 2))
+    library.check(library.lib().yalm_attn_sink_mix(
+        _need(q, "q", dt, (T, n_heads * head_dim)), _need(out, "out", dt, (T, n_heads * head_dim)),
+        _need(lse, "lse", torch.float32, (T, n_heads)), _need(sink_k, "sink_k", dt),
+        _need(sink_v, "sink_v", dt, (n_slots, n_kv_heads, n_sinks, head_dim)),
+        _need(tok_seq, "tok_seq", torch.int32, (T,)), _need(tok_pos, "tok_pos", torch.int32, (T,)),
+        _need(seq_slot, "seq_slot", torch.int32, (B,)), p_cs, n_pos, T, n_slots, n_heads, n_kv_heads, head_dim,
+        int(rotary_dim) if p_cs is not None else 0, int(window), n_sinks, dtype_code(dt), _stream()), "attn_sink_mix")
     return out
 
 

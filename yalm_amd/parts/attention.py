@@ -6,7 +6,14 @@ position; k and v stored in the cache; per query head h with KV head h // group:
 scores q.k / sqrt(head_dim) over the visible keys, softmax in float32, mix of
 the values; the output projection is added to the residual stream.  Key j is
 visible to the query at position i iff j <= i and (window == 0 or i - j <
-window) (the reference's kv_len rows, src/infer.cpp:486-488).
+window or j < sinks) (the reference's kv_len rows, src/infer.cpp:486-488).
+
+Sinks (src/infer.cpp:305-319: with a context of n the reference keeps positions
+0 and 1 and the last n - 2, and turns the kept keys one position further every
+step past n): a sink j that the window no longer covers is scored as if it lay
+window + sinks - 1 - j positions behind the query, whatever the query's
+position.  Its key is stored as it was rotated at j and turned by
+i - (window + sinks - 1) when it is read.
 
 The three projections are one matrix [q; k; v] (the reference fuses them by
 pointer, src/infer.cu:290-337); q/k rows are re-ordered at load if the folder
@@ -32,6 +39,11 @@ class GQAttention(Part):
         self.n_kv_heads = int(p["n_kv_heads"])
         self.head_dim = int(p["head_dim"])
         self.window = int(p.get("window", 0) or 0)
+        self.sinks = int(p.get("sinks", 0) or 0)
+        if self.sinks and not self.window:
+            raise ValueError("attention sinks (%d) need a window" % self.sinks)
+        if not 0 <= self.sinks <= kernels.MAX_SINKS:
+            raise ValueError("%d attention sinks asked for, at most %d are supported" % (self.sinks, kernels.MAX_SINKS))
         if self.n_heads % self.n_kv_heads:
             raise ValueError("n_heads %d is no multiple of n_kv_heads %d" % (self.n_heads, self.n_kv_heads))
         if self.head_dim % 2 or self.head_dim > kernels.MAX_HEAD_DIM:
@@ -63,11 +75,12 @@ class GQAttention(Part):
         return (self.wqkv.numel() + self.wo.numel()) * self.wqkv.element_size()
 
     def cache_request(self):
-        return KVRequest(self.n_kv_heads, self.head_dim, self.window)
+        return KVRequest(self.n_kv_heads, self.head_dim, self.window, self.sinks)
 
     def describe(self, compute_dtype):
         what = "attention, %d heads in %d groups of head size %d%s" % (
-            self.n_heads, self.n_kv_heads, self.head_dim, ", window %d" % self.window if self.window else "")
+            self.n_heads, self.n_kv_heads, self.head_dim,
+            (", window %d" % self.window if self.window else "") + (" + %d sinks" % self.sinks if self.sinks else ""))
         if compute_dtype != torch.bfloat16:
             return what + ": float32-arithmetic kernels", False
         group = self.n_heads // self.n_kv_heads
@@ -139,7 +152,7 @@ class GQAttention(Part):
                                   ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads,
                                   self.n_kv_heads, self.head_dim, pos.rotary_dim, slices=slices)
         o = ctx.ws.get("attn.o", (T, self.q_dim), self.wo.dtype)
-        self._decode_attention(q, o, ctx, group, k_pages, v_pages)
+        self._decode_attention(q, o, ctx, group, line, k_pages, v_pages, True)
         emit = self._emit_args(emit_for, ctx, T, self.dim)
         ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.q_dim) if emit is None else None
         if emit is not None and kernels.can_chain(T, self.q_dim, o.dtype):
@@ -153,14 +166,25 @@ class GQAttention(Part):
         else:
             self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)
 
-    def _decode_attention(self, q, o, ctx, group, k_pages, v_pages):
+    def _decode_attention(self, q, o, ctx, group, line, k_pages, v_pages, writes_cache):
         T = q.shape[0]
         n_splits = self.decode_splits(T, min(group.ring_pages, ctx.pages_bucket))
         partial = ctx.ws.get("attn.partial",
                              (kernels.attn_decode_workspace_floats(T, self.n_heads, self.head_dim, n_splits),),
                              torch.float32)
+        lse = ctx.ws.get("attn.lse", (T, self.n_heads), torch.float32) if self.sinks else None
+        if self.sinks and writes_cache:      # a sequence still at its first positions has just written a sink
+            sink_k, sink_v = group.line_sinks(line)
+            kernels.sink_store(k_pages, v_pages, group.table, ctx.seq_slot, ctx.seq_len, sink_k, sink_v, True)
         kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o, partial,
-                            self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits)
+                            self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits, lse=lse)
+        if self.sinks:
+            self._mix_sinks(q, o, lse, ctx, group, line)
+
+    def _mix_sinks(self, q, o, lse, ctx, group, line):
+        sink_k, sink_v = group.line_sinks(line)
+        kernels.attn_sink_mix(q, o, lse, sink_k, sink_v, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, self.position.table,
+                              self.n_heads, self.position.rotary_dim, self.window)
 
     def forward(self, h, x, ctx, line, writes_cache=True):
         T = h.shape[0]
@@ -198,8 +222,14 @@ class GQAttention(Part):
                                   pos.rotary_dim)
         o = ws.get("attn.o", (T, self.q_dim), act)
         if prefill:
+            lse = ws.get("attn.lse", (T, self.n_heads), torch.float32) if self.sinks else None
+            if self.sinks and writes_cache:
+                sink_k, sink_v = group.line_sinks(line)
+                kernels.sink_store(kst, vst, ctx.seq_tile0, ctx.seq_slot, ctx.seq_len, sink_k, sink_v, False)
             kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, ctx.seq_tile0, ctx.tok_seq, ctx.tok_pos,
-                                 self.n_heads, self.n_kv_heads, self.head_dim, self.window, ctx.tile_order)
+                                 self.n_heads, self.n_kv_heads, self.head_dim, self.window, ctx.tile_order, lse=lse)
+            if self.sinks:
+                self._mix_sinks(q, o, lse, ctx, group, line)
         else:
-            self._decode_attention(q, o, ctx, group, k_pages, v_pages)
+            self._decode_attention(q, o, ctx, group, line, k_pages, v_pages, writes_cache)
         self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)
