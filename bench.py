@@ -81,6 +81,9 @@ def main():
     ap.add_argument("--prefill-len", type=int, default=PREFILL, help="tokens of the timed prompt")
     ap.add_argument("--shape", default="mistral-7b-v0.2", choices=sorted(SHAPES),
                     help="the layer sizes: the Mistral-7B-v0.2 shape (default), Llama-3.2-3B or Mistral-7B-v0.1")
+    ap.add_argument("--context", type=int, default=0,
+                    help="the reference's -T: past this many positions two attention sinks and the last "
+                         "<context> - 2 positions are attended to (0: the shape's own window, if any)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this library runs on one GPU; --gpus %d is not measured" % args.gpus, flush=True)
@@ -92,6 +95,9 @@ def main():
 
     dtype = {"bf16": torch.bfloat16, "fp32": torch.float32}[args.dtype]
     CFG, shape_name, CONTEXT, (first, last) = SHAPES[args.shape]
+    if args.context:
+        CFG = dict(CFG, sliding_window=args.context - 2, attention_sinks=2)
+        shape_name += ", context %d (2 sinks)" % args.context
     # the timed steps' positions lie in the middle of the workload's range (all of it if they are as many)
     run = args.steps + args.warmup
     PROMPT = max(first, min((first + last - args.steps) // 2 - args.warmup, last - run))

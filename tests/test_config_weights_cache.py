@@ -53,7 +53,7 @@ def test_a_context_is_two_sinks_and_a_window():
     assert all(l.mixer.params["window"] == 38 and l.mixer.params["sinks"] == 2 for l in t.to_spec().layers)
     assert config_from_dict(t.to_dict()) == t                  # the folder of such a model keeps both
     assert c.with_window(16).attention_sinks == 0 and c.with_window(16, 3).attention_sinks == 3
-    for n in (1, 2):
+    for n in (1, 2, 3):
         with pytest.raises(ConfigError, match="sinks"):
             c.with_context(n)
     with pytest.raises(ConfigError, match="attention_sinks"):

@@ -755,7 +755,7 @@ def test_attn_prefill_with_sinks(n_heads, n_kv, hd, rd, window, sinks, lens, dty
     qd, ksd, vsd = q.to(DEV), ks.to(DEV), vs.to(DEV)
     k.FORCE_SIMPLE = simple
     try:
-        k.sink_store(ksd, vsd, i32(tile0), i32(slots), i32(lens), sink_k, sink_v, False)
+        k.sink_store(ksd, vsd, i32(tile0), i32(slots), i32(lens), sink_k, sink_v)
         k.attn_prefill(qd, ksd, vsd, out, i32(cu), i32(tile0), i32(seq), i32(pos), n_heads, n_kv, hd, window, lse=lse)
         plain_window = out.clone()
         k.attn_sink_mix(qd, out, lse, sink_k, sink_v, i32(seq), i32(pos), i32(slots), table, n_heads, rd, window)
@@ -784,10 +784,11 @@ def test_attn_prefill_with_sinks(n_heads, n_kv, hd, rd, window, sinks, lens, dty
 @pytest.mark.parametrize("n_heads,n_kv,hd,rd,window,sinks,lens,splits", [
     (4, 2, 16, 16, 5, 2, [30, 7, 6, 1, 2], 1), (6, 3, 48, 24, 37, 3, [150, 41, 40, 39, 3], 2),
     (8, 2, 128, 128, 94, 2, [300, 96, 97, 95], 1), (32, 8, 128, 128, 94, 2, [700, 200], 3),
-    (4, 1, 64, 32, 70, 4, [200, 73, 74, 2], 2)])
+    (4, 1, 64, 32, 70, 4, [200, 73, 74, 2], 2), (2, 2, 32, 0, 9, 1, [40, 1], 70)])
 def test_attn_decode_with_sinks(n_heads, n_kv, hd, rd, window, sinks, lens, splits, dtype, simple):
     """A decode step's sinks: the sequences still at their first positions store the key they just wrote;
-    the others have theirs from before; every query mixes in the sinks its window no longer covers."""
+    the others have theirs from before; the merge of the splits takes in the sinks that a query's window
+    no longer covers."""
     k = K()
     B = len(lens)
     kp, vp, bt, slots, ring, keys, vals = paged_case(lens, n_kv, hd, window, dtype, 40)
@@ -800,20 +801,15 @@ def test_attn_decode_with_sinks(n_heads, n_kv, hd, rd, window, sinks, lens, spli
         sink_k[slots[b], :, :have] = keys[b][:have].transpose(0, 1)
         sink_v[slots[b], :, :have] = vals[b][:have].transpose(0, 1)
     sink_k, sink_v = sink_k.to(DEV), sink_v.to(DEV)
-    table = make_table(max(lens) + 1, hd, rd, 80.0).to(DEV)
+    table = make_table(max(lens) + 1, hd, rd, 80.0).to(DEV) if rd else None
     qd = torch.cat([q, torch.zeros((1, n_heads * hd), dtype=dtype)]).to(DEV)
     out = torch.full((B + 1, n_heads * hd), 5.0, dtype=dtype, device=DEV)
-    lse = torch.empty((B + 1, n_heads), dtype=torch.float32, device=DEV)
     partial = torch.empty(k.attn_decode_workspace_floats(B + 1, n_heads, hd, splits), device=DEV)
     seq_slot, seq_len = i32(slots + [-1]), i32(lens + [0])
-    kpd, vpd, btd = kp.to(DEV), vp.to(DEV), bt.to(DEV)
     k.FORCE_SIMPLE = simple
     try:
-        k.sink_store(kpd, vpd, btd, seq_slot, seq_len, sink_k, sink_v, True)
-        k.attn_decode(qd, kpd, vpd, btd, ring, seq_slot, seq_len, out, partial, n_heads, n_kv, hd, window, splits,
-                      lse=lse)
-        k.attn_sink_mix(qd, out, lse, sink_k, sink_v, i32(list(range(B + 1))), i32([n - 1 for n in lens] + [0]),
-                        seq_slot, table, n_heads, rd, window)
+        k.attn_decode(qd, kp.to(DEV), vp.to(DEV), bt.to(DEV), ring, seq_slot, seq_len, out, partial, n_heads, n_kv, hd,
+                      window, splits, sinks=(sink_k, sink_v, table, rd, True))
     finally:
         k.FORCE_SIMPLE = False
     inv = R.rope_inv_freq(hd, rd, 80.0)
@@ -825,8 +821,31 @@ def test_attn_decode_with_sinks(n_heads, n_kv, hd, rd, window, sinks, lens, spli
         qf[-1] = q[b].double().reshape(n_heads, hd)
         want = R.attention(qf, keys[b], vals[b], window, sinks, inv)[-1].reshape(-1)
         close(out[b], want, dtype, "decode attention with sinks, row %d (%d keys)" % (b, n))
-        close(lse[b], window_lse_float64(qf, keys[b], window)[-1], torch.float32, "log-sum-exp of row %d" % b)
     assert (out[B] == 0).all()
+
+
+@pytest.mark.parametrize("simple", [False, True])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attn_decode_leaves_the_log_sum_exp(dtype, simple):
+    k = K()
+    n_heads, n_kv, hd, window = 8, 2, 128, 94
+    for lens, splits in (([300, 5, 96], 1), ([300, 5, 96], 3)):
+        B = len(lens)
+        kp, vp, bt, slots, ring, keys, vals = paged_case(lens, n_kv, hd, window, dtype, 41)
+        q = rnd((B, n_heads * hd), 37, dtype)
+        out = torch.empty((B, n_heads * hd), dtype=dtype, device=DEV)
+        lse = torch.empty((B, n_heads), dtype=torch.float32, device=DEV)
+        partial = torch.empty(k.attn_decode_workspace_floats(B, n_heads, hd, splits), device=DEV)
+        k.FORCE_SIMPLE = simple
+        try:
+            k.attn_decode(q.to(DEV), kp.to(DEV), vp.to(DEV), bt.to(DEV), ring, i32(slots), i32(lens), out, partial,
+                          n_heads, n_kv, hd, window, splits, lse=lse)
+        finally:
+            k.FORCE_SIMPLE = False
+        for b, n in enumerate(lens):
+            qf = torch.zeros((n, n_heads, hd), dtype=torch.float64)
+            qf[-1] = q[b].double().reshape(n_heads, hd)
+            close(lse[b], window_lse_float64(qf, keys[b], window)[-1], torch.float32, "log-sum-exp of row %d" % b)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

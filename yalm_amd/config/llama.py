@@ -131,8 +131,8 @@ class LlamaConfig:
                               % (self.partial_rotary_factor, self.rotary_dim, self.head_dim))
         if self.sliding_window < 0:
             raise ConfigError("sliding_window must not be negative")
-        if self.attention_sinks < 0 or (self.attention_sinks and not self.sliding_window):
-            raise ConfigError("attention_sinks (%d) must not be negative and needs a sliding_window"
+        if self.attention_sinks < 0 or (self.attention_sinks and self.sliding_window < self.attention_sinks):
+            raise ConfigError("attention_sinks (%d) must not be negative and needs a sliding_window at least as wide"
                               % self.attention_sinks)
 
     @property
@@ -154,7 +154,7 @@ class LlamaConfig:
         positions and the last n - KV_SINKS."""
         if not n:
             return self
-        if int(n) <= KV_SINKS:
+        if int(n) < 2 * KV_SINKS:
             raise ConfigError("a context of %d positions leaves no window beside the %d attention sinks"
                               % (int(n), KV_SINKS))
         return self.with_window(int(n) - KV_SINKS, KV_SINKS)

@@ -16,11 +16,12 @@
 #include <math.h>
 #include <type_traits>
 #include "common.h"
+#include "sinks.h"
 #include "yalm_hip.h"
 
 // attention_simple.hip; base2: the partial results' maxima are exponents of 2, not of e
 int yalm_attn_decode_combine_bf16(const float* partial, void* out, float* lse, int B, int n_heads, int head_dim,
-                                  int n_splits, int base2, hipStream_t stream);
+                                  int n_splits, int base2, const SinkArgs& sinks, hipStream_t stream);
 
 namespace {
 
@@ -191,7 +192,7 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
     float lt = sm_l[0][j];
 #pragma unroll
     for (int w = 1; w < NW; ++w) lt += sm_l[w][j];
-    if (n_splits == 1) {                          // nothing to merge with: this is the result
+    if (n_splits == 1 && out != nullptr) {        // nothing to merge with: this is the result
       bf16* orow = out + ((size_t)b * n_heads + g * G + j) * HD;
       const float inv_l = lt > 0.f ? 1.0f / lt : 0.f;
       for (int dt = wave; dt < DT; dt += NW) {
@@ -558,18 +559,20 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
-                               int n_splits, int n_pages, hipStream_t stream) {
+                               int n_splits, int n_pages, const SinkArgs& sinks, hipStream_t stream) {
+  // with sinks the merge kernel always runs: it takes them in, also where there is one split
+  const bool merge = n_splits > 1 || sinks.n_sinks > 0;
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_heads / n_kv_heads > 16) return YALM_ERR_ARG;
   dim3 grid(n_splits, n_kv_heads, B);
 #define YALM_DECODE(HD_, NW_)                                                                                       \
   attn_decode_mfma_kernel<HD_, NW_><<<grid, NW_ * WAVE, 0, stream>>>(                                               \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot, \
-      seq_len, partial, (bf16*)out, lse, n_heads, n_kv_heads, window, n_splits, n_pages)
+      seq_len, partial, merge ? nullptr : (bf16*)out, lse, n_heads, n_kv_heads, window, n_splits, n_pages)
   // 4 waves a workgroup: 8 measured no faster with one split and slower with more (a CU draws about
   // 33 GB/s whatever its number of waves, so a small batch needs its workgroups spread over all CUs)
   if (head_dim == 128) YALM_DECODE(128, 4); else YALM_DECODE(64, 4);
 #undef YALM_DECODE
   int rc = launch_status();
-  if (rc != YALM_OK || n_splits == 1) return rc;   // one split writes the result itself
-  return yalm_attn_decode_combine_bf16(partial, out, lse, B, n_heads, head_dim, n_splits, 1, stream);
+  if (rc != YALM_OK || !merge) return rc;          // one split writes the result itself
+  return yalm_attn_decode_combine_bf16(partial, out, lse, B, n_heads, head_dim, n_splits, 1, sinks, stream);
 }

@@ -5,6 +5,7 @@
 #include <float.h>
 #include <mutex>
 #include "common.h"
+#include "sinks.h"
 #include "yalm_hip.h"
 
 int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out, float* lse,
@@ -14,7 +15,7 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
-                               int n_splits, int n_pages, hipStream_t stream);
+                               int n_splits, int n_pages, const SinkArgs& sinks, hipStream_t stream);
 
 namespace {
 constexpr int MAX_HD = 256;              // head sizes up to 256 (4 output elements per lane)
@@ -169,12 +170,17 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
   }
 }
 
-// BASE2: the maxima of the partial results are exponents of 2 (the matrix-core kernel's), else of e
+// BASE2: the maxima of the partial results are exponents of 2 (the matrix-core kernel's), else of e.
+// With sk.n_sinks > 0 the attention sinks that the query's window no longer covers count as further
+// splits of one key each (maximum = score, denominator 1, sum = value): their scores are worked out
+// here, with the keys turned, while the splits' loads are in flight; and a token at one of its
+// sequence's first positions stores its key and value as a sink (no query of the launch reads it: one
+// token a sequence, and the window, at least n_sinks wide, still covers it).
 template <typename T, bool BASE2 = false>
 __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(const float* __restrict__ partial,
                                                                              T* __restrict__ out,
                                                                              float* __restrict__ lse, int n_heads,
-                                                                             int hd, int n_splits) {
+                                                                             int hd, int n_splits, SinkArgs sk) {
   // One trip to memory: every wave asks for the maxima and denominators of all splits (lanes over
   // splits) and, before it waits for them, for the sums of its own first splits (waves share the
   // splits of the weighted sum and add their parts in a fixed order).
@@ -197,15 +203,49 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(co
   }
   const int s0 = min(lane, n_splits - 1);
   const float m0 = part[(size_t)s0 * stride + hd], l0 = part[(size_t)s0 * stride + hd + 1];
+  __shared__ float sink_score[YALM_MAX_SINKS];
+  int n_behind = 0;                               // sinks behind the window of this query
+  const T* sv = nullptr;
+  if (sk.n_sinks > 0) {                           // the same for the whole launch
+    const int slot = sk.seq_slot[b];
+    const int pos = sk.seq_len[b] - 1;
+    if (slot >= 0 && slot < sk.n_slots) {
+      const int kvh = h / (n_heads / sk.n_kv_heads);
+      if (sk.k_pages != nullptr && pos < sk.n_sinks && h < sk.n_kv_heads) {
+        const int page = sk.block_table[(size_t)slot * sk.table_stride];
+        if (page >= 0 && page < sk.n_pages)
+          copy_sink((const T*)sk.k_pages, (const T*)sk.v_pages, page, h, pos, slot, (T*)sk.sink_k, (T*)sk.sink_v,
+                    sk.n_kv_heads, hd, sk.n_sinks, (int)threadIdx.x, COMBINE_THREADS);
+      }
+      n_behind = max(0, min(sk.n_sinks, pos - sk.window + 1));
+      if (n_behind > 0) {
+        const int turn = max(0, pos - sk.window - sk.n_sinks + 1);
+        const int half_rot = sk.rotary_dim / 2;
+        const float2* cs = sk.cos_sin != nullptr && turn > 0 && turn < sk.n_positions
+                               ? sk.cos_sin + (size_t)turn * half_rot : nullptr;
+        const T* qr = (const T*)sk.q + ((size_t)b * n_heads + h) * hd;
+        const T* kbase = (const T*)sk.sink_k + ((size_t)slot * sk.n_kv_heads + kvh) * sk.n_sinks * hd;
+        sv = (const T*)sk.sink_v + ((size_t)slot * sk.n_kv_heads + kvh) * sk.n_sinks * hd;
+        const float to_exponent = (BASE2 ? 1.4426950408889634f : 1.0f) / sqrtf((float)hd);
+        for (int j = g; j < n_behind; j += NWV) {
+          const float d = sink_dot(qr, kbase + (size_t)j * hd, cs, hd, half_rot, lane);
+          if (lane == 0) sink_score[j] = d * to_exponent;
+        }
+      }
+    }
+    __syncthreads();
+  }
   float m = lane < n_splits ? m0 : -FLT_MAX;
   for (int sp = lane + WAVE; sp < n_splits; sp += WAVE) m = fmaxf(m, part[(size_t)sp * stride + hd]);
   m = wave_max(m);
+  for (int j = 0; j < n_behind; ++j) m = fmaxf(m, sink_score[j]);
   float l = lane < n_splits ? l0 * weight(m0 - m) : 0.f;
   for (int sp = lane + WAVE; sp < n_splits; sp += WAVE) {
     const float* ps = part + (size_t)sp * stride;
     l += ps[hd + 1] * weight(ps[hd] - m);
   }
   l = wave_sum(l);
+  for (int j = 0; j < n_behind; ++j) l += weight(sink_score[j] - m);
   const float inv_l = l > 0.f ? 1.0f / l : 0.f;
   if (lse != nullptr && threadIdx.x == 0)
     lse[(size_t)b * n_heads + h] = l > 0.f ? (BASE2 ? m * 0.6931471805599453f : m) + logf(l) : -FLT_MAX;
@@ -241,6 +281,7 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(co
       float t = accs[0][d];
 #pragma unroll
       for (int w = 1; w < NWV; ++w) t += accs[w][d];
+      for (int s = 0; s < n_behind; ++s) t = fmaf(weight(sink_score[s] - m), to_f32(sv[(size_t)s * hd + d]), t);
       out[((size_t)b * n_heads + h) * hd + d] = from_f32<T>(t * inv_l);
     }
   }
@@ -290,12 +331,14 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
 
 // merges the partial results of the splits (also used by the MFMA kernel)
 int yalm_attn_decode_combine_bf16(const float* partial, void* out, float* lse, int B, int n_heads, int head_dim,
-                                  int n_splits, int base2, hipStream_t stream) {
+                                  int n_splits, int base2, const SinkArgs& sinks, hipStream_t stream) {
   dim3 cgrid(B, n_heads);
   if (base2)
-    attn_decode_combine_kernel<bf16, true><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim, n_splits);
+    attn_decode_combine_kernel<bf16, true><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads,
+                                                                                  head_dim, n_splits, sinks);
   else
-    attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim, n_splits);
+    attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads,
+                                                                            head_dim, n_splits, sinks);
   return launch_status();
 }
 
@@ -303,11 +346,11 @@ extern "C" long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int
   return (long)B * n_heads * n_splits * (head_dim + 2) * (long)sizeof(float);
 }
 
-extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
-                                    int table_stride, int ring_pages, const int* seq_slot, const int* seq_len,
-                                    void* out, float* lse, float* partial, int B, int n_heads, int n_kv_heads,
-                                    int head_dim, int window, int n_splits, int n_pages, int dtype, int force_simple,
-                                    hipStream_t stream) {
+namespace {
+int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, const int* block_table, int table_stride,
+                    int ring_pages, const int* seq_slot, const int* seq_len, void* out, float* lse, float* partial,
+                    int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits, int n_pages,
+                    int dtype, int force_simple, const SinkArgs& sinks, hipStream_t stream) {
   if (B <= 0) return YALM_OK;
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0)
     return YALM_ERR_ARG;
@@ -316,21 +359,35 @@ extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const vo
     attn_decode_simple_kernel<float><<<grid, WAVE, 0, stream>>>(
         (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
         seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
-    attn_decode_combine_kernel<float><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (float*)out, lse, n_heads, head_dim, n_splits);
+    attn_decode_combine_kernel<float><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (float*)out, lse, n_heads,
+                                                                             head_dim, n_splits, sinks);
     return launch_status();
   }
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
   if (!force_simple) {
     int rc = yalm_attn_decode_bf16_mfma(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len,
                                         out, lse, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits,
-                                        n_pages, stream);
+                                        n_pages, sinks, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   attn_decode_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
       seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
-  attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim, n_splits);
+  attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim,
+                                                                          n_splits, sinks);
   return launch_status();
+}
+}  // namespace
+
+extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                                    int table_stride, int ring_pages, const int* seq_slot, const int* seq_len,
+                                    void* out, float* lse, float* partial, int B, int n_heads, int n_kv_heads,
+                                    int head_dim, int window, int n_splits, int n_pages, int dtype, int force_simple,
+                                    hipStream_t stream) {
+  SinkArgs none = {};
+  return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, lse,
+                         partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, dtype, force_simple,
+                         none, stream);
 }
 
 extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -340,6 +397,40 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
   return yalm_attn_decode_lse(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out,
                               nullptr, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, dtype,
                               force_simple, stream);
+}
+
+extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                                      int table_stride, int ring_pages, const int* seq_slot, const int* seq_len,
+                                      void* out, float* partial, void* sink_k, void* sink_v, int store,
+                                      const float* cos_sin, int n_positions, int n_slots, int rotary_dim, int n_sinks,
+                                      int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits,
+                                      int n_pages, int dtype, int force_simple, hipStream_t stream) {
+  if (n_sinks <= 0 || n_sinks > YALM_MAX_SINKS || window < n_sinks || n_slots <= 0 || sink_k == nullptr ||
+      sink_v == nullptr || rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2 || head_dim % 2)
+    return YALM_ERR_ARG;
+  SinkArgs sk = {};
+  sk.q = q;
+  sk.sink_k = sink_k;
+  sk.sink_v = sink_v;
+  if (store) {
+    sk.k_pages = k_pages;
+    sk.v_pages = v_pages;
+    sk.block_table = block_table;
+    sk.table_stride = table_stride;
+    sk.n_pages = n_pages;
+  }
+  sk.seq_slot = seq_slot;
+  sk.seq_len = seq_len;
+  sk.cos_sin = rotary_dim > 0 ? (const float2*)cos_sin : nullptr;
+  sk.n_positions = n_positions;
+  sk.n_slots = n_slots;
+  sk.n_kv_heads = n_kv_heads;
+  sk.rotary_dim = rotary_dim;
+  sk.window = window;
+  sk.n_sinks = n_sinks;
+  return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, nullptr,
+                         partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, dtype, force_simple, sk,
+                         stream);
 }
 
 // ---------------------------------------------------------------------------

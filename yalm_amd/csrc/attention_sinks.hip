@@ -1,40 +1,33 @@
-// Attention sinks beside a window: the first positions of a sequence stay visible after the
-// window has moved past them.  Their keys and values live in a small per-slot store of their own
-// (the ring of pages overwrites their places); a pass behind the attention kernel mixes them into
-// its result with the log-sum-exp that the attention kernel left.  Few keys (two in the reference,
-// src/model.h:12), so a wave per (token, head) in float32 arithmetic does for every storage type.
+// Attention sinks beside a window, for a step of whole prompts: the first positions of a sequence
+// stay visible after the window has moved past them.  Their keys and values live in a small
+// per-slot store of their own (the ring of pages overwrites their places); a pass behind the
+// attention kernel mixes them into its result with the log-sum-exp that the attention kernel left.
+// Few keys (two in the reference, src/model.h:12), so a wave per (token, head) in float32 arithmetic
+// does for every storage type.  (A decode step takes its sinks in where it merges the attention's
+// splits, attention_simple.hip.)
 #include <float.h>
 #include "common.h"
+#include "sinks.h"
 #include "yalm_hip.h"
 
 namespace {
 constexpr int MAX_HD = 256;
-constexpr int MAX_SINKS = 16;
+constexpr int MAX_SINKS = YALM_MAX_SINKS;
 
-// grid (sequence, kv head, sink); a wave copies one key row and one value column
+// a step of whole prompts; grid (sequence, kv head, sink); a wave copies one key row and one value column
 template <typename T>
-__global__ __launch_bounds__(WAVE) void sink_store_kernel(const T* __restrict__ k_src, const T* __restrict__ v_src,
-                                                          const int* __restrict__ page0, int page0_stride,
+__global__ __launch_bounds__(WAVE) void sink_store_kernel(const T* __restrict__ k_stage, const T* __restrict__ v_stage,
+                                                          const int* __restrict__ seq_tile0,
                                                           const int* __restrict__ seq_slot,
                                                           const int* __restrict__ seq_len, T* __restrict__ sink_k,
-                                                          T* __restrict__ sink_v, int decode, int n_src_pages,
-                                                          int n_slots, int n_kv_heads, int hd, int n_sinks) {
+                                                          T* __restrict__ sink_v, int n_tiles, int n_slots,
+                                                          int n_kv_heads, int hd, int n_sinks) {
   const int b = blockIdx.x, g = blockIdx.y, j = blockIdx.z;
   const int slot = seq_slot[b];
-  if (slot < 0 || slot >= n_slots) return;
-  const int L = seq_len[b];
-  const bool fresh = decode ? j == L - 1 : j < L;      // position j was written by this step
-  if (!fresh) return;
-  const int page = decode ? page0[(size_t)slot * page0_stride] : page0[b];
-  if (page < 0 || page >= n_src_pages) return;
-  const T* kr = k_src + (((size_t)page * n_kv_heads + g) * PAGE + j) * hd;       // [page][head][row][element]
-  const T* vc = v_src + ((size_t)page * n_kv_heads + g) * hd * PAGE + j;         // [page][head][element][row]
-  T* dk = sink_k + (((size_t)slot * n_kv_heads + g) * n_sinks + j) * hd;
-  T* dv = sink_v + (((size_t)slot * n_kv_heads + g) * n_sinks + j) * hd;
-  for (int i = threadIdx.x; i < hd; i += WAVE) {
-    dk[i] = kr[i];
-    dv[i] = vc[(size_t)i * PAGE];
-  }
+  if (slot < 0 || slot >= n_slots || j >= seq_len[b]) return;
+  const int tile = seq_tile0[b];
+  if (tile < 0 || tile >= n_tiles) return;
+  copy_sink(k_stage, v_stage, tile, g, j, slot, sink_k, sink_v, n_kv_heads, hd, n_sinks, (int)threadIdx.x, WAVE);
 }
 
 // grid (token, head); lanes over the head's elements, pairs (2p, 2p + 1) in one lane
@@ -68,19 +61,7 @@ __global__ __launch_bounds__(WAVE) void attn_sink_mix_kernel(const T* __restrict
   float top = seen;
   for (int j = 0; j < n_out; ++j) {
     const T* kr = sink_k + (((size_t)slot * n_kv_heads + g) * n_sinks + j) * hd;
-    float d = 0.f;
-    for (int p = lane; p < hd / 2; p += WAVE) {
-      float k0 = to_f32(kr[2 * p]), k1 = to_f32(kr[2 * p + 1]);
-      if (turn && p < half_rot) {
-        const float2 c = cos_sin[(size_t)shift * half_rot + p];
-        const float y0 = k0 * c.x - k1 * c.y, y1 = k0 * c.y + k1 * c.x;
-        k0 = y0;
-        k1 = y1;
-      }
-      d = fmaf(to_f32(qr[2 * p]), k0, d);
-      d = fmaf(to_f32(qr[2 * p + 1]), k1, d);
-    }
-    d = wave_sum(d) / inv;
+    const float d = sink_dot(qr, kr, turn ? cos_sin + (size_t)shift * half_rot : nullptr, hd, half_rot, lane) / inv;
     if (lane == 0) w[j] = d;
     top = fmaxf(top, d);
   }
@@ -101,23 +82,20 @@ bool bad_shape(int n_kv_heads, int hd, int n_sinks) {
 }
 }  // namespace
 
-extern "C" int yalm_sink_store(const void* k_src, const void* v_src, const int* page0, int page0_stride,
-                               const int* seq_slot, const int* seq_len, void* sink_k, void* sink_v, int decode, int B,
-                               int n_src_pages, int n_slots, int n_kv_heads, int head_dim, int n_sinks, int dtype,
-                               hipStream_t stream) {
+extern "C" int yalm_sink_store(const void* k_stage, const void* v_stage, const int* seq_tile0, const int* seq_slot,
+                               const int* seq_len, void* sink_k, void* sink_v, int B, int n_tiles, int n_slots,
+                               int n_kv_heads, int head_dim, int n_sinks, int dtype, hipStream_t stream) {
   if (B <= 0) return YALM_OK;
-  if (bad_shape(n_kv_heads, head_dim, n_sinks) || n_sinks > PAGE || n_src_pages <= 0 || n_slots <= 0 ||
-      (decode && page0_stride <= 0))
-    return YALM_ERR_ARG;
+  if (bad_shape(n_kv_heads, head_dim, n_sinks) || n_sinks > PAGE || n_tiles <= 0 || n_slots <= 0) return YALM_ERR_ARG;
   dim3 grid(B, n_kv_heads, n_sinks);
   if (dtype == YALM_F32)
-    sink_store_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)k_src, (const float*)v_src, page0, page0_stride,
-                                                        seq_slot, seq_len, (float*)sink_k, (float*)sink_v, decode,
-                                                        n_src_pages, n_slots, n_kv_heads, head_dim, n_sinks);
+    sink_store_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)k_stage, (const float*)v_stage, seq_tile0,
+                                                        seq_slot, seq_len, (float*)sink_k, (float*)sink_v, n_tiles,
+                                                        n_slots, n_kv_heads, head_dim, n_sinks);
   else if (dtype == YALM_BF16)
-    sink_store_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)k_src, (const bf16*)v_src, page0, page0_stride,
-                                                       seq_slot, seq_len, (bf16*)sink_k, (bf16*)sink_v, decode,
-                                                       n_src_pages, n_slots, n_kv_heads, head_dim, n_sinks);
+    sink_store_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)k_stage, (const bf16*)v_stage, seq_tile0,
+                                                       seq_slot, seq_len, (bf16*)sink_k, (bf16*)sink_v, n_tiles,
+                                                       n_slots, n_kv_heads, head_dim, n_sinks);
   else
     return YALM_ERR_DTYPE;
   return launch_status();
@@ -128,7 +106,7 @@ extern "C" int yalm_attn_sink_mix(const void* q, void* out, const float* lse, co
                                   int n_positions, int T, int n_slots, int n_heads, int n_kv_heads, int head_dim,
                                   int rotary_dim, int window, int n_sinks, int dtype, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
-  if (bad_shape(n_kv_heads, head_dim, n_sinks) || n_heads <= 0 || n_heads % n_kv_heads || window <= 0 ||
+  if (bad_shape(n_kv_heads, head_dim, n_sinks) || n_heads <= 0 || n_heads % n_kv_heads || window < n_sinks ||
       n_slots <= 0 || rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2)
     return YALM_ERR_ARG;
   dim3 grid(T, n_heads);

@@ -152,21 +152,31 @@ int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages
 // turns the stored sink keys one position further every step; here they are kept as they were
 // written and turned by the whole distance when they are read, which rounds once instead of once a step.
 //
-// yalm_sink_store copies the keys and values of positions < n_sinks that this step wrote into
-//   sink_k, sink_v [slots, n_kv_heads, n_sinks, hd].  A sequence's new positions are [0, seq_len[b]) with
-//   decode == 0 and seq_len[b] - 1 with decode != 0; the page that holds positions 0..63 is
-//   page0[b] (decode == 0: the staging area's tile) or page0[seq_slot[b] * page0_stride] (the block table).
-// yalm_attn_sink_mix adds the sinks that the window no longer covers to a finished attention result:
+// The store: sink_k, sink_v [slots, n_kv_heads, n_sinks, hd].  1 <= n_sinks <= 16, window >= n_sinks.
+// A step of whole prompts:
+//   yalm_sink_store copies the keys and values of positions < min(n_sinks, seq_len[b]) from the staging
+//   area (tile seq_tile0[b]) into the store of seq_slot[b].
+//   yalm_attn_sink_mix adds the sinks that the window no longer covers to a finished attention result:
 //   for token t at position p the sinks j < min(n_sinks, p - window + 1), keys turned by
 //   max(0, p - window - n_sinks + 1) positions with cos_sin (null or rotary_dim 0: not turned);
 //   out[t, h] = (e^lse out + sum_j e^s_j v_j) / (e^lse + sum_j e^s_j), s_j = q . k_j / sqrt(hd).
-int yalm_sink_store(const void* k_src, const void* v_src, const int* page0, int page0_stride, const int* seq_slot,
-                    const int* seq_len, void* sink_k, void* sink_v, int decode, int B, int n_src_pages, int n_slots,
-                    int n_kv_heads, int head_dim, int n_sinks, int dtype, hipStream_t stream);
+// A decode step: yalm_attn_decode_sinks is yalm_attn_decode whose merge of the splits takes those sinks in
+//   as further splits of one key each (no rounding in between, no launch more; the merge runs with one
+//   split too); with store != 0 a token at a position < n_sinks first stores its own key and value from its
+//   page.
+int yalm_sink_store(const void* k_stage, const void* v_stage, const int* seq_tile0, const int* seq_slot,
+                    const int* seq_len, void* sink_k, void* sink_v, int B, int n_tiles, int n_slots, int n_kv_heads,
+                    int head_dim, int n_sinks, int dtype, hipStream_t stream);
 int yalm_attn_sink_mix(const void* q, void* out, const float* lse, const void* sink_k, const void* sink_v,
                        const int* tok_seq, const int* tok_pos, const int* seq_slot, const float* cos_sin,
                        int n_positions, int T, int n_slots, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
                        int window, int n_sinks, int dtype, hipStream_t stream);
+int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
+                           int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
+                           float* partial, void* sink_k, void* sink_v, int store, const float* cos_sin,
+                           int n_positions, int n_slots, int rotary_dim, int n_sinks, int B, int n_heads,
+                           int n_kv_heads, int head_dim, int window, int n_splits, int n_pages, int dtype,
+                           int force_simple, hipStream_t stream);
 
 // yalm_attn_decode without a workspace argument, for callers that cannot allocate device memory
 // (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no

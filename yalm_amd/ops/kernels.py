@@ -492,8 +492,12 @@ def attn_decode_workspace_floats(B, n_heads, head_dim, n_splits):
 
 
 def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len, out, partial, n_heads, n_kv_heads,
-                head_dim, window, n_splits, lse=None):
-    """One query per sequence over the cache pages; seq_len counts the new key.  lse as in attn_prefill."""
+                head_dim, window, n_splits, lse=None, sinks=None):
+    """One query per sequence over the cache pages; seq_len counts the new key.  lse as in attn_prefill.
+    sinks = (sink_k, sink_v [slots, n_kv_heads, n_sinks, head_dim], cos_sin or None, rotary_dim, store):
+    the attention sinks that a query's window no longer covers are taken in where the splits are merged
+    (their keys turned by max(0, position - window - n_sinks + 1) positions with the table cos_sin); with
+    `store` a token at one of its sequence's first n_sinks positions stores its key and value there."""
     _check_heads(n_heads, n_kv_heads, head_dim)
     B = q.shape[0]
     dt = q.dtype
@@ -512,53 +516,66 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
     p_w = _need(partial, "partial", torch.float32)
     if partial.numel() < need:
         raise ValueError("attn_decode workspace too small: %d floats, %d needed" % (partial.numel(), need))
-    p_lse = None if lse is None else _need(lse, "lse", torch.float32, (B, n_heads))
-    library.check(library.lib().yalm_attn_decode_lse(
-        p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_lse, p_w, B, n_heads, n_kv_heads, head_dim,
-        int(window), int(n_splits), n_pages, dtype_code(dt), 1 if FORCE_SIMPLE else 0, _stream()), "attn_decode")
+    force = 1 if FORCE_SIMPLE else 0
+    if sinks is None:
+        p_lse = None if lse is None else _need(lse, "lse", torch.float32, (B, n_heads))
+        library.check(library.lib().yalm_attn_decode_lse(
+            p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_lse, p_w, B, n_heads, n_kv_heads, head_dim,
+            int(window), int(n_splits), n_pages, dtype_code(dt), force, _stream()), "attn_decode")
+        return out
+    if lse is not None:
+        raise ValueError("attn_decode leaves no lse when it takes the sinks in itself")
+    sink_k, sink_v, cos_sin, rotary_dim, store = sinks
+    n_slots, _, n_sinks, _ = sink_k.shape
+    if window < n_sinks:
+        raise ValueError("a window of %d is narrower than the %d sinks beside it" % (window, n_sinks))
+    if block_table.shape[0] < n_slots:
+        raise ValueError("the block table has %d rows for %d slots" % (block_table.shape[0], n_slots))
+    n_pos, p_cs = 0, None
+    if cos_sin is not None and rotary_dim > 0:
+        n_pos = cos_sin.shape[0]
+        p_cs = _need(cos_sin, "cos_sin", torch.float32, (n_pos, rotary_dim // 2, 2))
+    library.check(library.lib().yalm_attn_decode_sinks(
+        p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_w,
+        _need(sink_k, "sink_k", dt, (n_slots, n_kv_heads, n_sinks, head_dim)),
+        _need(sink_v, "sink_v", dt, (n_slots, n_kv_heads, n_sinks, head_dim)), 1 if store else 0, p_cs, n_pos, n_slots,
+        int(rotary_dim) if p_cs is not None else 0, n_sinks, B, n_heads, n_kv_heads, head_dim, int(window),
+        int(n_splits), n_pages, dtype_code(dt), force, _stream()), "attn_decode with sinks")
     return out
 
 
 MAX_SINKS = 16
 
 
-def sink_store(k_src, v_src, page0, seq_slot, seq_len, sink_k, sink_v, decode):
-    """Copies the keys and values of positions < n_sinks that this step wrote from their page into the
-    per-slot store sink_k, sink_v [slots, n_kv_heads, n_sinks, head_dim].  k_src, v_src: pages in the
-    cache's format.  decode: page0 is the block table (the page of positions 0..63 of slot s is
-    page0[s, 0]) and the step wrote position seq_len - 1; else page0[b] is sequence b's first tile of
-    the staging area and the step wrote positions 0 .. seq_len - 1."""
+def sink_store(k_stage, v_stage, seq_tile0, seq_slot, seq_len, sink_k, sink_v):
+    """A step of whole prompts: copies the keys and values of positions < min(n_sinks, seq_len) from the
+    staging area (sequence b's first tile is seq_tile0[b]) into the per-slot store sink_k, sink_v
+    [slots, n_kv_heads, n_sinks, head_dim]."""
     n_slots, n_kv_heads, n_sinks, head_dim = sink_k.shape
     dt = sink_k.dtype
-    n_src = k_src.shape[0]
+    n_tiles = k_stage.shape[0]
     B = seq_slot.shape[0]
-    p_k = _need(k_src, "k_src", dt, (n_src, n_kv_heads, PAGE, head_dim))
-    p_v = _need(v_src, "v_src", dt, (n_src, n_kv_heads, head_dim, PAGE))
-    if decode:
-        p_p0 = _need(page0, "page0", torch.int32, (None, None))
-        if page0.shape[0] < n_slots:
-            raise ValueError("the block table has %d rows for %d slots" % (page0.shape[0], n_slots))
-        stride = page0.shape[1]
-    else:
-        p_p0 = _need(page0, "page0", torch.int32, (B + 1,))
-        stride = 0
     library.check(library.lib().yalm_sink_store(
-        p_k, p_v, p_p0, stride, _need(seq_slot, "seq_slot", torch.int32, (B,)),
+        _need(k_stage, "k_stage", dt, (n_tiles, n_kv_heads, PAGE, head_dim)),
+        _need(v_stage, "v_stage", dt, (n_tiles, n_kv_heads, head_dim, PAGE)),
+        _need(seq_tile0, "seq_tile0", torch.int32, (B + 1,)), _need(seq_slot, "seq_slot", torch.int32, (B,)),
         _need(seq_len, "seq_len", torch.int32, (B,)), _need(sink_k, "sink_k", dt),
-        _need(sink_v, "sink_v", dt, (n_slots, n_kv_heads, n_sinks, head_dim)), 1 if decode else 0, B, n_src, n_slots,
-        n_kv_heads, head_dim, n_sinks, dtype_code(dt), _stream()), "sink_store")
+        _need(sink_v, "sink_v", dt, (n_slots, n_kv_heads, n_sinks, head_dim)), B, n_tiles, n_slots, n_kv_heads,
+        head_dim, n_sinks, dtype_code(dt), _stream()), "sink_store")
 
 
 def attn_sink_mix(q, out, lse, sink_k, sink_v, tok_seq, tok_pos, seq_slot, cos_sin, n_heads, rotary_dim, window):
-    """Adds the attention sinks that the window no longer covers to the attention result `out`
-    (in place): for the token at position p the sinks j < min(n_sinks, p - window + 1), their keys
-    turned by max(0, p - window - n_sinks + 1) positions with the table cos_sin (None: not turned).
-    lse is what attn_prefill / attn_decode left for these queries."""
+    """A step of whole prompts: adds the attention sinks that the window no longer covers to the attention
+    result `out` (in place): for the token at position p the sinks j < min(n_sinks, p - window + 1), their
+    keys turned by max(0, p - window - n_sinks + 1) positions with the table cos_sin (None: not turned).
+    lse is what attn_prefill left for these queries."""
     n_slots, n_kv_heads, n_sinks, head_dim = sink_k.shape
     _check_heads(n_heads, n_kv_heads, head_dim)
     T = q.shape[0]
     dt = q.dtype
     B = seq_slot.shape[0]
+    if window < n_sinks:
+        raise ValueError("a window of %d is narrower than the %d sinks beside it" % (window, n_sinks))
     n_pos, p_cs = 0, None
     if cos_sin is not None and rotary_dim > 0:
         n_pos = cos_sin.shape[0]

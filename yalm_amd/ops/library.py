@@ -40,15 +40,17 @@ _SIGNATURES = {
     "yalm_attn_prefill_lse": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I,
                                    _P]),
     "yalm_attn_decode_lse": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
-    "yalm_sink_store": (_I, [_P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_sink_store": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_sink_mix": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_attn_decode_sinks": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I,
+                                    _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_static": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_argmax": (_I, [_P, _P, _I, _I, _P]),
     "yalm_sample": (_I, [_P, _P, _F, _P, _I, _I, _P]),
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
 }
 
-ABI_VERSION = 14
+ABI_VERSION = 16
 
 
 class KernelError(RuntimeError):

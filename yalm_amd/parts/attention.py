@@ -40,8 +40,8 @@ class GQAttention(Part):
         self.head_dim = int(p["head_dim"])
         self.window = int(p.get("window", 0) or 0)
         self.sinks = int(p.get("sinks", 0) or 0)
-        if self.sinks and not self.window:
-            raise ValueError("attention sinks (%d) need a window" % self.sinks)
+        if self.sinks and self.window < self.sinks:
+            raise ValueError("%d attention sinks need a window at least as wide (window %d)" % (self.sinks, self.window))
         if not 0 <= self.sinks <= kernels.MAX_SINKS:
             raise ValueError("%d attention sinks asked for, at most %d are supported" % (self.sinks, kernels.MAX_SINKS))
         if self.n_heads % self.n_kv_heads:
@@ -172,19 +172,12 @@ class GQAttention(Part):
         partial = ctx.ws.get("attn.partial",
                              (kernels.attn_decode_workspace_floats(T, self.n_heads, self.head_dim, n_splits),),
                              torch.float32)
-        lse = ctx.ws.get("attn.lse", (T, self.n_heads), torch.float32) if self.sinks else None
-        if self.sinks and writes_cache:      # a sequence still at its first positions has just written a sink
-            sink_k, sink_v = group.line_sinks(line)
-            kernels.sink_store(k_pages, v_pages, group.table, ctx.seq_slot, ctx.seq_len, sink_k, sink_v, True)
+        sinks = None
+        if self.sinks:       # taken in where the splits are merged; a sequence still at its first positions
+            sink_k, sink_v = group.line_sinks(line)        # has just written a sink, which is stored on the way
+            sinks = (sink_k, sink_v, self.position.table, self.position.rotary_dim, writes_cache)
         kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o, partial,
-                            self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits, lse=lse)
-        if self.sinks:
-            self._mix_sinks(q, o, lse, ctx, group, line)
-
-    def _mix_sinks(self, q, o, lse, ctx, group, line):
-        sink_k, sink_v = group.line_sinks(line)
-        kernels.attn_sink_mix(q, o, lse, sink_k, sink_v, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, self.position.table,
-                              self.n_heads, self.position.rotary_dim, self.window)
+                            self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits, sinks=sinks)
 
     def forward(self, h, x, ctx, line, writes_cache=True):
         T = h.shape[0]
@@ -225,11 +218,13 @@ class GQAttention(Part):
             lse = ws.get("attn.lse", (T, self.n_heads), torch.float32) if self.sinks else None
             if self.sinks and writes_cache:
                 sink_k, sink_v = group.line_sinks(line)
-                kernels.sink_store(kst, vst, ctx.seq_tile0, ctx.seq_slot, ctx.seq_len, sink_k, sink_v, False)
+                kernels.sink_store(kst, vst, ctx.seq_tile0, ctx.seq_slot, ctx.seq_len, sink_k, sink_v)
             kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, ctx.seq_tile0, ctx.tok_seq, ctx.tok_pos,
                                  self.n_heads, self.n_kv_heads, self.head_dim, self.window, ctx.tile_order, lse=lse)
             if self.sinks:
-                self._mix_sinks(q, o, lse, ctx, group, line)
+                sink_k, sink_v = group.line_sinks(line)
+                kernels.attn_sink_mix(q, o, lse, sink_k, sink_v, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, pos.table,
+                                      self.n_heads, pos.rotary_dim, self.window)
         else:
             self._decode_attention(q, o, ctx, group, line, k_pages, v_pages, writes_cache)
         self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)
