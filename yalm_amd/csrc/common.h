@@ -18,6 +18,14 @@
 
 typedef __bf16 bf16;
 
+// Cache policy bits of a global load (the `aux` operand of the load-to-LDS builtin).  READ_ONCE marks data
+// that a launch reads once and nobody reads again soon (a decode step's weights): non-temporal, so that it
+// does not push out of the second-level cache what is read again (the activations).  Measured on the decode
+// GEMMs: gate/up at 8 rows 41.1 -> 37.0 us (5.7 -> 6.4 TB/s), at 64 rows 53.7 -> 49.7.
+#ifndef YALM_READ_ONCE
+#define YALM_READ_ONCE 2
+#endif
+
 __device__ __forceinline__ float to_f32(float v) { return v; }
 __device__ __forceinline__ float to_f32(bf16 v) { return static_cast<float>(v); }
 template <typename T> __device__ __forceinline__ T from_f32(float v);

@@ -220,7 +220,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_batch_dma_kernel(const bf16* _
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass drops a template that names this builtin, and its launch stub with it
 #pragma unroll
     for (int u = 0; u < 2 * NTW; ++u)
-      __builtin_amdgcn_global_load_lds(gw[u] + (size_t)i * KD, wring + buf * WSTAGE + u * 1024, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(gw[u] + (size_t)i * KD, wring + buf * WSTAGE + u * 1024, 16, 0, YALM_READ_ONCE);
 #pragma unroll
     for (int u = 0; u < XI; ++u)
       __builtin_amdgcn_global_load_lds(gx[u] + (size_t)i * KD, xring + buf * XSTAGE + (wave * XI + u) * 1024, 16, 0, 0);

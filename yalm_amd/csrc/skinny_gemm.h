@@ -195,7 +195,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass drops a template that names this builtin, and its launch stub with it
 #pragma unroll
       for (int u = 0; u < 2 * TW; ++u)
-        __builtin_amdgcn_global_load_lds(gw[u] + (size_t)c * KD, dst + u * 1024, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(gw[u] + (size_t)c * KD, dst + u * 1024, 16, 0, YALM_READ_ONCE);
 #pragma unroll
       for (int u = 0; u < XI; ++u)
         __builtin_amdgcn_global_load_lds(gx[u] + (size_t)c * KD, dst + (2 * TW + u) * 1024, 16, 0, 0);
