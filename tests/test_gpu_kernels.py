@@ -43,6 +43,53 @@ def i32(x):
     return torch.tensor(x, dtype=torch.int32, device=DEV)
 
 
+# The cache's pages as the kernels store them.  Head sizes that are multiples of 32 are kept in blocks:
+# keys [element // 32][place(row)][element % 32], values [row // 32][element][row % 32], where place(row) is
+# the row's place in the order in which the matrix-core decode attention takes the rows of a page
+# (16 rows an instruction: rows 8 a + b (+ 4) (+ 32) for a, b < 4).  Other head sizes: keys [row][element],
+# values [element][row], which is also how the tests fill and read pages.
+def row_place(r):
+    return 16 * (2 * (r >> 5) + ((r >> 2) & 1)) + 4 * ((r >> 3) & 3) + (r & 3)
+
+
+def pages_as_stored(kp, vp):
+    """[pages, heads, 64, hd] keys and [pages, heads, hd, 64] values in rows -> the same shapes in storage order."""
+    P, H, R, hd = kp.shape
+    if hd % 32:
+        return kp, vp
+    place = torch.tensor([row_place(r) for r in range(R)], device=kp.device)
+    ks = torch.empty_like(kp).view(P, H, hd // 32, R, 32)
+    ks[:, :, :, place, :] = kp.view(P, H, R, hd // 32, 32).permute(0, 1, 3, 2, 4)
+    vs = vp.view(P, H, hd, R // 32, 32).permute(0, 1, 3, 2, 4).contiguous()
+    return ks.view(P, H, R, hd), vs.view(P, H, hd, R)
+
+
+def pages_as_rows(kp, vp):
+    """The inverse of pages_as_stored."""
+    P, H, R, hd = kp.shape
+    if hd % 32:
+        return kp, vp
+    place = torch.tensor([row_place(r) for r in range(R)], device=kp.device)
+    kr = kp.view(P, H, hd // 32, R, 32)[:, :, :, place, :].permute(0, 1, 3, 2, 4).contiguous().view(P, H, R, hd)
+    vr = vp.view(P, H, R // 32, hd, 32).permute(0, 1, 3, 2, 4).contiguous().view(P, H, hd, R)
+    return kr, vr
+
+
+def test_page_layout_helpers_invert_each_other():
+    assert sorted(row_place(r) for r in range(64)) == list(range(64))
+    assert [row_place(r) for r in (0, 1, 4, 8, 32, 63)] == [0, 1, 16, 4, 32, 63]
+    for hd in (16, 64, 128):
+        kp, vp = rnd((3, 2, 64, hd), 1), rnd((3, 2, hd, 64), 2)
+        ks, vs = pages_as_stored(kp, vp)
+        assert (hd % 32 != 0) == torch.equal(ks, kp)
+        a, b = pages_as_rows(ks, vs)
+        assert torch.equal(a, kp) and torch.equal(b, vp)
+        if hd % 32 == 0:        # the formula of the layout, element by element
+            for (r, e) in ((0, 0), (5, 33), (63, hd - 1), (36, 31)):
+                assert ks[1, 1].reshape(-1)[((e // 32) * 64 + row_place(r)) * 32 + e % 32] == kp[1, 1, r, e]
+                assert vs[1, 1].reshape(-1)[((r // 32) * hd + e) * 32 + r % 32] == vp[1, 1, e, r]
+
+
 # ------------------------------------------------------------------ embedding, norm
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -308,6 +355,7 @@ def test_rope_kv_write(n_heads, n_kv, hd, rd, dtype):
     v_want = qkv[:, Q + KV:].double().reshape(T, n_kv, hd)
     close(q_out, q_want, dtype, "q")
     kp, vp, ks, vs = kp.cpu(), vp.cpu(), ks.cpu(), vs.cpu()
+    kp, vp = pages_as_rows(kp, vp)
     for t in range(T):
         page, tile, r = page_of[seq[t]][pos[t] // PAGE], tile_of[seq[t]][pos[t] // PAGE], pos[t] % PAGE
         close(ks[tile, :, r, :], k_want[t], dtype, "staged k")
@@ -418,7 +466,7 @@ def test_rope_kv_write_ring_keeps_the_last_pages_only():
     q_out = torch.empty((L, hd), device=DEV)
     k.rope_kv_write(qkv.to(DEV), q_out, None, None, None, kp, vp, bt.to(DEV), ring, i32([0] * L),
                     i32(list(range(L))), i32([0]), i32([L]), None, 1, n_kv, hd, 0)
-    kp = kp.cpu()
+    kp = pages_as_rows(kp.cpu(), vp.cpu())[0]
     # absolute page 2 -> column 0 (page 4), page 3 -> column 1 (page 6)
     assert torch.equal(kp[4, 0], qkv[2 * PAGE:3 * PAGE, hd:2 * hd])
     assert torch.equal(kp[6, 0, :5], qkv[3 * PAGE:, hd:2 * hd])
@@ -552,9 +600,10 @@ def test_attn_prefill_in_a_given_tile_order(n_heads, n_kv, hd, window, lens):
     assert torch.equal(outs[0], outs[1])
 
 
-def paged_case(lens, n_kv, hd, window, dtype, seed, poison=True):
+def paged_case(lens, n_kv, hd, window, dtype, seed, poison=True, stored=True):
     """Random keys/values of sequences of the given lengths laid out in pages the way
-    the cache does (ring for a window), the rest of the pool poisoned with NaN."""
+    the cache does (ring for a window), the rest of the pool poisoned with NaN.  stored=False: the pages in
+    rows, for a caller that changes them before pages_as_stored."""
     k = K()
     PAGE = k.PAGE
     B = len(lens)
@@ -582,6 +631,8 @@ def paged_case(lens, n_kv, hd, window, dtype, seed, poison=True):
             for p in rows:
                 kp[page, :, p % PAGE, :] = kb[p]
                 vp[page, :, :, p % PAGE] = vb[p]
+    if stored:
+        kp, vp = pages_as_stored(kp, vp)
     return kp, vp, bt, [int(s) for s in slots], ring, keys, vals
 
 
@@ -654,7 +705,7 @@ def test_attn_window_edge_decides(hd, window, n, dtype, simple):
     k.FORCE_SIMPLE = simple
     try:
         # decode: the query at position n - 1 sees positions n - window ... n - 1
-        kp, vp, bt, slots, ring, keys, vals = paged_case([n], n_kv, hd, window, dtype, 40)
+        kp, vp, bt, slots, ring, keys, vals = paged_case([n], n_kv, hd, window, dtype, 40, stored=False)
         inside, outside = n - window, n - window - 1
         PAGE = k.PAGE
         for pos, strength, value in ((inside, 30.0, 7.0), (outside, 60.0, 1000.0)):
@@ -662,6 +713,7 @@ def test_attn_window_edge_decides(hd, window, n, dtype, simple):
             if pos // PAGE > (n - 1) // PAGE - ring:          # the ring still holds this position's page
                 kp[page, :, pos % PAGE, :] = (unit * strength).to(dtype)
                 vp[page, :, :, pos % PAGE] = value
+        kp, vp = pages_as_stored(kp, vp)
         q = (unit * 8.0).to(dtype).repeat(n_heads)[None]
         out = torch.empty((1, n_heads * hd), dtype=dtype, device=DEV)
         partial = torch.empty(k.attn_decode_workspace_floats(1, n_heads, hd, 3), device=DEV)
@@ -1024,7 +1076,7 @@ def test_gemm_norm_qkv_rope(n_heads, n_kv, hd, rd, D):
     k_want = R.rope_interleaved(qkv[:, Q:Q + KV].reshape(M, n_kv, hd), p, f)
     v_want = qkv[:, Q + KV:].reshape(M, n_kv, hd)
     close(q_out, q_want, torch.bfloat16, "q", factor=1.5)
-    kp, vp = kp.cpu(), vp.cpu()
+    kp, vp = pages_as_rows(kp.cpu(), vp.cpu())
     touched = torch.zeros((n_pages, PAGE), dtype=torch.bool)
     for m in range(M):
         if slots[m] < 0:
@@ -1076,7 +1128,7 @@ def test_gemm_chain_qkv_rope(n_heads, n_kv, hd, rd, D, M):
     k_want = R.rope_interleaved(qkv[:, Q:Q + KV].reshape(M, n_kv, hd), p, f)
     v_want = qkv[:, Q + KV:].reshape(M, n_kv, hd)
     close(q_out, q_want, torch.bfloat16, "q", factor=1.5)
-    kp, vp = kp.cpu(), vp.cpu()
+    kp, vp = pages_as_rows(kp.cpu(), vp.cpu())
     touched = torch.zeros((n_pages, PAGE), dtype=torch.bool)
     for m in range(M):
         if slots[m] < 0:

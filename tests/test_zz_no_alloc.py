@@ -50,7 +50,7 @@ def test_static_scratch_decode_attention_twice(dtype, simple):
     n_heads, n_kv, hd = 8, 2, 128
     # first call: four sequences (one row of padding), seven splits
     lens = [1000, 3, 517, 64]
-    kp, vp, bt, slots, ring, _, _ = paged_case(lens, n_kv, hd, 0, dtype, 41)
+    kp, vp, bt, slots, ring, _, _ = paged_case(lens, n_kv, hd, 0, dtype, 41, stored=False)
     q = rnd((len(lens) + 1, n_heads * hd), 42, dtype).to(DEV)
     want, got = _both(lib, q, kp.to(DEV), vp.to(DEV), bt.to(DEV), ring, slots + [-1], lens + [0], n_heads, n_kv, hd, 0,
                       7, dtype, simple)
@@ -58,7 +58,7 @@ def test_static_scratch_decode_attention_twice(dtype, simple):
     assert (got[-1] == 0).all()
     # second call, smaller in every size: the array still holds the first call's partial results
     lens2 = [130, 70]
-    kp2, vp2, bt2, slots2, ring2, _, _ = paged_case(lens2, n_kv, hd, 100, dtype, 43)
+    kp2, vp2, bt2, slots2, ring2, _, _ = paged_case(lens2, n_kv, hd, 100, dtype, 43, stored=False)
     q2 = rnd((2, n_heads * hd), 44, dtype).to(DEV)
     want2, got2 = _both(lib, q2, kp2.to(DEV), vp2.to(DEV), bt2.to(DEV), ring2, slots2, lens2, n_heads, n_kv, hd, 100,
                         2, dtype, simple)

@@ -31,6 +31,10 @@ constexpr float LN2 = 0.6931471805599453f;      // the kernels' maxima are expon
 
 __device__ __forceinline__ bf16x8 ld8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x8 zero8() { return (bf16x8){0, 0, 0, 0, 0, 0, 0, 0}; }
+// a load of data that the launch reads once: non-temporal
+__device__ __forceinline__ bf16x8 ld8_once(const bf16* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p));
+}
 
 // page row that MFMA row i (0..15) of key tile t (0..3) reads
 __device__ __forceinline__ int key_row(int t, int i) { return 32 * (t >> 1) + 8 * (i >> 2) + 4 * (t & 1) + (i & 3); }
@@ -41,7 +45,10 @@ __device__ __forceinline__ int key_row(int t, int i) { return 32 * (t >> 1) + 8 
 // under no branch (the last page is done by a copy of the body without them), else the compiler
 // waits for every load in flight at each use.
 // ---------------------------------------------------------------------------
-template <int HD, int NW>
+// BLOCKS: the pages are laid out in blocks (YALM_PAGE_BLOCKS): every load instruction reads 1 KB of consecutive
+// bytes, and asks for them non-temporally (a step reads a page once; with pieces of lines the hint costs more
+// than it gains: the other half of a line would be fetched again).
+template <int HD, int NW, bool BLOCKS>
 __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_kernel(   // 2 waves a SIMD: head size 128 needs their registers
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
@@ -90,7 +97,9 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 #pragma unroll
       for (int t = 0; t < 4; ++t)
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) kreg[t][ks] = ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
+        for (int ks = 0; ks < KS; ++ks)
+          kreg[t][ks] = BLOCKS ? ld8_once(kp + ((ks * PAGE + t * 16 + j) * 32 + qd * 8))
+                               : ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
     };
     int ap = p_begin + wave;
     int phys = ap < p_end ? page_of(ap) : 0;
@@ -103,7 +112,9 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int s = 0; s < 2; ++s) vreg[dt][s] = ld8(vp + (dt * 16 + j) * PAGE + s * 32 + qd * 8);
+        for (int s = 0; s < 2; ++s)
+          vreg[dt][s] = BLOCKS ? ld8_once(vp + ((s * HD + dt * 16 + j) * 32 + qd * 8))
+                               : ld8(vp + (dt * 16 + j) * PAGE + s * 32 + qd * 8);
       int physn = 0;
       if constexpr (decltype(has_next)::value) physn = page_of(ap + NW);
       __builtin_amdgcn_sched_barrier(0);         // the values are asked for before the keys are waited for
@@ -559,18 +570,23 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
-                               int n_splits, int n_pages, const SinkArgs& sinks, hipStream_t stream) {
+                               int n_splits, int n_pages, int page_layout, const SinkArgs& sinks,
+                               hipStream_t stream) {
   // with sinks the merge kernel always runs: it takes them in, also where there is one split
   const bool merge = n_splits > 1 || sinks.n_sinks > 0;
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_heads / n_kv_heads > 16) return YALM_ERR_ARG;
   dim3 grid(n_splits, n_kv_heads, B);
-#define YALM_DECODE(HD_, NW_)                                                                                       \
-  attn_decode_mfma_kernel<HD_, NW_><<<grid, NW_ * WAVE, 0, stream>>>(                                               \
+#define YALM_DECODE(HD_, NW_, BLOCKS_)                                                                              \
+  attn_decode_mfma_kernel<HD_, NW_, BLOCKS_><<<grid, NW_ * WAVE, 0, stream>>>(                                      \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot, \
       seq_len, partial, merge ? nullptr : (bf16*)out, lse, n_heads, n_kv_heads, window, n_splits, n_pages)
   // 4 waves a workgroup: 8 measured no faster with one split and slower with more (a CU draws about
   // 33 GB/s whatever its number of waves, so a small batch needs its workgroups spread over all CUs)
-  if (head_dim == 128) YALM_DECODE(128, 4); else YALM_DECODE(64, 4);
+  if (page_layout == YALM_PAGE_BLOCKS) {
+    if (head_dim == 128) YALM_DECODE(128, 4, true); else YALM_DECODE(64, 4, true);
+  } else {
+    if (head_dim == 128) YALM_DECODE(128, 4, false); else YALM_DECODE(64, 4, false);
+  }
 #undef YALM_DECODE
   int rc = launch_status();
   if (rc != YALM_OK || !merge) return rc;          // one split writes the result itself

@@ -15,7 +15,7 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
-                               int n_splits, int n_pages, const SinkArgs& sinks, hipStream_t stream);
+                               int n_splits, int n_pages, int page_layout, const SinkArgs& sinks, hipStream_t stream);
 
 namespace {
 constexpr int MAX_HD = 256;              // head sizes up to 256 (4 output elements per lane)
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_len, float* __restrict__ partial, int n_heads, int n_kv_heads, int hd, int window,
-    int n_splits, int n_pages) {
+    int n_splits, int n_pages, int page_layout) {
   __shared__ float qs[MAX_HD];
   __shared__ float ps[WAVE];
   const int b = blockIdx.x, h = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
@@ -131,9 +131,8 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
       bool valid = pos >= lo && pos < L;
       float s = -FLT_MAX;
       if (valid) {
-        const T* kr = kp + (size_t)lane * hd;
         float d = 0.f;
-        for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kr[i]), d);
+        for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kp[page_k_offset(page_layout, lane, i, hd)]), d);
         s = d / inv;
       }
       float m_new = fmaxf(m, wave_max(s));
@@ -148,11 +147,10 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
       for (int a = 0; a < ACC; ++a) {
         int d = lane + a * WAVE;
         if (d < hd) {
-          const T* vr = vp + (size_t)d * PAGE;
           float s2 = 0.f;
           for (int jj = 0; jj < PAGE; ++jj) {
-            float pj = ps[jj];
-            if (pj != 0.f) s2 = fmaf(pj, to_f32(vr[jj]), s2);   // rows outside the mask may hold anything
+            float pj = ps[jj];                                   // rows outside the mask may hold anything
+            if (pj != 0.f) s2 = fmaf(pj, to_f32(vp[page_v_offset(page_layout, jj, d, hd)]), s2);
           }
           acc[a] = acc[a] * corr + s2;
         }
@@ -214,8 +212,8 @@ __global__ __launch_bounds__(COMBINE_THREADS) void attn_decode_combine_kernel(co
       if (sk.k_pages != nullptr && pos < sk.n_sinks && h < sk.n_kv_heads) {
         const int page = sk.block_table[(size_t)slot * sk.table_stride];
         if (page >= 0 && page < sk.n_pages)
-          copy_sink((const T*)sk.k_pages, (const T*)sk.v_pages, page, h, pos, slot, (T*)sk.sink_k, (T*)sk.sink_v,
-                    sk.n_kv_heads, hd, sk.n_sinks, (int)threadIdx.x, COMBINE_THREADS);
+          copy_sink((const T*)sk.k_pages, (const T*)sk.v_pages, sk.page_layout, page, h, pos, slot, (T*)sk.sink_k,
+                    (T*)sk.sink_v, sk.n_kv_heads, hd, sk.n_sinks, (int)threadIdx.x, COMBINE_THREADS);
       }
       n_behind = max(0, min(sk.n_sinks, pos - sk.window + 1));
       if (n_behind > 0) {
@@ -350,15 +348,16 @@ namespace {
 int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, const int* block_table, int table_stride,
                     int ring_pages, const int* seq_slot, const int* seq_len, void* out, float* lse, float* partial,
                     int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits, int n_pages,
-                    int dtype, int force_simple, const SinkArgs& sinks, hipStream_t stream) {
+                    int page_layout, int dtype, int force_simple, const SinkArgs& sinks, hipStream_t stream) {
   if (B <= 0) return YALM_OK;
-  if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0)
+  if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0 ||
+      !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
   dim3 grid(B, n_heads, n_splits), cgrid(B, n_heads);
   if (dtype == YALM_F32) {
     attn_decode_simple_kernel<float><<<grid, WAVE, 0, stream>>>(
         (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
-        seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
+        seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout);
     attn_decode_combine_kernel<float><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (float*)out, lse, n_heads,
                                                                              head_dim, n_splits, sinks);
     return launch_status();
@@ -367,12 +366,12 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
   if (!force_simple) {
     int rc = yalm_attn_decode_bf16_mfma(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len,
                                         out, lse, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits,
-                                        n_pages, sinks, stream);
+                                        n_pages, page_layout, sinks, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   attn_decode_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
-      seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages);
+      seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout);
   attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim,
                                                                           n_splits, sinks);
   return launch_status();
@@ -382,12 +381,12 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
 extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                     int table_stride, int ring_pages, const int* seq_slot, const int* seq_len,
                                     void* out, float* lse, float* partial, int B, int n_heads, int n_kv_heads,
-                                    int head_dim, int window, int n_splits, int n_pages, int dtype, int force_simple,
-                                    hipStream_t stream) {
+                                    int head_dim, int window, int n_splits, int n_pages, int page_layout, int dtype,
+                                    int force_simple, hipStream_t stream) {
   SinkArgs none = {};
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, lse,
-                         partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, dtype, force_simple,
-                         none, stream);
+                         partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
+                         force_simple, none, stream);
 }
 
 extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -395,8 +394,8 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
                                 float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                                 int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream) {
   return yalm_attn_decode_lse(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out,
-                              nullptr, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, dtype,
-                              force_simple, stream);
+                              nullptr, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages,
+                              YALM_PAGE_ROWS, dtype, force_simple, stream);
 }
 
 extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -404,7 +403,8 @@ extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const 
                                       void* out, float* partial, void* sink_k, void* sink_v, int store,
                                       const float* cos_sin, int n_positions, int n_slots, int rotary_dim, int n_sinks,
                                       int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits,
-                                      int n_pages, int dtype, int force_simple, hipStream_t stream) {
+                                      int n_pages, int page_layout, int dtype, int force_simple,
+                                      hipStream_t stream) {
   if (n_sinks <= 0 || n_sinks > YALM_MAX_SINKS || window < n_sinks || n_slots <= 0 || sink_k == nullptr ||
       sink_v == nullptr || rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2 || head_dim % 2)
     return YALM_ERR_ARG;
@@ -418,6 +418,7 @@ extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const 
     sk.block_table = block_table;
     sk.table_stride = table_stride;
     sk.n_pages = n_pages;
+    sk.page_layout = page_layout;
   }
   sk.seq_slot = seq_slot;
   sk.seq_len = seq_len;
@@ -429,8 +430,8 @@ extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const 
   sk.window = window;
   sk.n_sinks = n_sinks;
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, nullptr,
-                         partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, dtype, force_simple, sk,
-                         stream);
+                         partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
+                         force_simple, sk, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -27,7 +27,8 @@ __global__ __launch_bounds__(WAVE) void sink_store_kernel(const T* __restrict__ 
   if (slot < 0 || slot >= n_slots || j >= seq_len[b]) return;
   const int tile = seq_tile0[b];
   if (tile < 0 || tile >= n_tiles) return;
-  copy_sink(k_stage, v_stage, tile, g, j, slot, sink_k, sink_v, n_kv_heads, hd, n_sinks, (int)threadIdx.x, WAVE);
+  copy_sink(k_stage, v_stage, YALM_PAGE_ROWS, tile, g, j, slot, sink_k, sink_v, n_kv_heads, hd, n_sinks,
+            (int)threadIdx.x, WAVE);
 }
 
 // grid (token, head); lanes over the head's elements, pairs (2p, 2p + 1) in one lane

@@ -26,6 +26,29 @@ typedef __bf16 bf16;
 #define YALM_READ_ONCE 2
 #endif
 
+// Where the key and the value of row r (0..63) lie inside a cache page of one KV head (elements from the
+// page's start).
+//   YALM_PAGE_ROWS:   keys [row][element], values [element][row] (the staging area of a prompt step always).
+//   YALM_PAGE_BLOCKS: head sizes that are multiples of 32.  Keys [element / 32][place(row)][element % 32],
+//     place(row) being the row's place in the order in which the matrix-core decode attention takes the
+//     rows of a page (16 rows an instruction: rows 8a + b (+4) (+32) for a, b < 4); values
+//     [row / 32][element][row % 32].  Each of that kernel's load instructions then reads 1 KB of
+//     consecutive bytes, whole 128-byte lines, instead of 16 pieces of 64 bytes.
+#define YALM_PAGE_ROWS 0
+#define YALM_PAGE_BLOCKS 1
+__host__ __device__ __forceinline__ int page_row_place(int r) {
+  return 16 * (2 * (r >> 5) + ((r >> 2) & 1)) + 4 * ((r >> 3) & 3) + (r & 3);
+}
+__host__ __device__ __forceinline__ int page_k_offset(int layout, int r, int e, int hd) {
+  return layout == YALM_PAGE_BLOCKS ? ((e >> 5) * PAGE + page_row_place(r)) * 32 + (e & 31) : r * hd + e;
+}
+__host__ __device__ __forceinline__ int page_v_offset(int layout, int r, int e, int hd) {
+  return layout == YALM_PAGE_BLOCKS ? ((r >> 5) * hd + e) * 32 + (r & 31) : e * PAGE + r;
+}
+__host__ __device__ __forceinline__ bool page_layout_ok(int layout, int hd) {
+  return layout == YALM_PAGE_ROWS || (layout == YALM_PAGE_BLOCKS && hd % 32 == 0);
+}
+
 __device__ __forceinline__ float to_f32(float v) { return v; }
 __device__ __forceinline__ float to_f32(bf16 v) { return static_cast<float>(v); }
 template <typename T> __device__ __forceinline__ T from_f32(float v);

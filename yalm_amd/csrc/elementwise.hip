@@ -140,7 +140,8 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
                                      const int* __restrict__ tok_seq, const int* __restrict__ tok_pos,
                                      const int* __restrict__ seq_slot, const int* __restrict__ seq_len,
                                      const float2* __restrict__ cos_sin, int n_positions, int n_heads,
-                                     int n_kv_heads, int hd, int rotary_dim, int n_pages, int slices, long plane) {
+                                     int n_kv_heads, int hd, int rotary_dim, int n_pages, int page_layout, int slices,
+                                     long plane) {
   // qkv may be `slices` partial products [slices][T][Q + 2 KV] of a GEMM that split K: added here, in order
   auto rd = [&](const float* p) {
     float v = p[0];
@@ -220,8 +221,9 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
         kst[r * hd + 2 * p + 1] = bb;
       }
       if (kpage) {
-        kpage[r * hd + 2 * p] = a;
-        kpage[r * hd + 2 * p + 1] = bb;
+        const int o = page_k_offset(page_layout, r, 2 * p, hd);     // a pair never straddles a block of 32
+        kpage[o] = a;
+        kpage[o + 1] = bb;
       }
     }
   } else {
@@ -229,7 +231,7 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
     for (int i = threadIdx.x; i < hd; i += WAVE) {
       T a = from_f32<T>(rd(src + i));
       if (vst) vst[(size_t)i * PAGE + r] = a;
-      if (vpage) vpage[(size_t)i * PAGE + r] = a;      // values are kept transposed inside a page
+      if (vpage) vpage[page_v_offset(page_layout, r, i, hd)] = a;      // values are kept transposed inside a page
     }
   }
 }
@@ -258,7 +260,7 @@ __global__ __launch_bounds__(256) void rope_kv_tiles_kernel(
     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_tile0, T* __restrict__ k_pages,
     T* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride, int ring_pages,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_len, const float2* __restrict__ cos_sin,
-    int n_positions, int B, int n_heads, int n_kv_heads, int hd, int rotary_dim, int n_pages) {
+    int n_positions, int B, int n_heads, int n_kv_heads, int hd, int rotary_dim, int n_pages, int page_layout) {
   extern __shared__ __attribute__((aligned(16))) unsigned char vt_raw[];
   T* vt = reinterpret_cast<T*>(vt_raw);           // [hd][VT_ROW]
   const int gt = blockIdx.x, job = blockIdx.y, tid = threadIdx.x;
@@ -319,7 +321,7 @@ __global__ __launch_bounds__(256) void rope_kv_tiles_kernel(
     const int r = e / pairs, p = e % pairs;
     const float2 y = rotated(src0 + (size_t)r * W + Q + g * hd, p0 + r, p);
     store_pair(kst + r * hd + 2 * p, y.x, y.y);
-    if (kpage) store_pair(kpage + r * hd + 2 * p, y.x, y.y);
+    if (kpage) store_pair(kpage + page_k_offset(page_layout, r, 2 * p, hd), y.x, y.y);
     const float2 v = *reinterpret_cast<const float2*>(src0 + (size_t)r * W + Q + KV + g * hd + 2 * p);
     vt[(2 * p) * VT_ROW + r] = from_f32<T>(v.x);
     vt[(2 * p + 1) * VT_ROW + r] = from_f32<T>(v.y);
@@ -333,7 +335,8 @@ __global__ __launch_bounds__(256) void rope_kv_tiles_kernel(
 #pragma unroll
     for (int u = 0; u < PER; ++u) piece[u] = c0 + u < rows ? vt[i * VT_ROW + c0 + u] : from_f32<T>(0.f);
     *reinterpret_cast<uint4*>(vst + (size_t)i * PAGE + c0) = *reinterpret_cast<const uint4*>(piece);
-    if (vpage) *reinterpret_cast<uint4*>(vpage + (size_t)i * PAGE + c0) = *reinterpret_cast<const uint4*>(piece);
+    if (vpage)       // 16 bytes of consecutive rows stay consecutive in either layout
+      *reinterpret_cast<uint4*>(vpage + page_v_offset(page_layout, c0, i, hd)) = *reinterpret_cast<const uint4*>(piece);
   }
 }
 
@@ -342,12 +345,13 @@ extern "C" int yalm_rope_kv_write_tiles(const float* qkv, void* q_out, void* k_s
                                         const int* block_table, int table_stride, int ring_pages,
                                         const int* seq_slot, const int* seq_len, const float* cos_sin,
                                         int n_positions, int T, int B, int n_tiles, int n_heads, int n_kv_heads,
-                                        int head_dim, int rotary_dim, int n_pages, int dtype, hipStream_t stream) {
+                                        int head_dim, int rotary_dim, int n_pages, int page_layout, int dtype,
+                                        hipStream_t stream) {
   if (T <= 0 || B <= 0 || n_tiles <= 0) return YALM_OK;
   if (head_dim <= 0 || (head_dim & 1) || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > head_dim ||
       n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || k_stage == nullptr || v_stage == nullptr ||
       cu_seqlens == nullptr || seq_tile0 == nullptr || n_heads + n_kv_heads > 65535 ||
-      ((n_heads + 2 * n_kv_heads) * head_dim) % 2 != 0)
+      ((n_heads + 2 * n_kv_heads) * head_dim) % 2 != 0 || !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
   const size_t esize = dtype == YALM_F32 ? 4 : 2;
   const size_t lds = (size_t)head_dim * VT_ROW * esize;
@@ -357,12 +361,12 @@ extern "C" int yalm_rope_kv_write_tiles(const float* qkv, void* q_out, void* k_s
     rope_kv_tiles_kernel<float><<<grid, 256, lds, stream>>>(
         qkv, (float*)q_out, (float*)k_stage, (float*)v_stage, cu_seqlens, seq_tile0, (float*)k_pages, (float*)v_pages,
         block_table, table_stride, ring_pages, seq_slot, seq_len, (const float2*)cos_sin, n_positions, B, n_heads,
-        n_kv_heads, head_dim, rotary_dim, n_pages);
+        n_kv_heads, head_dim, rotary_dim, n_pages, page_layout);
   else if (dtype == YALM_BF16)
     rope_kv_tiles_kernel<bf16><<<grid, 256, lds, stream>>>(
         qkv, (bf16*)q_out, (bf16*)k_stage, (bf16*)v_stage, cu_seqlens, seq_tile0, (bf16*)k_pages, (bf16*)v_pages,
         block_table, table_stride, ring_pages, seq_slot, seq_len, (const float2*)cos_sin, n_positions, B, n_heads,
-        n_kv_heads, head_dim, rotary_dim, n_pages);
+        n_kv_heads, head_dim, rotary_dim, n_pages, page_layout);
   else
     return YALM_ERR_DTYPE;
   return launch_status();
@@ -372,11 +376,11 @@ extern "C" int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_stage, 
                                   const int* seq_tile0, void* k_pages, void* v_pages, const int* block_table, int table_stride, int ring_pages,
                                   const int* tok_seq, const int* tok_pos, const int* seq_slot, const int* seq_len,
                                   const float* cos_sin, int n_positions, int T, int n_heads, int n_kv_heads,
-                                  int head_dim, int rotary_dim, int n_pages, int slices, int dtype,
+                                  int head_dim, int rotary_dim, int n_pages, int page_layout, int slices, int dtype,
                                   hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (head_dim <= 0 || (head_dim & 1) || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > head_dim ||
-      n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || slices < 1)
+      n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || slices < 1 || !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
   const long plane = (long)T * (n_heads + 2 * n_kv_heads) * head_dim;
   dim3 grid(T, n_heads + 2 * n_kv_heads);
@@ -384,12 +388,12 @@ extern "C" int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_stage, 
     rope_kv_write_kernel<float><<<grid, WAVE, 0, stream>>>(
         qkv, (float*)q_out, (float*)k_stage, (float*)v_stage, seq_tile0, (float*)k_pages, (float*)v_pages, block_table,
         table_stride, ring_pages, tok_seq, tok_pos, seq_slot, seq_len, (const float2*)cos_sin, n_positions, n_heads,
-        n_kv_heads, head_dim, rotary_dim, n_pages, slices, plane);
+        n_kv_heads, head_dim, rotary_dim, n_pages, page_layout, slices, plane);
   else if (dtype == YALM_BF16)
     rope_kv_write_kernel<bf16><<<grid, WAVE, 0, stream>>>(
         qkv, (bf16*)q_out, (bf16*)k_stage, (bf16*)v_stage, seq_tile0, (bf16*)k_pages, (bf16*)v_pages, block_table, table_stride,
         ring_pages, tok_seq, tok_pos, seq_slot, seq_len, (const float2*)cos_sin, n_positions, n_heads, n_kv_heads,
-        head_dim, rotary_dim, n_pages, slices, plane);
+        head_dim, rotary_dim, n_pages, page_layout, slices, plane);
   else
     return YALM_ERR_DTYPE;
   return launch_status();

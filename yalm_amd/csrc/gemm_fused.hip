@@ -201,9 +201,9 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_norm_kernel(const float* _
               const size_t base = ((size_t)phys * ra.n_kv_heads + head) * PAGE * ra.hd;
               const int row = pos & (PAGE - 1);
               if (region == 1)
-                ra.k_pages[base + (size_t)row * ra.hd + i] = yb;
+                ra.k_pages[base + page_k_offset(ra.page_layout, row, i, ra.hd)] = yb;
               else
-                ra.v_pages[base + (size_t)i * PAGE + row] = yb;
+                ra.v_pages[base + page_v_offset(ra.page_layout, row, i, ra.hd)] = yb;
             }
           }
         }
@@ -247,11 +247,11 @@ extern "C" int yalm_gemm_norm_qkv_rope(const float* x, const float* norm_w, floa
                                        void* k_pages, void* v_pages, const int* block_table, int table_stride,
                                        int ring_pages, const int* tok_pos, const int* seq_slot, const float* cos_sin,
                                        int n_positions, int M, int K, int n_heads, int n_kv_heads, int head_dim,
-                                       int rotary_dim, int n_pages, hipStream_t stream) {
+                                       int rotary_dim, int n_pages, int page_layout, hipStream_t stream) {
   const int N = (n_heads + 2 * n_kv_heads) * head_dim;
   if (!shape_ok(x, norm_w, Wqkv, M, N, K)) return YALM_ERR_ARG;
   if (head_dim <= 0 || head_dim % 16 != 0 || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > head_dim ||
-      n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || n_pages <= 0)
+      n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || n_pages <= 0 || !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
   RopeArgs ra;
   ra.q_out = (bf16*)q_out;
@@ -269,6 +269,7 @@ extern "C" int yalm_gemm_norm_qkv_rope(const float* x, const float* norm_w, floa
   ra.hd = head_dim;
   ra.rotary_dim = rotary_dim;
   ra.n_pages = n_pages;
+  ra.page_layout = page_layout;
   return launch_norm<EPI_ROPE>(x, norm_w, eps, (const bf16*)Wqkv, nullptr, M, N, K, 0, ra, stream);
 }
 
@@ -311,13 +312,13 @@ extern "C" int yalm_gemm_chain_qkv_rope(const void* X, const float* ss_in, int n
                                         const int* block_table, int table_stride, int ring_pages,
                                         const int* tok_pos, const int* seq_slot, const float* cos_sin,
                                         int n_positions, int M, int K, int n_heads, int n_kv_heads, int head_dim,
-                                        int rotary_dim, int n_pages, hipStream_t stream) {
+                                        int rotary_dim, int n_pages, int page_layout, hipStream_t stream) {
   const int N = (n_heads + 2 * n_kv_heads) * head_dim;
   if (M < 1 || M > 64 || K <= 0 || K % 8 != 0 || ((uintptr_t)X & 15) || ((uintptr_t)Wqkv & 15) || ss_in == nullptr ||
       n_parts_in <= 0 || block_table == nullptr || tok_pos == nullptr || seq_slot == nullptr)
     return YALM_ERR_ARG;
   if (head_dim <= 0 || head_dim % 16 != 0 || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > head_dim ||
-      n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || n_pages <= 0)
+      n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || n_pages <= 0 || !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
   ChainArgs ca = {};
   ca.ss_in = ss_in;
@@ -339,6 +340,7 @@ extern "C" int yalm_gemm_chain_qkv_rope(const void* X, const float* ss_in, int n
   ra.hd = head_dim;
   ra.rotary_dim = rotary_dim;
   ra.n_pages = n_pages;
+  ra.page_layout = page_layout;
   return skinny::launch<EPI_ROPE>((const bf16*)X, (const bf16*)Wqkv, nullptr, M, N, K, 0, ca, stream);
 }
 

@@ -16,6 +16,7 @@ struct SinkArgs {
   const int* block_table;
   int table_stride;
   int n_pages;
+  int page_layout;            // of k_pages, v_pages
   const int* seq_slot;        // [B]
   const int* seq_len;         // [B], the new token included: its position is seq_len - 1
   const float2* cos_sin;      // (cos, sin) [n_positions, rotary_dim / 2], or null
@@ -27,18 +28,20 @@ struct SinkArgs {
   int n_sinks;
 };
 
-// copies key row j and value column j of a page into the store of `slot`; threads tid, tid + n_threads, ...
+// copies the key and the value of row j of a page (of the given layout) into the store of `slot`; threads
+// tid, tid + n_threads, ...
 template <typename T>
-__device__ __forceinline__ void copy_sink(const T* __restrict__ k_src, const T* __restrict__ v_src, int page, int g,
-                                          int j, int slot, T* __restrict__ sink_k, T* __restrict__ sink_v,
-                                          int n_kv_heads, int hd, int n_sinks, int tid, int n_threads) {
-  const T* kr = k_src + (((size_t)page * n_kv_heads + g) * PAGE + j) * hd;       // [page][head][row][element]
-  const T* vc = v_src + ((size_t)page * n_kv_heads + g) * hd * PAGE + j;         // [page][head][element][row]
+__device__ __forceinline__ void copy_sink(const T* __restrict__ k_src, const T* __restrict__ v_src, int layout,
+                                          int page, int g, int j, int slot, T* __restrict__ sink_k,
+                                          T* __restrict__ sink_v, int n_kv_heads, int hd, int n_sinks, int tid,
+                                          int n_threads) {
+  const T* kp = k_src + ((size_t)page * n_kv_heads + g) * PAGE * hd;
+  const T* vp = v_src + ((size_t)page * n_kv_heads + g) * PAGE * hd;
   T* dk = sink_k + (((size_t)slot * n_kv_heads + g) * n_sinks + j) * hd;
   T* dv = sink_v + (((size_t)slot * n_kv_heads + g) * n_sinks + j) * hd;
   for (int i = tid; i < hd; i += n_threads) {
-    dk[i] = kr[i];
-    dv[i] = vc[(size_t)i * PAGE];
+    dk[i] = kp[page_k_offset(layout, j, i, hd)];
+    dv[i] = vp[page_v_offset(layout, j, i, hd)];
   }
 }
 

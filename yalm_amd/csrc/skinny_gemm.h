@@ -51,7 +51,7 @@ struct RopeArgs {                                // epilogue of the fused q/k/v 
   const int* tok_pos;
   const int* seq_slot;
   const float2* cos_sin;
-  int table_stride, ring_pages, n_positions, n_heads, n_kv_heads, hd, rotary_dim, n_pages;
+  int table_stride, ring_pages, n_positions, n_heads, n_kv_heads, hd, rotary_dim, n_pages, page_layout;
 };
 
 struct ChainArgs {
@@ -392,9 +392,9 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
             const size_t base = ((size_t)phys * ra.n_kv_heads + head) * PAGE * ra.hd;
             const int row = pos & (PAGE - 1);
             if (region == 1)
-              ra.k_pages[base + (size_t)row * ra.hd + i] = yb;
+              ra.k_pages[base + page_k_offset(ra.page_layout, row, i, ra.hd)] = yb;
             else
-              ra.v_pages[base + (size_t)i * PAGE + row] = yb;
+              ra.v_pages[base + page_v_offset(ra.page_layout, row, i, ra.hd)] = yb;
           }
         }
       }

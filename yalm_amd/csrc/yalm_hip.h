@@ -53,7 +53,7 @@ int yalm_gemm_norm_qkv_rope(const float* x, const float* norm_w, float eps, cons
                             void* k_pages, void* v_pages, const int* block_table, int table_stride, int ring_pages,
                             const int* tok_pos, const int* seq_slot, const float* cos_sin, int n_positions, int M,
                             int K, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, int n_pages,
-                            hipStream_t stream);
+                            int page_layout, hipStream_t stream);
 
 // Residual add and the next RMSNorm in one for 17..64 rows, or more with K a multiple of 64 (bfloat16): C float32 [M,N] += A[M,K] * W[N,K]^T, then
 // h_out bfloat16 [M,N] = C_new * rsqrt(mean(C_new^2) + eps) * norm_w.  workspace: at least M * N floats (more lets
@@ -81,7 +81,7 @@ int yalm_gemm_chain_qkv_rope(const void* X, const float* ss_in, int n_parts_in, 
                              void* q_out, void* k_pages, void* v_pages, const int* block_table, int table_stride,
                              int ring_pages, const int* tok_pos, const int* seq_slot, const float* cos_sin,
                              int n_positions, int M, int K, int n_heads, int n_kv_heads, int head_dim,
-                             int rotary_dim, int n_pages, hipStream_t stream);
+                             int rotary_dim, int n_pages, int page_layout, hipStream_t stream);
 
 // Rotates q and k of every token (adjacent pairs, angles from the table), writes q,
 // optionally k and v into a staging area in page format (for attention over the step's
@@ -90,7 +90,10 @@ int yalm_gemm_chain_qkv_rope(const void* X, const float* ss_in, int n_parts_in, 
 //   k_stage [n_tiles, n_kv_heads, PAGE, head_dim], v_stage [n_tiles, n_kv_heads, head_dim, PAGE] or null
 //   qkv      float32 [T, (n_heads + 2 n_kv_heads) * head_dim]
 //   cos_sin  float32 [n_positions, rotary_dim/2, 2] or null (no rotation)
-//   k_pages  [n_pages, n_kv_heads, PAGE, head_dim], v_pages [n_pages, n_kv_heads, head_dim, PAGE]
+//   k_pages  [n_pages, n_kv_heads, PAGE, head_dim], v_pages [n_pages, n_kv_heads, head_dim, PAGE]; inside a
+//            page of a head the elements lie as page_layout says (common.h: YALM_PAGE_ROWS as these shapes
+//            read, YALM_PAGE_BLOCKS in blocks of 32 elements or rows for head sizes that are multiples of
+//            32); the staging area is always YALM_PAGE_ROWS
 //   block_table int32 [n_slots, table_stride]; page of position p: table[slot][(p / PAGE) % ring_pages]
 //   a token is written iff its page is among the last ring_pages pages of its sequence
 // reference: fused_rope_and_cache_update (src/infer.cu:660-705)
@@ -100,7 +103,7 @@ int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_stage, void* v_sta
                        void* k_pages, void* v_pages, const int* block_table, int table_stride, int ring_pages, const int* tok_seq,
                        const int* tok_pos, const int* seq_slot, const int* seq_len, const float* cos_sin,
                        int n_positions, int T, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
-                       int n_pages, int slices, int dtype, hipStream_t stream);
+                       int n_pages, int page_layout, int slices, int dtype, hipStream_t stream);
 
 // The same for a step of whole prompts (every sequence from position 0; cu_seqlens [B + 1] token offsets,
 // n_tiles = seq_tile0[B]): whole page-shaped tiles at a time.  Needs a staging area; refuses
@@ -109,7 +112,8 @@ int yalm_rope_kv_write_tiles(const float* qkv, void* q_out, void* k_stage, void*
                              const int* seq_tile0, void* k_pages, void* v_pages, const int* block_table,
                              int table_stride, int ring_pages, const int* seq_slot, const int* seq_len,
                              const float* cos_sin, int n_positions, int T, int B, int n_tiles, int n_heads,
-                             int n_kv_heads, int head_dim, int rotary_dim, int n_pages, int dtype, hipStream_t stream);
+                             int n_kv_heads, int head_dim, int rotary_dim, int n_pages, int page_layout, int dtype,
+                             hipStream_t stream);
 
 // Causal attention of a step's tokens over the same step's keys (sequences that
 // start at position 0), packed without padding.  window 0 = all keys.
@@ -128,6 +132,7 @@ int yalm_attn_prefill(const void* q, const void* k_stage, const void* v_stage, v
 //   q, out [B, n_heads, hd]; seq_len[b] = keys of sequence b including the new one;
 //   seq_slot[b] < 0 marks a padding row (out = 0).
 //   partial: float32 workspace of yalm_attn_decode_workspace(...) bytes
+//   the pages are YALM_PAGE_ROWS (the variants below take a page_layout)
 int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                      int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                      float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits,
@@ -144,7 +149,8 @@ int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stag
 int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                          int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                          float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
-                         int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream);
+                         int n_splits, int n_pages, int page_layout, int dtype, int force_simple,
+                         hipStream_t stream);
 
 // Attention sinks beside a window (src/infer.cpp:305-319, 486-488): the first n_sinks positions of a
 // sequence stay visible when the window has moved past them, and each then counts as lying
@@ -175,8 +181,8 @@ int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pag
                            int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                            float* partial, void* sink_k, void* sink_v, int store, const float* cos_sin,
                            int n_positions, int n_slots, int rotary_dim, int n_sinks, int B, int n_heads,
-                           int n_kv_heads, int head_dim, int window, int n_splits, int n_pages, int dtype,
-                           int force_simple, hipStream_t stream);
+                           int n_kv_heads, int head_dim, int window, int n_splits, int n_pages, int page_layout,
+                           int dtype, int force_simple, hipStream_t stream);
 
 // yalm_attn_decode without a workspace argument, for callers that cannot allocate device memory
 // (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no

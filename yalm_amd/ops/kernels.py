@@ -154,8 +154,27 @@ def gemm_norm(x, norm_w, eps, w, out, epilogue, hidden=0):
     return out
 
 
+PAGE_ROWS, PAGE_BLOCKS = 0, 1
+
+
+def page_layout(head_dim):
+    """How keys and values lie inside a cache page of a head: PAGE_ROWS (keys [row][element], values
+    [element][row]) or, for head sizes that are multiples of 32, PAGE_BLOCKS (keys [element // 32][place of the
+    row in the order the matrix-core decode attention takes rows][element % 32], values [row // 32][element]
+    [row % 32]), in which every load instruction of that kernel reads 1 KB of consecutive bytes.  The tensors'
+    shapes stay [pages, heads, PAGE, head_dim] and [pages, heads, head_dim, PAGE] either way."""
+    return PAGE_BLOCKS if head_dim % 32 == 0 else PAGE_ROWS
+
+
+def _layout(layout, head_dim):
+    layout = page_layout(head_dim) if layout is None else int(layout)
+    if layout not in (PAGE_ROWS, PAGE_BLOCKS) or (layout == PAGE_BLOCKS and head_dim % 32):
+        raise ValueError("page layout %r does not fit head_dim %d" % (layout, head_dim))
+    return layout
+
+
 def gemm_norm_qkv_rope(x, norm_w, eps, wqkv, q_out, k_pages, v_pages, block_table, ring_pages, tok_pos, seq_slot,
-                       cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim):
+                       cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim, layout=None):
     """A decode step's rmsnorm + q/k/v projection + rotation + cache write in one kernel
     (row m is sequence m; see rope_kv_write for the operands)."""
     _check_heads(n_heads, n_kv_heads, head_dim)
@@ -184,7 +203,7 @@ def gemm_norm_qkv_rope(x, norm_w, eps, wqkv, q_out, k_pages, v_pages, block_tabl
         rotary_dim = 0
     library.check(library.lib().yalm_gemm_norm_qkv_rope(
         p_x, p_n, float(eps), p_w, p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_tp, p_ss, p_cs, n_pos, M, K, n_heads,
-        n_kv_heads, head_dim, rotary_dim, n_pages, _stream()), "gemm_norm_qkv_rope")
+        n_kv_heads, head_dim, rotary_dim, n_pages, _layout(layout, head_dim), _stream()), "gemm_norm_qkv_rope")
 
 
 CHAIN_MAX_ROWS = 16
@@ -293,7 +312,7 @@ def gemm_chain(x, w, out, epilogue, hidden=0, scale_from=None, emit=None):
 
 
 def gemm_chain_qkv_rope(xn, scale_from, wqkv, q_out, k_pages, v_pages, block_table, ring_pages, tok_pos, seq_slot,
-                        cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim):
+                        cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim, layout=None):
     """gemm_norm_qkv_rope for activations a producer emitted (see gemm_chain)."""
     _check_heads(n_heads, n_kv_heads, head_dim)
     if head_dim % 16:
@@ -323,7 +342,8 @@ def gemm_chain_qkv_rope(xn, scale_from, wqkv, q_out, k_pages, v_pages, block_tab
         rotary_dim = 0
     library.check(library.lib().yalm_gemm_chain_qkv_rope(
         p_x, p_ss, n_parts, float(eps), p_w, p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_tp, p_sl, p_cs, n_pos, M, K,
-        n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, _stream()), "gemm_chain_qkv_rope")
+        n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, _layout(layout, head_dim), _stream()),
+        "gemm_chain_qkv_rope")
 
 
 def _check_heads(n_heads, n_kv_heads, head_dim):
@@ -334,7 +354,7 @@ def _check_heads(n_heads, n_kv_heads, head_dim):
 
 
 def rope_kv_write(qkv, q_out, k_stage, v_stage, seq_tile0, k_pages, v_pages, block_table, ring_pages, tok_seq, tok_pos,
-                  seq_slot, seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim, slices=1):
+                  seq_slot, seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim, slices=1, layout=None):
     """Rotates q and k by the angles of `cos_sin` at each token's position, writes q in
     q_out's dtype, k and v into the staging area (page format, tile seq_tile0[sequence] +
     position // PAGE) if one is given, and into the pages of the cache if given.
@@ -385,12 +405,12 @@ def rope_kv_write(qkv, q_out, k_stage, v_stage, seq_tile0, k_pages, v_pages, blo
         rotary_dim = 0
     library.check(library.lib().yalm_rope_kv_write(
         p_qkv, p_q, p_ks, p_vs, p_t0, p_kp, p_vp, p_bt, stride, max(ring_pages, 1), p_ts, p_tp, p_ss, p_sl, p_cs,
-        n_pos, T, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, int(slices), dtype_code(dt), _stream()),
-        "rope_kv_write")
+        n_pos, T, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, _layout(layout, head_dim), int(slices),
+        dtype_code(dt), _stream()), "rope_kv_write")
 
 
 def rope_kv_write_tiles(qkv, q_out, k_stage, v_stage, cu_seqlens, seq_tile0, k_pages, v_pages, block_table, ring_pages,
-                        seq_slot, seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim):
+                        seq_slot, seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim, layout=None):
     """rope_kv_write for a step of whole prompts (every sequence from position 0), a page-shaped
     tile of 64 positions at a time.  False if the kernel refuses the head size (the caller then
     uses rope_kv_write)."""
@@ -431,7 +451,8 @@ def rope_kv_write_tiles(qkv, q_out, k_stage, v_stage, cu_seqlens, seq_tile0, k_p
         rotary_dim = 0
     library.check(library.lib().yalm_rope_kv_write_tiles(
         p_qkv, p_q, p_ks, p_vs, p_cu, p_t0, p_kp, p_vp, p_bt, stride, max(ring_pages, 1), p_ss, p_sl, p_cs, n_pos, T, B,
-        n_tiles, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, dtype_code(dt), _stream()), "rope_kv_write_tiles")
+        n_tiles, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, _layout(layout, head_dim), dtype_code(dt),
+        _stream()), "rope_kv_write_tiles")
     return True
 
 
@@ -492,8 +513,9 @@ def attn_decode_workspace_floats(B, n_heads, head_dim, n_splits):
 
 
 def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len, out, partial, n_heads, n_kv_heads,
-                head_dim, window, n_splits, lse=None, sinks=None):
-    """One query per sequence over the cache pages; seq_len counts the new key.  lse as in attn_prefill.
+                head_dim, window, n_splits, lse=None, sinks=None, layout=None):
+    """One query per sequence over the cache pages (laid out as `layout` says, default page_layout(head_dim));
+    seq_len counts the new key.  lse as in attn_prefill.
     sinks = (sink_k, sink_v [slots, n_kv_heads, n_sinks, head_dim], cos_sin or None, rotary_dim, store):
     the attention sinks that a query's window no longer covers are taken in where the splits are merged
     (their keys turned by max(0, position - window - n_sinks + 1) positions with the table cos_sin); with
@@ -521,7 +543,8 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
         p_lse = None if lse is None else _need(lse, "lse", torch.float32, (B, n_heads))
         library.check(library.lib().yalm_attn_decode_lse(
             p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_lse, p_w, B, n_heads, n_kv_heads, head_dim,
-            int(window), int(n_splits), n_pages, dtype_code(dt), force, _stream()), "attn_decode")
+            int(window), int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, _stream()),
+            "attn_decode")
         return out
     if lse is not None:
         raise ValueError("attn_decode leaves no lse when it takes the sinks in itself")
@@ -540,7 +563,7 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
         _need(sink_k, "sink_k", dt, (n_slots, n_kv_heads, n_sinks, head_dim)),
         _need(sink_v, "sink_v", dt, (n_slots, n_kv_heads, n_sinks, head_dim)), 1 if store else 0, p_cs, n_pos, n_slots,
         int(rotary_dim) if p_cs is not None else 0, n_sinks, B, n_heads, n_kv_heads, head_dim, int(window),
-        int(n_splits), n_pages, dtype_code(dt), force, _stream()), "attn_decode with sinks")
+        int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, _stream()), "attn_decode with sinks")
     return out
 
 

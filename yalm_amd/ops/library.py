@@ -21,36 +21,31 @@ _SIGNATURES = {
     "yalm_rmsnorm": (_I, [_P, _P, _I, _P, _I, _P, _I, _I, _F, _P]),
     "yalm_gemm": (_I, [_P, _P, _P, _P, ctypes.c_long, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_gemm_norm": (_I, [_P, _P, _F, _P, _P, _I, _I, _I, _I, _I, _P]),
-    "yalm_gemm_norm_qkv_rope": (_I, [_P, _P, _F, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I,
-                                     _I, _P]),
+    "yalm_gemm_norm_qkv_rope": (_I, [_P, _P, _F, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_gemm_chain": (_I, [_P, _P, _P, _I, _I, _I, _I, _I, _P, _I, _F, _P, _P, _P, _P]),
     "yalm_gemm_chain_parts": (_I, [_I]),
-    "yalm_gemm_chain_qkv_rope": (_I, [_P, _P, _I, _F, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I,
-                                      _I, _I, _P]),
-    "yalm_rope_kv_write": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I,
-                                _I, _I, _I, _P]),
+    "yalm_gemm_chain_qkv_rope": (_I, [_P, _P, _I, _F, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_rope_kv_write": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_gemm_partial": (_I, [_P, _P, _P, ctypes.c_long, _I, _I, _I, _P, _P]),
     "yalm_gemm_bf16_dma_workspace": (ctypes.c_long, [_I, _I, _I]),
     "yalm_gemm_add_norm": (_I, [_P, _P, _P, _P, ctypes.c_long, _I, _I, _I, _P, _F, _P, _P]),
-    "yalm_rope_kv_write_tiles": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I,
-                                      _I, _I, _I, _I, _P]),
+    "yalm_rope_kv_write_tiles": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_prefill": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_workspace": (ctypes.c_long, [_I, _I, _I, _I]),
     "yalm_attn_prefill_lse": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I,
                                    _P]),
-    "yalm_attn_decode_lse": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_attn_decode_lse": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_sink_store": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_sink_mix": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
-    "yalm_attn_decode_sinks": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I,
-                                    _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_attn_decode_sinks": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_static": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_argmax": (_I, [_P, _P, _I, _I, _P]),
     "yalm_sample": (_I, [_P, _P, _F, _P, _I, _I, _P]),
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
 }
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 
 class KernelError(RuntimeError):
