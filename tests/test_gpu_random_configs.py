@@ -1,6 +1,7 @@
 """The engine against the plain implementation for configurations drawn at random (seeded):
 head sizes in steps of 16, group sizes that are no power of two, widths with and without the
-factors that choose a kernel's path (8, 64), windows, tied and untied heads.  Each is replayed
+factors that choose a kernel's path (8, 64), windows with and without attention sinks, heads rotated whole
+or by half, tied and untied heads.  Each is replayed
 whole, with its last tokens one by one and as a batch of unequal lengths, in both dtypes."""
 import numpy as np
 import pytest
@@ -36,11 +37,18 @@ def random_config(seed):
     }
     if window:
         cfg["sliding_window"] = window
+    # drawn after everything else, so that the seeds keep the sizes they had before these options existed
+    sinks = pick([0, 1, 2, 4])
+    if window and sinks:
+        cfg["attention_sinks"] = sinks
+    rotary = pick([1.0, 1.0, 0.5])
+    if rotary != 1.0:
+        cfg["partial_rotary_factor"] = rotary
     return cfg
 
 
 LENGTHS = [40, 1, 130, 67, 18]
-SEEDS = [101, 102, 103, 104, 105, 106]
+SEEDS = [101, 102, 103, 104, 105, 106, 107, 127, 135, 185]
 
 
 @pytest.fixture(scope="module")
