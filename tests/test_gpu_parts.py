@@ -255,7 +255,10 @@ def define_toy_parts():
 
 class ToyConfig:
     """A toy architecture: layer 0 mixes with the running mean, layer 1 with
-    attention; the schedule runs layer 1 twice (two cache lines)."""
+    attention; the schedule runs layer 1 twice (two cache lines) and then a third
+    time as a reader of the first run's line: its queries are the present ones, its
+    keys and values those that the first run stored.  `window` / `sinks` (optional)
+    give the attention a window with attention sinks beside it."""
 
     def __init__(self, d):
         self.d = d
@@ -275,7 +278,8 @@ class ToyConfig:
         pos = PartSpec("rope", {"head_dim": 16, "rotary_dim": 16, "theta": 100.0, "scaling": None,
                                 "weight_rows": "interleaved"})
         mixers = [PartSpec(d.get("mean_mixer", "toy_running_mean"), {}, prefix="mean."),
-                  PartSpec("gqa_attention", {"n_heads": 2, "n_kv_heads": 1, "head_dim": 16, "window": 0,
+                  PartSpec("gqa_attention", {"n_heads": 2, "n_kv_heads": 1, "head_dim": 16,
+                                             "window": d.get("window", 0), "sinks": d.get("sinks", 0),
                                              "position": pos}, prefix="attn.")]
         layers = [LayerSpec("prenorm_residual", m, PartSpec("swiglu", {"hidden": d["hidden"]}, prefix="ff."),
                             PartSpec("rmsnorm", norm, prefix="n1."), PartSpec("rmsnorm", norm, prefix="n2."),
@@ -284,7 +288,8 @@ class ToyConfig:
                          PartSpec("token_embedding", {"vocab_size": d["vocab"]}, prefix="toy.emb."), layers,
                          PartSpec("rmsnorm", norm, prefix="toy.norm."),
                          PartSpec("lm_head", {"vocab_size": d["vocab"], "tied": True}),
-                         schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1), ScheduleEntry(1, 2)])
+                         schedule=[ScheduleEntry(0, 0), ScheduleEntry(1, 1), ScheduleEntry(1, 2),
+                                   ScheduleEntry(1, 1, writes_cache=False)])
 
 
 def toy_plain_forward(w, d, tokens):
@@ -300,19 +305,25 @@ def toy_plain_forward(w, d, tokens):
 
     x = x + toy_mixer_plain(R.rmsnorm(x, w["toy.0.n1.weight"], d["eps"]), w["toy.0.mean.w.weight"])
     x = x + ffn(x, "toy.0.")
-    for _ in range(2):
+    first_kv = None
+    for run in range(3):
         h = R.rmsnorm(x, w["toy.1.n1.weight"], d["eps"])
         q = (h @ w["toy.1.attn.q_proj.weight"].double().T).reshape(T, 2, 16)
-        k = (h @ w["toy.1.attn.k_proj.weight"].double().T).reshape(T, 1, 16)
+        k = R.rope_interleaved((h @ w["toy.1.attn.k_proj.weight"].double().T).reshape(T, 1, 16), pos, f)
         v = (h @ w["toy.1.attn.v_proj.weight"].double().T).reshape(T, 1, 16)
-        a = R.attention(R.rope_interleaved(q, pos, f), R.rope_interleaved(k, pos, f), v)
+        if run == 0:
+            first_kv = (k, v)
+        if run == 2:                       # the reader: keys and values as the first run stored them
+            k, v = first_kv
+        a = R.attention(R.rope_interleaved(q, pos, f), k, v, d.get("window", 0), d.get("sinks", 0), f)
         x = x + a.reshape(T, 32) @ w["toy.1.attn.o_proj.weight"].double().T
         x = x + ffn(x, "toy.1.")
     return R.rmsnorm(x, w["toy.norm.weight"], d["eps"]) @ w["toy.emb.weight"].double().T
 
 
+@pytest.mark.parametrize("window,sinks", [(0, 0), (9, 2)])
 @pytest.mark.parametrize("mixer", ["toy_running_mean", "toy_running_mean_on_device"])
-def test_toy_mixer_and_architecture_from_outside(tmp_path, mixer):
+def test_toy_mixer_and_architecture_from_outside(tmp_path, mixer, window, sinks):
     """Layer 0 carries state of its own.  With the host-driven mixer only that layer runs kernel by
     kernel in a decode step and the layers around it are replayed from graphs; with the device-driven
     one the whole step is one graph and the state is advanced inside it, once a step."""
@@ -324,17 +335,18 @@ def test_toy_mixer_and_architecture_from_outside(tmp_path, mixer):
     register_architecture("ToyForCausalLM", ToyConfig, replace=True)
     try:
         d = {"architectures": ["ToyForCausalLM"], "width": 40, "hidden": 48, "vocab": 61, "positions": 200,
-             "eps": 1e-5, "mean_mixer": mixer}
+             "eps": 1e-5, "mean_mixer": mixer, "window": window, "sinks": sinks}
         folder = write_random_model(str(tmp_path / "toy"), d, seed=2)
         model = Model.from_folder(folder, dtype=torch.float32, device=DEV)
         engine = Engine(model, max_tokens=1024)
         if mixer == "toy_running_mean":
             assert not model.graph_safe()
-            assert engine._segments == [(True, 0, 1), (False, 1, 2), (True, 2, 5)]
+            assert engine._segments == [(True, 0, 1), (False, 1, 2), (True, 2, 6)]
         else:
-            assert model.graph_safe() and engine._segments == [(True, 0, 5)]
+            assert model.graph_safe() and engine._segments == [(True, 0, 6)]
         assert len(engine.cache.state_groups) == 1 and isinstance(engine.cache.group_of(0), StateGroup)
         assert engine.cache.group_of(1) is engine.cache.group_of(2)          # the layer that runs twice: two lines
+        assert engine.cache.group_of(1).lines == [1, 2]                      # the reader has no line of its own
         cfg, w = R.read_folder(folder)
         requests = {"a": [5, 9, 60, 3, 3, 17, 44, 8, 0, 31], "b": [7, 7, 2], "c": list(range(40, 61)) + list(range(30)),
                     "d": [60, 0, 1, 59, 2, 58]}
