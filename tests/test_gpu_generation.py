@@ -240,9 +240,9 @@ def test_a_context_shorter_than_the_text(folders):
     """The reference's -T <n>: the first two positions stay as sinks beside the last n - 2.  Greedy
     generation far past a context of 24 through the Python entry point and through the command line,
     against the plain implementation with the same sinks and window."""
-    from yalm_amd import Engine, Model, generate
-    folder = folders["tiny_wide_heads"]          # an untied head: the next token is not simply the last one again
-    cfg, w = R.read_folder(folder)
+    from yalm_amd import Engine, Model, StepError, generate
+    folder = folders["tiny_mistral"]             # an untied head: the next token is not simply the last one again;
+    cfg, w = R.read_folder(folder)               # 64 positions of its own, which the text runs past
     prompt = [1, 17, 200, 33, 5]
     n_new, context = 90, 24
 
@@ -254,10 +254,17 @@ def test_a_context_shorter_than_the_text(folders):
     for _ in range(n_new):
         want.append(R.sample_argmax(plain(seq)[-1]))
         seq.append(want[-1])
-    unlimited = plain_greedy(folder, prompt, n_new)
-    assert want[:context - len(prompt)] == unlimited[:context - len(prompt)] and want != unlimited
+    unlimited, seq = [], list(prompt)            # every key visible: the same up to the context's end, then another text
+    for _ in range(60):
+        unlimited.append(R.sample_argmax(R.forward(w, cfg, seq, window_override=0)[-1]))
+        seq.append(unlimited[-1])
+    assert want[:context - len(prompt)] == unlimited[:context - len(prompt)] and want[:60] != unlimited
     model = Model.from_folder(folder, dtype=torch.float32, device="cuda:0", context=context)
-    engine = Engine(model, max_tokens=512)
+    with pytest.raises(StepError, match="window"):            # without a window on every attention: the model's positions
+        Engine(Model.from_folder(folders["tiny_llama"], dtype=torch.float32, device="cuda:0"), max_tokens=512,
+               positions=1000)
+    engine = Engine(model, max_tokens=512, positions=len(prompt) + n_new + 1)
+    assert engine.n_positions == len(prompt) + n_new + 1 > cfg["max_position_embeddings"]
     assert generate(engine, [prompt], max_new_tokens=n_new, temperature=0.0, stop_ids=[])[0] == want
     # a prompt that is itself longer than the context, with company
     long_prompt = prompt + want[:50]

@@ -157,10 +157,10 @@ def _prompts(a, model):
     return [tokenizer().encode(text, True)], tokenizer()
 
 
-def _engine(a, model, need_tokens):
+def _engine(a, model, need_tokens, positions=None):
     from .engine import Engine
     budget = a["max_tokens"] or need_tokens
-    return Engine(model, max_tokens=max(64, budget))
+    return Engine(model, max_tokens=max(64, budget), positions=positions if a["context"] else None)
 
 
 def run_completion(a):
@@ -172,8 +172,11 @@ def run_completion(a):
     steps = a["num_steps"]
     if steps == 0 or steps == -1:                                   # main.cpp:71-74; -1 ends when the context is full
         steps = max_len
-    need = sum(min(max_len, len(p) + steps) + 64 for p in prompts)
-    engine = _engine(a, model, need)
+    if a["context"]:                                                # under -T a text may run past the model's positions
+        max_len = max(max_len, max(len(p) for p in prompts) + steps)
+    held = (a["context"] // 64 + 2) * 64 if a["context"] else max_len      # a window's ring of pages holds no more
+    need = sum(min(max_len, len(p) + steps, max(held, len(p))) + 64 for p in prompts)
+    engine = _engine(a, model, need, positions=max_len)
     seed = a["seed"] if a["seed"] is not None else int(time.time() * 1000)          # main.cpp:66
     stats = GenerationStats()
     stop = list(model.spec.eos_token_ids)
@@ -223,7 +226,7 @@ def run_perplexity(a):
     token; ppl = exp(-sum/N), error = ppl * sqrt((ss - sum^2/N)/N/N), N = len - 1."""
     model = _load(a)
     prompts, _ = _prompts(a, model)
-    engine = _engine(a, model, max(len(p) + 64 for p in prompts))
+    engine = _engine(a, model, max(len(p) + 64 for p in prompts), positions=max(len(p) for p in prompts) + 1)
     results = []
     for p in prompts:
         if len(p) < 2:

@@ -73,9 +73,12 @@ class Engine:
     """max_tokens: the most tokens live sequences hold at any time (each rounded up to a page);
     max_batch: the most sequences alive at once; use_graphs: replay decode steps from captured
     graphs; max_graphs: the most (batch bucket, pages bucket) graphs kept (the least recently
-    used one goes first)."""
+    used one goes first); positions: how far a sequence may run (default: the model's
+    max_position_embeddings) - more than the model's own only if every attention keeps a window,
+    whose scores depend on distances alone (the reference's -T lets a text run on without end,
+    src/infer.cpp:484-488)."""
 
-    def __init__(self, model, max_tokens, max_batch=None, use_graphs=True, max_graphs=24):
+    def __init__(self, model, max_tokens, max_batch=None, use_graphs=True, max_graphs=24, positions=None):
         if model.device is None:
             raise StepError("the model has no weights yet")
         if model.device.type != "cuda":
@@ -88,6 +91,11 @@ class Engine:
                                   self.device, n_slots=max_batch)
         n_positions = model.spec.max_positions if self.cache.unbounded else \
             min(model.spec.max_positions, self.cache.max_seq_len)
+        if positions is not None and int(positions) > n_positions:
+            if not self.cache.unbounded:
+                raise StepError("%d positions asked for, the model has %d: more need a window on every attention "
+                                "(a context shorter than the text)" % (int(positions), model.spec.max_positions))
+            n_positions = int(positions)
         self.n_positions = n_positions
         model.prepare(n_positions)                      # tables only ever grow: other engines of the model keep theirs
         self._tables_version = model.tables_version
