@@ -9,7 +9,9 @@ have pools and tables of their own.  A windowed group keeps, per sequence, a rin
 of ceil(window / PAGE) + 1 pages: position p lives in table column (p // PAGE)
 % ring_pages; if it also keeps attention sinks (the first positions of a
 sequence, visible behind the window), their keys and values have a place of
-their own per slot, because the ring overwrites their pages.  Beside the pages there is per-sequence state of fixed size
+their own per slot, because the ring overwrites their pages.  How the elements
+lie inside a page is the kernels' matter (ops.kernels.page_layout); nothing here
+looks inside one.  Beside the pages there is per-sequence state of fixed size
 (StateGroup) for mixers that carry one; it is cleared when a slot is acquired,
 because unlike keys behind the length, stale state is not harmless.
 
