@@ -375,21 +375,30 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, void* __
   }
 }
 
+// K slices wanted for n_blocks row blocks: until every CU has a workgroup, while the partial sums stay small
+// beside the weights (slices * M * N * 4 bytes against N * K * 2) and a slice keeps at least 2 chunks
+int wanted_slices(int n_blocks, int M, int K) {
+  const int chunks = ceil_div(K, KC);
+  int slices = 1;
+  while (n_blocks * slices < 200 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
+    slices *= 2;
+  return slices;
+}
+// k a slice covers (whole chunks), and how many slices that makes
+void slice_k(int K, int wanted, int* k_per_slice, int* slices) {
+  *k_per_slice = ceil_div(ceil_div(K, KC), wanted) * KC;
+  *slices = ceil_div(K, *k_per_slice);
+}
+
 template <int MT, int EPI, int NW>
 int launch_nw(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
               hipStream_t stream) {
   constexpr int NTW = EPI == 3 ? 2 : 1;
   const int rows_per_wg = NW * 16 * NTW;
   const int n_blocks = ceil_div(N, rows_per_wg);
-  const int chunks = ceil_div(K, KC);
-  // slices: until every CU has a workgroup, while the partial sums stay small beside the weights
-  // (slices * M * N * 4 bytes against N * K * 2) and a slice keeps at least 2 chunks
-  int slices = 1;
-  while (n_blocks * slices < 200 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
-    slices *= 2;
+  int slices = wanted_slices(n_blocks, M, K), k_per_slice;
   if (ws == nullptr || (long)slices * M * N > ws_floats) slices = 1;
-  const int k_per_slice = ceil_div(chunks, slices) * KC;
-  slices = ceil_div(K, k_per_slice);
+  slice_k(K, slices, &k_per_slice, &slices);
   dim3 grid(n_blocks, slices);
   int rc = launch_kernel<MT, NTW, EPI, NW>(grid, X, W, C, ws, M, N, K, H, k_per_slice, 0, stream);
   if (rc != YALM_OK || slices == 1) return rc;
@@ -472,14 +481,10 @@ template <int MT, int NW>
 int launch_add_norm_nw(const bf16* X, const bf16* W, float* C, float* ws, long ws_floats, int M, int N, int K,
                        const float* norm_w, float eps, bf16* h, hipStream_t stream) {
   const int n_blocks = ceil_div(N, NW * 16);
-  const int chunks = ceil_div(K, KC);
-  int slices = 1;
-  while (n_blocks * slices < 200 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
-    slices *= 2;
+  int slices = wanted_slices(n_blocks, M, K), k_per_slice;
   while (slices > 1 && (long)slices * M * N > ws_floats) slices /= 2;
   if (ws == nullptr || (long)slices * M * N > ws_floats) return YALM_ERR_ARG;
-  const int k_per_slice = ceil_div(chunks, slices) * KC;
-  slices = ceil_div(K, k_per_slice);
+  slice_k(K, slices, &k_per_slice, &slices);
   dim3 grid(n_blocks, slices);
   int rc = launch_kernel<MT, 1, 2, NW>(grid, X, W, C, ws, M, N, K, 0, k_per_slice, 1, stream);
   if (rc != YALM_OK) return rc;
@@ -501,14 +506,10 @@ template <int MT, int NW>
 int launch_partial_nw(const bf16* X, const bf16* W, float* ws, long ws_floats, int M, int N, int K, int* slices_out,
                       hipStream_t stream) {
   const int n_blocks = ceil_div(N, NW * 16);
-  const int chunks = ceil_div(K, KC);
-  int slices = 1;
-  while (n_blocks * slices < 200 && slices * 2 <= K / (8 * M) && slices * 2 <= chunks / 2 && slices < 16)
-    slices *= 2;
+  int slices = wanted_slices(n_blocks, M, K), k_per_slice;
   while (slices > 1 && (long)slices * M * N > ws_floats) slices /= 2;
   if (ws == nullptr || (long)slices * M * N > ws_floats) return YALM_ERR_ARG;
-  const int k_per_slice = ceil_div(chunks, slices) * KC;
-  slices = ceil_div(K, k_per_slice);
+  slice_k(K, slices, &k_per_slice, &slices);
   *slices_out = slices;
   dim3 grid(n_blocks, slices);
   return launch_kernel<MT, 1, 0, NW>(grid, X, W, ws, ws, M, N, K, 0, k_per_slice, 1, stream);
