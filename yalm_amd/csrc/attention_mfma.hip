@@ -390,30 +390,32 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
       auto softmax_tile = [&](auto masked) {
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
+          // the maximum is taken over the raw dot products and scaled once (the scale is positive); every
+          // score is then scaled and has the maximum taken off in one fused multiply-add
           float mx = -FLT_MAX;
 #pragma unroll
           for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              float v = sc[c][t][r] * score_scale;
+              float v = sc[c][t][r];
               if (decltype(masked)::value) {
                 int kpos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
                 bool vis = kpos <= pos_q[c] && (window == 0 || pos_q[c] - kpos < window) && q_ok[c];
                 v = vis ? v : -INFINITY;
+                sc[c][t][r] = v;
               }
-              sc[c][t][r] = v;
               mx = fmaxf(mx, v);
             }
           mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
           mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-          const float m_new = fmaxf(m[c], mx);
+          const float m_new = fmaxf(m[c], mx * score_scale);
           corr[c] = __builtin_amdgcn_exp2f(m[c] - m_new);
           float psum = 0.f;
 #pragma unroll
           for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              float p = __builtin_amdgcn_exp2f(sc[c][2 * s2 + (e >> 2)][e & 3] - m_new);
+              float p = __builtin_amdgcn_exp2f(fmaf(sc[c][2 * s2 + (e >> 2)][e & 3], score_scale, -m_new));
               psum += p;
               pb[c][s2][e] = static_cast<bf16>(p);
             }
