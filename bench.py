@@ -156,15 +156,22 @@ def main():
         for i in range(0, B, n):
             logits = engine.step(slots[i:i + n], prompts[i:i + n])
             tokens += sampler.sample(logits, 0.0, ids[i:i + n], [0] * len(slots[i:i + n]))
-        for _ in range(warmup):
-            logits = engine.step(slots, [[t] for t in tokens])
-            tokens = sampler.sample(logits, 0.0, ids, [0] * B)
+        # decode steps as generate() runs them: each step takes its tokens from the draw before on the
+        # device, and the host reads every draw while the step behind it runs
+        def advance(n, drawn):
+            for _ in range(n):
+                logits = engine.step_from(slots, drawn.tokens)
+                ahead = sampler.draw(logits, 0.0, ids, [0] * B)
+                drawn.tolist()
+                drawn = ahead
+            return drawn
+
+        drawn = sampler.draw(engine.step(slots, [[t] for t in tokens]), 0.0, ids, [0] * B)
+        drawn = advance(warmup, drawn)
         sync()
         start_len = engine.length(slots[0])
         t = time.perf_counter()
-        for _ in range(steps):
-            logits = engine.step(slots, [[t_] for t_ in tokens])
-            tokens = sampler.sample(logits, 0.0, ids, [0] * B)
+        advance(steps, drawn)
         sync()
         sec = time.perf_counter() - t
         end_len = engine.length(slots[0])

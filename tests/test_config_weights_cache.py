@@ -454,15 +454,80 @@ def test_generation_loop_decisions():
     assert generate(e2, [[1]], max_new_tokens=0, sampler=ArgmaxSampler()) == [[]]
 
 
-def test_a_failed_step_gives_the_slots_back():
-    class Failing(ScriptedEngine):
+class ScriptedAheadEngine(ScriptedEngine):
+    """Takes a step's tokens from the tensor of the draw before, as the engine's step_from does."""
+
+    def step_from(self, slots, source, rows=None):
+        rows = list(range(len(slots))) if rows is None else list(rows)
+        assert len(rows) == len(slots) and all(self.lens[s] > 0 for s in slots)
+        return self.step(slots, [[int(source[r])] for r in rows])
+
+
+class DrawingSampler(ArgmaxSampler):
+    """draw() as the sampler's: the tokens as a tensor at once, as a list on demand."""
+
+    class _Drawn:
+        def __init__(self, tokens, reads):
+            self.tokens, self._reads = tokens, reads
+
+        def tolist(self):
+            self._reads.append(len(self.tokens))
+            return self.tokens.tolist()
+
+    def __init__(self):
+        self.reads = []
+        self.draws = []
+
+    def draw(self, logits, temperature, request_ids, steps):
+        self.draws.append((list(request_ids), list(steps)))
+        return self._Drawn(logits.argmax(dim=1).to(torch.int32), self.reads)
+
+
+def test_generation_loop_a_step_ahead():
+    """The same tokens as the loop that reads every token first; a stop token is seen one step
+    late (its sequence is in one more step), an end by count is known beforehand."""
+    prompts = [[1, 2, 3], [7], [4, 5], [0], [8]]
+    e = ScriptedAheadEngine()
+    sampler = DrawingSampler()
+    out = generate(e, prompts, max_new_tokens=4, sampler=sampler, batch_size=3)
+    assert out == [[4, 5, 6, 7], [8, 9], [6, 7, 8, 9], [1, 2, 3, 4], [9]]
+    assert e.log[0] == ([0, 1, 2], [3, 1, 2])
+    assert e.log[1] == ([0, 1, 2], [1, 1, 1])
+    assert e.log[2] == ([0, 1, 2], [1, 1, 1])            # the 9 of request 1 is read while this step runs
+    assert e.log[3] == ([0, 2], [1, 1])
+    assert e.log[4][1] == [1, 1] and len(e.log) == 8     # no step for a fourth token's successor
+    assert not e.lens and sorted(e.free) == [0, 1, 2]
+    # every draw is read once, after the step behind it was queued; the draw numbers count a request's tokens
+    assert sampler.reads == [3, 3, 3, 2, 2, 2, 1, 1]
+    assert sampler.draws[:4] == [([0, 1, 2], [0, 0, 0]), ([0, 1, 2], [1, 1, 1]), ([0, 1, 2], [2, 2, 2]), ([0, 2], [3, 3])]
+    behind = generate(ScriptedAheadEngine(), prompts, max_new_tokens=4, sampler=DrawingSampler(), batch_size=3,
+                      ahead=False)
+    assert behind == out
+    # the context ends a request by its count: no step beyond the last position
+    e2 = ScriptedAheadEngine(n_positions=6)
+    assert generate(e2, [[1, 2, 3]], max_new_tokens=50, sampler=DrawingSampler(), stop_ids=[]) == [[4, 5, 6]]
+    assert not e2.lens and [n for _, n in e2.log] == [[3], [1], [1]]
+    with pytest.raises(ValueError, match="step_from"):
+        generate(ScriptedEngine(), prompts, max_new_tokens=4, sampler=DrawingSampler(), ahead=True)
+    # a callback sees the tokens in the same order
+    seen_a, seen_b = [], []
+    generate(ScriptedAheadEngine(), prompts, max_new_tokens=4, sampler=DrawingSampler(), batch_size=3,
+             on_token=lambda i, t: seen_a.append((i, t)))
+    generate(ScriptedEngine(), prompts, max_new_tokens=4, sampler=ArgmaxSampler(), batch_size=3,
+             on_token=lambda i, t: seen_b.append((i, t)))
+    assert seen_a == seen_b
+
+
+@pytest.mark.parametrize("base, sampler", [(ScriptedEngine, ArgmaxSampler), (ScriptedAheadEngine, DrawingSampler)])
+def test_a_failed_step_gives_the_slots_back(base, sampler):
+    class Failing(base):
         def step(self, slots, tokens, want=None):
             if len(self.log) == 3:
                 raise RuntimeError("step failed")
             return super().step(slots, tokens, want)
     eng = Failing()
     with pytest.raises(RuntimeError, match="step failed"):
-        generate(eng, [[1], [7, 8], [3]], max_new_tokens=6, sampler=ArgmaxSampler())
+        generate(eng, [[1], [7, 8], [3]], max_new_tokens=6, sampler=sampler())
     assert sorted(eng.free) == [0, 1, 2] and not eng.lens          # also the one that had ended before
 
 

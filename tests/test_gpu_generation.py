@@ -103,6 +103,56 @@ def test_stop_tokens_end_a_request_early_and_batches_follow_each_other(folders):
     assert stats.batches >= 3 and sum(stats.batch_sizes) == len(prompts) and max(stats.batch_sizes) <= 3
     assert stats.prompt_tokens == sum(map(len, prompts)) and stats.new_tokens == sum(map(len, out))
     assert not engine.cache.slots.held and all(g.pool.n_free == g.n_pages for g in engine.cache.kv_groups)
+    # the loop that reads every token before it queues the next step gives the same, in fewer rows of work
+    behind = GenerationStats()
+    assert generate(engine, prompts, max_new_tokens=12, temperature=0.0, stop_ids=[stop], stats=behind,
+                    ahead=False) == out
+    assert behind.new_tokens == stats.new_tokens and behind.bytes_read < stats.bytes_read
+    assert not engine.cache.slots.held and all(g.pool.n_free == g.n_pages for g in engine.cache.kv_groups)
+
+
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_a_step_from_the_tokens_on_the_device(folders, use_graphs):
+    """step_from takes a step's tokens from the vector of a draw, whole or by rows, and gives the
+    logits of the step that is handed the same tokens as a list."""
+    from yalm_amd import Engine, Model, Sampler, StepError
+    name = "tiny_mistral"
+    model = Model.from_folder(folders[name], dtype=torch.bfloat16, device="cuda:0")
+    by_list = Engine(model, max_tokens=1024, max_batch=4, use_graphs=use_graphs, positions=160)
+    by_device = Engine(model, max_tokens=1024, max_batch=4, use_graphs=use_graphs, positions=160)
+    prompts = list(helpers.random_requests(tiny_configs.ALL[name], [7, 61, 30, 2], seed=5).values())
+    sampler = Sampler(0)
+    a, b = by_list.start(4), by_device.start(4)
+    tokens = sampler.argmax(by_list.step(a, prompts))
+    drawn = sampler.draw(by_device.step(b, prompts), 0.0, [0, 1, 2, 3], [0] * 4)
+    live = [0, 1, 2, 3]                               # the requests that still run
+    for step in range(70):                            # past a page's end and the window
+        rows = None
+        if step in (20, 40):                          # a sequence leaves: the rows of the draw are no longer 0..n-1
+            gone = live[1] if step == 20 else live[0]
+            rows = [k for k, i in enumerate(live) if i != gone]
+            tokens = [tokens[k] for k in rows]
+            live = [i for i in live if i != gone]
+            by_list.release([a[gone]])
+            by_device.release([b[gone]])
+        want = by_list.step([a[i] for i in live], [[t] for t in tokens])
+        got = by_device.step_from([b[i] for i in live], drawn.tokens, rows)
+        assert torch.equal(got, want), step
+        tokens = sampler.argmax(want)
+        drawn = sampler.draw(got, 0.0, live, [step + 1] * len(live))
+        assert drawn.tolist() == tokens
+    a, b = [a[i] for i in live], [b[i] for i in live]
+    fresh = by_device.start(1)
+    with pytest.raises(StepError, match="after its prompt"):
+        by_device.step_from(fresh, drawn.tokens[:1])
+    with pytest.raises(StepError, match="int32"):
+        by_device.step_from(b, drawn.tokens.to(torch.int64))
+    with pytest.raises(StepError, match="one row"):
+        by_device.step_from(b, drawn.tokens, [0, 2])
+    with pytest.raises(StepError, match="one row"):
+        by_device.step_from(b, drawn.tokens[:1])
+    lengths = [by_device.length(s) for s in b]
+    assert lengths == [by_list.length(s) for s in a]                   # a refused step changes nothing
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

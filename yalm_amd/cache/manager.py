@@ -81,6 +81,9 @@ class SlotAllocator:
     def is_held(self, slot):
         return slot in self._held
 
+    def holds_all(self, slots):
+        return self._held.issuperset(slots)
+
     @property
     def n_free(self):
         return len(self._free)
@@ -283,25 +286,32 @@ class CacheManager:
     def extend(self, slots, n_new):
         """Makes room for n_new[i] more tokens of slots[i] and advances the lengths.
         Nothing changes if the pages do not suffice.  Returns the new lengths."""
-        new_lens = []
-        for s, n in zip(slots, n_new):
-            if not self.slots.is_held(s):
-                raise CacheError("slot %r is not held by a live sequence" % (s,))
-            new = self.seq_len[s] + n
-            if not self.unbounded and new > self.max_seq_len:
-                raise CacheFull("a sequence of %d tokens exceeds the longest the cache holds (%d)"
-                                % (new, self.max_seq_len))
-            new_lens.append(new)
+        if not self.slots.holds_all(slots):
+            bad = [s for s in slots if not self.slots.is_held(s)]
+            raise CacheError("slot %r is not held by a live sequence" % (bad[0],))
+        seq_len = self.seq_len
+        old_lens = [seq_len[s] for s in slots]
+        new_lens = [o + n for o, n in zip(old_lens, n_new)]
+        if not self.unbounded and max(new_lens) > self.max_seq_len:
+            raise CacheFull("a sequence of %d tokens exceeds the longest the cache holds (%d)"
+                            % (max(new_lens), self.max_seq_len))
+        # only a sequence that passes a page's end can need a page, in whatever group
+        growing = [i for i, (o, n) in enumerate(zip(old_lens, new_lens)) if (o + PAGE - 1) // PAGE != (n + PAGE - 1) // PAGE]
+        if growing:
+            g_slots = [slots[i] for i in growing]
+            g_old = [old_lens[i] for i in growing]
+            g_new = [new_lens[i] for i in growing]
+            for g in self.kv_groups:
+                need = sum(g.pages_needed(o, n) for o, n in zip(g_old, g_new))
+                if need > g.pool.n_free:
+                    raise CacheFull("the step needs %d more cache pages, %d are free of %d (max_tokens too small)"
+                                    % (need, g.pool.n_free, g.n_pages))
+            for g in self.kv_groups:
+                g.grow(g_slots, g_old, g_new)
         for g in self.kv_groups:
-            need = sum(g.pages_needed(self.seq_len[s], nl) for s, nl in zip(slots, new_lens))
-            if need > g.pool.n_free:
-                raise CacheFull("the step needs %d more cache pages, %d are free of %d (max_tokens too small)"
-                                % (need, g.pool.n_free, g.n_pages))
-        for g in self.kv_groups:
-            g.grow(slots, [self.seq_len[s] for s in slots], new_lens)
             g.flush()
         for s, nl in zip(slots, new_lens):
-            self.seq_len[s] = nl
+            seq_len[s] = nl
         return new_lens
 
     def tokens_held(self):

@@ -31,26 +31,30 @@ class StepError(ValueError):
 
 
 class _BucketBuffers:
-    """The step metadata of one batch-size bucket: a pinned host copy and the device tensor
-    that every graph of the bucket reads."""
+    """The step metadata of one batch-size bucket: the device tensor that every graph of the bucket
+    reads, and two pinned host copies that are filled in turn, so that the host can write a step's
+    metadata while the upload of the step before is still queued."""
 
     def __init__(self, engine, bucket):
         self.bucket = bucket
         n_meta = 6 * bucket + 1
-        self.meta_host = torch.empty(n_meta, dtype=torch.int32, pin_memory=True)
+        self.meta_host = [torch.empty(n_meta, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self.copied = [None, None]    # the event after the last upload of each host copy
+        self.turn = 0
         self.meta = torch.zeros(n_meta, dtype=torch.int32, device=engine.device)
-        self.copied = None            # event after the last upload of meta_host
 
     def host(self):
-        if self.copied is not None:
-            self.copied.synchronize()                    # the last upload has read the pinned buffer
-        return self.meta_host.numpy()
+        """The host copy to fill for the next upload."""
+        if self.copied[self.turn] is not None:
+            self.copied[self.turn].synchronize()         # its last upload has read the pinned buffer
+        return self.meta_host[self.turn].numpy()
 
     def upload(self):
-        self.meta.copy_(self.meta_host, non_blocking=True)
-        if self.copied is None:
-            self.copied = torch.cuda.Event()
-        self.copied.record()
+        self.meta.copy_(self.meta_host[self.turn], non_blocking=True)
+        if self.copied[self.turn] is None:
+            self.copied[self.turn] = torch.cuda.Event()
+        self.copied[self.turn].record()
+        self.turn ^= 1
 
 
 class _DecodeGraph:
@@ -161,22 +165,15 @@ class Engine:
         (src/sampler.cpp:11-25), and the logits are made and used a block of rows at a time: what a
         text's perplexity needs, in memory that does not grow with the text."""
         B = len(slots)
-        if B == 0:
-            raise StepError("a step needs at least one sequence")
+        starts = self._starts(slots)
         if len(tokens) != B or (want is not None and len(want) != B):
             raise StepError("slots, tokens and want must have the same length")
-        if len(set(slots)) != B:
-            raise StepError("a slot occurs twice in the step")
         n_tok = [len(t) for t in tokens]
         if min(n_tok) < 1:
             raise StepError("every sequence of a step brings at least one token")
-        starts = []
-        for s in slots:
-            if not self.cache.slots.is_held(s):
-                raise StepError("slot %r is not held by a live sequence" % (s,))
-            starts.append(self.cache.seq_len[s])
         V = self.model.vocab_size
-        if max(n_tok) == 1:                               # a decode step: one comparison pair for the batch
+        decode = max(n_tok) == 1
+        if decode:                                        # one comparison pair for the batch
             firsts = [t[0] for t in tokens]
             if not (0 <= min(firsts) and max(firsts) < V):
                 bad = [tok for tok in firsts if not 0 <= tok < V]
@@ -187,39 +184,80 @@ class Engine:
                 if ids.ndim != 1 or ids.min() < 0 or ids.max() >= V:
                     bad = [tok for tok in t if not 0 <= tok < V]
                     raise StepError("token id %r is outside the vocabulary of %d" % (bad[0] if bad else t, V))
-        if want is None:
-            want = [[n - 1] for n in n_tok]
-        for w, n in zip(want, n_tok):
-            for j in w:
-                if not 0 <= j < n:
-                    raise StepError("wanted place %r is outside the %d tokens of its sequence" % (j, n))
+        if want is not None:
+            for w, n in zip(want, n_tok):
+                for j in w:
+                    if not 0 <= j < n:
+                        raise StepError("wanted place %r is outside the %d tokens of its sequence" % (j, n))
         if targets is not None:
+            if want is None:
+                want = [[n - 1] for n in n_tok]
             if len(targets) != B or any(len(t) != len(w) for t, w in zip(targets, want)):
                 raise StepError("targets must name one token for every wanted place")
             if any(not 0 <= tok < V for t in targets for tok in t):
                 raise StepError("a target token is outside the vocabulary of %d" % V)
-        if all(s == 0 for s in starts):
+        if max(starts) == 0:
             mode = "prefill"
-        elif all(n == 1 for n in n_tok):
+        elif decode:
             mode = "decode"
         else:
             raise StepError("the sequences of a step either all start at their first token or all go on by one "
                             "token (lengths so far %s, tokens brought %s)" % (starts, n_tok))
-        max_pos = max(s + n for s, n in zip(starts, n_tok)) - 1
-        if max_pos >= self.n_positions:
-            raise StepError("position %d is beyond the %d positions of this engine (max_position_embeddings / "
-                            "max_tokens)" % (max_pos, self.n_positions))
-        try:
-            new_lens = self.cache.extend(slots, n_tok)
-        except CacheError as e:
-            raise StepError(str(e)) from None
+        max_pos = max(starts) if decode else max(s + n for s, n in zip(starts, n_tok)) - 1
+        new_lens = self._extend(slots, n_tok, max_pos)
         if mode == "decode":
-            logits = self._decode(slots, tokens, want, starts, new_lens)
+            logits = self._decode(slots, firsts, want, starts, new_lens)
             if targets is None:
                 return logits
             flat = torch.tensor([tok for t in targets for tok in t], dtype=torch.int32, device=self.device)
             return kernels.token_prob(logits, flat, torch.empty(flat.shape[0], dtype=torch.float32, device=self.device))
+        if want is None:
+            want = [[n - 1] for n in n_tok]
         return self._prefill(slots, tokens, want, n_tok, new_lens, targets)
+
+    def step_from(self, slots, source, rows=None):
+        """A decode step whose tokens lie on the device: slots[i] goes on by the token source[rows[i]]
+        (rows None: source[i]).  source: int32 [n] on the engine's device, as a sampling kernel has
+        written it; the host need not have seen the tokens, so the step can be queued while the step
+        that made them still runs.  Returns the logits of every sequence, float32 [len(slots), vocab],
+        valid until the next step.  A token outside the vocabulary (no sampling kernel makes one)
+        is not reported: its embedding is a row of zeros."""
+        B = len(slots)
+        starts = self._starts(slots)
+        if not (torch.is_tensor(source) and source.is_cuda and source.dtype == torch.int32 and source.dim() == 1
+                and source.is_contiguous()):
+            raise StepError("the tokens of step_from are a contiguous int32 vector on the device")
+        n_src = source.shape[0]
+        if rows is None:
+            rows = range(B)
+        if len(rows) != B or min(rows) < 0 or max(rows) >= n_src:
+            raise StepError("step_from needs one row of its %d tokens for each of the %d sequences" % (n_src, B))
+        if min(starts) < 1:
+            raise StepError("a sequence goes on only after its prompt (lengths so far %s)" % (starts,))
+        new_lens = self._extend(slots, [1] * B, max(starts))
+        return self._decode(slots, None, None, starts, new_lens, source, rows)
+
+    def _starts(self, slots):
+        """The lengths so far of the sequences of a step, after the checks on its slots."""
+        B = len(slots)
+        if B == 0:
+            raise StepError("a step needs at least one sequence")
+        if len(set(slots)) != B:
+            raise StepError("a slot occurs twice in the step")
+        if not self.cache.slots.holds_all(slots):
+            bad = [s for s in slots if not self.cache.slots.is_held(s)]
+            raise StepError("slot %r is not held by a live sequence" % (bad[0],))
+        seq_len = self.cache.seq_len
+        return [seq_len[s] for s in slots]
+
+    def _extend(self, slots, n_tok, max_pos):
+        if max_pos >= self.n_positions:
+            raise StepError("position %d is beyond the %d positions of this engine (max_position_embeddings / "
+                            "max_tokens)" % (max_pos, self.n_positions))
+        try:
+            return self.cache.extend(slots, n_tok)
+        except CacheError as e:
+            raise StepError(str(e)) from None
 
     HEAD_ROWS = 1024        # rows of logits made at a time when only token probabilities are asked for
 
@@ -301,18 +339,20 @@ class Engine:
             pages_bucket *= 2
         return pages_bucket
 
-    def _decode(self, slots, tokens, want, starts, new_lens):
+    def _decode(self, slots, firsts, want, starts, new_lens, source=None, source_rows=None):
+        """firsts: the sequences' tokens, or None: they are source[source_rows] on the device."""
         B = len(slots)
         use_graph = self.use_graphs and self._any_graph
         Bk = self._bucket(B) if use_graph else B
         pages_bucket = self._pages_bucket(max(new_lens))
-        firsts = [t[0] for t in tokens]
-        rows = [i for i, w in enumerate(want) if len(w) > 0]
+        if firsts is None:
+            firsts = 0                                                # a place holder; fed below
         if not use_graph:
             host = np.empty(6 * Bk + 1, dtype=np.int32)
             self._fill_decode_meta(host, Bk, firsts, starts, slots, new_lens)
             meta = self.ws.get("meta", (6 * Bk + 1,), torch.int32)
             meta.copy_(torch.from_numpy(host))
+            self._feed(meta, B, source, source_rows)
             ctx = self._context("decode", self.ws, meta, Bk, Bk, max(starts))
             ctx.pages_bucket = pages_bucket
             ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), [1] * B, list(starts)
@@ -322,6 +362,7 @@ class Engine:
             g = self._graph(Bk, pages_bucket)
             self._fill_decode_meta(g.bufs.host(), Bk, firsts, starts, slots, new_lens)
             g.bufs.upload()
+            self._feed(g.bufs.meta, B, source, source_rows)
             for graph, lo, hi in g.segments:
                 if graph is not None:
                     graph.replay()
@@ -332,11 +373,24 @@ class Engine:
                     ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), [1] * B, list(starts)
                     self.model.run_units(ctx, lo, hi, None, g.logits)
             logits = g.logits
-        if rows == list(range(B)):
+        if want is None:
+            return logits[:B]
+        rows = [i for i, w in enumerate(want) if len(w) > 0]
+        if len(rows) == B:
             return logits[:B]
         if not rows:
             return torch.empty((0, self.model.vocab_size), dtype=torch.float32, device=self.device)
         return logits[torch.tensor(rows, device=self.device)]
+
+    def _feed(self, meta, B, source, source_rows):
+        """Puts the tokens that lie on the device into the step's metadata."""
+        if source is None:
+            return
+        if isinstance(source_rows, range) or list(source_rows) == list(range(B)):
+            meta[0:B].copy_(source[0:B])
+        else:
+            index = torch.tensor(list(source_rows), dtype=torch.int64, device=self.device)
+            torch.index_select(source, 0, index, out=meta[0:B])
 
     # ------------------------------------------------------------------ captured decode steps
     def _graph(self, Bk, pages_bucket):

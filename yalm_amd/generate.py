@@ -2,9 +2,15 @@
 requests): batches of unequal prompts, whole prompts in the first step, then
 one token a step for every sequence that still runs; a sequence ends when it
 samples a stop token (which is kept, src/main.cpp:120-126), has its number of
-new tokens, or fills the context; it leaves the batch at once and its slot and
-pages go back to the cache; when a batch has drained the next one starts, as
-many as there are requests."""
+new tokens, or fills the context; it leaves the batch and its slot and pages go
+back to the cache; when a batch has drained the next one starts, as many as
+there are requests.
+
+The loop runs one step ahead of the host where the engine and the sampler allow
+it: a step's tokens stay on the device and feed the next step from there, and
+the host reads them while that step runs, so the device never waits for the
+host between two steps.  A sequence that samples a stop token is then seen one
+step late: it has taken part in one more step, whose token is dropped."""
 import time
 from dataclasses import dataclass, field
 from typing import List
@@ -61,10 +67,13 @@ def plan_batches(prompt_lens, max_new_tokens, batch_size, max_tokens, n_slots, m
 
 
 def generate(engine, prompts, max_new_tokens=256, temperature=0.0, seed=0, stop_ids=None, batch_size=None,
-             sampler=None, on_token=None, stats=None, request_ids=None):
+             sampler=None, on_token=None, stats=None, request_ids=None, ahead=None):
     """Generates for every prompt (a list of token ids).  Returns the new tokens of
     each request, in the order of the prompts.  stop_ids None means the model's own
-    (config eos); on_token(request index, token) is called for every new token."""
+    (config eos); on_token(request index, token) is called for every new token.
+    ahead: queue each step before the host has read the tokens of the step before
+    (default: if the engine has step_from and the sampler has draw); the tokens are
+    the same either way."""
     from .sampling import Sampler
     sampler = sampler or Sampler(seed)
     stats = stats if stats is not None else GenerationStats()
@@ -74,6 +83,11 @@ def generate(engine, prompts, max_new_tokens=256, temperature=0.0, seed=0, stop_
     ids = list(request_ids) if request_ids is not None else list(range(len(prompts)))
     max_len = engine.n_positions
     step_bytes = getattr(engine, "step_bytes", lambda slots: 0)
+    can_ahead = hasattr(engine, "step_from") and hasattr(sampler, "draw")
+    if ahead is None:
+        ahead = can_ahead
+    elif ahead and not can_ahead:
+        raise ValueError("running a step ahead needs an engine with step_from and a sampler with draw")
     results = [[] for _ in prompts]
     if max_new_tokens <= 0 or not prompts:
         return results
@@ -89,35 +103,62 @@ def generate(engine, prompts, max_new_tokens=256, temperature=0.0, seed=0, stop_
             t0 = time.perf_counter()
             logits = engine.step(slots, [prompts[i] for i in batch])
             stats.bytes_read += step_bytes(slots)
-            tokens = sampler.sample(logits, temperature, [ids[i] for i, _ in live], [0] * len(live))
+            if ahead:
+                drawn = sampler.draw(logits, temperature, [ids[i] for i, _ in live], [0] * len(live))
+                tokens = None
+            else:
+                tokens = sampler.sample(logits, temperature, [ids[i] for i, _ in live], [0] * len(live))
             stats.prefill_seconds += time.perf_counter() - t0
             stats.prompt_tokens += sum(len(prompts[i]) for i in batch)
             stats.batches_first_tokens += len(batch)
             t0 = time.perf_counter()
-            while True:
-                still = []
-                ended = []
-                for (i, slot), tok in zip(live, tokens):
+            rows = list(range(len(live)))                 # where each live sequence's token lies in the last draw
+            while live:
+                # who goes on: by the counts alone when the tokens are not read yet
+                going, going_rows = [], []
+                for (i, slot), r in zip(live, rows):
+                    n = len(results[i]) + 1               # with the token just sampled
+                    if n < max_new_tokens and len(prompts[i]) + n < max_len and (ahead or tokens[r] not in stop):
+                        going.append((i, slot))
+                        going_rows.append(r)
+                next_drawn = next_tokens = None
+                if going:
+                    going_slots = [s for _, s in going]
+                    if ahead:
+                        logits = engine.step_from(going_slots, drawn.tokens, going_rows)
+                    else:
+                        logits = engine.step(going_slots, [[tokens[r]] for r in going_rows])
+                    stats.bytes_read += step_bytes(going_slots)
+                    stats.decode_steps += 1
+                    draw_ids = [ids[i] for i, _ in going]
+                    draw_steps = [len(results[i]) + 1 for i, _ in going]
+                    if ahead:
+                        next_drawn = sampler.draw(logits, temperature, draw_ids, draw_steps)
+                if ahead:
+                    tokens = drawn.tolist()               # lands while the step just queued runs
+                still, still_rows, ended = [], [], []
+                k = 0                                     # walks `going`, which keeps the order of `live`
+                for (i, slot), r in zip(live, rows):
+                    tok = tokens[r]
                     results[i].append(tok)
                     stats.new_tokens += 1
                     if on_token is not None:
                         on_token(i, tok)
-                    full = len(prompts[i]) + len(results[i]) >= max_len        # no room for the token just sampled
-                    if tok in stop or len(results[i]) >= max_new_tokens or full:
-                        ended.append(slot)
+                    if k < len(going) and going[k][0] == i:
+                        if tok in stop:                   # seen a step late: its row of the next draw is dropped
+                            ended.append(slot)
+                        else:
+                            still.append((i, slot))
+                            still_rows.append(k)
+                        k += 1
                     else:
-                        still.append((i, slot))
+                        ended.append(slot)
                 if ended:
                     engine.release(ended)
                     held.difference_update(ended)
-                live = still
-                if not live:
-                    break
-                logits = engine.step([s for _, s in live], [[results[i][-1]] for i, _ in live])
-                stats.bytes_read += step_bytes([s for _, s in live])
-                tokens = sampler.sample(logits, temperature, [ids[i] for i, _ in live],
-                                        [len(results[i]) for i, _ in live])
-                stats.decode_steps += 1
+                if going and not ahead:                   # sampled only now: the tokens just appended are not in it
+                    next_tokens = sampler.sample(logits, temperature, draw_ids, draw_steps)
+                live, rows, drawn, tokens = still, still_rows, next_drawn, next_tokens
         except BaseException:
             engine.release(sorted(held))                  # a failed batch gives back what it still holds
             raise

@@ -25,13 +25,51 @@ def uniform(seed, request_id, step):
     return (h >> 40) / float(1 << 24)
 
 
+class Drawn:
+    """The tokens of one draw: on the device at once (`tokens`, int32 [R]), on the host once the
+    copy that follows the sampling kernel has landed (`tolist()` waits for it, and for nothing
+    that was queued later)."""
+
+    def __init__(self, tokens, host, landed, sampler, turn):
+        self.tokens = tokens
+        self._host = host
+        self._landed = landed
+        self._sampler, self._turn = sampler, turn
+        self._list = None
+
+    def tolist(self):
+        if self._list is None:
+            if self._sampler._turn - self._turn >= Sampler.HOST_BUFFERS:
+                raise RuntimeError("the tokens of a draw are read after %d later draws have taken its host buffer"
+                                   % Sampler.HOST_BUFFERS)
+            self._landed.synchronize()
+            self._list = self._host.tolist()
+        return self._list
+
+
 class Sampler:
+    HOST_BUFFERS = 4          # draws whose host copies may be unread at the same time
+
     def __init__(self, seed=0):
         self.seed = int(seed)
+        self._host = []           # pinned buffers and the events after the copies into them, used in turn
+        self._turn = 0
 
-    def sample(self, logits, temperature, request_ids, steps):
-        """One token for each row of logits [R, vocab] (device, float32).
-        temperature 0 is argmax.  Returns a list of ints."""
+    def _host_buffer(self, R):
+        if len(self._host) < self.HOST_BUFFERS:
+            self._host.append([torch.empty(max(R, 64), dtype=torch.int32, pin_memory=True), torch.cuda.Event()])
+            entry = self._host[-1]
+        else:
+            entry = self._host[self._turn % self.HOST_BUFFERS]
+            entry[1].synchronize()
+            if entry[0].shape[0] < R:
+                entry[0] = torch.empty(R, dtype=torch.int32, pin_memory=True)
+        return entry
+
+    def draw(self, logits, temperature, request_ids, steps):
+        """One token for each row of logits [R, vocab] (device, float32); temperature 0 is argmax.
+        Nothing waits for the device here: the tokens can feed the next step from where they lie
+        while the host reads them a step later."""
         R = logits.shape[0]
         out = torch.empty(R, dtype=torch.int32, device=logits.device)
         if temperature == 0.0:
@@ -39,7 +77,15 @@ class Sampler:
         else:
             u = torch.tensor([uniform(self.seed, r, s) for r, s in zip(request_ids, steps)], dtype=torch.float32)
             kernels.sample(logits, u.to(logits.device), float(temperature), out)
-        return out.tolist()
+        host, landed = self._host_buffer(R)
+        host[:R].copy_(out, non_blocking=True)
+        landed.record()
+        self._turn += 1
+        return Drawn(out, host[:R], landed, self, self._turn)
+
+    def sample(self, logits, temperature, request_ids, steps):
+        """As draw, but returns the tokens as a list of ints."""
+        return self.draw(logits, temperature, request_ids, steps).tolist()
 
     def argmax(self, logits):
         out = torch.empty(logits.shape[0], dtype=torch.int32, device=logits.device)
