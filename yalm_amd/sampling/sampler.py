@@ -55,15 +55,19 @@ class Sampler:
         self._host = []           # pinned buffers and the events after the copies into them, used in turn
         self._turn = 0
 
-    def _host_buffer(self, R):
+    def _host_buffers(self, R):
+        """The next pinned pair in turn: int32 for the tokens on their way back, float32 for the
+        uniform numbers on their way out, and the event behind the draw that used them last."""
         if len(self._host) < self.HOST_BUFFERS:
-            self._host.append([torch.empty(max(R, 64), dtype=torch.int32, pin_memory=True), torch.cuda.Event()])
-            entry = self._host[-1]
-        else:
-            entry = self._host[self._turn % self.HOST_BUFFERS]
-            entry[1].synchronize()
-            if entry[0].shape[0] < R:
-                entry[0] = torch.empty(R, dtype=torch.int32, pin_memory=True)
+            n = max(R, 64)
+            self._host.append([torch.empty(n, dtype=torch.int32, pin_memory=True),
+                               torch.empty(n, dtype=torch.float32, pin_memory=True), torch.cuda.Event()])
+            return self._host[-1]
+        entry = self._host[self._turn % self.HOST_BUFFERS]
+        entry[2].synchronize()
+        if entry[0].shape[0] < R:
+            entry[0] = torch.empty(R, dtype=torch.int32, pin_memory=True)
+            entry[1] = torch.empty(R, dtype=torch.float32, pin_memory=True)
         return entry
 
     def draw(self, logits, temperature, request_ids, steps):
@@ -72,12 +76,15 @@ class Sampler:
         while the host reads them a step later."""
         R = logits.shape[0]
         out = torch.empty(R, dtype=torch.int32, device=logits.device)
+        host, host_u, landed = self._host_buffers(R)
         if temperature == 0.0:
             kernels.argmax(logits, out)
         else:
-            u = torch.tensor([uniform(self.seed, r, s) for r, s in zip(request_ids, steps)], dtype=torch.float32)
-            kernels.sample(logits, u.to(logits.device), float(temperature), out)
-        host, landed = self._host_buffer(R)
+            host_u[:R] = torch.tensor([uniform(self.seed, r, s) for r, s in zip(request_ids, steps)],
+                                      dtype=torch.float32)
+            u = torch.empty(R, dtype=torch.float32, device=logits.device)
+            u.copy_(host_u[:R], non_blocking=True)          # from pinned memory: the host does not wait for the queue
+            kernels.sample(logits, u, float(temperature), out)
         host[:R].copy_(out, non_blocking=True)
         landed.record()
         self._turn += 1
