@@ -452,6 +452,21 @@ def test_rope_kv_write_tiles(n_heads, n_kv, hd, rd, lens, ring, dtype):
                        (vp0, vp1, "v pages")):
         assert torch.equal(a, b), what
     assert q0.abs().sum() > 0 and kp0.abs().sum() > 0
+    # the K slices of a product instead of the product: added in order, as the per-token kernel adds them
+    parts = torch.stack([rnd((T, Q + 2 * KV), 30 + s).to(DEV) for s in range(3)]).reshape(-1)
+    kp2, vp2, ks2, vs2, q2 = buffers()
+    k.rope_kv_write(parts, q2, ks2, vs2, i32(tile0), kp2, vp2, bt.to(DEV), ring, i32(seq), i32(pos), i32(slots),
+                    i32(lens), table, n_heads, n_kv, hd, rd, slices=3)
+    kp3, vp3, ks3, vs3, q3 = buffers()
+    assert k.rope_kv_write_tiles(parts, q3, ks3, vs3, i32(cu), i32(tile0), kp3, vp3, bt.to(DEV), ring, i32(slots),
+                                 i32(lens), table, n_heads, n_kv, hd, rd, slices=3)
+    for a, b, what in ((q2, q3, "q"), (ks2, ks3, "staged k"), (vs2, vs3, "staged v"), (kp2, kp3, "k pages"),
+                       (vp2, vp3, "v pages")):
+        assert torch.equal(a, b), what + " from slices"
+    assert not torch.equal(q2, q0)
+    with pytest.raises(ValueError):
+        k.rope_kv_write_tiles(parts[:2 * T * (Q + 2 * KV)], q3, ks3, vs3, i32(cu), i32(tile0), kp3, vp3, bt.to(DEV),
+                              ring, i32(slots), i32(lens), table, n_heads, n_kv, hd, rd, slices=3)
 
 
 def test_rope_kv_write_ring_keeps_the_last_pages_only():

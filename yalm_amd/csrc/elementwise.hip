@@ -1,4 +1,6 @@
 // Embedding gather, RMSNorm and the fused rotation + cache write.
+#include <type_traits>
+
 #include "common.h"
 #include "yalm_hip.h"
 
@@ -254,13 +256,60 @@ __device__ __forceinline__ void store_pair(bf16* dst, float a, float b) {
   *reinterpret_cast<bf16x2*>(dst) = v;
 }
 
-template <typename T>
+// 2 * PP consecutive values
+template <int PP>
+__device__ __forceinline__ void store_values(float* dst, const float* v) {
+  if constexpr (PP == 2) *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+  else store_pair(dst, v[0], v[1]);
+}
+template <int PP>
+__device__ __forceinline__ void store_values(bf16* dst, const float* v) {
+  if constexpr (PP == 2) {
+    typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+    bf16x4 o = {static_cast<bf16>(v[0]), static_cast<bf16>(v[1]), static_cast<bf16>(v[2]), static_cast<bf16>(v[3])};
+    *reinterpret_cast<bf16x4*>(dst) = o;
+  } else {
+    store_pair(dst, v[0], v[1]);
+  }
+}
+
+// 2 * PP consecutive floats at `at`, or the sum of the `slices` planes that hold them as the K slices of a
+// product, added in order (four loads asked for before the first is added: a slice more costs no trip to
+// memory of its own)
+template <int PP>
+__device__ __forceinline__ void load_slices(const float* at, int slices, long plane, float* v) {
+  typedef typename std::conditional<PP == 2, float4, float2>::type V;
+  V x = *reinterpret_cast<const V*>(at);
+  float* xs = reinterpret_cast<float*>(&x);
+  for (int s = 1; s < slices; s += 4) {
+    V y[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (s + u < slices) {
+        y[u] = *reinterpret_cast<const V*>(at + (size_t)(s + u) * plane);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 2 * PP; ++c) reinterpret_cast<float*>(&y[u])[c] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int c = 0; c < 2 * PP; ++c) xs[c] += reinterpret_cast<const float*>(&y[u])[c];
+  }
+#pragma unroll
+  for (int c = 0; c < 2 * PP; ++c) v[c] = xs[c];
+}
+
+// PP: pairs a thread takes at a time (2: 16-byte loads; head sizes that are multiples of 4)
+template <typename T, int PP>
 __global__ __launch_bounds__(256) void rope_kv_tiles_kernel(
     const float* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_stage, T* __restrict__ v_stage,
     const int* __restrict__ cu_seqlens, const int* __restrict__ seq_tile0, T* __restrict__ k_pages,
     T* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride, int ring_pages,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_len, const float2* __restrict__ cos_sin,
-    int n_positions, int B, int n_heads, int n_kv_heads, int hd, int rotary_dim, int n_pages, int page_layout) {
+    int n_positions, int B, int n_heads, int n_kv_heads, int hd, int rotary_dim, int n_pages, int page_layout,
+    int slices, long plane) {
   extern __shared__ __attribute__((aligned(16))) unsigned char vt_raw[];
   T* vt = reinterpret_cast<T*>(vt_raw);           // [hd][VT_ROW]
   const int gt = blockIdx.x, job = blockIdx.y, tid = threadIdx.x;
@@ -282,21 +331,28 @@ __global__ __launch_bounds__(256) void rope_kv_tiles_kernel(
   const int half_rot = rotary_dim / 2, pairs = hd / 2;
   const float* src0 = qkv + (size_t)(start + p0) * W;
 
-  auto rotated = [&](const float* row, int pos, int p) {
-    float2 x = *reinterpret_cast<const float2*>(row + 2 * p);
-    if (cos_sin != nullptr && p < half_rot && pos < n_positions) {
-      const float2 c = cos_sin[(size_t)pos * half_rot + p];
-      x = make_float2(x.x * c.x - x.y * c.y, x.x * c.y + x.y * c.x);
+  // qkv may come as the K slices of its product ([slices] planes of `plane` floats), added here in order
+  auto rotate = [&](float* v, int pos, int p) {   // the pairs p .. p + PP - 1 of a head at position pos
+#pragma unroll
+    for (int u = 0; u < PP; ++u) {
+      if (cos_sin != nullptr && p + u < half_rot && pos < n_positions) {
+        const float2 c = cos_sin[(size_t)pos * half_rot + p + u];
+        const float a = v[2 * u], b2 = v[2 * u + 1];
+        v[2 * u] = a * c.x - b2 * c.y;
+        v[2 * u + 1] = a * c.y + b2 * c.x;
+      }
     }
-    return x;
   };
+  const int groups = pairs / PP;
 
   if (job >= n_kv_heads) {                        // a query head
     const int h = job - n_kv_heads;
-    for (int e = tid; e < rows * pairs; e += 256) {
-      const int r = e / pairs, p = e % pairs;
-      const float2 y = rotated(src0 + (size_t)r * W + h * hd, p0 + r, p);
-      store_pair(q_out + (size_t)(start + p0 + r) * Q + h * hd + 2 * p, y.x, y.y);
+    for (int e = tid; e < rows * groups; e += 256) {
+      const int r = e / groups, p = (e % groups) * PP;
+      float v[2 * PP];
+      load_slices<PP>(src0 + (size_t)r * W + h * hd + 2 * p, slices, plane, v);
+      rotate(v, p0 + r, p);
+      store_values<PP>(q_out + (size_t)(start + p0 + r) * Q + h * hd + 2 * p, v);
     }
     return;
   }
@@ -317,14 +373,16 @@ __global__ __launch_bounds__(256) void rope_kv_tiles_kernel(
       }
     }
   }
-  for (int e = tid; e < rows * pairs; e += 256) {
-    const int r = e / pairs, p = e % pairs;
-    const float2 y = rotated(src0 + (size_t)r * W + Q + g * hd, p0 + r, p);
-    store_pair(kst + r * hd + 2 * p, y.x, y.y);
-    if (kpage) store_pair(kpage + page_k_offset(page_layout, r, 2 * p, hd), y.x, y.y);
-    const float2 v = *reinterpret_cast<const float2*>(src0 + (size_t)r * W + Q + KV + g * hd + 2 * p);
-    vt[(2 * p) * VT_ROW + r] = from_f32<T>(v.x);
-    vt[(2 * p + 1) * VT_ROW + r] = from_f32<T>(v.y);
+  for (int e = tid; e < rows * groups; e += 256) {
+    const int r = e / groups, p = (e % groups) * PP;
+    float v[2 * PP];
+    load_slices<PP>(src0 + (size_t)r * W + Q + g * hd + 2 * p, slices, plane, v);
+    rotate(v, p0 + r, p);
+    store_values<PP>(kst + r * hd + 2 * p, v);
+    if (kpage) store_values<PP>(kpage + page_k_offset(page_layout, r, 2 * p, hd), v);   // 4 elements from a multiple of 4 lie together in either layout
+    load_slices<PP>(src0 + (size_t)r * W + Q + KV + g * hd + 2 * p, slices, plane, v);
+#pragma unroll
+    for (int c = 0; c < 2 * PP; ++c) vt[(2 * p + c) * VT_ROW + r] = from_f32<T>(v[c]);
   }
   __syncthreads();
   // values, transposed: element i of the head is a row of 64 positions; positions behind the prompt's end get zeros
@@ -345,9 +403,11 @@ extern "C" int yalm_rope_kv_write_tiles(const float* qkv, void* q_out, void* k_s
                                         const int* block_table, int table_stride, int ring_pages,
                                         const int* seq_slot, const int* seq_len, const float* cos_sin,
                                         int n_positions, int T, int B, int n_tiles, int n_heads, int n_kv_heads,
-                                        int head_dim, int rotary_dim, int n_pages, int page_layout, int dtype,
-                                        hipStream_t stream) {
+                                        int head_dim, int rotary_dim, int n_pages, int page_layout, int slices,
+                                        int dtype, hipStream_t stream) {
   if (T <= 0 || B <= 0 || n_tiles <= 0) return YALM_OK;
+  if (slices < 1) return YALM_ERR_ARG;
+  const long plane = (long)T * (n_heads + 2 * n_kv_heads) * head_dim;
   if (head_dim <= 0 || (head_dim & 1) || rotary_dim < 0 || (rotary_dim & 1) || rotary_dim > head_dim ||
       n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || k_stage == nullptr || v_stage == nullptr ||
       cu_seqlens == nullptr || seq_tile0 == nullptr || n_heads + n_kv_heads > 65535 ||
@@ -357,18 +417,29 @@ extern "C" int yalm_rope_kv_write_tiles(const float* qkv, void* q_out, void* k_s
   const size_t lds = (size_t)head_dim * VT_ROW * esize;
   if (lds > 64 * 1024) return YALM_ERR_ARG;
   dim3 grid(n_tiles, n_kv_heads + n_heads);
+  // two pairs a thread where every address it touches is a multiple of 16 bytes (8 for bfloat16 stores)
+  const bool wide = head_dim % 4 == 0 && ((uintptr_t)qkv & 15) == 0 && ((uintptr_t)q_out & 15) == 0 &&
+                    ((uintptr_t)k_stage & 15) == 0 && ((uintptr_t)k_pages & 15) == 0;
+#define YALM_ROPE_TILES(T_)                                                                                         \
+  do {                                                                                                              \
+    if (wide)                                                                                                       \
+      rope_kv_tiles_kernel<T_, 2><<<grid, 256, lds, stream>>>(                                                      \
+          qkv, (T_*)q_out, (T_*)k_stage, (T_*)v_stage, cu_seqlens, seq_tile0, (T_*)k_pages, (T_*)v_pages,           \
+          block_table, table_stride, ring_pages, seq_slot, seq_len, (const float2*)cos_sin, n_positions, B,         \
+          n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, page_layout, slices, plane);                          \
+    else                                                                                                            \
+      rope_kv_tiles_kernel<T_, 1><<<grid, 256, lds, stream>>>(                                                      \
+          qkv, (T_*)q_out, (T_*)k_stage, (T_*)v_stage, cu_seqlens, seq_tile0, (T_*)k_pages, (T_*)v_pages,           \
+          block_table, table_stride, ring_pages, seq_slot, seq_len, (const float2*)cos_sin, n_positions, B,         \
+          n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, page_layout, slices, plane);                          \
+  } while (0)
   if (dtype == YALM_F32)
-    rope_kv_tiles_kernel<float><<<grid, 256, lds, stream>>>(
-        qkv, (float*)q_out, (float*)k_stage, (float*)v_stage, cu_seqlens, seq_tile0, (float*)k_pages, (float*)v_pages,
-        block_table, table_stride, ring_pages, seq_slot, seq_len, (const float2*)cos_sin, n_positions, B, n_heads,
-        n_kv_heads, head_dim, rotary_dim, n_pages, page_layout);
+    YALM_ROPE_TILES(float);
   else if (dtype == YALM_BF16)
-    rope_kv_tiles_kernel<bf16><<<grid, 256, lds, stream>>>(
-        qkv, (bf16*)q_out, (bf16*)k_stage, (bf16*)v_stage, cu_seqlens, seq_tile0, (bf16*)k_pages, (bf16*)v_pages,
-        block_table, table_stride, ring_pages, seq_slot, seq_len, (const float2*)cos_sin, n_positions, B, n_heads,
-        n_kv_heads, head_dim, rotary_dim, n_pages, page_layout);
+    YALM_ROPE_TILES(bf16);
   else
     return YALM_ERR_DTYPE;
+#undef YALM_ROPE_TILES
   return launch_status();
 }
 

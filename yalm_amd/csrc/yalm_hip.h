@@ -107,13 +107,13 @@ int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_stage, void* v_sta
 
 // The same for a step of whole prompts (every sequence from position 0; cu_seqlens [B + 1] token offsets,
 // n_tiles = seq_tile0[B]): whole page-shaped tiles at a time.  Needs a staging area; refuses
-// (YALM_ERR_ARG) head sizes whose transposed tile does not fit 64 KB of LDS.
+// (YALM_ERR_ARG) head sizes whose transposed tile does not fit 64 KB of LDS.  slices as above.
 int yalm_rope_kv_write_tiles(const float* qkv, void* q_out, void* k_stage, void* v_stage, const int* cu_seqlens,
                              const int* seq_tile0, void* k_pages, void* v_pages, const int* block_table,
                              int table_stride, int ring_pages, const int* seq_slot, const int* seq_len,
                              const float* cos_sin, int n_positions, int T, int B, int n_tiles, int n_heads,
-                             int n_kv_heads, int head_dim, int rotary_dim, int n_pages, int page_layout, int dtype,
-                             hipStream_t stream);
+                             int n_kv_heads, int head_dim, int rotary_dim, int n_pages, int page_layout, int slices,
+                             int dtype, hipStream_t stream);
 
 // Causal attention of a step's tokens over the same step's keys (sequences that
 // start at position 0), packed without padding.  window 0 = all keys.

@@ -410,19 +410,25 @@ def rope_kv_write(qkv, q_out, k_stage, v_stage, seq_tile0, k_pages, v_pages, blo
 
 
 def rope_kv_write_tiles(qkv, q_out, k_stage, v_stage, cu_seqlens, seq_tile0, k_pages, v_pages, block_table, ring_pages,
-                        seq_slot, seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim, layout=None):
+                        seq_slot, seq_len, cos_sin, n_heads, n_kv_heads, head_dim, rotary_dim, slices=1, layout=None):
     """rope_kv_write for a step of whole prompts (every sequence from position 0), a page-shaped
     tile of 64 positions at a time.  False if the kernel refuses the head size (the caller then
-    uses rope_kv_write)."""
+    uses rope_kv_write).  slices as in rope_kv_write."""
     _check_heads(n_heads, n_kv_heads, head_dim)
-    T = qkv.shape[0]
+    T = q_out.shape[0]
     Q, KV = n_heads * head_dim, n_kv_heads * head_dim
     dt = q_out.dtype
     if head_dim * (PAGE + 8) * dt.itemsize > 64 * 1024:
         return False
     B = seq_slot.shape[0]
     n_tiles = k_stage.shape[0]
-    p_qkv = _need(qkv, "qkv", torch.float32, (T, Q + 2 * KV))
+    if slices == 1 and qkv.dim() == 2:
+        p_qkv = _need(qkv, "qkv", torch.float32, (T, Q + 2 * KV))
+    else:
+        p_qkv = _need(qkv, "qkv", torch.float32, (None,))
+        if slices < 1 or qkv.numel() < slices * T * (Q + 2 * KV):
+            raise ValueError("qkv holds %d floats, %d slices of %d rows need %d"
+                             % (qkv.numel(), slices, T, slices * T * (Q + 2 * KV)))
     p_q = _need(q_out, "q_out", dt, (T, Q))
     p_ks = _need(k_stage, "k_stage", dt, (n_tiles, n_kv_heads, PAGE, head_dim))
     p_vs = _need(v_stage, "v_stage", dt, (n_tiles, n_kv_heads, head_dim, PAGE))
@@ -451,8 +457,8 @@ def rope_kv_write_tiles(qkv, q_out, k_stage, v_stage, cu_seqlens, seq_tile0, k_p
         rotary_dim = 0
     library.check(library.lib().yalm_rope_kv_write_tiles(
         p_qkv, p_q, p_ks, p_vs, p_cu, p_t0, p_kp, p_vp, p_bt, stride, max(ring_pages, 1), p_ss, p_sl, p_cs, n_pos, T, B,
-        n_tiles, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, _layout(layout, head_dim), dtype_code(dt),
-        _stream()), "rope_kv_write_tiles")
+        n_tiles, n_heads, n_kv_heads, head_dim, rotary_dim, n_pages, _layout(layout, head_dim), int(slices),
+        dtype_code(dt), _stream()), "rope_kv_write_tiles")
     return True
 
 

@@ -29,7 +29,7 @@ _SIGNATURES = {
     "yalm_gemm_partial": (_I, [_P, _P, _P, ctypes.c_long, _I, _I, _I, _P, _P]),
     "yalm_gemm_bf16_dma_workspace": (ctypes.c_long, [_I, _I, _I]),
     "yalm_gemm_add_norm": (_I, [_P, _P, _P, _P, ctypes.c_long, _I, _I, _I, _P, _F, _P, _P]),
-    "yalm_rope_kv_write_tiles": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
+    "yalm_rope_kv_write_tiles": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_prefill": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_workspace": (ctypes.c_long, [_I, _I, _I, _I]),
@@ -45,7 +45,7 @@ _SIGNATURES = {
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
 }
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 
 class KernelError(RuntimeError):

@@ -100,15 +100,27 @@ class GQAttention(Part):
         return max(1, min(max_pages, TARGET_WORKGROUPS // max(1, B * self.n_heads)))
 
     def fuses_norm(self, norm, x, ctx):
-        if not hasattr(norm, "fused") or ctx.mode != "decode" or self.head_dim % 16:
+        if not hasattr(norm, "fused") or self.head_dim % 16:
             return False
         T = x.shape[0]
+        if ctx.mode == "prefill":             # takes the norm's output where the product before has left it
+            return kernels.can_add_norm(T, self.dim, self.wo.dtype)
+        if ctx.mode != "decode":
+            return False
         return kernels.can_chain(T, self.dim, self.wo.dtype) or kernels.can_add_norm(T, self.dim, self.wo.dtype)
 
     def forward_prenorm(self, x, norm, ctx, line, writes_cache=True, emit_for=None):
         """A decode step from the residual stream: norm, q/k/v, rotation and cache write in
         one kernel, attention over the cache, output projection added to x (which may
         prepare the activations of the next norm, emit_for)."""
+        if ctx.mode == "prefill":                 # whole prompts: the norm, unless its output is ready, then the plain way
+            src = ctx.normed.pop(id(norm), None)
+            if src is not None and src[1] is None:
+                h = src[0]
+            else:
+                h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
+                norm.forward(x, h, ctx)
+            return self.forward(h, x, ctx, line, writes_cache, emit_for=emit_for)
         if not writes_cache:                      # a reader of another entry's line: the plain way
             ctx.normed.pop(id(norm), None)
             h = ctx.ws.get("block.h", (x.shape[0], self.dim), ctx.act_dtype)
@@ -179,7 +191,7 @@ class GQAttention(Part):
         kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o, partial,
                             self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits, sinks=sinks)
 
-    def forward(self, h, x, ctx, line, writes_cache=True):
+    def forward(self, h, x, ctx, line, writes_cache=True, emit_for=None):
         T = h.shape[0]
         act = h.dtype
         ws = ctx.ws
@@ -187,12 +199,19 @@ class GQAttention(Part):
         if pos.table is not None and ctx.max_position >= pos.n_positions:
             raise ValueError("position %d is beyond the %d positions the rotation table holds"
                              % (ctx.max_position, pos.n_positions))
-        qkv = ws.get("attn.qkv", (T, self.q_dim + 2 * self.kv_dim), torch.float32)
-        self._gemm(ctx, h, self.wqkv, qkv, kernels.EPI_STORE_F32)
+        prefill = ctx.mode == "prefill"
+        n_qkv = self.q_dim + 2 * self.kv_dim
+        slices = 1
+        if prefill and kernels.can_gemm_partial(T, self.dim, act):
+            # the product's K slices (a short prompt's has some) go to the rotation kernel as they are, which adds them
+            qkv = ws.get("gemm.partial", (kernels.fused_workspace_floats(T, n_qkv, self.dim),), torch.float32)
+            slices = kernels.gemm_partial(h, self.wqkv, qkv)
+        else:
+            qkv = ws.get("attn.qkv", (T, n_qkv), torch.float32)
+            self._gemm(ctx, h, self.wqkv, qkv, kernels.EPI_STORE_F32)
         q = ws.get("attn.q", (T, self.q_dim), act)
         group = ctx.cache.group_of(line)
         k_pages, v_pages = group.line_pages(line)
-        prefill = ctx.mode == "prefill"
         if prefill:
             # the step's own keys and values in page format; a line that later entries read
             # keeps them for those entries
@@ -204,15 +223,16 @@ class GQAttention(Part):
         if writes_cache:
             done = prefill and kernels.rope_kv_write_tiles(
                 qkv, q, kst, vst, ctx.cu_seqlens, ctx.seq_tile0, k_pages, v_pages, group.table, group.ring_pages,
-                ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads, self.head_dim, pos.rotary_dim)
+                ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads, self.head_dim, pos.rotary_dim,
+                slices=slices)
             if not done:
                 kernels.rope_kv_write(qkv, q, kst, vst, ctx.seq_tile0, k_pages, v_pages, group.table,
                                       group.ring_pages, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table,
-                                      self.n_heads, self.n_kv_heads, self.head_dim, pos.rotary_dim)
+                                      self.n_heads, self.n_kv_heads, self.head_dim, pos.rotary_dim, slices=slices)
         else:
             kernels.rope_kv_write(qkv, q, None, None, None, None, None, None, 0, ctx.tok_seq, ctx.tok_pos,
                                   ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads, self.head_dim,
-                                  pos.rotary_dim)
+                                  pos.rotary_dim, slices=slices)
         o = ws.get("attn.o", (T, self.q_dim), act)
         if prefill:
             lse = ws.get("attn.lse", (T, self.n_heads), torch.float32) if self.sinks else None
@@ -227,4 +247,10 @@ class GQAttention(Part):
                                       self.n_heads, pos.rotary_dim, self.window)
         else:
             self._decode_attention(q, o, ctx, group, line, k_pages, v_pages, writes_cache)
-        self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)
+        ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.q_dim) if prefill else None
+        if ready is not None:                     # the product splits K: its slices are added with the next norm behind
+            nw2, eps2, h2, ws2 = ready
+            kernels.gemm_add_norm(o, self.wo, x, nw2, eps2, h2, ws2)
+            ctx.normed[id(emit_for)] = (h2, None, None)
+        else:
+            self._gemm(ctx, o, self.wo, x, kernels.EPI_ADD_F32)

@@ -126,10 +126,12 @@ class Part:
         """Operands for a residual-add GEMM [T, K] x [width, K] of more than 16 rows that also does the norm
         `emit_for` (the next one on the residual stream) and leaves its activations ready, or None."""
         from ..ops import kernels
-        if emit_for is None or not hasattr(emit_for, "fused") or ctx.mode != "decode":
+        if emit_for is None or not hasattr(emit_for, "fused") or ctx.mode not in ("decode", "prefill"):
             return None
         if not kernels.can_add_norm(T, K, ctx.act_dtype):
             return None
+        if ctx.mode == "prefill" and kernels.gemm_workspace_floats(T, width, K) == 0:
+            return None      # a prompt's product that does not split K adds to the residual stream itself: cheaper
         import torch
         nw, eps = emit_for.fused()
         h = ctx.ws.get("chain.h", (T, width), torch.bfloat16)          # read by the consumer before the next is written

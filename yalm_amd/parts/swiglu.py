@@ -50,9 +50,11 @@ class SwiGLU(Part):
         return 3 * self.hidden * self.dim * self.w_down.element_size()
 
     def fuses_norm(self, norm, x, ctx):
-        if not hasattr(norm, "fused") or ctx.mode != "decode":
+        if not hasattr(norm, "fused") or ctx.mode not in ("decode", "prefill"):
             return False
         T = x.shape[0]
+        if ctx.mode == "prefill":             # takes the norm's output where the product before has left it
+            return kernels.can_add_norm(T, self.dim, self.w_down.dtype)
         return kernels.can_chain(T, self.dim, self.w_down.dtype) or kernels.can_add_norm(T, self.dim, self.w_down.dtype)
 
     def forward_prenorm(self, x, norm, ctx, emit_for=None):
