@@ -1257,7 +1257,7 @@ def test_gemm_of_more_than_64_rows_splits_k(M, N, Kd):
         acc = res.to(DEV).clone()
         k.gemm(a.to(DEV), w.to(DEV), acc, k.EPI_ADD_F32, workspace=ws)
         close(acc, want + res.double(), torch.float32, "add, %d floats" % floats)
-    assert k.gemm_workspace_floats(2048, 4096, 4096) == 0       # enough tiles: no slices
+    assert k.gemm_workspace_floats(8192, 4096, 4096) == 0       # enough tiles: no slices
 
 
 @pytest.mark.parametrize("M,H,D", [(100, 1000, 4096), (128, 176, 2048), (65, 3000, 1024)])

@@ -14,7 +14,7 @@
 #include "yalm_hip.h"
 
 int yalm_gemm_bf16_dma_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N,
-                               int K, int* slices_out, hipStream_t stream);   // gemm_dma.hip
+                               int K, int* slices_out, int residual, hipStream_t stream);   // gemm_dma.hip
 
 namespace {
 
@@ -560,7 +560,7 @@ int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace
 extern "C" int yalm_gemm_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N,
                                  int K, int* slices, hipStream_t stream) {
   if (M > 128 || (M > 64 && K % 64 != 0))
-    return yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, slices, stream);
+    return yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, slices, 0, stream);
   if (M <= 16 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || slices == nullptr)
     return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
@@ -585,7 +585,7 @@ extern "C" int yalm_gemm_add_norm(const void* A, const void* W, float* C, float*
   if (norm_w == nullptr || h_out == nullptr) return YALM_ERR_ARG;
   if (M > 128 || (M > 64 && K % 64 != 0)) {        // the tiled kernel's slices, then the same reduction
     int slices = 0;
-    int rc = yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, &slices, stream);
+    int rc = yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, &slices, 1, stream);
     if (rc != YALM_OK) return rc;
     reduce_add_norm_kernel<<<M, RN_THREADS, 0, stream>>>(workspace, C, norm_w, eps, (bf16*)h_out, M, N, slices);
     return launch_status();

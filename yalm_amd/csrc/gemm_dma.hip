@@ -743,24 +743,31 @@ double ring_time(long tiles, int iters, int tn) {
 }
 
 // Splits K where the tiles alone leave most CUs without work (short prompts, narrow outputs): a second kernel then
-// adds the slices (about (slices + 2) * M * N * 4 bytes at 4 TB/s).
-RingPlan ring_plan(int M, int N, int K, long workspace_floats) {
+// adds the slices (about (slices + 2) * M * N * 4 bytes at 4 TB/s).  residual: the product is added to the float32
+// residual stream.  Unsplit, the tiles read and write that stream in their epilogue, M * N * 8 bytes that no loop
+// hides (2,048 x 4,096 x 4,096 on tiles of 128 columns: 87 us, the same tiles with the gated epilogue 65); split,
+// the kernel that adds the slices also does the norm behind them, whose own pass (M * N * 6 bytes) is saved.
+RingPlan ring_plan(int M, int N, int K, long workspace_floats, bool residual) {
   const int mt = ceil_div(M, 256), nk = K / TK;
   RingPlan best;
   double best_t = 1e30;
+  const double in_epilogue = residual ? (double)M * N * 8.0 / 4.0e6 : 0.0;
+  const double norm_saved = residual ? (double)M * N * 6.0 / 5.0e6 : 0.0;
   for (int tn : {256, 192, 128}) {
     const long tiles = (long)mt * ceil_div(N, tn);
     for (int s = 1; s <= 8; s *= 2) {
       if (s > 1 && (tiles * s > 256 || nk / s < 8 || (long)s * M * N > workspace_floats)) break;
       const int iters = ceil_div(nk, s);
-      const double t = ring_time(tiles * s, iters, tn) + (s > 1 ? 3.0 + (double)(s + 2) * M * N * 4.0 / 4.0e6 : 0.0);
+      const double t = ring_time(tiles * s, iters, tn) +
+                       (s > 1 ? 3.0 + (double)(s + 2) * M * N * 4.0 / 4.0e6 - norm_saved : in_epilogue);
       if (t < best_t) { best_t = t; best.tn = tn; best.slices = s; best.nt_main = 0; }
     }
   }
   const int nt = ceil_div(N, 256);
   const int nt_main = (int)(((long)mt * nt / 256) * 256 / mt);
   if (nt_main > 0 && nt_main < nt) {
-    const double t = ring_time((long)mt * nt_main, nk, 256) + ring_time((long)mt * (ceil_div(N, 128) - 2 * nt_main), nk, 128);
+    const double t = ring_time((long)mt * nt_main, nk, 256) +
+                     ring_time((long)mt * (ceil_div(N, 128) - 2 * nt_main), nk, 128) + in_epilogue;
     if (t < best_t) { best_t = t; best.tn = 256; best.slices = 1; best.nt_main = nt_main; }
   }
   return best;
@@ -770,9 +777,9 @@ RingPlan ring_plan(int M, int N, int K, long workspace_floats) {
 // stay there unadded (one slice: the product itself), *slices_out says how many
 template <int EPI>
 int launch_ring_shape(const bf16* A, const bf16* W, void* C, float* partial, long partial_floats, int M, int N, int K,
-                      int H, hipStream_t stream, int* slices_out = nullptr) {
+                      int H, hipStream_t stream, int* slices_out = nullptr, bool residual = EPI == 2) {
   const bool keep = slices_out != nullptr;
-  const RingPlan p = ring_plan(M, N, K, partial != nullptr ? partial_floats : 0);
+  const RingPlan p = ring_plan(M, N, K, partial != nullptr ? partial_floats : 0, residual);
   if (p.nt_main > 0) {
     if (keep) *slices_out = 1;
     int rc = launch_ring<EPI, 256, 4>(A, W, C, M, N, K, H, stream, 0, p.nt_main);
@@ -807,11 +814,12 @@ int launch(const bf16* A, const bf16* W, void* C, float* ws, long ws_floats, int
 
 }  // namespace
 
-// floats of scratch with which yalm_gemm_bf16_dma would split K (0: it would not)
+// floats of scratch with which yalm_gemm_bf16_dma would split K (0: it would not) as a product that is added to
+// the residual stream; other products split as much or less
 long yalm_gemm_bf16_dma_workspace(int M, int N, int K) {
   if (M <= 64 || K < TK || K % TK != 0) return 0;
   if (takes_ring(M)) {
-    const int s = ring_plan(M, N, K, (long)1 << 40).slices;
+    const int s = ring_plan(M, N, K, (long)1 << 40, true).slices;
     return s > 1 ? (long)s * M * N : 0;
   }
   const int slices = slices_for(M, N, K, (long)1 << 40);
@@ -820,20 +828,22 @@ long yalm_gemm_bf16_dma_workspace(int M, int N, int K) {
 
 // The product's K slices, left unadded, as [*slices][M][N] float32 in the workspace (one slice: the product
 // itself), for a consumer that adds them.  More than 64 rows, K a multiple of 64, at least M * N floats.
+// residual: the consumer adds them to the residual stream (see ring_plan).
 int yalm_gemm_bf16_dma_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N,
-                               int K, int* slices_out, hipStream_t stream) {
+                               int K, int* slices_out, int residual, hipStream_t stream) {
   if (M <= 64 || K < TK || K % TK != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || workspace == nullptr ||
       workspace_floats < (long)M * N || slices_out == nullptr)
     return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   if (takes_ring(M)) {              // one slice: the ring kernel stores the product itself, to the workspace
-    const RingPlan p = ring_plan(M, N, K, workspace_floats);
+    const RingPlan p = ring_plan(M, N, K, workspace_floats, residual != 0);
     if (p.slices == 1) {
       *slices_out = 1;
       return launch_ring_shape<0>(a, w, workspace, nullptr, 0, M, N, K, 0, stream);
     }
-    return launch_ring_shape<0>(a, w, nullptr, workspace, workspace_floats, M, N, K, 0, stream, slices_out);
+    return launch_ring_shape<0>(a, w, nullptr, workspace, workspace_floats, M, N, K, 0, stream, slices_out,
+                                residual != 0);
   }
   int slices = slices_for(M, N, K, workspace_floats);
   const int tiles_per_slice = ceil_div(K / TK, slices);
