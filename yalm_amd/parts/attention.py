@@ -248,7 +248,7 @@ class GQAttention(Part):
         else:
             self._decode_attention(q, o, ctx, group, line, k_pages, v_pages, writes_cache)
         ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.q_dim) if prefill else None
-        if ready is not None:                     # the product splits K: its slices are added with the next norm behind
+        if ready is not None:                     # the product's K slices (or the product) are added with the next norm behind
             nw2, eps2, h2, ws2 = ready
             kernels.gemm_add_norm(o, self.wo, x, nw2, eps2, h2, ws2)
             ctx.normed[id(emit_for)] = (h2, None, None)

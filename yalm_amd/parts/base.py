@@ -130,8 +130,6 @@ class Part:
             return None
         if not kernels.can_add_norm(T, K, ctx.act_dtype):
             return None
-        if ctx.mode == "prefill" and kernels.gemm_workspace_floats(T, width, K) == 0:
-            return None      # a prompt's product that does not split K adds to the residual stream itself: cheaper
         import torch
         nw, eps = emit_for.fused()
         h = ctx.ws.get("chain.h", (T, width), torch.bfloat16)          # read by the consumer before the next is written
