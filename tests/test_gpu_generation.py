@@ -111,6 +111,28 @@ def test_stop_tokens_end_a_request_early_and_batches_follow_each_other(folders):
     assert not engine.cache.slots.held and all(g.pool.n_free == g.n_pages for g in engine.cache.kv_groups)
 
 
+def test_a_draw_stays_on_the_device_and_is_read_in_time():
+    """draw() gives what sample() gives, as a device vector at once and as a list on demand; its host
+    buffer is one of four used in turn, and a draw read after four later ones says so."""
+    from yalm_amd import Sampler
+    gen = torch.Generator().manual_seed(11)
+    logits = torch.randn((5, 300), generator=gen).to("cuda:0")
+    ids, steps = [3, 1, 4, 1, 5], [0, 7, 2, 9, 9]
+    sampler = Sampler(21)
+    for temperature in (0.0, 0.7):
+        want = Sampler(21).sample(logits, temperature, ids, steps)
+        drawn = sampler.draw(logits, temperature, ids, steps)
+        assert drawn.tokens.dtype == torch.int32 and drawn.tokens.is_cuda
+        assert drawn.tolist() == want == drawn.tokens.tolist()
+    first = sampler.draw(logits, 0.0, ids, steps)
+    later = [sampler.draw(logits[:2], 0.0, ids[:2], steps[:2]) for _ in range(Sampler.HOST_BUFFERS)]
+    with pytest.raises(RuntimeError, match="later draws"):
+        first.tolist()
+    assert later[-1].tolist() == logits[:2].argmax(1).tolist()
+    wide = sampler.draw(torch.randn((200, 50), generator=gen).to("cuda:0"), 0.0, range(200), [0] * 200)
+    assert len(wide.tolist()) == 200                  # more rows than a buffer held so far
+
+
 @pytest.mark.parametrize("use_graphs", [True, False])
 def test_a_step_from_the_tokens_on_the_device(folders, use_graphs):
     """step_from takes a step's tokens from the vector of a draw, whole or by rows, and gives the
