@@ -111,6 +111,19 @@ def test_unequal_batches_with_reuse(folders, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("min_tokens", [0, 1 << 30])
+@pytest.mark.parametrize("name", ["tiny_sinks", "tiny_wide_heads", "tiny_long", "small_sinks"])
+def test_prompt_steps_with_either_rotation_kernel(folders, name, min_tokens, dtype, monkeypatch):
+    """A prompt step rotates and stores a page-shaped tile at a time from a number of tokens on and token by
+    token below it: the same logits with the choice forced either way."""
+    from yalm_amd.parts import attention
+    monkeypatch.setattr(attention, "ROPE_TILES_MIN_TOKENS", min_tokens)
+    cfg = tiny_configs.ALL[name]
+    requests = helpers.random_requests(cfg, LENGTHS[name], seed=5)
+    compare(folders, name, dtype, schedules.whole(requests), requests, engine_for(folders, name, dtype), "whole")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name,n_requests", [("tiny_llama", 20), ("tiny_mistral", 40), ("tiny_wide_heads", 70),
                                              ("tiny_llama", 130), ("small_windowed", 24), ("small_windowed", 66)])
 def test_batches_of_many_requests(folders, name, n_requests, dtype):

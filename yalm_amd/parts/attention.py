@@ -28,6 +28,10 @@ from .base import Part, build_part, part
 # decode attention is split over pages so that about this many workgroups run
 TARGET_WORKGROUPS = 256
 RESIDENT_WORKGROUPS = 512       # decode-attention workgroups that the chip holds at once (two a compute unit)
+# A prompt step of fewer tokens rotates and stores token by token: the kernel that works a page-shaped tile at a
+# time has a workgroup per (tile, head), too few to fill the chip below this (64 tokens: 4.78 against 4.46 ms a
+# step, 128: 5.75 against 5.48, 256: 6.87 against 6.76, 384: the same)
+ROPE_TILES_MIN_TOKENS = 320
 
 
 @part("mixer", "gqa_attention")
@@ -221,7 +225,7 @@ class GQAttention(Part):
         else:
             kst = vst = None
         if writes_cache:
-            done = prefill and kernels.rope_kv_write_tiles(
+            done = prefill and T >= ROPE_TILES_MIN_TOKENS and kernels.rope_kv_write_tiles(
                 qkv, q, kst, vst, ctx.cu_seqlens, ctx.seq_tile0, k_pages, v_pages, group.table, group.ring_pages,
                 ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads, self.head_dim, pos.rotary_dim,
                 slices=slices)
