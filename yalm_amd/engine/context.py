@@ -15,11 +15,16 @@ class Workspace:
     def __init__(self, device):
         self.device = device
         self._flat = {}
+        self._views = {}              # (name, dtype, shape) -> the view that was handed out last time
         self._retired = []
         self.frozen = False           # set while a graph is captured on these buffers
         self.pinned = False           # set once a captured graph uses these buffers
 
     def _buffer(self, name, shape, dtype, zeroed):
+        shape = tuple(shape)
+        view = self._views.get((name, dtype, shape))
+        if view is not None:
+            return view
         n = 1
         for s in shape:
             n *= int(s)
@@ -33,7 +38,13 @@ class Workspace:
             make = torch.zeros if zeroed else torch.empty
             buf = make(max(n, 1), dtype=dtype, device=self.device)
             self._flat[key] = buf
-        return buf[:n].view(*shape)
+            for k in [k for k in self._views if k[0] == name and k[1] == dtype]:
+                del self._views[k]                 # views of the buffer that was replaced
+        if len(self._views) > 4096:                # many shapes (prompts of every length): start afresh
+            self._views.clear()
+        view = buf[:n].view(*shape)
+        self._views[(name, dtype, shape)] = view
+        return view
 
     def get(self, name, shape, dtype):
         return self._buffer(name, shape, dtype, False)

@@ -28,11 +28,33 @@ def dtype_code(dtype):
         raise TypeError("unsupported dtype %s (float32 or bfloat16)" % dtype) from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream():
+    """The current stream's handle (a launch asks for it: the short way, where torch has one)."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
 def _need(t, name, dtype=None, shape=None):
+    """The address of a tensor after the checks every kernel argument gets; the first lines are the way of an
+    argument that passes them (a step of a short prompt is a few hundred launches that the host has to keep up with)."""
+    try:
+        fine = t.is_cuda and t.is_contiguous() and (dtype is None or t.dtype == dtype)
+    except AttributeError:
+        fine = False
+    if fine:
+        if shape is None:
+            return t.data_ptr()
+        have = t.shape
+        if len(have) == len(shape):
+            for s, d in zip(shape, have):
+                if s is not None and s != d:
+                    break
+            else:
+                return t.data_ptr()
     if not isinstance(t, torch.Tensor):
         raise TypeError("%s: expected a tensor" % name)
     if not t.is_cuda:
