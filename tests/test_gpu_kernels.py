@@ -410,7 +410,8 @@ def test_gemm_partial_and_rotation_that_adds_the_slices(M, n_heads, n_kv, hd, D)
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_heads,n_kv,hd,rd,lens,ring", [(4, 2, 16, 16, [5, 130, 64], 3), (3, 1, 48, 24, [200, 1], 2),
-                                                          (8, 2, 128, 128, [70, 257], 8), (2, 2, 64, 64, [300], 3)])
+                                                          (8, 2, 128, 128, [70, 257], 8), (2, 2, 64, 64, [300], 3),
+                                                          (2, 1, 16, 6, [70, 5], 2), (3, 3, 18, 10, [130], 3)])
 def test_rope_kv_write_tiles(n_heads, n_kv, hd, rd, lens, ring, dtype):
     """Whole prompts, a tile of 64 positions at a time: the same q, staging area and cache pages as the
     per-token kernel (which the tests above pin to the plain rotation), also where a prompt ends inside a
