@@ -747,7 +747,12 @@ double ring_time(long tiles, int iters, int tn) {
 // residual stream.  Unsplit, the tiles read and write that stream in their epilogue, M * N * 8 bytes that no loop
 // hides (2,048 x 4,096 x 4,096 on tiles of 128 columns: 87 us, the same tiles with the gated epilogue 65); split,
 // the kernel that adds the slices also does the norm behind them, whose own pass (M * N * 6 bytes) is saved.
-RingPlan ring_plan(int M, int N, int K, long workspace_floats, bool residual) {
+// consumer: who takes the product.  RING_PLAIN: the epilogue, or a kernel that adds the slices; RING_RESIDUAL:
+// as described above; RING_READER: a kernel that reads the product anyway adds the slices as it reads (the
+// rotation kernel behind q/k/v), a slice more is M * N * 4 bytes more for it to read.
+enum { RING_PLAIN = 0, RING_RESIDUAL = 1, RING_READER = 2 };
+RingPlan ring_plan(int M, int N, int K, long workspace_floats, int consumer) {
+  const bool residual = consumer == RING_RESIDUAL;
   const int mt = ceil_div(M, 256), nk = K / TK;
   RingPlan best;
   double best_t = 1e30;
@@ -758,8 +763,9 @@ RingPlan ring_plan(int M, int N, int K, long workspace_floats, bool residual) {
     for (int s = 1; s <= 8; s *= 2) {
       if (s > 1 && (tiles * s > 256 || nk / s < 8 || (long)s * M * N > workspace_floats)) break;
       const int iters = ceil_div(nk, s);
-      const double t = ring_time(tiles * s, iters, tn) +
-                       (s > 1 ? 3.0 + (double)(s + 2) * M * N * 4.0 / 4.0e6 - norm_saved : in_epilogue);
+      const double adding = consumer == RING_READER ? (double)(s - 1) * M * N * 4.0 / 5.0e6
+                                                    : 3.0 + (double)(s + 2) * M * N * 4.0 / 4.0e6 - norm_saved;
+      const double t = ring_time(tiles * s, iters, tn) + (s > 1 ? adding : in_epilogue);
       if (t < best_t) { best_t = t; best.tn = tn; best.slices = s; best.nt_main = 0; }
     }
   }
@@ -777,9 +783,10 @@ RingPlan ring_plan(int M, int N, int K, long workspace_floats, bool residual) {
 // stay there unadded (one slice: the product itself), *slices_out says how many
 template <int EPI>
 int launch_ring_shape(const bf16* A, const bf16* W, void* C, float* partial, long partial_floats, int M, int N, int K,
-                      int H, hipStream_t stream, int* slices_out = nullptr, bool residual = EPI == 2) {
+                      int H, hipStream_t stream, int* slices_out = nullptr,
+                      int consumer = EPI == 2 ? RING_RESIDUAL : RING_PLAIN) {
   const bool keep = slices_out != nullptr;
-  const RingPlan p = ring_plan(M, N, K, partial != nullptr ? partial_floats : 0, residual);
+  const RingPlan p = ring_plan(M, N, K, partial != nullptr ? partial_floats : 0, consumer);
   if (p.nt_main > 0) {
     if (keep) *slices_out = 1;
     int rc = launch_ring<EPI, 256, 4>(A, W, C, M, N, K, H, stream, 0, p.nt_main);
@@ -819,7 +826,8 @@ int launch(const bf16* A, const bf16* W, void* C, float* ws, long ws_floats, int
 long yalm_gemm_bf16_dma_workspace(int M, int N, int K) {
   if (M <= 64 || K < TK || K % TK != 0) return 0;
   if (takes_ring(M)) {
-    const int s = ring_plan(M, N, K, (long)1 << 40, true).slices;
+    const int s = max(ring_plan(M, N, K, (long)1 << 40, RING_RESIDUAL).slices,
+                      ring_plan(M, N, K, (long)1 << 40, RING_READER).slices);
     return s > 1 ? (long)s * M * N : 0;
   }
   const int slices = slices_for(M, N, K, (long)1 << 40);
@@ -828,7 +836,8 @@ long yalm_gemm_bf16_dma_workspace(int M, int N, int K) {
 
 // The product's K slices, left unadded, as [*slices][M][N] float32 in the workspace (one slice: the product
 // itself), for a consumer that adds them.  More than 64 rows, K a multiple of 64, at least M * N floats.
-// residual: the consumer adds them to the residual stream (see ring_plan).
+// residual: the consumer adds them to the residual stream; else it is a kernel that reads the product anyway
+// (see ring_plan).
 int yalm_gemm_bf16_dma_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N,
                                int K, int* slices_out, int residual, hipStream_t stream) {
   if (M <= 64 || K < TK || K % TK != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || workspace == nullptr ||
@@ -837,13 +846,14 @@ int yalm_gemm_bf16_dma_partial(const void* A, const void* W, float* workspace, l
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   if (takes_ring(M)) {              // one slice: the ring kernel stores the product itself, to the workspace
-    const RingPlan p = ring_plan(M, N, K, workspace_floats, residual != 0);
+    const int consumer = residual ? RING_RESIDUAL : RING_READER;
+    const RingPlan p = ring_plan(M, N, K, workspace_floats, consumer);
     if (p.slices == 1) {
       *slices_out = 1;
       return launch_ring_shape<0>(a, w, workspace, nullptr, 0, M, N, K, 0, stream);
     }
     return launch_ring_shape<0>(a, w, nullptr, workspace, workspace_floats, M, N, K, 0, stream, slices_out,
-                                residual != 0);
+                                consumer);
   }
   int slices = slices_for(M, N, K, workspace_floats);
   const int tiles_per_slice = ceil_div(K / TK, slices);
