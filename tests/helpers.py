@@ -31,10 +31,12 @@ def make_folder(tmp, name, cfg, seed=0, stored=torch.float32, device="cpu"):
 def _folder_weights(folder, rounded):
     """The folder's tensors for the plain implementation, which widens each to float64 where it
     uses it (layer by layer: a model of billions of elements never stands in float64 as a whole).
-    rounded: the values the engine's bfloat16 path stores."""
+    rounded: the values the engine's bfloat16 path stores: matrices rounded to bfloat16, while a vector
+    that the folder keeps in 32-bit (the norm weights of the folders here) stays as it is."""
     if rounded:
         cfg, w = _folder_weights(folder, False)           # tensors stored in bfloat16 are shared, not read again
-        return cfg, {k: v if v.dtype == torch.bfloat16 else v.to(torch.bfloat16) for k, v in w.items()}
+        return cfg, {k: v if v.dtype == torch.bfloat16 or (v.dim() <= 1 and v.dtype in (torch.float32, torch.float64))
+                     else v.to(torch.bfloat16) for k, v in w.items()}
     return R.read_folder(folder)
 
 
@@ -47,8 +49,8 @@ def forget_plain_results():
 @functools.lru_cache(maxsize=None)
 def plain_logits(folder, tokens, dtype="float32"):
     """float32 numpy [T, vocab] of the plain implementation; with dtype bfloat16
-    the weights are rounded to bfloat16 first, as the engine stores them
-    (vectors stored in 32-bit would stay; the folders here are rounded whole)."""
+    the matrices are rounded to bfloat16 first, as the engine stores them (vectors
+    that a folder keeps in 32-bit stay in 32-bit, there as here)."""
     cfg, w = _folder_weights(folder, dtype == "bfloat16")
     return R.forward(w, cfg, list(tokens)).to(torch.float32).numpy()
 

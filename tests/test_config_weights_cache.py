@@ -518,6 +518,25 @@ def test_generation_loop_a_step_ahead():
     assert seen_a == seen_b
 
 
+def test_the_prompt_clock_covers_the_prompt_step_when_the_loop_runs_ahead():
+    """A draw does not wait for the device; the prompt step is over only when its tokens have landed.
+    Here every landing takes 30 ms: the prompt's share of it must be in prefill_seconds, not in decode_seconds."""
+    import time
+    from yalm_amd.generate import GenerationStats
+
+    class SlowLanding(DrawingSampler):
+        class _Drawn(DrawingSampler._Drawn):
+            def tolist(self):
+                time.sleep(0.03)
+                return super().tolist()
+
+    stats = GenerationStats()
+    out = generate(ScriptedAheadEngine(), [[1, 2, 3]], max_new_tokens=3, sampler=SlowLanding(), stats=stats, stop_ids=[])
+    assert out == [[4, 5, 6]]
+    assert stats.prefill_seconds >= 0.03
+    assert stats.decode_seconds >= 0.06                      # the two later draws
+
+
 @pytest.mark.parametrize("base, sampler", [(ScriptedEngine, ArgmaxSampler), (ScriptedAheadEngine, DrawingSampler)])
 def test_a_failed_step_gives_the_slots_back(base, sampler):
     class Failing(base):

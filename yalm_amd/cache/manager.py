@@ -143,6 +143,14 @@ class KVGroup:
         self.table_host = np.full((n_slots, self.ring_pages), -1, dtype=np.int32)
         self.table = torch.full((n_slots, self.ring_pages), -1, dtype=torch.int32, device=device)
         self._dirty = set()
+        # changed rows travel through two pinned copies of the table used in turn, so that the upload is queued
+        # without the host waiting for the steps still running (a copy from pageable memory would wait)
+        self._staging = self._staged = None
+        if torch.device(device).type == "cuda":
+            self._staging = [torch.empty((n_slots, self.ring_pages), dtype=torch.int32, pin_memory=True)
+                             for _ in range(2)]
+            self._staged = [None, None]               # the event behind the last upload from each copy
+        self._turn = 0
         self.sinks = request.sinks if self.window > 0 else 0
         # A slot's sinks need no clearing when the slot is taken again: a sink is read only once its
         # position lies behind the window, and by then the slot's present sequence has written it.
@@ -199,7 +207,18 @@ class KVGroup:
         if not self._dirty:
             return
         lo, hi = min(self._dirty), max(self._dirty) + 1
-        self.table[lo:hi].copy_(torch.from_numpy(self.table_host[lo:hi]))
+        if self._staging is None:
+            self.table[lo:hi].copy_(torch.from_numpy(self.table_host[lo:hi]))
+        else:
+            t = self._turn
+            if self._staged[t] is not None:
+                self._staged[t].synchronize()         # the upload before last: long done while the host is a step ahead
+            else:
+                self._staged[t] = torch.cuda.Event()
+            self._staging[t].numpy()[lo:hi] = self.table_host[lo:hi]
+            self.table[lo:hi].copy_(self._staging[t][lo:hi], non_blocking=True)
+            self._staged[t].record()
+            self._turn = t ^ 1
         self._dirty.clear()
 
     def bytes_per_token(self):

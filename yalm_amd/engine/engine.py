@@ -401,6 +401,8 @@ class Engine:
         key = (Bk, pages_bucket)
         g = self._graphs.get(key)
         if g is None:
+            if len(self._graphs) >= self.max_graphs or not self._graphs:
+                torch.cuda.synchronize(self.device)      # a graph's last replay may still be queued: the host runs ahead
             while len(self._graphs) >= self.max_graphs:
                 self._graphs.popitem(last=False)
             if not self._graphs:
@@ -472,7 +474,8 @@ class Engine:
         return self.graphs_captured - before
 
     def drop_graphs(self):
-        """Forgets every captured graph and the buffers only they used."""
+        """Forgets every captured graph and the buffers only they used (after their last replays have ended)."""
+        torch.cuda.synchronize(self.device)
         self._graphs.clear()
         self.graph_ws.drop_retired()
 

@@ -10,7 +10,10 @@ The loop runs one step ahead of the host where the engine and the sampler allow
 it: a step's tokens stay on the device and feed the next step from there, and
 the host reads them while that step runs, so the device never waits for the
 host between two steps.  A sequence that samples a stop token is then seen one
-step late: it has taken part in one more step, whose token is dropped."""
+step late: it has taken part in one more step, whose token is dropped.  The one
+place where the host does wait is the end of a batch's prompt step, so that the
+time of the prompt and the time of decoding are told apart on the device's clock
+(src/main.cpp:133-147 reports them so)."""
 import time
 from dataclasses import dataclass, field
 from typing import List
@@ -103,9 +106,11 @@ def generate(engine, prompts, max_new_tokens=256, temperature=0.0, seed=0, stop_
             t0 = time.perf_counter()
             logits = engine.step(slots, [prompts[i] for i in batch])
             stats.bytes_read += step_bytes(slots)
+            landed = None
             if ahead:
                 drawn = sampler.draw(logits, temperature, [ids[i] for i, _ in live], [0] * len(live))
                 tokens = None
+                landed = drawn.tolist()                   # waits for the prompt step: its clock stops on the device's time
             else:
                 tokens = sampler.sample(logits, temperature, [ids[i] for i, _ in live], [0] * len(live))
             stats.prefill_seconds += time.perf_counter() - t0
@@ -134,8 +139,9 @@ def generate(engine, prompts, max_new_tokens=256, temperature=0.0, seed=0, stop_
                     draw_steps = [len(results[i]) + 1 for i, _ in going]
                     if ahead:
                         next_drawn = sampler.draw(logits, temperature, draw_ids, draw_steps)
-                if ahead:
-                    tokens = drawn.tolist()               # lands while the step just queued runs
+                if ahead:                                 # lands while the step just queued runs (a batch's first
+                    tokens = drawn.tolist() if landed is None else landed       # draw was read with the prompt step)
+                    landed = None
                 still, still_rows, ended = [], [], []
                 k = 0                                     # walks `going`, which keeps the order of `live`
                 for (i, slot), r in zip(live, rows):
