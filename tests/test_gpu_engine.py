@@ -249,3 +249,78 @@ def test_token_probabilities_in_blocks_of_rows(folders, dtype):
     assert got.shape == (len(want),) and (got > 0).all()
     assert np.abs(np.log(got.astype(np.float64)) - np.asarray(want)).max() <= tol
     assert np.abs(np.log(after.cpu().numpy().astype(np.float64)) - np.asarray(want_after)).max() <= tol
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_batch_in_the_largest_graph_bucket(tmp_path_factory, dtype):
+    """520 sequences of 3 to 90 tokens decode together: the graph bucket of 1,024 rows, half of them
+    padding.  Every 40th request is compared with the plain implementation at every place."""
+    from yalm_amd.engine import Engine, Model
+    folder = helpers.make_folder(tmp_path_factory.mktemp("bucket_1024"), "many_rows", MANY_ROWS, seed=10)
+    rng = np.random.default_rng(21)
+    n = 520
+    lengths = [int(x) for x in rng.integers(3, 91, size=n)]
+    requests = helpers.random_requests(MANY_ROWS, lengths, seed=22)
+    first = {rid: len(t) - 2 for rid, t in requests.items()}
+    steps = schedules.batches(requests, [list(requests)], first)
+    for s in steps:
+        for e in s["entries"]:
+            if int(e["id"][1:]) % 40:
+                e["want"] = []
+    model = Model.from_folder(folder, dtype=helpers.torch_dtype(dtype), device="cuda:0")
+    engine = Engine(model, max_tokens=schedules.max_tokens_needed(steps), max_batch=n)
+    out = schedules.replay_in_process(engine, steps)
+    assert 1024 in {k[0] for k in engine._graphs}
+    got = {rid: [] for rid in requests if int(rid[1:]) % 40 == 0}
+    for s in steps:
+        r = 0
+        for e in s["entries"]:
+            for _ in e["want"]:
+                got[e["id"]].append(out[s["step"]][r])
+                r += 1
+    assert len(got) == 13
+    for rid, rows in got.items():
+        want = helpers.plain_logits(folder, tuple(requests[rid]), dtype)
+        helpers.check_logits(np.stack(rows), want, dtype, "bucket 1024 %s request %s" % (dtype, rid))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["tiny_llama", "tiny_mistral"])
+def test_a_sequence_at_its_first_token_beside_sequences_that_go_on(folders, name, dtype):
+    """A step of one token each in which one sequence has nothing in the cache yet: the step function
+    takes it as a decode step (position 0 beside later positions); that sequence's first page is
+    new, the others' pages are old."""
+    engine = make_engine(folders, name, dtype, max_tokens=1024)
+    requests = helpers.random_requests(tiny_configs.ALL[name], [40, 12, 9], seed=23)
+    a, b, c = (requests[r] for r in ("r0", "r1", "r2"))
+    sa, sb = engine.start(2)
+    rows = {"a": [], "b": [], "c": []}
+    first = engine.step([sa, sb], [a[:30], b[:5]], [list(range(30)), list(range(5))]).cpu().numpy()
+    rows["a"] += list(first[:30])
+    rows["b"] += list(first[30:])
+    (sc,) = engine.start(1)
+    for k in range(7):                                     # c joins at its position 0, then all go on
+        out = engine.step([sa, sc, sb], [[a[30 + k]], [c[k]], [b[5 + k]]]).cpu().numpy()
+        rows["a"].append(out[0])
+        rows["c"].append(out[1])
+        rows["b"].append(out[2])
+    engine.release([sa, sb, sc])
+    for key, toks in (("a", a), ("b", b), ("c", c)):
+        want = helpers.plain_logits(folders[name], tuple(toks), dtype)[:len(rows[key])]
+        helpers.check_logits(np.stack(rows[key]), want, dtype, "%s %s joined at position 0, sequence %s" % (name, dtype, key))
+
+
+def test_a_step_whose_widest_buffer_would_pass_the_checked_size_is_refused(folders):
+    from yalm_amd.engine.engine import StepError
+    engine = make_engine(folders, "tiny_llama", "float32", max_tokens=1024)
+    assert engine.MAX_ELEMENTS == 1 << 31 and engine._widest_row == 176       # the feed-forward's hidden width
+    engine.MAX_ELEMENTS = 176 * 20
+    slots = engine.start(1)
+    with pytest.raises(StepError, match="2\\^31"):
+        engine.step(slots, [list(range(20))])
+    assert engine.length(slots[0]) == 0                    # refused before anything was taken
+    engine.step(slots, [list(range(13))])                  # 13 x 176 and one row of 256 logits fit
+    with pytest.raises(StepError, match="2\\^31"):         # the logits alone: 14 rows x 256 reach 176 x 20
+        s2 = engine.start(1)
+        engine.step(s2, [list(range(15))], [list(range(14))])
+    engine.release(slots + s2)

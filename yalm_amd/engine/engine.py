@@ -107,6 +107,7 @@ class Engine:
         self.graph_ws = Workspace(self.device)          # shared by all captured graphs (they never run together)
         self.use_graphs = use_graphs
         self.max_graphs = max(1, int(max_graphs))
+        self._widest_row = model.widest_row()
         self._segments = model.decode_segments()        # the parts are fixed from here on: asked once, not every step
         self._any_graph = any(safe for safe, _, _ in self._segments)
         for text in model.describe()[1]:                # a slow fallback is said once, not hidden
@@ -203,6 +204,12 @@ class Engine:
         else:
             raise StepError("the sequences of a step either all start at their first token or all go on by one "
                             "token (lengths so far %s, tokens brought %s)" % (starts, n_tok))
+        n_wanted = B if want is None else sum(len(w) for w in want)
+        if sum(n_tok) * self._widest_row >= self.MAX_ELEMENTS or (targets is None and n_wanted * V >= self.MAX_ELEMENTS):
+            raise StepError("a step of %d tokens with %d rows of logits is refused: its widest buffer (%d elements a "
+                            "token, %d logits a row) would reach 2^31 elements, more than any step that was ever "
+                            "checked; cut the batch, or ask for fewer logits"
+                            % (sum(n_tok), n_wanted, self._widest_row, V))
         max_pos = max(starts) if decode else max(s + n for s, n in zip(starts, n_tok)) - 1
         new_lens = self._extend(slots, n_tok, max_pos)
         if mode == "decode":
@@ -260,6 +267,7 @@ class Engine:
             raise StepError(str(e)) from None
 
     HEAD_ROWS = 1024        # rows of logits made at a time when only token probabilities are asked for
+    MAX_ELEMENTS = 1 << 31  # a step whose widest buffer reaches this many elements is refused
 
     def _prefill(self, slots, tokens, want, n_tok, new_lens, targets=None):
         B, T = len(slots), sum(n_tok)

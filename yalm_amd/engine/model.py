@@ -178,6 +178,11 @@ class Model:
                     slow.append(text)
         return lines, slow
 
+    def widest_row(self):
+        """The most elements any part keeps for one token of a step (a part says so with `row_elements()`;
+        the residual stream's width stands for the others)."""
+        return max([self.dim] + [int(p.row_elements()) for p in self.all_parts() if hasattr(p, "row_elements")])
+
     def weight_bytes(self):
         """Bytes of weights a step reads: every weight once, one embedding row."""
         total = self.embedding.weight_bytes() + self.final_norm.weight_bytes() + self.head.weight_bytes()

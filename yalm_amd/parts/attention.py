@@ -81,6 +81,10 @@ class GQAttention(Part):
     def cache_request(self):
         return KVRequest(self.n_kv_heads, self.head_dim, self.window, self.sinks)
 
+    def row_elements(self):
+        """The widest buffer a token has in this part: q, k and v side by side."""
+        return self.q_dim + 2 * self.kv_dim
+
     def describe(self, compute_dtype):
         what = "attention, %d heads in %d groups of head size %d%s" % (
             self.n_heads, self.n_kv_heads, self.head_dim,

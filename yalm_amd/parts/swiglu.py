@@ -49,6 +49,9 @@ class SwiGLU(Part):
     def weight_bytes(self):
         return 3 * self.hidden * self.dim * self.w_down.element_size()
 
+    def row_elements(self):
+        return self.hidden
+
     def fuses_norm(self, norm, x, ctx):
         if not hasattr(norm, "fused") or ctx.mode not in ("decode", "prefill"):
             return False
