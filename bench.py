@@ -7,6 +7,12 @@ shape with its window of 4,096 positions and prompts of 6,000 tokens).
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers N] [--dtype bf16|fp32] [--shape NAME]
                     [--prompt-len N] [--prefill-len N] [--batch B] [--points B,B] [--no-prefill]
+                    [--kernels] [--ragged] [--sweep]
+
+--kernels adds the time of every kernel of a decode step and of a prompt step, each taken alone at the
+shape's sizes (src/test.cpp:340-405 times single kernels so), with its rate against the peak;
+--ragged adds generate() over 64 requests of unequal lengths beside the same batch at equal lengths;
+--sweep adds the shape's whole workload end to end (src/main.cpp:104-147 times a whole run).
 
 A step is one decode step as generation does it: the step function for a batch
 of sequences (one token each, from the cache), greedy sampling on the device
@@ -15,7 +21,9 @@ positions (2,048 to 4,096 for the default shape); a run of K steps takes the K
 positions in the middle of that range, so that its mean context is the whole
 range's (K = 2,048 is the range itself), by prefilling that many random tokens.
 One JSON line is printed.  Peaks are MI355X's
-published ones: HBM 8 TB/s; dense MFMA bf16/fp16 2.5 PFLOP/s, fp32 157.3 TFLOP/s."""
+published ones: HBM 8 TB/s; dense MFMA bf16/fp16 2.5 PFLOP/s, fp32 157.3 TFLOP/s; beside them the line
+names what a kernel that only reads memory and a loop of matrix-core instructions reach in this run
+(`peak_measured`)."""
 import argparse
 import json
 import os
@@ -65,6 +73,140 @@ def prefill_flops(cfg, n_layers, T):
     return n_layers * (per_layer + attn) + 2 * D * V
 
 
+def measured_peaks(torch, dtype):
+    """(GB/s of a kernel that only reads 2 GB once, TFLOP/s of the better matrix-core loop on registers)."""
+    from yalm_amd.ops import kernels
+    buf = torch.empty(1 << 31, dtype=torch.uint8, device="cuda:0")
+    buf.zero_()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best_read = 0.0
+    for wg in (1024, 2048, 4096):
+        for _ in range(3):
+            e0.record()
+            n = kernels.probe_read(buf, wg)
+            e1.record()
+            e1.synchronize()
+            best_read = max(best_read, n / (e0.elapsed_time(e1) * 1e-3) / 1e9)
+    del buf
+    best_mfma = 0.0
+    if dtype == "bf16":
+        for shape in (32, 16):
+            for _ in range(3):
+                e0.record()
+                fl = kernels.probe_mfma(shape, 16384, 1024)
+                e1.record()
+                e1.synchronize()
+                best_mfma = max(best_mfma, fl / (e0.elapsed_time(e1) * 1e-3) / 1e12)
+    return round(best_read, 1), round(best_mfma, 1)
+
+
+KERNEL_FACES = ("embed", "rmsnorm", "gemm", "gemm_norm", "gemm_norm_qkv_rope", "gemm_add_norm", "gemm_partial",
+                "gemm_chain", "gemm_chain_qkv_rope", "rope_kv_write", "rope_kv_write_tiles", "attn_prefill",
+                "attn_decode", "sink_store", "attn_sink_mix", "argmax")
+
+
+def record_kernel_calls(run):
+    """Runs `run()` with every face of ops.kernels wrapped; returns the calls it made, in order, as
+    (face name, function, args, kwargs)."""
+    from yalm_amd.ops import kernels
+    calls, saved = [], {n: getattr(kernels, n) for n in KERNEL_FACES}
+
+    def wrap(name, fn):
+        def face(*a, **kw):
+            calls.append((name, fn, a, kw))
+            return fn(*a, **kw)
+        return face
+    for n, fn in saved.items():
+        setattr(kernels, n, wrap(n, fn))
+    try:
+        run()
+    finally:
+        for n, fn in saved.items():
+            setattr(kernels, n, fn)
+    return calls
+
+
+def kernel_cost(name, a, kw, kv_tokens, torch):
+    """(label, bytes the call has to move, flops it has to do) from the call's own operands.  kv_tokens: the keys
+    a decode attention reads, summed over its sequences."""
+    def nbytes(*ts):
+        return sum(t.numel() * t.element_size() for t in ts if torch.is_tensor(t))
+    gemm_w = {"gemm": 1, "gemm_chain": 1, "gemm_add_norm": 1, "gemm_partial": 1, "gemm_norm": 3,
+              "gemm_norm_qkv_rope": 3, "gemm_chain_qkv_rope": 2}
+    if name in gemm_w:
+        x, w = a[0], a[gemm_w[name]]
+        M, K = x.shape
+        N = w.shape[0]
+        out_bytes = M * N * 4
+        return "%s %dx%dx%d" % (name, M, N, K), nbytes(x, w) + out_bytes, 2.0 * M * N * K
+    if name == "attn_decode":
+        q, kp = a[0], a[1]
+        n_kv, hd = kp.shape[1], kp.shape[3]
+        return "attn_decode %d rows" % q.shape[0], 2 * kv_tokens * n_kv * hd * kp.element_size() + 2 * nbytes(q), \
+            4.0 * q.shape[1] * kv_tokens
+    if name == "attn_prefill":
+        q, cu = a[0], a[4]
+        lens = (cu[1:] - cu[:-1]).tolist()
+        pairs = sum(n * (n + 1) // 2 for n in lens)
+        window = a[11]
+        if window:
+            pairs = sum(sum(min(i + 1, window) for i in range(n)) for n in lens)
+        return "attn_prefill %d tokens" % q.shape[0], nbytes(q, a[1], a[2], a[3]), 4.0 * q.shape[1] * pairs
+    if name in ("rope_kv_write", "rope_kv_write_tiles"):
+        q_out = a[1]
+        T, Q = q_out.shape
+        n_kv, hd = a[15 if name == "rope_kv_write" else 14], a[16 if name == "rope_kv_write" else 15]
+        width = Q + 2 * n_kv * hd
+        slices = kw.get("slices", 1)
+        return "%s %d tokens, %d slices" % (name, T, slices), T * width * (4 * slices + 2 * q_out.element_size()), 0.0
+    if name == "rmsnorm":
+        return "rmsnorm %dx%d" % tuple(a[2].shape), nbytes(a[2]) + a[2].numel() * 4, 0.0
+    if name == "embed":
+        return "embed %d" % a[1].shape[0], 2 * nbytes(a[2]), 0.0
+    if name == "argmax":
+        return "argmax %dx%d" % tuple(a[0].shape), nbytes(a[0]), 0.0
+    return name, nbytes(*a), 0.0
+
+
+def time_kernel_groups(calls, kv_tokens, torch, dtype, reps=5):
+    """Every kernel of a step alone: the calls with the same face and shapes (one a layer) are captured into one
+    graph in the order of the step, so that each reads weights that no call just before it has read, and the
+    graph is replayed between two events.  Returns {label: {calls, us, GB/s, TFLOP/s, frac, bound}}."""
+    groups = {}
+    for name, fn, a, kw in calls:
+        label, nb, fl = kernel_cost(name, a, kw, kv_tokens, torch)
+        g = groups.setdefault(label, {"calls": [], "bytes": nb, "flops": fl})
+        g["calls"].append((fn, a, kw))
+    flush = torch.empty(1 << 29, dtype=torch.uint8, device="cuda:0")        # 512 MB: more than the caches hold
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    out = {}
+    for label, g in groups.items():
+        graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph):
+            for fn, a, kw in g["calls"]:
+                fn(*a, **kw)
+        graph.replay()
+        total = 0.0
+        for _ in range(reps):
+            flush.zero_()
+            e0.record()
+            graph.replay()
+            e1.record()
+            e1.synchronize()
+            total += e0.elapsed_time(e1)
+        n = len(g["calls"])
+        us = total / reps / n * 1e3
+        gbs = g["bytes"] / us / 1e3
+        tfs = g["flops"] / us / 1e6
+        frac_hbm, frac_mfma = gbs * 1e9 / HBM_PEAK, tfs * 1e12 / FLOP_PEAK[dtype]
+        bound = "hbm" if frac_hbm >= frac_mfma else "mfma"
+        out[label] = {"calls": n, "us": round(us, 2), "GB/s": round(gbs, 1), "TFLOP/s": round(tfs, 2),
+                      "bound": bound, "frac": round(max(frac_hbm, frac_mfma), 4)}
+        del graph
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -81,6 +223,15 @@ def main():
     ap.add_argument("--prefill-len", type=int, default=PREFILL, help="tokens of the timed prompt")
     ap.add_argument("--shape", default="mistral-7b-v0.2", choices=sorted(SHAPES),
                     help="the layer sizes: the Mistral-7B-v0.2 shape (default), Llama-3.2-3B or Mistral-7B-v0.1")
+    ap.add_argument("--kernels", action="store_true",
+                    help="also time every kernel of a decode step (at --batch) and of the prompt step alone")
+    ap.add_argument("--ragged", action="store_true",
+                    help="also run generate() over 64 requests of 1,024 to 3,072 tokens beside the same batch at "
+                         "equal lengths")
+    ap.add_argument("--ragged-new", type=int, default=128, help="new tokens of each request of --ragged")
+    ap.add_argument("--sweep", action="store_true",
+                    help="also run the shape's whole workload end to end at --batch: the prompts, then every "
+                         "decode step of its range of positions")
     ap.add_argument("--context", type=int, default=0,
                     help="the reference's -T: past this many positions two attention sinks and the last "
                          "<context> - 2 positions are attended to (0: the shape's own window, if any)")
@@ -146,13 +297,14 @@ def main():
         sys.stderr.write("[bench] prefill %s\n" % prefill)
 
     # ---------------------------------------------------------------- decode
-    def decode(B, steps, warmup):
-        prompts = [torch.randint(0, V, (PROMPT,), generator=gen).tolist() for _ in range(B)]
+    def decode(B, steps, warmup, prompt_len=None):
+        PROMPT_B = prompt_len or PROMPT
+        prompts = [torch.randint(0, V, (PROMPT_B,), generator=gen).tolist() for _ in range(B)]
         slots = engine.start(B)
         ids = list(range(B))
         # prompts in chunks of sequences, so that the prefill workspace stays small
         tokens = []
-        n = max(1, min(8, 48000 // PROMPT))
+        n = max(1, min(8, 48000 // PROMPT_B))
         for i in range(0, B, n):
             logits = engine.step(slots[i:i + n], prompts[i:i + n])
             tokens += sampler.sample(logits, 0.0, ids[i:i + n], [0] * len(slots[i:i + n]))

@@ -117,6 +117,36 @@ def test_spec_is_data_layer_by_layer():
                   spec.final_norm, spec.head, schedule=[ScheduleEntry(0, 1, writes_cache=False)])
 
 
+def test_a_layer_names_its_members_and_parts_that_follow_from_their_spec_are_shared():
+    from yalm_amd.config import LayerSpec, PartSpec
+    from yalm_amd.engine.model import Model
+    norm = PartSpec("rmsnorm", {"eps": 1e-5}, prefix="n.")
+    ff = PartSpec("swiglu", {"hidden": 32}, prefix="ff.")
+    layer = LayerSpec("some_block", {"norm": norm}, prefix="l.", feed_forward=ff)
+    assert layer.norm is norm and layer.part("feed_forward") is ff and layer.part("mixer") is None
+    assert sorted(layer.parts) == ["feed_forward", "norm"] and layer.prefix == "l." and layer.block == "some_block"
+    with pytest.raises(AttributeError, match="no member 'mixer'"):
+        layer.mixer
+    with pytest.raises(AttributeError):
+        layer.block = "other"
+    with pytest.raises(TypeError, match="PartSpec"):
+        LayerSpec("some_block", mixer="attention")
+    assert layer == LayerSpec("some_block", prefix="l.", norm=norm, feed_forward=ff)
+    # the reference's block keeps its four names
+    spec = config_from_dict(tiny_configs.TINY_MISTRAL).to_spec()
+    assert sorted(spec.layers[0].parts) == ["feed_forward", "feed_forward_norm", "mixer", "mixer_norm"]
+    # one position part for the layers that name the same spec; parts with tensors stay one each
+    model = Model(spec)
+    positions = {id(b.mixer.position) for b in model.blocks}
+    assert len(positions) == 1 and len({id(b.mixer_norm) for b in model.blocks}) == 3
+    assert sum(1 for p in model.all_parts() if p is model.blocks[0].mixer.position) == 1
+    other = Model(spec)                                    # another model has its own
+    assert other.blocks[0].mixer.position is not model.blocks[0].mixer.position
+    assert [m.name for m in model.prompt_tables()] == ["kv_tiles"]
+    tables = model.prompt_tables()[0]([130, 1, 64])
+    assert list(tables["seq_tile0"]) == [0, 3, 4, 5] and tables["n_tiles"] == 5 and sorted(tables["tile_order"]) == [0, 2, 3, 4]
+
+
 # ------------------------------------------------------------------ weights
 
 def test_random_model_folder_round_trip(tmp_path):
@@ -643,3 +673,29 @@ def test_prefill_tile_order_names_every_second_tile_once_the_longest_first():
     for b in runs:
         w = [x for x, s in zip(work, seqs) if s == b]
         assert w == sorted(w, reverse=True)
+
+
+def test_a_library_built_from_other_sources_is_built_again(tmp_path, monkeypatch):
+    """The digest of the kernel sources is kept beside the built library; a library whose digest is another
+    (or that has none) is not loaded but built again."""
+    from yalm_amd.csrc import build
+
+    class Reached(Exception):
+        pass
+
+    def no_compiler():
+        raise Reached()
+    lib = tmp_path / build.LIB_NAME
+    lib.write_bytes(b"not a library")
+    monkeypatch.setattr(build, "_candidates", lambda: [str(lib)])
+    monkeypatch.setattr(build, "_hipcc", no_compiler)
+    with pytest.raises(Reached):                          # no digest beside it: stale
+        build.build(force=False)
+    (tmp_path / (build.LIB_NAME + ".sources")).write_text("0" * 64 + "\n")
+    with pytest.raises(Reached):                          # another digest: stale
+        build.build(force=False)
+    (tmp_path / (build.LIB_NAME + ".sources")).write_text(build.sources_digest() + "\n")
+    assert build.build(force=False) == str(lib)           # built from these sources: taken as it is
+    with pytest.raises(Reached):
+        build.build(force=True)
+    assert len(build.sources_digest()) == 64

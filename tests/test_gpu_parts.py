@@ -35,7 +35,7 @@ def make_ctx(cache, lens, dtype, mode="prefill", starts=None):
     ctx.seq_len = i32(new_lens)
     ctx.cu_seqlens = i32(np.concatenate([[0], np.cumsum(lens)]))
     tile0 = np.concatenate([[0], np.cumsum([(n + 63) // 64 for n in lens])])
-    ctx.seq_tile0, ctx.n_tiles = i32(tile0), int(tile0[-1])
+    ctx.tables["kv_tiles"] = {"seq_tile0": i32(tile0), "n_tiles": int(tile0[-1])}
     ctx.max_position = max(new_lens) - 1
     ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), list(lens), list(starts)
     return ctx, slots
@@ -281,9 +281,11 @@ class ToyConfig:
                   PartSpec("gqa_attention", {"n_heads": 2, "n_kv_heads": 1, "head_dim": 16,
                                              "window": d.get("window", 0), "sinks": d.get("sinks", 0),
                                              "position": pos}, prefix="attn.")]
-        layers = [LayerSpec("prenorm_residual", m, PartSpec("swiglu", {"hidden": d["hidden"]}, prefix="ff."),
-                            PartSpec("rmsnorm", norm, prefix="n1."), PartSpec("rmsnorm", norm, prefix="n2."),
-                            "toy.%d." % i) for i, m in enumerate(mixers)]
+        layers = [LayerSpec("prenorm_residual", prefix="toy.%d." % i, mixer=m,
+                            feed_forward=PartSpec("swiglu", {"hidden": d["hidden"]}, prefix="ff."),
+                            mixer_norm=PartSpec("rmsnorm", norm, prefix="n1."),
+                            feed_forward_norm=PartSpec("rmsnorm", norm, prefix="n2."))
+                  for i, m in enumerate(mixers)]
         return ModelSpec("ToyForCausalLM", D, d["vocab"], d["positions"],
                          PartSpec("token_embedding", {"vocab_size": d["vocab"]}, prefix="toy.emb."), layers,
                          PartSpec("rmsnorm", norm, prefix="toy.norm."),
@@ -468,8 +470,9 @@ class RoutedToyConfig:
                                               "position": pos}, prefix="attn.")
         ffs = [PartSpec("swiglu", {"hidden": d["hidden"]}, prefix="ff."),
                PartSpec("toy_top1_experts", {"n_experts": d["experts"], "hidden": d["hidden"]}, prefix="moe.")]
-        layers = [LayerSpec("prenorm_residual", attn(w), ff, PartSpec("rmsnorm", norm, prefix="n1."),
-                            PartSpec("rmsnorm", norm, prefix="n2."), "toy.%d." % i)
+        layers = [LayerSpec("prenorm_residual", prefix="toy.%d." % i, mixer=attn(w), feed_forward=ff,
+                            mixer_norm=PartSpec("rmsnorm", norm, prefix="n1."),
+                            feed_forward_norm=PartSpec("rmsnorm", norm, prefix="n2."))
                   for i, (w, ff) in enumerate(zip((0, 9), ffs))]
         return ModelSpec("RoutedToyForCausalLM", d["width"], d["vocab"], d["positions"],
                          PartSpec("token_embedding", {"vocab_size": d["vocab"]}, prefix="toy.emb."), layers,
@@ -539,3 +542,154 @@ def test_toy_routed_feed_forward_and_position_encoding_from_outside(tmp_path):
         unregister_architecture("RoutedToyForCausalLM")
         unregister_part("feed_forward", "toy_top1_experts")
         unregister_part("position", "toy_linear_frequencies")
+
+
+# ---------------------------------------------------------------------------
+# toy arrangements of a layer with other members than the reference's block has
+# ---------------------------------------------------------------------------
+
+def define_toy_blocks():
+    from yalm_amd.parts import Part, build_part, register_part
+
+    class ParallelBlock(Part):
+        """x += mixer(norm(x)) + feed_forward(norm(x)): ONE norm, and both branches read its output.
+        Members: norm, mixer, feed_forward."""
+
+        def __init__(self, layer_spec, dim, prefix=""):
+            super().__init__(None, dim, layer_spec.prefix)
+            p = layer_spec.prefix
+            self.norm = build_part("norm", layer_spec.norm, dim, p)
+            self.mixer = build_part("mixer", layer_spec.mixer, dim, p)
+            self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, dim, p)
+
+        def children(self):
+            return [self.norm, self.mixer, self.feed_forward]
+
+        def forward(self, x, ctx, line, writes_cache=True):
+            h = ctx.ws.get("toy.parallel.h", (x.shape[0], self.dim), ctx.act_dtype)
+            self.norm.forward(x, h, ctx)
+            self.mixer.forward(h, x, ctx, line, writes_cache)
+            self.feed_forward.forward(h, x, ctx)
+
+    class FeedForwardOnlyBlock(Part):
+        """x += feed_forward(norm(x)): no mixer, so the layer keeps nothing in the cache.
+        Members: norm, feed_forward."""
+
+        def __init__(self, layer_spec, dim, prefix=""):
+            super().__init__(None, dim, layer_spec.prefix)
+            self.norm = build_part("norm", layer_spec.norm, dim, layer_spec.prefix)
+            self.feed_forward = build_part("feed_forward", layer_spec.feed_forward, dim, layer_spec.prefix)
+
+        def children(self):
+            return [self.norm, self.feed_forward]
+
+        def forward(self, x, ctx, line, writes_cache=True):
+            h = ctx.ws.get("toy.ffonly.h", (x.shape[0], self.dim), ctx.act_dtype)
+            self.norm.forward(x, h, ctx)
+            self.feed_forward.forward(h, x, ctx)
+
+    register_part("block", "toy_parallel", ParallelBlock, replace=True)
+    register_part("block", "toy_feed_forward_only", FeedForwardOnlyBlock, replace=True)
+
+
+class BlocksToyConfig:
+    """Three layers, three arrangements: the parallel block, the block without a mixer, and the
+    reference's own.  Both attentions name the same position encoding."""
+
+    def __init__(self, d):
+        self.d = d
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d)
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def to_spec(self):
+        from yalm_amd.config import LayerSpec, ModelSpec, PartSpec
+        d = self.d
+        norm = {"eps": d["eps"]}
+        pos = PartSpec("rope", {"head_dim": 16, "rotary_dim": 8, "theta": 50.0, "scaling": None,
+                                "weight_rows": "interleaved"})
+        attn = PartSpec("gqa_attention", {"n_heads": 4, "n_kv_heads": 2, "head_dim": 16, "window": 0, "position": pos},
+                        prefix="attn.")
+        ff = PartSpec("swiglu", {"hidden": d["hidden"]}, prefix="ff.")
+        layers = [LayerSpec("toy_parallel", prefix="toy.0.", norm=PartSpec("rmsnorm", norm, prefix="n."),
+                            mixer=attn, feed_forward=ff),
+                  LayerSpec("toy_feed_forward_only", {"norm": PartSpec("rmsnorm", norm, prefix="n."), "feed_forward": ff},
+                            prefix="toy.1."),
+                  LayerSpec("prenorm_residual", prefix="toy.2.", mixer=attn, feed_forward=ff,
+                            mixer_norm=PartSpec("rmsnorm", norm, prefix="n1."),
+                            feed_forward_norm=PartSpec("rmsnorm", norm, prefix="n2."))]
+        return ModelSpec("BlocksToyForCausalLM", d["width"], d["vocab"], d["positions"],
+                         PartSpec("token_embedding", {"vocab_size": d["vocab"]}, prefix="toy.emb."), layers,
+                         PartSpec("rmsnorm", norm, prefix="toy.norm."),
+                         PartSpec("lm_head", {"vocab_size": d["vocab"], "tied": True}))
+
+
+def blocks_toy_plain_forward(w, d, tokens):
+    T = len(tokens)
+    x = R.embedding(w["toy.emb.weight"], torch.tensor(tokens))
+    f = R.rope_inv_freq(16, 8, 50.0)
+    pos = torch.arange(T)
+
+    def attention(h, p):
+        q = (h @ w[p + "attn.q_proj.weight"].double().T).reshape(T, 4, 16)
+        k = (h @ w[p + "attn.k_proj.weight"].double().T).reshape(T, 2, 16)
+        v = (h @ w[p + "attn.v_proj.weight"].double().T).reshape(T, 2, 16)
+        a = R.attention(R.rope_interleaved(q, pos, f), R.rope_interleaved(k, pos, f), v, 0)
+        return a.reshape(T, 64) @ w[p + "attn.o_proj.weight"].double().T
+
+    def ffn(h, p):
+        return R.swiglu_ffn(h, w[p + "ff.gate_proj.weight"], w[p + "ff.down_proj.weight"], w[p + "ff.up_proj.weight"])
+
+    h = R.rmsnorm(x, w["toy.0.n.weight"], d["eps"])
+    x = x + attention(h, "toy.0.") + ffn(h, "toy.0.")              # both branches from the one norm
+    x = x + ffn(R.rmsnorm(x, w["toy.1.n.weight"], d["eps"]), "toy.1.")
+    x = x + attention(R.rmsnorm(x, w["toy.2.n1.weight"], d["eps"]), "toy.2.")
+    x = x + ffn(R.rmsnorm(x, w["toy.2.n2.weight"], d["eps"]), "toy.2.")
+    return R.rmsnorm(x, w["toy.norm.weight"], d["eps"]) @ w["toy.emb.weight"].double().T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_blocks_with_other_members_from_outside(tmp_path, dtype):
+    """Arrangements whose members are not the reference's four (one norm for two parallel branches; no mixer
+    at all) are registered here, named by a configuration layer by layer, and stepped under every schedule.
+    The two attentions share one table of angles, and the step's index tables are made once."""
+    from yalm_amd import Engine, Model, register_architecture, write_random_model
+    from yalm_amd.config import unregister_architecture
+    from yalm_amd.parts import unregister_part
+    define_toy_blocks()
+    register_architecture("BlocksToyForCausalLM", BlocksToyConfig, replace=True)
+    try:
+        d = {"architectures": ["BlocksToyForCausalLM"], "width": 48, "hidden": 80, "vocab": 97, "positions": 160,
+             "eps": 3e-6}
+        folder = write_random_model(str(tmp_path / "blocks_toy"), d, seed=6)
+        model = Model.from_folder(folder, dtype=helpers.torch_dtype(dtype), device=DEV)
+        assert model.graph_safe()
+        engine = Engine(model, max_tokens=1024)
+        assert engine.cache.group_of(1) is None and engine.cache.group_of(0) is engine.cache.group_of(2)
+        assert model.blocks[0].mixer.position is model.blocks[2].mixer.position          # one table for both
+        assert model.blocks[0].mixer.position.table.shape[0] == 160
+        assert [m.name for m in engine._prompt_tables] == ["kv_tiles"]                   # asked twice, made once
+        cfg, w = R.read_folder(folder)
+        if dtype == "bfloat16":
+            w = {k: v if v.dim() <= 1 else v.to(torch.bfloat16) for k, v in w.items()}
+        rng = np.random.default_rng(5)
+        requests = {rid: [int(t) for t in rng.integers(0, d["vocab"], size=n)]
+                    for rid, n in (("a", 40), ("b", 2), ("c", 130), ("d", 65))}
+        for steps in (schedules.whole(requests), schedules.tail_one_by_one(requests, 32),
+                      schedules.batches(requests, [["a", "b"], ["c", "d"]], {"a": 9, "b": 1, "c": 100, "d": 64}),
+                      schedules.interleaved(requests, [["a", "b"], ["c", "d"]], {"a": 9, "b": 1, "c": 100, "d": 64},
+                                            [0, 3])):
+            out = schedules.replay_in_process(engine, steps)
+            got = schedules.per_request(steps, out, requests)
+            for rid, toks in requests.items():
+                want = blocks_toy_plain_forward(w, d, toks).float().numpy()
+                helpers.check_logits(got[rid], want, dtype, "blocks toy %s %s" % (dtype, rid))
+        assert engine.graphs_captured > 0
+    finally:
+        unregister_architecture("BlocksToyForCausalLM")
+        unregister_part("block", "toy_parallel")
+        unregister_part("block", "toy_feed_forward_only")

@@ -19,15 +19,43 @@ class PartSpec:
         return hash((self.kind, self.prefix, repr(sorted(self.params.items(), key=lambda kv: kv[0]))))
 
 
-@dataclass(frozen=True)
 class LayerSpec:
-    """A layer: the arrangement (block kind) and the parts it arranges."""
-    block: str                      # e.g. "prenorm_residual"
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
-    prefix: str                     # e.g. "model.layers.3."
+    """A layer: the arrangement (block kind), the members it arranges, by the names that block
+    kind knows, and the layer's place in the tensor names.  The reference's arrangement
+    ("prenorm_residual") has the members mixer, feed_forward, mixer_norm and feed_forward_norm;
+    another block kind has the members it needs (one norm in front of a mixer and a feed-forward
+    that run side by side, no feed-forward at all, ...) and reads only those.  Members are given by
+    name, `LayerSpec("prenorm_residual", prefix="model.layers.3.", mixer=..., ...)`, or as a
+    dictionary `parts`, and read back as attributes or with `part(name)`.  The member called
+    `mixer`, if there is one, is the one whose cache line the schedule speaks of."""
+
+    def __init__(self, block, parts=None, prefix="", **members):
+        merged = dict(parts or {})
+        merged.update(members)
+        for name, spec in merged.items():
+            if not isinstance(spec, PartSpec):
+                raise TypeError("member %r of a layer is a %s, not a PartSpec" % (name, type(spec).__name__))
+        self.__dict__["block"] = block                 # e.g. "prenorm_residual"
+        self.__dict__["parts"] = merged
+        self.__dict__["prefix"] = prefix               # e.g. "model.layers.3."
+
+    def part(self, name, default=None):
+        return self.parts.get(name, default)
+
+    def __getattr__(self, name):
+        parts = self.__dict__.get("parts")
+        if parts is not None and name in parts:
+            return parts[name]
+        raise AttributeError("this layer (%s) has no member %r" % (self.__dict__.get("block"), name))
+
+    def __setattr__(self, name, value):
+        raise AttributeError("a LayerSpec is not changed after it is made")
+
+    def __eq__(self, other):
+        return isinstance(other, LayerSpec) and (self.block, self.parts, self.prefix) == (other.block, other.parts, other.prefix)
+
+    def __repr__(self):
+        return "LayerSpec(%r, %r, prefix=%r)" % (self.block, self.parts, self.prefix)
 
 
 @dataclass(frozen=True)
@@ -74,7 +102,8 @@ class ModelSpec:
             elif e.cache not in writers:
                 raise ValueError("schedule entry %d reads cache line %d before any entry wrote it" % (i, e.cache))
             else:
-                a = self.layers[self.schedule[writers[e.cache]].layer].mixer
-                b = self.layers[e.layer].mixer
-                if a.kind != b.kind:
-                    raise ValueError("schedule entry %d (%s) cannot read the cache line of a %s" % (i, b.kind, a.kind))
+                a = self.layers[self.schedule[writers[e.cache]].layer].part("mixer")
+                b = self.layers[e.layer].part("mixer")
+                if a is None or b is None or a.kind != b.kind:
+                    raise ValueError("schedule entry %d (%s) cannot read the cache line of a %s"
+                                     % (i, getattr(b, "kind", "no mixer"), getattr(a, "kind", "layer without a mixer")))

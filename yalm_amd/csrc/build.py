@@ -1,11 +1,14 @@
 """Builds the gfx950 kernel library with hipcc (no torch headers, no pybind).
 
 `library_path()` returns the built library, compiling it first if there is
-none; `build(force=True)` always compiles.  The library is placed in-tree
+none or if the one there was built from other sources (a digest of the .hip
+and .h files and of the compiler flags is kept beside the library);
+`build(force=True)` always compiles.  The library is placed in-tree
 (`yalm_amd/lib/`); if the tree cannot be written, in a per-user folder under
 the system's temporary directory.
 """
 import concurrent.futures
+import hashlib
 import os
 import shutil
 import subprocess
@@ -23,6 +26,25 @@ FLAGS = ["--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC", "-Xclang", "-ta
 
 def sources():
     return sorted(f for f in os.listdir(HERE) if f.endswith(".hip"))
+
+
+def sources_digest():
+    """A digest of everything the library is built from: the .hip and .h files of this folder and the flags."""
+    h = hashlib.sha256(" ".join(FLAGS).encode())
+    for name in sorted(f for f in os.listdir(HERE) if f.endswith((".hip", ".h"))):
+        h.update(name.encode())
+        with open(os.path.join(HERE, name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
+
+
+def _built_from(lib):
+    """The digest recorded beside a built library, or None."""
+    try:
+        with open(lib + ".sources") as f:
+            return f.read().strip()
+    except OSError:
+        return None
 
 
 def _hipcc():
@@ -65,10 +87,16 @@ def _compile_one(hipcc, src, obj):
 
 def build(force=True, jobs=None):
     """Compiles every .hip file of this folder and links the library."""
+    digest = sources_digest()
     if not force:
+        stale = []
         for c in _candidates():
             if os.path.exists(c):
-                return c
+                if _built_from(c) == digest:
+                    return c
+                stale.append(c)
+        if stale:
+            _say("%s was built from other sources than the ones here: building again" % stale[0])
     hipcc = _hipcc()
     out_dir = _writable_dir()
     obj_dir = os.path.join(out_dir, "_build")
@@ -101,6 +129,9 @@ def build(force=True, jobs=None):
         raise RuntimeError("linking the kernel library failed:\n" + p.stderr)
     lib = os.path.join(out_dir, LIB_NAME)
     os.replace(tmp, lib)
+    with open(lib + ".sources.tmp%d" % os.getpid(), "w") as f:
+        f.write(digest + "\n")
+    os.replace(lib + ".sources.tmp%d" % os.getpid(), lib + ".sources")
     shutil.rmtree(obj_dir, ignore_errors=True)
     _say("built %s in %.0f s" % (lib, time.time() - t0))
     return lib

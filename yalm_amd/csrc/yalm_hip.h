@@ -55,14 +55,15 @@ int yalm_gemm_norm_qkv_rope(const float* x, const float* norm_w, float eps, cons
                             int K, int n_heads, int n_kv_heads, int head_dim, int rotary_dim, int n_pages,
                             int page_layout, hipStream_t stream);
 
-// Residual add and the next RMSNorm in one for 17..64 rows, or more with K a multiple of 64 (bfloat16): C float32 [M,N] += A[M,K] * W[N,K]^T, then
-// h_out bfloat16 [M,N] = C_new * rsqrt(mean(C_new^2) + eps) * norm_w.  workspace: at least M * N floats (more lets
-// it split K).  Refuses (YALM_ERR_ARG) other shapes.
-// The K slices of A[M,K] * W[N,K]^T for 17..64 rows, or more with K a multiple of 64 (bfloat16), left unadded: workspace [*slices][M][N] float32, for a
-// consumer that adds them itself (yalm_rope_kv_write).  Needs at least M * N floats; refuses (YALM_ERR_ARG) other shapes.
+// The K slices of A[M,K] * W[N,K]^T for 17..64 rows, or more with K a multiple of 64 (bfloat16), left unadded:
+// workspace [*slices][M][N] float32, for a consumer that adds them itself (yalm_rope_kv_write).  Needs at least
+// M * N floats; refuses (YALM_ERR_ARG) other shapes.
 int yalm_gemm_partial(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N, int K,
                       int* slices, hipStream_t stream);
 
+// Residual add and the next RMSNorm in one for 17..64 rows, or more with K a multiple of 64 (bfloat16):
+// C float32 [M,N] += A[M,K] * W[N,K]^T, then h_out bfloat16 [M,N] = C_new * rsqrt(mean(C_new^2) + eps) * norm_w.
+// workspace: at least M * N floats (more lets it split K).  Refuses (YALM_ERR_ARG) other shapes.
 int yalm_gemm_add_norm(const void* A, const void* W, float* C, float* workspace, long workspace_floats, int M, int N,
                        int K, const float* norm_w, float eps, void* h_out, hipStream_t stream);
 
@@ -207,6 +208,12 @@ int yalm_argmax(const float* logits, int* out, int R, int V, hipStream_t stream)
 int yalm_sample(const float* logits, const float* u, float temperature, int* out, int R, int V, hipStream_t stream);
 // prob[r] = softmax(logits[r, :])[index[r]] (src/sampler.cpp:11-25)
 int yalm_token_prob(const float* logits, const int* index, float* prob, int R, int V, hipStream_t stream);
+
+// Yardsticks for the measurement (probes.hip): a kernel that only reads `bytes` bytes once with `workgroups`
+// workgroups (out: 1,024 words of scratch), and a loop of matrix-core instructions on registers (shape 32:
+// v_mfma_f32_32x32x16_bf16, 16: v_mfma_f32_16x16x32_bf16; *flops, host memory, receives the launch's operations).
+int yalm_probe_read(const void* src, long bytes, unsigned int* out, int workgroups, hipStream_t stream);
+int yalm_probe_mfma(int shape, int iters, int workgroups, float* out, double* flops, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -66,9 +66,10 @@ class StepContext:
     """mode: 'prefill' (sequences that start at position 0, whole prompts, packed)
     or 'decode' (one token per sequence).  Device tensors, all int32:
       tokens[T], tok_seq[T] (row of the batch), tok_pos[T] (position in its sequence),
-      seq_slot[B] (-1: padding row), seq_len[B] (length after this step), cu_seqlens[B+1],
-      seq_tile0[B+1] (prefill: first 64-token tile of each sequence in the staging area; n_tiles in all),
-      tile_order (prefill, may be None: the order in which attention should take the tiles).
+      seq_slot[B] (-1: padding row), seq_len[B] (length after this step), cu_seqlens[B+1].
+    tables: prefill only; {maker's name: {key: int32 device tensor or host value}}, the index tables that parts
+    asked for through their `prompt_tables` (made once a step and uploaded with the tensors above; the
+    attention's staging tiles and the order in which it takes them are such a table).
     max_position: the largest position in the step (host value, for table checks).
     host_slots, host_n_tokens, host_start: the step's real sequences as host lists (a decode step's
     padding rows, seq_slot -1, are not in them), for parts whose launches depend on host values.
@@ -82,9 +83,7 @@ class StepContext:
         self.act_dtype = act_dtype
         self.shared_lines = set(shared_lines)
         self.tokens = self.tok_seq = self.tok_pos = self.seq_slot = self.seq_len = self.cu_seqlens = None
-        self.seq_tile0 = None
-        self.tile_order = None
-        self.n_tiles = 0
+        self.tables = {}
         self.x = None                     # the residual stream of the step, float32 [T, dim]
         self.normed = {}                  # id(norm part) -> (xn, ss, eps): activations a producer emitted for it
         self.pages_bucket = 1 << 30       # decode: no sequence of the step has more pages than this

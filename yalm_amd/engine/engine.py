@@ -108,6 +108,7 @@ class Engine:
         self.use_graphs = use_graphs
         self.max_graphs = max(1, int(max_graphs))
         self._widest_row = model.widest_row()
+        self._prompt_tables = model.prompt_tables()     # index tables that parts want made for a step of whole prompts
         self._segments = model.decode_segments()        # the parts are fixed from here on: asked once, not every step
         self._any_graph = any(safe for safe, _, _ in self._segments)
         for text in model.describe()[1]:                # a slow fallback is said once, not hidden
@@ -277,10 +278,16 @@ class Engine:
         for i, w in enumerate(want):
             rows.extend(int(cu[i]) + j for j in w)
         R = len(rows)
-        tile0 = np.zeros(B + 1, dtype=np.int32)
-        np.cumsum([(n + PAGE - 1) // PAGE for n in n_tok], out=tile0[1:])
-        order = kernels.prefill_tile_order(n_tok)
-        n_meta = 3 * T + 4 * B + 2 + R + len(order)
+        # what the parts asked for beside the common tables: made once a step, whoever and however many ask
+        extra, host_values = [], {}
+        for make in self._prompt_tables:
+            values = host_values[make.name] = {}
+            for key, v in make(n_tok).items():
+                if isinstance(v, np.ndarray):
+                    extra.append((make.name, key, np.ascontiguousarray(v, dtype=np.int32).ravel()))
+                else:
+                    values[key] = v
+        n_meta = 3 * T + 3 * B + 1 + R + sum(len(a) for _, _, a in extra)
         host = np.empty(n_meta, dtype=np.int32)
         host[0:T] = np.concatenate([np.asarray(t, dtype=np.int32) for t in tokens])
         host[T:2 * T] = np.repeat(np.arange(B, dtype=np.int32), n_tok)
@@ -289,18 +296,23 @@ class Engine:
         host[o:o + B] = slots
         host[o + B:o + 2 * B] = new_lens
         host[o + 2 * B:o + 3 * B + 1] = cu
-        host[o + 3 * B + 1:o + 4 * B + 2] = tile0
-        host[o + 4 * B + 2:o + 4 * B + 2 + R] = rows
-        host[o + 4 * B + 2 + R:] = order
+        at = o + 3 * B + 1
+        host[at:at + R] = rows
+        at += R
+        for _, _, a in extra:
+            host[at:at + len(a)] = a
+            at += len(a)
         meta = self.ws.get("meta", (n_meta,), torch.int32)
         meta.copy_(torch.from_numpy(host))
         ctx = self._context("prefill", self.ws, meta, T, B, max(n_tok) - 1)
-        ctx.seq_tile0 = meta[o + 3 * B + 1:o + 4 * B + 2]
-        ctx.tile_order = meta[o + 4 * B + 2 + R:]
-        ctx.n_tiles = int(tile0[-1])
+        at = o + 3 * B + 1 + R
+        ctx.tables = host_values
+        for name, key, a in extra:
+            ctx.tables[name][key] = meta[at:at + len(a)]
+            at += len(a)
         ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), list(n_tok), [0] * B
         V = self.model.vocab_size
-        want_rows = meta[o + 4 * B + 2:o + 4 * B + 2 + R]
+        want_rows = meta[o + 3 * B + 1:o + 3 * B + 1 + R]
         if targets is not None:
             probs = torch.empty(R, dtype=torch.float32, device=self.device)
             flat = torch.tensor([tok for t in targets for tok in t], dtype=torch.int32, device=self.device)

@@ -32,10 +32,11 @@ class Model:
         self.config = config
         self.dim = spec.dim
         self.vocab_size = spec.vocab_size
-        self.embedding = build_part("embedding", spec.embedding, spec.dim, "")
-        self.blocks = [build_block(ls, spec.dim) for ls in spec.layers]
-        self.final_norm = build_part("norm", spec.final_norm, spec.dim, "")
-        self.head = build_part("head", spec.head, spec.dim, "", embedding=self.embedding)
+        with parts_base.sharing():        # parts that follow from their spec alone are built once (position tables)
+            self.embedding = build_part("embedding", spec.embedding, spec.dim, "")
+            self.blocks = [build_block(ls, spec.dim) for ls in spec.layers]
+            self.final_norm = build_part("norm", spec.final_norm, spec.dim, "")
+            self.head = build_part("head", spec.head, spec.dim, "", embedding=self.embedding)
         self.schedule = list(spec.schedule)
         import inspect
         self._takes_next_norm = ["next_norm" in inspect.signature(b.forward).parameters for b in self.blocks]
@@ -53,8 +54,13 @@ class Model:
         return [self.embedding] + self.blocks + [self.final_norm, self.head]
 
     def all_parts(self):
-        for p in self.top_parts():
-            yield from _walk(p)
+        """Every part once (a part that several others share is named by each of them)."""
+        seen = set()
+        for top in self.top_parts():
+            for p in _walk(top):
+                if id(p) not in seen:
+                    seen.add(id(p))
+                    yield p
 
     def param_specs(self):
         seen, out = set(), []
@@ -116,7 +122,8 @@ class Model:
         out = {}
         for e in self.schedule:
             if e.writes_cache:
-                out[e.cache] = self.blocks[e.layer].mixer.cache_request()
+                mixer = getattr(self.blocks[e.layer], "mixer", None)     # a block without a mixer keeps nothing
+                out[e.cache] = mixer.cache_request() if mixer is not None else None
         return out
 
     def prepare(self, n_positions):
@@ -177,6 +184,17 @@ class Model:
                 if is_slow and text not in slow:
                     slow.append(text)
         return lines, slow
+
+    def prompt_tables(self):
+        """The makers of index tables that parts ask for in a step of whole prompts (a part names them in
+        `prompt_tables`), each once, by its name.  A maker is called with the step's token counts and gives
+        {key: int32 array (uploaded with the step's metadata) or host value}; parts find the result in
+        ctx.tables[maker.name]."""
+        out = {}
+        for p in self.all_parts():
+            for make in getattr(p, "prompt_tables", ()):
+                out.setdefault(make.name, make)
+        return list(out.values())
 
     def widest_row(self):
         """The most elements any part keeps for one token of a step (a part says so with `row_elements()`;

@@ -664,3 +664,36 @@ def token_prob(logits, index, out):
                                                 _need(index, "index", torch.int32, (R,)),
                                                 _need(out, "out", torch.float32, (R,)), R, V, _stream()), "token_prob")
     return out
+
+
+def probe_read(src, workgroups=2048):
+    """Queues a kernel that reads the tensor `src` once and does nothing else (a yardstick for what the
+    memory gives a kernel).  Returns the bytes it reads."""
+    n = src.numel() * src.element_size()
+    piece = 256 * 8 * 16
+    if n < piece:
+        raise ValueError("probe_read needs at least %d bytes" % piece)
+    out = _probe_scratch(src.device)
+    library.check(library.lib().yalm_probe_read(_need(src, "src"), n, out.data_ptr(), int(workgroups), _stream()),
+                  "probe_read")
+    return n // piece * piece
+
+
+def probe_mfma(shape, iters, workgroups=2048):
+    """Queues a loop of matrix-core instructions on registers (shape 32: 32x32x16, 16: 16x16x32, bfloat16).
+    Returns the floating-point operations of the launch."""
+    out = _probe_scratch(torch.device("cuda", torch.cuda.current_device()))
+    flops = ctypes.c_double(0.0)
+    library.check(library.lib().yalm_probe_mfma(int(shape), int(iters), int(workgroups), out.data_ptr(),
+                                                ctypes.byref(flops), _stream()), "probe_mfma")
+    return flops.value
+
+
+_probe_out = {}
+
+
+def _probe_scratch(device):
+    key = str(device)
+    if key not in _probe_out:
+        _probe_out[key] = torch.zeros(1024, dtype=torch.int32, device=device)
+    return _probe_out[key]

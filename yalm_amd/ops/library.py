@@ -43,9 +43,11 @@ _SIGNATURES = {
     "yalm_argmax": (_I, [_P, _P, _I, _I, _P]),
     "yalm_sample": (_I, [_P, _P, _F, _P, _I, _I, _P]),
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
+    "yalm_probe_read": (_I, [_P, ctypes.c_long, _P, _I, _P]),
+    "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 
 class KernelError(RuntimeError):

@@ -34,8 +34,24 @@ RESIDENT_WORKGROUPS = 512       # decode-attention workgroups that the chip hold
 ROPE_TILES_MIN_TOKENS = 320
 
 
+def kv_tiles(n_tok):
+    """The index tables a step of whole prompts needs for attention over its own keys and values, which are
+    staged in page-shaped tiles of 64 positions: seq_tile0[B + 1], the first tile of each sequence (n_tiles in
+    all), and tile_order, the order in which the attention kernel should take the tiles of queries."""
+    import numpy as np
+    tile0 = np.zeros(len(n_tok) + 1, dtype=np.int32)
+    np.cumsum([(n + kernels.PAGE - 1) // kernels.PAGE for n in n_tok], out=tile0[1:])
+    return {"seq_tile0": tile0, "tile_order": np.asarray(kernels.prefill_tile_order(n_tok), dtype=np.int32),
+            "n_tiles": int(tile0[-1])}
+
+
+kv_tiles.name = "kv_tiles"
+
+
 @part("mixer", "gqa_attention")
 class GQAttention(Part):
+    prompt_tables = (kv_tiles,)
+
     def __init__(self, spec, dim, prefix):
         super().__init__(spec, dim, prefix)
         p = spec.params
@@ -223,18 +239,20 @@ class GQAttention(Part):
         if prefill:
             # the step's own keys and values in page format; a line that later entries read
             # keeps them for those entries
+            tiles = ctx.tables["kv_tiles"]
+            seq_tile0, n_tiles = tiles["seq_tile0"], tiles["n_tiles"]
             tag = "attn.stage%d" % line if ctx.line_is_shared(line) else "attn.stage"
-            kst = ws.get(tag + ".k", (ctx.n_tiles, self.n_kv_heads, kernels.PAGE, self.head_dim), act)
-            vst = ws.get(tag + ".v", (ctx.n_tiles, self.n_kv_heads, self.head_dim, kernels.PAGE), act)
+            kst = ws.get(tag + ".k", (n_tiles, self.n_kv_heads, kernels.PAGE, self.head_dim), act)
+            vst = ws.get(tag + ".v", (n_tiles, self.n_kv_heads, self.head_dim, kernels.PAGE), act)
         else:
-            kst = vst = None
+            kst = vst = seq_tile0 = None
         if writes_cache:
             done = prefill and T >= ROPE_TILES_MIN_TOKENS and kernels.rope_kv_write_tiles(
-                qkv, q, kst, vst, ctx.cu_seqlens, ctx.seq_tile0, k_pages, v_pages, group.table, group.ring_pages,
+                qkv, q, kst, vst, ctx.cu_seqlens, seq_tile0, k_pages, v_pages, group.table, group.ring_pages,
                 ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads, self.n_kv_heads, self.head_dim, pos.rotary_dim,
                 slices=slices)
             if not done:
-                kernels.rope_kv_write(qkv, q, kst, vst, ctx.seq_tile0, k_pages, v_pages, group.table,
+                kernels.rope_kv_write(qkv, q, kst, vst, seq_tile0, k_pages, v_pages, group.table,
                                       group.ring_pages, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table,
                                       self.n_heads, self.n_kv_heads, self.head_dim, pos.rotary_dim, slices=slices)
         else:
@@ -246,9 +264,10 @@ class GQAttention(Part):
             lse = ws.get("attn.lse", (T, self.n_heads), torch.float32) if self.sinks else None
             if self.sinks and writes_cache:
                 sink_k, sink_v = group.line_sinks(line)
-                kernels.sink_store(kst, vst, ctx.seq_tile0, ctx.seq_slot, ctx.seq_len, sink_k, sink_v)
-            kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, ctx.seq_tile0, ctx.tok_seq, ctx.tok_pos,
-                                 self.n_heads, self.n_kv_heads, self.head_dim, self.window, ctx.tile_order, lse=lse)
+                kernels.sink_store(kst, vst, seq_tile0, ctx.seq_slot, ctx.seq_len, sink_k, sink_v)
+            kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, seq_tile0, ctx.tok_seq, ctx.tok_pos,
+                                 self.n_heads, self.n_kv_heads, self.head_dim, self.window, tiles.get("tile_order"),
+                                 lse=lse)
             if self.sinks:
                 sink_k, sink_v = group.line_sinks(line)
                 kernels.attn_sink_mix(q, o, lse, sink_k, sink_v, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, pos.table,

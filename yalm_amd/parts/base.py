@@ -5,7 +5,9 @@ residual stream and the prefix of its tensor names.  No part knows which model
 it is in.  Kinds of parts and the methods each must have:
 
   norm           forward(x_f32[R, dim], out[R, dim], ctx, row_index=None)
-  position       prepare(n_positions, device); used by a mixer, which owns it
+  position       prepare(n_positions, device); used by the mixers that name it (one instance per distinct
+                 PartSpec of a model if the class says `share_by_spec = True`: it then has no tensors
+                 of its own and its prefix means nothing)
   mixer          cache_request() -> KVRequest | StateRequest | None
                  forward(h[T, dim], x_f32[T, dim], ctx, line, writes_cache): adds its output to x
   feed_forward   forward(h[T, dim], x_f32[T, dim], ctx): adds its output to x
@@ -32,6 +34,7 @@ the cache or on per-sequence state.
 All of them: param_specs() -> [ParamSpec], load(get, compute_dtype, device),
 weight_bytes().  `h` is in the compute dtype (bfloat16 or float32); the
 residual stream `x` is always float32."""
+import threading
 from typing import Callable, Dict, List
 
 from ..config.spec import PartSpec
@@ -62,12 +65,43 @@ def part(role, kind):
     return deco
 
 
+_building = threading.local()        # .pools: the pools of the models this thread is building (innermost last)
+
+
+def _pools():
+    if not hasattr(_building, "pools"):
+        _building.pools = []
+    return _building.pools
+
+
+class sharing:
+    """While a model is built inside `with sharing():`, parts whose class says `share_by_spec = True`
+    (parts without tensors of their own, whose state follows from their PartSpec alone: the position
+    encodings) are built once per distinct (role, PartSpec, width) and handed to everyone who asks
+    for that spec.  The thirty-two attentions of a model then read one table of angles."""
+
+    def __enter__(self):
+        _pools().append({})
+        return _pools()[-1]
+
+    def __exit__(self, *exc):
+        _pools().pop()
+        return False
+
+
 def build_part(role, spec: PartSpec, dim: int, prefix: str, **extra):
     try:
         cls = _REGISTRY[role][spec.kind]
     except KeyError:
         raise ValueError("no %s part named %r is registered (known: %s)"
                          % (role, spec.kind, sorted(_REGISTRY[role]))) from None
+    pools = _pools()
+    if pools and getattr(cls, "share_by_spec", False) and not extra:
+        key = (role, spec, dim)
+        made = pools[-1].get(key)
+        if made is None:
+            made = pools[-1][key] = cls(spec, dim, prefix + spec.prefix)
+        return made
     return cls(spec, dim, prefix + spec.prefix, **extra)
 
 

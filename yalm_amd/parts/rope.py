@@ -45,6 +45,8 @@ def interleave_rows(w, n_heads, head_dim, rotary_dim):
 
 @part("position", "rope")
 class RotaryEncoding(Part):
+    share_by_spec = True              # no tensors of its own: mixers that name the same spec share one table
+
     def __init__(self, spec, dim, prefix):
         super().__init__(spec, dim, prefix)
         p = spec.params
@@ -80,6 +82,7 @@ class RotaryEncoding(Part):
 @part("position", "none")
 class NoPositionEncoding(Part):
     """No rotation at all (a mixer that needs no positions, or test parts)."""
+    share_by_spec = True
     rotary_dim = 0
     table = None
     n_positions = 0
