@@ -171,7 +171,7 @@ def kernel_cost(name, a, kw, kv_tokens, torch):
 def time_kernel_groups(calls, kv_tokens, torch, dtype, reps=5):
     """Every kernel of a step alone: the calls with the same face and shapes (one a layer) are captured into one
     graph in the order of the step, so that each reads weights that no call just before it has read, and the
-    graph is replayed between two events.  Returns {label: {calls, us, GB/s, TFLOP/s, frac, bound}}."""
+    graph is replayed between two events (the best of `reps` replays counts).  Returns {label: {calls, us, GB/s, TFLOP/s, frac, bound}}."""
     groups = {}
     for name, fn, a, kw in calls:
         label, nb, fl = kernel_cost(name, a, kw, kv_tokens, torch)
@@ -179,22 +179,35 @@ def time_kernel_groups(calls, kv_tokens, torch, dtype, reps=5):
         g["calls"].append((fn, a, kw))
     flush = torch.empty(1 << 29, dtype=torch.uint8, device="cuda:0")        # 512 MB: more than the caches hold
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def timed(graph):
+        graph.replay()
+        best = None
+        for _ in range(reps):
+            e0.record()
+            graph.replay()
+            e1.record()
+            e1.synchronize()
+            t = e0.elapsed_time(e1)
+            best = t if best is None else min(best, t)
+        return best
+
+    # every graph begins by overwriting 512 MB, so that no kernel finds its operands in a cache; the time of a
+    # graph that does only that is taken off (with it goes what starting a graph costs)
+    empty = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.graph(empty):
+        flush.zero_()
+    base = timed(empty)
     out = {}
     for label, g in groups.items():
         graph = torch.cuda.CUDAGraph()
         torch.cuda.synchronize()
         with torch.cuda.graph(graph):
+            flush.zero_()
             for fn, a, kw in g["calls"]:
                 fn(*a, **kw)
-        graph.replay()
-        total = 0.0
-        for _ in range(reps):
-            flush.zero_()
-            e0.record()
-            graph.replay()
-            e1.record()
-            e1.synchronize()
-            total += e0.elapsed_time(e1)
+        total = max(timed(graph) - base, 1e-4) * reps
         n = len(g["calls"])
         us = total / reps / n * 1e3
         gbs = g["bytes"] / us / 1e3
@@ -263,7 +276,14 @@ def main():
     torch.cuda.synchronize()
     sys.stderr.write("[bench] %d layers of random weights in %.1f s\n" % (n_layers, time.time() - t0))
     batches = sorted({args.batch} | {int(b) for b in args.points.split(",") if b})
-    engine = Engine(model, max_tokens=max(batches) * CONTEXT, max_batch=max(batches))
+    RAGGED_B, RAGGED_LENS = 64, (1024, 3072)
+    if args.ragged:
+        CONTEXT = max(CONTEXT, RAGGED_LENS[1] + args.ragged_new + 64)
+    most = max(batches + ([RAGGED_B] if args.ragged else []))
+    engine = Engine(model, max_tokens=most * CONTEXT, max_batch=most)
+    read_peak, mfma_peak = measured_peaks(torch, args.dtype)
+    sys.stderr.write("[bench] measured here: a kernel that only reads memory %.0f GB/s, a loop of matrix-core "
+                     "instructions %.0f TFLOP/s\n" % (read_peak, mfma_peak))
     t0 = time.time()
     n_graphs = engine.warmup(batches, min_len=PROMPT + 1, max_len=PROMPT + args.steps + args.warmup + 1)
     torch.cuda.synchronize()
@@ -294,6 +314,9 @@ def main():
         fl = prefill_flops(CFG, n_layers, PREFILL_LEN)
         prefill = {"value": round(PREFILL_LEN / sec, 1), "tokens": PREFILL_LEN, "ms": round(sec * 1e3, 3),
                    "frac": round(fl / sec / FLOP_PEAK[args.dtype], 4)}
+        if mfma_peak:
+            prefill["peak_measured"] = mfma_peak
+            prefill["peak_measured_unit"] = "TFLOP/s"
         sys.stderr.write("[bench] prefill %s\n" % prefill)
 
     # ---------------------------------------------------------------- decode
@@ -361,7 +384,7 @@ def main():
             "decode_mean_context": round(main_r["ctx"], 1), "kv_dtype": args.dtype, "page_tokens": PAGE,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(achieved * 1e9 / HBM_PEAK, 4)},
+                     "frac": round(achieved * 1e9 / HBM_PEAK, 4), "peak_measured": read_peak},
         "points": {"decode_b%d" % B: round(r["tok_s"], 1) for B, r in results.items() if B != args.batch},
         "points_roofline_frac": {"decode_b%d" % B: round(r["bytes"] / (r["ms"] * 1e-3) / HBM_PEAK, 4)
                                  for B, r in results.items()},
@@ -369,6 +392,91 @@ def main():
     }
     if prefill is not None:
         line["prefill"] = prefill
+
+    # ---------------------------------------------------------------- every kernel of a step alone
+    if args.kernels:
+        B = args.batch
+        L = int(main_r["ctx"])
+        slots = engine.start(B)
+        n = max(1, min(8, 48000 // L))
+        tokens = []
+        for i in range(0, B, n):
+            part = [torch.randint(0, V, (L - 1,), generator=gen).tolist() for _ in slots[i:i + n]]
+            tokens += sampler.sample(engine.step(slots[i:i + n], part), 0.0, list(range(len(part))), [0] * len(part))
+        graphs_on, engine.use_graphs = engine.use_graphs, False
+        try:
+            calls = record_kernel_calls(
+                lambda: sampler.draw(engine.step(slots, [[t] for t in tokens]), 0.0, list(range(B)), [0] * B))
+        finally:
+            engine.use_graphs = graphs_on
+        sync()
+        per_kernel = time_kernel_groups(calls, B * L, torch, args.dtype)
+        engine.release(slots)
+        total = sum(k["us"] * k["calls"] for k in per_kernel.values())
+        line["kernels"] = {"decode_b%d" % B: dict(per_kernel, sum_us=round(total, 1),
+                                                    step_us=round(main_r["ms"] * 1e3, 1), context=L)}
+        for label, k in per_kernel.items():
+            sys.stderr.write("[bench] decode B=%d  %-44s x%-3d %8.2f us  %8.1f GB/s  %7.2f TFLOP/s  %.3f of %s\n"
+                             % (B, label, k["calls"], k["us"], k["GB/s"], k["TFLOP/s"], k["frac"], k["bound"]))
+        sys.stderr.write("[bench] decode B=%d: kernels alone %.0f us, the step %.0f us\n" % (B, total, main_r["ms"] * 1e3))
+        if not args.no_prefill:
+            slots = engine.start(1)
+            prompt = torch.randint(0, V, (PREFILL_LEN,), generator=gen).tolist()
+            calls = record_kernel_calls(lambda: sampler.draw(engine.step(slots, [prompt]), 0.0, [0], [0]))
+            sync()
+            per_kernel = time_kernel_groups(calls, 0, torch, args.dtype)
+            engine.release(slots)
+            total = sum(k["us"] * k["calls"] for k in per_kernel.values())
+            line["kernels"]["prefill_%d" % PREFILL_LEN] = dict(per_kernel, sum_us=round(total, 1),
+                                                               step_us=round(prefill["ms"] * 1e3, 1))
+            for label, k in per_kernel.items():
+                sys.stderr.write("[bench] prefill %d  %-44s x%-3d %8.2f us  %8.1f GB/s  %7.2f TFLOP/s  %.3f of %s\n"
+                                 % (PREFILL_LEN, label, k["calls"], k["us"], k["GB/s"], k["TFLOP/s"], k["frac"],
+                                    k["bound"]))
+            sys.stderr.write("[bench] prefill %d: kernels alone %.0f us, the step %.0f us\n"
+                             % (PREFILL_LEN, total, prefill["ms"] * 1e3))
+
+    # ---------------------------------------------------------------- requests of unequal lengths through generate()
+    if args.ragged:
+        from yalm_amd.generate import GenerationStats, generate
+        lens = torch.randint(RAGGED_LENS[0], RAGGED_LENS[1] + 1, (RAGGED_B,), generator=gen).tolist()
+        prompts = [torch.randint(0, V, (n,), generator=gen).tolist() for n in lens]
+        engine.warmup([RAGGED_B], min_len=min(lens), max_len=max(lens) + args.ragged_new + 1)
+        stats = GenerationStats()
+        generate(engine, prompts, max_new_tokens=args.ragged_new, temperature=0.0, stop_ids=(), batch_size=RAGGED_B,
+                 sampler=sampler, stats=stats)
+        mean_len = int(sum(lens) / len(lens))
+        equal = decode(RAGGED_B, args.ragged_new - 8, 8, prompt_len=mean_len)
+        line["ragged"] = {
+            "requests": RAGGED_B, "prompt_min": min(lens), "prompt_max": max(lens), "prompt_mean": mean_len,
+            "new_tokens": args.ragged_new, "decode_tok_s": round(stats.decode_tokens_per_second, 1),
+            "ms_per_step": round(stats.decode_seconds / max(1, stats.decode_steps) * 1e3, 4),
+            "prefill_tok_s": round(stats.prefill_tokens_per_second, 1),
+            "equal_length_decode_tok_s": round(equal["tok_s"], 1), "equal_length_ms_per_step": round(equal["ms"], 4),
+            "roofline_frac": round(stats.bytes_read / max(1, stats.decode_steps + 1)
+                                   / (stats.decode_seconds / max(1, stats.decode_steps)) / HBM_PEAK, 4)}
+        sys.stderr.write("[bench] ragged %s\n" % line["ragged"])
+
+    # ---------------------------------------------------------------- the shape's whole workload, end to end
+    if args.sweep:
+        from yalm_amd.generate import GenerationStats, generate
+        B = args.batch
+        prompts = [torch.randint(0, V, (first,), generator=gen).tolist() for _ in range(B)]
+        engine.warmup([B], min_len=first, max_len=last + 1)
+        stats = GenerationStats()
+        t = time.perf_counter()
+        generate(engine, prompts, max_new_tokens=last - first, temperature=0.0, stop_ids=(), batch_size=B,
+                 sampler=sampler, stats=stats)
+        sync()
+        sec = time.perf_counter() - t
+        line["sweep"] = {
+            "batch": B, "prompt_tokens": first, "new_tokens": last - first, "seconds": round(sec, 3),
+            "tok_s_prompt_and_new": round((stats.prompt_tokens + stats.new_tokens) / sec, 1),       # src/main.cpp:139
+            "prefill_tok_s": round(stats.prefill_tokens_per_second, 1),
+            "decode_tok_s": round(stats.decode_tokens_per_second, 1),
+            "decode_ms_per_step": round(stats.decode_seconds / max(1, stats.decode_steps) * 1e3, 4),
+            "GB_per_s": round(stats.bytes_read / sec / 1e9, 1)}
+        sys.stderr.write("[bench] sweep %s\n" % line["sweep"])
     print(json.dumps(line), flush=True)
     return 0
 
