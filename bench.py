@@ -100,7 +100,7 @@ def measured_peaks(torch, dtype):
     return round(best_read, 1), round(best_mfma, 1)
 
 
-KERNEL_FACES = ("embed", "rmsnorm", "gemm", "gemm_norm", "gemm_norm_qkv_rope", "gemm_add_norm", "gemm_partial",
+KERNEL_FACES = ("embed", "rmsnorm", "gemm", "gemm_norm", "gemm_norm_qkv_rope", "gemm_add_norm", "gemm_add_emit", "gemm_partial",
                 "gemm_chain", "gemm_chain_qkv_rope", "rope_kv_write", "rope_kv_write_tiles", "attn_prefill",
                 "attn_decode", "sink_store", "attn_sink_mix", "argmax")
 
@@ -131,7 +131,7 @@ def kernel_cost(name, a, kw, kv_tokens, torch):
     a decode attention reads, summed over its sequences."""
     def nbytes(*ts):
         return sum(t.numel() * t.element_size() for t in ts if torch.is_tensor(t))
-    gemm_w = {"gemm": 1, "gemm_chain": 1, "gemm_add_norm": 1, "gemm_partial": 1, "gemm_norm": 3,
+    gemm_w = {"gemm": 1, "gemm_chain": 1, "gemm_add_norm": 1, "gemm_add_emit": 1, "gemm_partial": 1, "gemm_norm": 3,
               "gemm_norm_qkv_rope": 3, "gemm_chain_qkv_rope": 2}
     if name in gemm_w:
         x, w = a[0], a[gemm_w[name]]

@@ -324,3 +324,44 @@ def test_a_step_whose_widest_buffer_would_pass_the_checked_size_is_refused(folde
         s2 = engine.start(1)
         engine.step(s2, [list(range(15))], [list(range(14))])
     engine.release(slots + s2)
+
+
+# widths that let every product of a decode step of 17..128 rows take the kernels that split K and chain the norms
+# (K a multiple of 64 beyond 64 rows), and one that does not (hidden 144: beyond 64 rows its down projection goes
+# another way)
+MID_ROWS = dict(MANY_ROWS, intermediate_size=192)
+MID_ROWS_ODD = dict(MANY_ROWS, intermediate_size=144, hidden_size=136, num_attention_heads=2, num_key_value_heads=1)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("n,which", [(40, "even"), (100, "even"), (23, "odd"), (90, "odd")])
+def test_decode_batches_of_17_to_128_rows(tmp_path_factory, n, which, dtype):
+    """Decode steps of 17..128 sequences: the products whose K is split over workgroups, the kernel that adds the
+    slices to the residual stream and prepares the next norm, and the consumers that scale their sums row by row.
+    Sequences of unequal lengths, the shorter ones end earlier (the batch shrinks through the buckets); every fifth
+    request is compared with the plain implementation at every place."""
+    from yalm_amd.engine import Engine, Model
+    cfg = MID_ROWS if which == "even" else MID_ROWS_ODD
+    folder = helpers.make_folder(tmp_path_factory.mktemp("mid_rows"), "mid_rows_" + which, cfg, seed=30)
+    rng = np.random.default_rng(31 + n)
+    lengths = [int(x) for x in rng.integers(6, 80, size=n)]
+    requests = helpers.random_requests(cfg, lengths, seed=32)
+    first = {rid: max(1, len(t) - 5 - (i % 7)) for i, (rid, t) in enumerate(requests.items())}
+    steps = schedules.batches(requests, [list(requests)], first)
+    for s in steps:
+        for e in s["entries"]:
+            if int(e["id"][1:]) % 5:
+                e["want"] = []
+    model = Model.from_folder(folder, dtype=helpers.torch_dtype(dtype), device="cuda:0")
+    engine = Engine(model, max_tokens=schedules.max_tokens_needed(steps), max_batch=n)
+    out = schedules.replay_in_process(engine, steps)
+    got = {rid: [] for rid in requests if int(rid[1:]) % 5 == 0}
+    for s in steps:
+        r = 0
+        for e in s["entries"]:
+            for _ in e["want"]:
+                got[e["id"]].append(out[s["step"]][r])
+                r += 1
+    for rid, rows in got.items():
+        want = helpers.plain_logits(folder, tuple(requests[rid]), dtype)
+        helpers.check_logits(np.stack(rows), want, dtype, "%d rows (%s) %s request %s" % (n, which, dtype, rid))

@@ -1297,3 +1297,57 @@ def test_gemm_add_norm(M, N, Kd, small_workspace):
     close(h, R.rmsnorm(want_x, nw, eps), torch.bfloat16, "normed")
     with pytest.raises(ValueError):
         k.gemm_add_norm(a.to(DEV), w.to(DEV), x, nw.to(DEV), eps, h, torch.empty(M * N - 1, device=DEV))
+
+
+@pytest.mark.parametrize("small_workspace", [False, True])
+@pytest.mark.parametrize("M,N,Kd,N2", [(17, 4096, 4096, 6144), (64, 104, 264, 48), (40, 4096, 14336, 320),
+                                       (33, 96, 64, 200), (65, 4096, 4096, 1000), (128, 1088, 1024, 96)])
+def test_gemm_add_emit_and_its_consumers(M, N, Kd, N2, small_workspace):
+    """The norm chain of 17..128 rows: x += a W^T with the next norm only prepared (activations times the norm's
+    weights, partial sums of squares), and the consumers that scale their sums row by row: a plain product, a gated
+    one, and K slices left for another kernel to add.  Together they must give what a finished norm in front of the
+    same products gives."""
+    k = K()
+    a = rnd((M, Kd), 90, torch.bfloat16)
+    w = rnd((N, Kd), 91, torch.bfloat16, scale=1 / math.sqrt(Kd))
+    x0 = rnd((M, N), 92, scale=2.0)
+    x0[M // 2] *= 37.0                                   # rows of very different sizes: every row has its own scale
+    x0[0] *= 1e-3
+    nw = (1 + 0.1 * rnd((N,), 93)).float()
+    eps = 1e-5
+    x = x0.clone().to(DEV)
+    xn = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
+    parts = k.gemm_add_emit_parts(N)
+    assert parts == (N + 1023) // 1024
+    ss = torch.full((M, parts), float("nan"), device=DEV)
+    ws = torch.empty(M * N if small_workspace else k.fused_workspace_floats(M, N, Kd), device=DEV)
+    assert k.can_add_emit(M, Kd, torch.bfloat16) and not k.can_add_emit(16, Kd, torch.bfloat16)
+    k.gemm_add_emit(a.to(DEV), w.to(DEV), x, nw.to(DEV), xn, ss, ws)
+    want_x = x0.double() + a.double() @ w.double().T
+    close(x, want_x, torch.float32, "residual", factor=4)
+    close(xn, want_x * nw.double(), torch.bfloat16, "activations times the norm's weights")
+    close(ss.sum(dim=1), (want_x ** 2).sum(dim=1), torch.float32, "sums of squares", factor=4)
+    h = R.rmsnorm(want_x, nw, eps)                       # what the consumers' products must be products of
+    # a plain consumer (the head's epilogue) and the K slices of one
+    w2 = rnd((N2, N), 94, torch.bfloat16, scale=1 / math.sqrt(N))
+    want = h @ w2.double().T
+    out = torch.empty((M, N2), device=DEV)
+    ws2 = torch.full((k.gemm_workspace_floats(M, N2, N),), float("nan"), device=DEV)
+    k.gemm(xn, w2.to(DEV), out, k.EPI_STORE_F32, workspace=ws2, scale_from=(ss, eps))
+    close(out, want, torch.bfloat16, "scaled product")
+    if k.can_gemm_partial(M, N, torch.bfloat16):
+        ws3 = torch.full((k.fused_workspace_floats(M, N2, N),), float("nan"), device=DEV)
+        slices = k.gemm_partial(xn, w2.to(DEV), ws3, scale_from=(ss, eps))
+        close(ws3[:slices * M * N2].view(slices, M, N2).sum(dim=0), want, torch.bfloat16, "scaled slices")
+    # a gated consumer
+    H = 72
+    wg = rnd((H, N), 95, torch.bfloat16, scale=1 / math.sqrt(N))
+    wu = rnd((H, N), 96, torch.bfloat16, scale=1 / math.sqrt(N))
+    from yalm_amd.parts.swiglu import interleave_gate_up
+    wgu = interleave_gate_up(wg, wu).to(DEV)
+    mid = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
+    ws4 = torch.full((k.gemm_workspace_floats(M, wgu.shape[0], N),), float("nan"), device=DEV)
+    k.gemm(xn, wgu, mid, k.EPI_GATED, hidden=H, workspace=ws4, scale_from=(ss, eps))
+    close(mid, R.silu(h @ wg.double().T) * (h @ wu.double().T), torch.bfloat16, "scaled gated product", factor=2)
+    with pytest.raises(Exception):                        # a row scale is for these batches only
+        k.gemm(xn[:8].contiguous(), w2.to(DEV), out[:8].contiguous(), k.EPI_STORE_F32, scale_from=(ss[:8].contiguous(), eps))

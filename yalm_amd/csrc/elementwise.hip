@@ -130,12 +130,22 @@ extern "C" int yalm_rmsnorm(const float* x, const void* w, int w_dtype, void* ou
   return YALM_ERR_DTYPE;
 }
 
+__device__ __forceinline__ void store_pair(float* dst, float a, float b) {
+  *reinterpret_cast<float2*>(dst) = make_float2(a, b);
+}
+__device__ __forceinline__ void store_pair(bf16* dst, float a, float b) {
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+  bf16x2 v = {static_cast<bf16>(a), static_cast<bf16>(b)};
+  *reinterpret_cast<bf16x2*>(dst) = v;
+}
+
 // ---------------------------------------------------------------------------
 // rotation of q and k + write of k and v into the pages of the cache
-// grid (T, n_heads + 2 n_kv_heads); one wave per (token, head); a lane per pair
+// grid (T, ceil((n_heads + 2 n_kv_heads) / ROPE_JOBS)); one wave per (token, head); a lane per pair
 // ---------------------------------------------------------------------------
+constexpr int ROPE_JOBS = 1;                     // (token, head) jobs a workgroup: a wave each
 template <typename T>
-__global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_stage,
+__global__ __launch_bounds__(ROPE_JOBS * WAVE) void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restrict__ q_out, T* __restrict__ k_stage,
                                      T* __restrict__ v_stage, const int* __restrict__ seq_tile0,
                                      T* __restrict__ k_pages, T* __restrict__ v_pages,
                                      const int* __restrict__ block_table, int table_stride, int ring_pages,
@@ -144,14 +154,41 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
                                      const float2* __restrict__ cos_sin, int n_positions, int n_heads,
                                      int n_kv_heads, int hd, int rotary_dim, int n_pages, int page_layout, int slices,
                                      long plane) {
-  // qkv may be `slices` partial products [slices][T][Q + 2 KV] of a GEMM that split K: added here, in order
+  // qkv may be `slices` partial products [slices][T][Q + 2 KV] of a GEMM that split K: added here, in order;
+  // the loads of four slices are asked for together
   auto rd = [&](const float* p) {
     float v = p[0];
-    for (int s = 1; s < slices; ++s) v += p[(size_t)s * plane];
+    int s = 1;
+    for (; s + 4 <= slices; s += 4) {
+      const float a = p[(size_t)s * plane], b = p[(size_t)(s + 1) * plane], c = p[(size_t)(s + 2) * plane],
+                  d = p[(size_t)(s + 3) * plane];
+      v += a; v += b; v += c; v += d;
+    }
+    for (; s < slices; ++s) v += p[(size_t)s * plane];
     return v;
   };
-  int t = blockIdx.x;
-  int job = blockIdx.y;
+  const bool pairs_aligned = ((((uintptr_t)qkv) | ((uintptr_t)q_out)) & 7) == 0;
+  auto rd2 = [&](const float* p) {                // an adjacent pair (head sizes are even)
+    if (!pairs_aligned) return make_float2(rd(p), rd(p + 1));
+    float2 v = *reinterpret_cast<const float2*>(p);
+    int s = 1;
+    for (; s + 4 <= slices; s += 4) {
+      const float2 a = *reinterpret_cast<const float2*>(p + (size_t)s * plane),
+                   b = *reinterpret_cast<const float2*>(p + (size_t)(s + 1) * plane),
+                   c = *reinterpret_cast<const float2*>(p + (size_t)(s + 2) * plane),
+                   d = *reinterpret_cast<const float2*>(p + (size_t)(s + 3) * plane);
+      v.x += a.x; v.y += a.y; v.x += b.x; v.y += b.y; v.x += c.x; v.y += c.y; v.x += d.x; v.y += d.y;
+    }
+    for (; s < slices; ++s) {
+      const float2 a = *reinterpret_cast<const float2*>(p + (size_t)s * plane);
+      v.x += a.x; v.y += a.y;
+    }
+    return v;
+  };
+  const int t = blockIdx.x;
+  const int job = blockIdx.y * ROPE_JOBS + threadIdx.x / WAVE;       // a wave per (token, head)
+  const int lane = threadIdx.x % WAVE;
+  if (job >= n_heads + 2 * n_kv_heads) return;
   int pos = tok_pos[t];
   int Q = n_heads * hd, KV = n_kv_heads * hd;
   const float* row = qkv + (size_t)t * (Q + 2 * KV);
@@ -162,8 +199,9 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
   if (job < n_heads) {                       // a query head
     const float* src = row + job * hd;
     T* dst = q_out + (size_t)t * Q + job * hd;
-    for (int p = threadIdx.x; p < hd / 2; p += WAVE) {
-      float x0 = rd(src + 2 * p), x1 = rd(src + 2 * p + 1);
+    for (int p = lane; p < hd / 2; p += WAVE) {
+      const float2 x = rd2(src + 2 * p);
+      float x0 = x.x, x1 = x.y;
       if (rotate && p < half_rot) {
         float2 c = cs[p];
         float y0 = x0 * c.x - x1 * c.y;
@@ -171,8 +209,12 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
         x0 = y0;
         x1 = y1;
       }
-      dst[2 * p] = from_f32<T>(x0);
-      dst[2 * p + 1] = from_f32<T>(x1);
+      if (pairs_aligned) {
+        store_pair(dst + 2 * p, x0, x1);
+      } else {
+        dst[2 * p] = from_f32<T>(x0);
+        dst[2 * p + 1] = from_f32<T>(x1);
+      }
     }
     return;
   }
@@ -208,8 +250,9 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
 
   if (is_k) {
     const float* src = row + Q + g * hd;
-    for (int p = threadIdx.x; p < hd / 2; p += WAVE) {
-      float x0 = rd(src + 2 * p), x1 = rd(src + 2 * p + 1);
+    for (int p = lane; p < hd / 2; p += WAVE) {
+      const float2 x = rd2(src + 2 * p);
+      float x0 = x.x, x1 = x.y;
       if (rotate && p < half_rot) {
         float2 c = cs[p];
         float y0 = x0 * c.x - x1 * c.y;
@@ -230,7 +273,7 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
     }
   } else {
     const float* src = row + Q + KV + g * hd;
-    for (int i = threadIdx.x; i < hd; i += WAVE) {
+    for (int i = lane; i < hd; i += WAVE) {
       T a = from_f32<T>(rd(src + i));
       if (vst) vst[(size_t)i * PAGE + r] = a;
       if (vpage) vpage[page_v_offset(page_layout, r, i, hd)] = a;      // values are kept transposed inside a page
@@ -247,14 +290,6 @@ __global__ void rope_kv_write_kernel(const float* __restrict__ qkv, T* __restric
 // ---------------------------------------------------------------------------
 constexpr int VT_ROW = PAGE + 8;                  // LDS row of the transposed values (elements)
 
-__device__ __forceinline__ void store_pair(float* dst, float a, float b) {
-  *reinterpret_cast<float2*>(dst) = make_float2(a, b);
-}
-__device__ __forceinline__ void store_pair(bf16* dst, float a, float b) {
-  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-  bf16x2 v = {static_cast<bf16>(a), static_cast<bf16>(b)};
-  *reinterpret_cast<bf16x2*>(dst) = v;
-}
 
 // 2 * PP consecutive values
 template <int PP>
@@ -454,14 +489,14 @@ extern "C" int yalm_rope_kv_write(const float* qkv, void* q_out, void* k_stage, 
       n_heads <= 0 || n_kv_heads <= 0 || ring_pages <= 0 || slices < 1 || !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
   const long plane = (long)T * (n_heads + 2 * n_kv_heads) * head_dim;
-  dim3 grid(T, n_heads + 2 * n_kv_heads);
+  dim3 grid(T, ceil_div(n_heads + 2 * n_kv_heads, ROPE_JOBS));
   if (dtype == YALM_F32)
-    rope_kv_write_kernel<float><<<grid, WAVE, 0, stream>>>(
+    rope_kv_write_kernel<float><<<grid, ROPE_JOBS * WAVE, 0, stream>>>(
         qkv, (float*)q_out, (float*)k_stage, (float*)v_stage, seq_tile0, (float*)k_pages, (float*)v_pages, block_table,
         table_stride, ring_pages, tok_seq, tok_pos, seq_slot, seq_len, (const float2*)cos_sin, n_positions, n_heads,
         n_kv_heads, head_dim, rotary_dim, n_pages, page_layout, slices, plane);
   else if (dtype == YALM_BF16)
-    rope_kv_write_kernel<bf16><<<grid, WAVE, 0, stream>>>(
+    rope_kv_write_kernel<bf16><<<grid, ROPE_JOBS * WAVE, 0, stream>>>(
         qkv, (bf16*)q_out, (bf16*)k_stage, (bf16*)v_stage, seq_tile0, (bf16*)k_pages, (bf16*)v_pages, block_table, table_stride,
         ring_pages, tok_seq, tok_pos, seq_slot, seq_len, (const float2*)cos_sin, n_positions, n_heads, n_kv_heads,
         head_dim, rotary_dim, n_pages, page_layout, slices, plane);

@@ -21,6 +21,49 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
+// The norm chain for more than 16 rows: the activations came as bfloat16(x * w_norm) from a producer that also left
+// partial sums of squares of every row (yalm_gemm_add_emit); the sums of this product are scaled by
+// rsqrt(sum(ss[m, :]) / K + eps) per row before they are stored (as slices or through the epilogue: the scale is the
+// same for every slice of a row, so the sum of the scaled slices is the scaled sum).  ss null: no scale.
+struct RowScale {
+  const float* ss;                               // [M][n_parts]
+  int n_parts;
+  float eps;
+};
+
+// A thread per row adds the row's parts (row_sum: asked for BEFORE the first stages of the operands, so that waiting
+// for it does not mean waiting for them: loads return in order) and leaves the scale in LDS; the epilogue reads it
+// from there.  The workgroups have at least 16 * MT threads.
+__device__ __forceinline__ float row_sum(const RowScale& rs, int M, int rows) {
+  float t = 0.f;
+  if (rs.ss != nullptr && (int)threadIdx.x < rows && (int)threadIdx.x < M) {
+    const float* p = rs.ss + (size_t)threadIdx.x * rs.n_parts;
+    int i = 0;
+    for (; i + 4 <= rs.n_parts; i += 4) {
+      const float a = p[i], b = p[i + 1], c = p[i + 2], d = p[i + 3];
+      t += a; t += b; t += c; t += d;
+    }
+    for (; i < rs.n_parts; ++i) t += p[i];
+  }
+  return t;
+}
+__device__ __forceinline__ void row_scale_store(const RowScale& rs, float sum, int K, int rows, float* sm_scale) {
+  if (rs.ss != nullptr && (int)threadIdx.x < rows) sm_scale[threadIdx.x] = 1.0f / sqrtf(sum / (float)K + rs.eps);
+}
+template <int MT, int NTW>
+__device__ __forceinline__ void row_scales_apply(const RowScale& rs, const float* sm_scale, int q, f32x4 (&acc)[MT][NTW]) {
+  if (rs.ss == nullptr) return;
+  __syncthreads();
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float sc = sm_scale[mt * 16 + 4 * q + r];
+#pragma unroll
+      for (int t = 0; t < NTW; ++t) acc[mt][t][r] *= sc;
+    }
+}
+
 constexpr int NWAVES = 8;
 constexpr int KC = 128;                          // k per chunk
 constexpr int XROW = KC + 8;                     // LDS row stride (elements): 16 bytes of padding
@@ -57,7 +100,8 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_kernel(const bf16* _
                                                                     const bf16* __restrict__ W,
                                                                     void* __restrict__ Cv,
                                                                     float* __restrict__ partial, int M, int N, int K,
-                                                                    int H, int k_per_slice, int always_partial) {
+                                                                    int H, int k_per_slice, int always_partial,
+                                                                    RowScale rs) {
   __shared__ __attribute__((aligned(16))) bf16 xs[2][MT * 16 * XROW];
   constexpr int NTHREADS = NWAVES * WAVE;
   constexpr int XCHUNKS = MT * 16 * (KC / 8);    // 16-byte pieces of an activation chunk
@@ -107,6 +151,9 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_kernel(const bf16* _
     }
   };
 
+  __shared__ float sm_scale[MT * 16];
+  static_assert(NTHREADS >= MT * 16, "a thread per batch row");
+  row_scale_store(rs, row_sum(rs, M, MT * 16), K, MT * 16, sm_scale);
   if (k_begin < k_end) {
     load_w(k_begin, wv);
     load_x(k_begin);
@@ -142,6 +189,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_kernel(const bf16* _
   }
 
   // C[m][n]: lane (q, j) holds rows 4q..4q+3 of column j of every tile
+  row_scales_apply<MT, NTW>(rs, sm_scale, q, acc);
   if (gridDim.y == 1 && !always_partial) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -189,7 +237,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_batch_dma_kernel(const bf16* _
                                                                         void* __restrict__ Cv,
                                                                         float* __restrict__ partial, int M, int N,
                                                                         int K, int H, int k_per_slice,
-                                                                        int always_partial) {
+                                                                        int always_partial, RowScale rs) {
   constexpr int KD = 64;
   constexpr int WSTAGE = NTW * 2048;             // a wave's weight rows of a stage
   constexpr int XG0 = MT <= 2 ? 4 : (MT <= 4 ? 8 : 16);  // DMA instructions for the activations: 8 rows each, 32, 64 or
@@ -239,9 +287,13 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_batch_dma_kernel(const bf16* _
 #pragma unroll
     for (int t = 0; t < NTW; ++t) acc[mt][t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
+  __shared__ float sm_scale[MT * 16];
+  static_assert(NW * WAVE >= MT * 16, "a thread per batch row");
+  const float rsum = row_sum(rs, M, MT * 16);
 #pragma unroll
   for (int i = 0; i < S - 1; ++i)
     if (i < n_st) issue(i);
+  row_scale_store(rs, rsum, K, MT * 16, sm_scale);
   // fragment reads: lane (q, j) of step s wants chunk 4 s + q of row j, which lies at (4 s + q) ^ (j & 7)
   const int rd = j * 128, swz = j & 7;
   int buf = 0;
@@ -277,6 +329,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_batch_dma_kernel(const bf16* _
     if (++buf == S) buf = 0;
   }
 
+  row_scales_apply<MT, NTW>(rs, sm_scale, q, acc);
   if (gridDim.y == 1 && !always_partial) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -308,7 +361,7 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_batch_dma_kernel(const bf16* _
 // multiples of 64, else the register one (8 waves; up to 64 rows)
 template <int MT, int NTW, int EPI, int NW>
 int launch_kernel(dim3 grid, const bf16* X, const bf16* W, void* C, float* ws, int M, int N, int K, int H,
-                  int k_per_slice, int always_partial, hipStream_t stream) {
+                  int k_per_slice, int always_partial, const RowScale& rs, hipStream_t stream) {
   if (K % 64 == 0 && k_per_slice % 64 == 0) {
     constexpr int XG0 = MT <= 2 ? 4 : (MT <= 4 ? 8 : 16);
     constexpr int XG = XG0 < NW ? NW : XG0;
@@ -322,12 +375,12 @@ int launch_kernel(dim3 grid, const bf16* X, const bf16* W, void* C, float* ws, i
       if (e != hipSuccess) return (int)e;
       allowed = true;
     }
-    kernel<<<grid, NW * WAVE, lds, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice, always_partial);
+    kernel<<<grid, NW * WAVE, lds, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice, always_partial, rs);
     return launch_status();
   }
   if constexpr (MT <= 4 && NW == NWAVES) {
     gemm_batch_kernel<MT, NTW, EPI><<<grid, NWAVES * WAVE, 0, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice,
-                                                                        always_partial);
+                                                                        always_partial, rs);
     return launch_status();
   }
   return YALM_ERR_ARG;
@@ -399,17 +452,22 @@ void slice_k(int K, int wanted, int* k_per_slice, int* slices) {
   *slices = ceil_div(K, *k_per_slice);
 }
 
-template <int MT, int EPI, int NW>
+template <int MT, int EPI, int NW, int NTW_ = 0>
 int launch_nw(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
-              hipStream_t stream) {
-  constexpr int NTW = EPI == 3 ? 2 : 1;
+              const RowScale& rs, hipStream_t stream) {
+  constexpr int NTW = NTW_ ? NTW_ : (EPI == 3 ? 2 : 1);
+  if constexpr (NTW_ == 0 && EPI != 3 && MT <= 4 && NW <= 4) {
+    // a matrix with rows enough (the head): workgroups of 128 rows fill the chip by themselves, K unsplit
+    if (K % 64 == 0 && ceil_div(N, NW * 32) >= 200)
+      return launch_nw<MT, EPI, NW, 2>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
+  }
   const int rows_per_wg = NW * 16 * NTW;
   const int n_blocks = ceil_div(N, rows_per_wg);
   int slices = wanted_slices(n_blocks, M, K), k_per_slice;
   if (ws == nullptr || (long)slices * M * N > ws_floats) slices = 1;
   slice_k(K, slices, &k_per_slice, &slices);
   dim3 grid(n_blocks, slices);
-  int rc = launch_kernel<MT, NTW, EPI, NW>(grid, X, W, C, ws, M, N, K, H, k_per_slice, 0, stream);
+  int rc = launch_kernel<MT, NTW, EPI, NW>(grid, X, W, C, ws, M, N, K, H, k_per_slice, 0, rs, stream);
   if (rc != YALM_OK || slices == 1) return rc;
   const long items = (long)M * (EPI == 3 ? (N / 2) / 4 : (N + 3) / 4);
   splitk_reduce_kernel<EPI><<<ceil_div(items, 256), 256, 0, stream>>>(ws, C, M, N, H, slices);
@@ -418,14 +476,14 @@ int launch_nw(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, 
 
 template <int MT, int EPI>
 int launch_mt(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
-              hipStream_t stream) {
+              const RowScale& rs, hipStream_t stream) {
   // waves a workgroup of the DMA kernel (they share the activations' stage): measured at batch 64
   // 8 waves 8120, 4 waves 8580, 2 waves 8410 tokens a second; at batch 32 5490, 5740 and 5870; with more than 64
   // rows 8 waves where their rings fit (not the gated product's): batch 96 8,950 -> 9,060, batch 128 9,540 -> 9,590
   constexpr int NW = MT <= 2 ? 2 : (MT > 4 && EPI != 3 ? 8 : 4);
-  if (K % 64 == 0) return launch_nw<MT, EPI, NW>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+  if (K % 64 == 0) return launch_nw<MT, EPI, NW>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
   if constexpr (MT > 4) return YALM_ERR_ARG;
-  else return launch_nw<MT, EPI, 8>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+  else return launch_nw<MT, EPI, 8>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
 }
 
 // The residual add that also does the NEXT RMSNorm: a workgroup per row adds the K slices to
@@ -488,82 +546,279 @@ __global__ __launch_bounds__(RN_THREADS) void reduce_add_norm_kernel(const float
   }
 }
 
-template <int MT, int NW>
+// Workgroups of 32 weight rows a wave instead of 16 (twice the rows for the same stage of activations): what a CU
+// takes in is bounded (about 37 GB/s, whether the bytes come from memory or from the second-level cache), so the
+// activations' share is taken from the weights'; at 64 batch rows a workgroup of 64 weight rows spends half of it on
+// activations, one of 128 a third.  Such a workgroup's rings allow one workgroup a CU, so K is cut into as many slices
+// as bring the launch to at most 256 workgroups, and a slice must stay long enough to be worth its start (12 stages).
+// Measured at 64 rows of the 7B shape: down projection 31.4 -> 27.9 us, q/k/v 16.0 -> 12.7 (5 slices of 13 stages);
+// the output projection (8 slices of 8 stages) 15.3 -> 16.5, which the rule leaves out.  Returns the slices, 0: no.
+int wide_slices(int n_blocks_wide, int K) {
+  int s = 256 / (n_blocks_wide > 0 ? n_blocks_wide : 1);
+  if (s > 16) s = 16;
+  if (s < 1 || n_blocks_wide * s < 192 || K % 64 != 0 || K / s < 768) return 0;
+  return s;
+}
+
+// The same with a row's columns kept in registers between the two halves (N a multiple of 4, at most
+// THREADS * VPT * 4): the new row is written and never read again, and the norm's weights are asked for before the
+// sum of squares is known.  64 rows of 4,096 columns: 4.85 -> see the launcher.
+template <int THREADS, int VPT>
+__global__ __launch_bounds__(THREADS) void reduce_add_norm_reg_kernel(const float* __restrict__ partial,
+                                                                      float* __restrict__ C,
+                                                                      const float* __restrict__ norm_w, float eps,
+                                                                      bf16* __restrict__ h, int M, int N, int slices) {
+  __shared__ float red[THREADS / WAVE];
+  const int m = blockIdx.x;
+  const size_t plane = (size_t)M * N;
+  float* row = C + (size_t)m * N;
+  const float* prow = partial + (size_t)m * N;
+  float4 y[VPT], w[VPT];
+  int col[VPT];
+#pragma unroll
+  for (int v = 0; v < VPT; ++v) {
+    col[v] = (threadIdx.x + v * THREADS) * 4;
+    const bool ok = col[v] < N;
+    const int c = ok ? col[v] : 0;                  // every lane loads (a load under a branch holds up the others)
+    y[v] = *reinterpret_cast<const float4*>(row + c);
+    w[v] = *reinterpret_cast<const float4*>(norm_w + c);
+  }
+  int s = 0;
+  for (; s + 4 <= slices; s += 4) {
+    float4 p[4][VPT];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int v = 0; v < VPT; ++v)
+        p[u][v] = *reinterpret_cast<const float4*>(prow + (size_t)(s + u) * plane + (col[v] < N ? col[v] : 0));
+#pragma unroll
+    for (int u = 0; u < 4; ++u)                     // added in the order of the slices
+#pragma unroll
+      for (int v = 0; v < VPT; ++v) {
+        y[v].x += p[u][v].x; y[v].y += p[u][v].y; y[v].z += p[u][v].z; y[v].w += p[u][v].w;
+      }
+  }
+  for (; s < slices; ++s) {
+    float4 p[VPT];
+#pragma unroll
+    for (int v = 0; v < VPT; ++v)
+      p[v] = *reinterpret_cast<const float4*>(prow + (size_t)s * plane + (col[v] < N ? col[v] : 0));
+#pragma unroll
+    for (int v = 0; v < VPT; ++v) {
+      y[v].x += p[v].x; y[v].y += p[v].y; y[v].z += p[v].z; y[v].w += p[v].w;
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int v = 0; v < VPT; ++v)
+    if (col[v] < N) {
+      *reinterpret_cast<float4*>(row + col[v]) = y[v];
+      ss += y[v].x * y[v].x + y[v].y * y[v].y + y[v].z * y[v].z + y[v].w * y[v].w;
+    }
+  ss = block_sum<THREADS / WAVE>(ss, red);
+  const float scale = 1.0f / sqrtf(ss / (float)N + eps);
+  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+#pragma unroll
+  for (int v = 0; v < VPT; ++v)
+    if (col[v] < N) {
+      bf16x4 o = {static_cast<bf16>(y[v].x * scale * w[v].x), static_cast<bf16>(y[v].y * scale * w[v].y),
+                  static_cast<bf16>(y[v].z * scale * w[v].z), static_cast<bf16>(y[v].w * scale * w[v].w)};
+      *reinterpret_cast<bf16x4*>(h + (size_t)m * N + col[v]) = o;
+    }
+}
+
+// The residual add that prepares the next norm without waiting for it: a workgroup takes EMIT_COLS columns of a row,
+// adds the K slices to the residual stream, and writes xn = bfloat16(x_new * norm_w) and the sum of the squares of its
+// columns, ss[row][part].  The consumer scales its sums by rsqrt(sum(ss[row, :]) / N + eps) (RowScale).  No workgroup
+// waits for a whole row, so a batch of 64 rows is 256 small workgroups instead of 64 that each walk a row twice.
+constexpr int EMIT_THREADS = 256, EMIT_COLS = EMIT_THREADS * 4;
+__global__ __launch_bounds__(EMIT_THREADS) void reduce_add_emit_kernel(const float* __restrict__ partial,
+                                                                       float* __restrict__ C,
+                                                                       const float* __restrict__ norm_w,
+                                                                       bf16* __restrict__ xn, float* __restrict__ ss_out,
+                                                                       int M, int N, int slices) {
+  __shared__ float red[EMIT_THREADS / WAVE];
+  const int m = blockIdx.x, part = blockIdx.y, n_parts = gridDim.y;
+  const size_t plane = (size_t)M * N;
+  const int c = part * EMIT_COLS + threadIdx.x * 4;
+  float ss = 0.f;
+  {                                               // N is a multiple of 8 (the launcher sees to it)
+    const bool ok = c < N;
+    const int cc = ok ? c : 0;
+    float* row = C + (size_t)m * N + cc;
+    const float* prow = partial + (size_t)m * N + cc;
+    float4 y = *reinterpret_cast<const float4*>(row);
+    const float4 w = *reinterpret_cast<const float4*>(norm_w + cc);
+    int s = 0;
+    for (; s + 4 <= slices; s += 4) {
+      float4 p[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) p[u] = *reinterpret_cast<const float4*>(prow + (size_t)(s + u) * plane);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {                // added in the order of the slices
+        y.x += p[u].x; y.y += p[u].y; y.z += p[u].z; y.w += p[u].w;
+      }
+    }
+    for (; s < slices; ++s) {
+      const float4 p = *reinterpret_cast<const float4*>(prow + (size_t)s * plane);
+      y.x += p.x; y.y += p.y; y.z += p.z; y.w += p.w;
+    }
+    if (ok) {
+      *reinterpret_cast<float4*>(row) = y;
+      typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+      bf16x4 o = {static_cast<bf16>(y.x * w.x), static_cast<bf16>(y.y * w.y), static_cast<bf16>(y.z * w.z),
+                  static_cast<bf16>(y.w * w.w)};
+      *reinterpret_cast<bf16x4*>(xn + (size_t)m * N + c) = o;
+      ss = y.x * y.x + y.y * y.y + y.z * y.z + y.w * y.w;
+    }
+  }
+  ss = block_sum<EMIT_THREADS / WAVE>(ss, red);
+  if (threadIdx.x == 0) ss_out[(size_t)m * n_parts + part] = ss;
+}
+
+int emit_parts(int N) { return ceil_div(N, EMIT_COLS); }
+
+// emit_ss null: the new row's norm is finished here (h = its output); else h = bfloat16(x_new * norm_w) and emit_ss
+// receives the parts of the rows' sums of squares
+int launch_reduce_add_norm(const float* ws, float* C, const float* norm_w, float eps, bf16* h, int M, int N, int slices,
+                           hipStream_t stream, float* emit_ss = nullptr) {
+  if (emit_ss != nullptr) {
+    reduce_add_emit_kernel<<<dim3(M, emit_parts(N)), EMIT_THREADS, 0, stream>>>(ws, C, norm_w, h, emit_ss, M, N, slices);
+    return launch_status();
+  }
+  if ((N & 3) == 0 && N <= 1024 * 4 && !((uintptr_t)norm_w & 15))
+    reduce_add_norm_reg_kernel<1024, 1><<<M, 1024, 0, stream>>>(ws, C, norm_w, eps, h, M, N, slices);
+  else if ((N & 3) == 0 && N <= 1024 * 4 * 4 && !((uintptr_t)norm_w & 15))
+    reduce_add_norm_reg_kernel<1024, 4><<<M, 1024, 0, stream>>>(ws, C, norm_w, eps, h, M, N, slices);
+  else
+    reduce_add_norm_kernel<<<M, RN_THREADS, 0, stream>>>(ws, C, norm_w, eps, h, M, N, slices);
+  return launch_status();
+}
+
+template <int MT, int NW, int NTW = 1>
 int launch_add_norm_nw(const bf16* X, const bf16* W, float* C, float* ws, long ws_floats, int M, int N, int K,
-                       const float* norm_w, float eps, bf16* h, hipStream_t stream) {
-  const int n_blocks = ceil_div(N, NW * 16);
-  int slices = wanted_slices(n_blocks, M, K), k_per_slice;
+                       const float* norm_w, float eps, bf16* h, hipStream_t stream, float* emit_ss = nullptr) {
+  if constexpr (NTW == 1 && MT <= 4 && NW <= 4) {
+    const int wide = wide_slices(ceil_div(N, NW * 32), K);
+    if (wide > 0 && ws != nullptr && (long)wide * M * N <= ws_floats)
+      return launch_add_norm_nw<MT, NW, 2>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream, emit_ss);
+  }
+  const int n_blocks = ceil_div(N, NW * 16 * NTW);
+  int slices = NTW == 2 ? wide_slices(n_blocks, K) : wanted_slices(n_blocks, M, K), k_per_slice;
   while (slices > 1 && (long)slices * M * N > ws_floats) slices /= 2;
   if (ws == nullptr || (long)slices * M * N > ws_floats) return YALM_ERR_ARG;
   slice_k(K, slices, &k_per_slice, &slices);
   dim3 grid(n_blocks, slices);
-  int rc = launch_kernel<MT, 1, 2, NW>(grid, X, W, C, ws, M, N, K, 0, k_per_slice, 1, stream);
+  int rc = launch_kernel<MT, NTW, 2, NW>(grid, X, W, C, ws, M, N, K, 0, k_per_slice, 1, RowScale{nullptr, 0, 0.f}, stream);
   if (rc != YALM_OK) return rc;
-  reduce_add_norm_kernel<<<M, RN_THREADS, 0, stream>>>(ws, C, norm_w, eps, h, M, N, slices);
-  return launch_status();
+  return launch_reduce_add_norm(ws, C, norm_w, eps, h, M, N, slices, stream, emit_ss);
 }
 
 template <int MT>
 int launch_add_norm(const bf16* X, const bf16* W, float* C, float* ws, long ws_floats, int M, int N, int K,
-                    const float* norm_w, float eps, bf16* h, hipStream_t stream) {
+                    const float* norm_w, float eps, bf16* h, hipStream_t stream, float* emit_ss = nullptr) {
   if (K % 64 == 0 && MT > 2)
-    return launch_add_norm_nw<MT, (MT > 4 ? 8 : 4)>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream);
+    return launch_add_norm_nw<MT, (MT > 4 ? 8 : 4)>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream, emit_ss);
   if constexpr (MT > 4) return YALM_ERR_ARG;
-  else return launch_add_norm_nw<MT, NWAVES>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream);
+  else return launch_add_norm_nw<MT, NWAVES>(X, W, C, ws, ws_floats, M, N, K, norm_w, eps, h, stream, emit_ss);
 }
 
 // the K slices only: [slices][M][N] in ws, for a consumer that adds them
-template <int MT, int NW>
+template <int MT, int NW, int NTW = 1>
 int launch_partial_nw(const bf16* X, const bf16* W, float* ws, long ws_floats, int M, int N, int K, int* slices_out,
-                      hipStream_t stream) {
-  const int n_blocks = ceil_div(N, NW * 16);
-  int slices = wanted_slices(n_blocks, M, K), k_per_slice;
+                      const RowScale& rs, hipStream_t stream) {
+  if constexpr (NTW == 1 && MT <= 4 && NW <= 4) {
+    const int wide = wide_slices(ceil_div(N, NW * 32), K);
+    if (wide > 0 && ws != nullptr && (long)wide * M * N <= ws_floats)
+      return launch_partial_nw<MT, NW, 2>(X, W, ws, ws_floats, M, N, K, slices_out, rs, stream);
+  }
+  const int n_blocks = ceil_div(N, NW * 16 * NTW);
+  int slices = NTW == 2 ? wide_slices(n_blocks, K) : wanted_slices(n_blocks, M, K), k_per_slice;
   while (slices > 1 && (long)slices * M * N > ws_floats) slices /= 2;
   if (ws == nullptr || (long)slices * M * N > ws_floats) return YALM_ERR_ARG;
   slice_k(K, slices, &k_per_slice, &slices);
   *slices_out = slices;
   dim3 grid(n_blocks, slices);
-  return launch_kernel<MT, 1, 0, NW>(grid, X, W, ws, ws, M, N, K, 0, k_per_slice, 1, stream);
+  return launch_kernel<MT, NTW, 0, NW>(grid, X, W, ws, ws, M, N, K, 0, k_per_slice, 1, rs, stream);
 }
 
 template <int MT>
 int launch_partial(const bf16* X, const bf16* W, float* ws, long ws_floats, int M, int N, int K, int* slices_out,
-                   hipStream_t stream) {
+                   const RowScale& rs, hipStream_t stream) {
   if (K % 64 == 0)
-    return launch_partial_nw<MT, (MT <= 2 ? 2 : (MT > 4 ? 8 : 4))>(X, W, ws, ws_floats, M, N, K, slices_out, stream);
+    return launch_partial_nw<MT, (MT > 4 ? 8 : 4)>(X, W, ws, ws_floats, M, N, K, slices_out, rs, stream);
   if constexpr (MT > 4) return YALM_ERR_ARG;
-  else return launch_partial_nw<MT, NWAVES>(X, W, ws, ws_floats, M, N, K, slices_out, stream);
+  else return launch_partial_nw<MT, NWAVES>(X, W, ws, ws_floats, M, N, K, slices_out, rs, stream);
 }
 
 template <int EPI>
 int dispatch(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
-             hipStream_t stream) {
+             const RowScale& rs, hipStream_t stream) {
   switch ((M + 15) / 16) {
-    case 2: return launch_mt<2, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
-    case 3: return launch_mt<3, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
-    case 4: return launch_mt<4, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
-    case 5: return launch_mt<5, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
-    case 6: return launch_mt<6, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
-    case 7: return launch_mt<7, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
-    case 8: return launch_mt<8, EPI>(X, W, C, ws, ws_floats, M, N, K, H, stream);
+    case 2: return launch_mt<2, EPI>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
+    case 3: return launch_mt<3, EPI>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
+    case 4: return launch_mt<4, EPI>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
+    case 5: return launch_mt<5, EPI>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
+    case 6: return launch_mt<6, EPI>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
+    case 7: return launch_mt<7, EPI>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
+    case 8: return launch_mt<8, EPI>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
   }
   return YALM_ERR_ARG;
 }
 }  // namespace
 
 // 17..64 rows, and up to 128 with K a multiple of 64; workspace: float32 scratch for the K slices (may be
-// null: one slice then).  Refuses (YALM_ERR_ARG) what it does not take.
-int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
-                         int K, int epilogue, int H, hipStream_t stream) {
+// null: one slice then).  ss (may be null): the producer's partial sums of squares [M][n_parts] for the row scale.
+// Refuses (YALM_ERR_ARG) what it does not take.
+static int gemm_batch_scaled(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M,
+                             int N, int K, int epilogue, int H, const float* ss, int n_parts, float eps,
+                             hipStream_t stream) {
   if (M <= 16 || M > (K % 64 == 0 ? 128 : 64) || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15))
     return YALM_ERR_ARG;
+  if (ss != nullptr && n_parts <= 0) return YALM_ERR_ARG;
+  const RowScale rs = {ss, n_parts, eps};
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   switch (epilogue) {
-    case 0: return dispatch<0>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
-    case 1: return dispatch<1>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
-    case 2: return dispatch<2>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
-    case 3: return dispatch<3>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+    case 0: return dispatch<0>(a, w, C, workspace, workspace_floats, M, N, K, H, rs, stream);
+    case 1: return dispatch<1>(a, w, C, workspace, workspace_floats, M, N, K, H, rs, stream);
+    case 2: return dispatch<2>(a, w, C, workspace, workspace_floats, M, N, K, H, rs, stream);
+    case 3: return dispatch<3>(a, w, C, workspace, workspace_floats, M, N, K, H, rs, stream);
+  }
+  return YALM_ERR_ARG;
+}
+
+int yalm_gemm_bf16_batch(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
+                         int K, int epilogue, int H, hipStream_t stream) {
+  return gemm_batch_scaled(A, W, C, workspace, workspace_floats, M, N, K, epilogue, H, nullptr, 0, 0.f, stream);
+}
+
+// yalm_gemm for 17..128 bfloat16 rows (more than 64: K a multiple of 64) whose activations came from yalm_gemm_add_emit:
+// the sums are scaled per row by rsqrt(sum(ss[m, :]) / K + eps).  Refuses (YALM_ERR_ARG) other shapes.
+extern "C" int yalm_gemm_scaled(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M,
+                                int N, int K, int epilogue, int H, const float* ss, int n_parts, float eps,
+                                hipStream_t stream) {
+  if (ss == nullptr) return YALM_ERR_ARG;
+  if (epilogue == 3 && (H <= 0 || N != 32 * ((H + 15) / 16))) return YALM_ERR_ARG;
+  return gemm_batch_scaled(A, W, C, workspace, workspace_floats, M, N, K, epilogue, H, ss, n_parts, eps, stream);
+}
+
+static int gemm_partial_scaled(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N,
+                               int K, int* slices, const float* ss, int n_parts, float eps, hipStream_t stream) {
+  if (M <= 16 || M > (K % 64 == 0 ? 128 : 64) || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) ||
+      slices == nullptr || (ss != nullptr && n_parts <= 0))
+    return YALM_ERR_ARG;
+  const RowScale rs = {ss, n_parts, eps};
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  switch ((M + 15) / 16) {
+    case 2: return launch_partial<2>(a, w, workspace, workspace_floats, M, N, K, slices, rs, stream);
+    case 3: return launch_partial<3>(a, w, workspace, workspace_floats, M, N, K, slices, rs, stream);
+    case 4: return launch_partial<4>(a, w, workspace, workspace_floats, M, N, K, slices, rs, stream);
+    case 5: return launch_partial<5>(a, w, workspace, workspace_floats, M, N, K, slices, rs, stream);
+    case 6: return launch_partial<6>(a, w, workspace, workspace_floats, M, N, K, slices, rs, stream);
+    case 7: return launch_partial<7>(a, w, workspace, workspace_floats, M, N, K, slices, rs, stream);
+    case 8: return launch_partial<8>(a, w, workspace, workspace_floats, M, N, K, slices, rs, stream);
   }
   return YALM_ERR_ARG;
 }
@@ -572,49 +827,61 @@ extern "C" int yalm_gemm_partial(const void* A, const void* W, float* workspace,
                                  int K, int* slices, hipStream_t stream) {
   if (M > 128 || (M > 64 && K % 64 != 0))
     return yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, slices, 0, stream);
-  if (M <= 16 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15) || slices == nullptr)
-    return YALM_ERR_ARG;
-  const bf16* a = (const bf16*)A;
-  const bf16* w = (const bf16*)W;
-  switch ((M + 15) / 16) {
-    case 2: return launch_partial<2>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
-    case 3: return launch_partial<3>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
-    case 4: return launch_partial<4>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
-    case 5: return launch_partial<5>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
-    case 6: return launch_partial<6>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
-    case 7: return launch_partial<7>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
-    case 8: return launch_partial<8>(a, w, workspace, workspace_floats, M, N, K, slices, stream);
-  }
-  return YALM_ERR_ARG;
+  return gemm_partial_scaled(A, W, workspace, workspace_floats, M, N, K, slices, nullptr, 0, 0.f, stream);
+}
+
+// yalm_gemm_partial with the row scale of yalm_gemm_scaled applied to every slice (17..128 rows only).
+extern "C" int yalm_gemm_partial_scaled(const void* A, const void* W, float* workspace, long workspace_floats, int M,
+                                        int N, int K, int* slices, const float* ss, int n_parts, float eps,
+                                        hipStream_t stream) {
+  if (ss == nullptr) return YALM_ERR_ARG;
+  return gemm_partial_scaled(A, W, workspace, workspace_floats, M, N, K, slices, ss, n_parts, eps, stream);
 }
 
 // C (float32 residual stream) += A * W^T for more than 16 rows, and h = RMSNorm(C_new) * norm_w in bfloat16
 // for the next consumer.  Needs scratch for at least M * N floats; refuses (YALM_ERR_ARG) other shapes.
-extern "C" int yalm_gemm_add_norm(const void* A, const void* W, float* C, float* workspace, long workspace_floats,
-                                  int M, int N, int K, const float* norm_w, float eps, void* h_out,
-                                  hipStream_t stream) {
+static int gemm_add_norm_or_emit(const void* A, const void* W, float* C, float* workspace, long workspace_floats,
+                                 int M, int N, int K, const float* norm_w, float eps, void* h_out, float* emit_ss,
+                                 hipStream_t stream) {
   if (norm_w == nullptr || h_out == nullptr) return YALM_ERR_ARG;
   if (M > 128 || (M > 64 && K % 64 != 0)) {        // the tiled kernel's slices, then the same reduction
     int slices = 0;
     int rc = yalm_gemm_bf16_dma_partial(A, W, workspace, workspace_floats, M, N, K, &slices, 1, stream);
     if (rc != YALM_OK) return rc;
-    reduce_add_norm_kernel<<<M, RN_THREADS, 0, stream>>>(workspace, C, norm_w, eps, (bf16*)h_out, M, N, slices);
-    return launch_status();
+    return launch_reduce_add_norm(workspace, C, norm_w, eps, (bf16*)h_out, M, N, slices, stream, emit_ss);
   }
   if (M <= 16 || K % 8 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
   const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
+  bf16* h = (bf16*)h_out;
   switch ((M + 15) / 16) {
-    case 2: return launch_add_norm<2>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
-    case 3: return launch_add_norm<3>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
-    case 4: return launch_add_norm<4>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
-    case 5: return launch_add_norm<5>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
-    case 6: return launch_add_norm<6>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
-    case 7: return launch_add_norm<7>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
-    case 8: return launch_add_norm<8>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, (bf16*)h_out, stream);
+    case 2: return launch_add_norm<2>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, h, stream, emit_ss);
+    case 3: return launch_add_norm<3>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, h, stream, emit_ss);
+    case 4: return launch_add_norm<4>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, h, stream, emit_ss);
+    case 5: return launch_add_norm<5>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, h, stream, emit_ss);
+    case 6: return launch_add_norm<6>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, h, stream, emit_ss);
+    case 7: return launch_add_norm<7>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, h, stream, emit_ss);
+    case 8: return launch_add_norm<8>(a, w, C, workspace, workspace_floats, M, N, K, norm_w, eps, h, stream, emit_ss);
   }
   return YALM_ERR_ARG;
 }
+
+extern "C" int yalm_gemm_add_norm(const void* A, const void* W, float* C, float* workspace, long workspace_floats,
+                                  int M, int N, int K, const float* norm_w, float eps, void* h_out,
+                                  hipStream_t stream) {
+  return gemm_add_norm_or_emit(A, W, C, workspace, workspace_floats, M, N, K, norm_w, eps, h_out, nullptr, stream);
+}
+
+// The same product and residual add, but the next norm is only prepared: xn_out bfloat16 [M,N] = C_new * norm_w and
+// ss_out float32 [M, yalm_gemm_add_emit_parts(N)] = sums of squares of C_new over the columns of each part; the
+// consumer (yalm_gemm_scaled, yalm_gemm_partial_scaled) scales its sums.  Same shapes as yalm_gemm_add_norm.
+extern "C" int yalm_gemm_add_emit(const void* A, const void* W, float* C, float* workspace, long workspace_floats,
+                                  int M, int N, int K, const float* norm_w, void* xn_out, float* ss_out,
+                                  hipStream_t stream) {
+  if (ss_out == nullptr || N % 8 != 0 || ((uintptr_t)norm_w & 15)) return YALM_ERR_ARG;   // a consumer's K is this N
+  return gemm_add_norm_or_emit(A, W, C, workspace, workspace_floats, M, N, K, norm_w, 0.f, xn_out, ss_out, stream);
+}
+extern "C" int yalm_gemm_add_emit_parts(int N) { return emit_parts(N); }
 
 // Adds `slices` float32 partial products [slices][M][N] in order and applies the epilogue (for the
 // kernels that split K: this file's and the tiled one of gemm_dma.hip).

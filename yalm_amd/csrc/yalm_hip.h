@@ -67,6 +67,19 @@ int yalm_gemm_partial(const void* A, const void* W, float* workspace, long works
 int yalm_gemm_add_norm(const void* A, const void* W, float* C, float* workspace, long workspace_floats, int M, int N,
                        int K, const float* norm_w, float eps, void* h_out, hipStream_t stream);
 
+// The norm chain for 17..128 rows (more than 64: K a multiple of 64).  yalm_gemm_add_emit is yalm_gemm_add_norm that
+// only prepares the next norm: xn_out bfloat16 [M,N] = C_new * norm_w and ss_out float32
+// [M, yalm_gemm_add_emit_parts(N)] = sums of squares of C_new over the columns of each part.  A consumer given those
+// (ss, n_parts, eps; its K is the row's width) scales its float32 sums by rsqrt(sum(ss[m, :]) / K + eps) per row:
+// yalm_gemm_scaled (epilogues of yalm_gemm) and yalm_gemm_partial_scaled (slices of yalm_gemm_partial, each scaled).
+int yalm_gemm_add_emit(const void* A, const void* W, float* C, float* workspace, long workspace_floats, int M, int N,
+                       int K, const float* norm_w, void* xn_out, float* ss_out, hipStream_t stream);
+int yalm_gemm_add_emit_parts(int N);
+int yalm_gemm_scaled(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N, int K,
+                     int epilogue, int H, const float* ss, int n_parts, float eps, hipStream_t stream);
+int yalm_gemm_partial_scaled(const void* A, const void* W, float* workspace, long workspace_floats, int M, int N, int K,
+                             int* slices, const float* ss, int n_parts, float eps, hipStream_t stream);
+
 // Decode GEMMs (M <= 64, bfloat16) that chain norms without a norm kernel in between.
 // Producer: epilogue 2 (C float32 += product) with emit_nw given also writes
 // emit_xn[M,N] = bfloat16(C_new * emit_nw[n]) and emit_ss[M, parts] = sums of squares of

@@ -116,12 +116,14 @@ def gemm_workspace_floats(M, N, K):
     return 0
 
 
-def gemm(a, w, out, epilogue, hidden=0, workspace=None):
+def gemm(a, w, out, epilogue, hidden=0, workspace=None, scale_from=None):
     """out = a[M,K] @ w[N,K]^T with float32 accumulation and one of four epilogues:
     EPI_STORE_F32 (float32 out), EPI_STORE (out in a's dtype), EPI_ADD_F32
     (float32 out += product), EPI_GATED (w = gate/up rows interleaved in blocks of
     16; out[M, hidden] = silu(gate) * up in a's dtype).  workspace: float32 scratch of
-    gemm_workspace_floats(M, N, K) elements, with which small batches split K."""
+    gemm_workspace_floats(M, N, K) elements, with which small batches split K.
+    scale_from = (ss float32 [M, parts], eps), 17..128 bfloat16 rows only (can_add_emit): a was emitted by
+    gemm_add_emit, and the sums are scaled by rsqrt(sum(ss[m]) / K + eps) per row before the epilogue."""
     M, K = a.shape
     N = w.shape[0]
     dt = a.dtype
@@ -140,6 +142,14 @@ def gemm(a, w, out, epilogue, hidden=0, workspace=None):
     p_ws, n_ws = None, 0
     if workspace is not None:
         p_ws, n_ws = _need(workspace, "workspace", torch.float32), workspace.numel()
+    if scale_from is not None:
+        ss, eps = scale_from
+        if dt != torch.bfloat16:
+            raise TypeError("gemm: a row scale goes with bfloat16 activations")
+        p_ss = _need(ss, "ss", torch.float32, (M, None))
+        library.check(library.lib().yalm_gemm_scaled(p_a, p_w, p_o, p_ws, n_ws, M, N, K, epilogue, hidden, p_ss,
+                                                     ss.shape[1], float(eps), _stream()), "gemm with a row scale")
+        return out
     library.check(library.lib().yalm_gemm(p_a, p_w, p_o, p_ws, n_ws, M, N, K, dtype_code(dt), epilogue, hidden,
                                           1 if FORCE_SIMPLE else 0, _stream()), "gemm")
     return out
@@ -268,16 +278,48 @@ def gemm_add_norm(a, w, x, norm_w, eps, h_out, workspace):
     return h_out
 
 
+def can_add_emit(M, K, dtype):
+    """Whether gemm_add_emit takes this shape, and gemm / gemm_partial a row scale for M rows: batches beyond the
+    norm chain of gemm_chain (16 rows) up to 128 rows."""
+    return can_add_norm(M, K, dtype) and M <= 128
+
+
+def gemm_add_emit_parts(N):
+    """Columns of the partial sums of squares that gemm_add_emit leaves for rows of N columns."""
+    return library.lib().yalm_gemm_add_emit_parts(int(N))
+
+
+def gemm_add_emit(a, w, x, norm_w, xn_out, ss_out, workspace):
+    """x float32 [M, N] += a[M, K] @ w[N, K]^T (shapes as gemm_add_norm), xn_out bfloat16 [M, N] = x_new * norm_w and
+    ss_out float32 [M, gemm_add_emit_parts(N)] = partial sums of squares of x_new: the next norm prepared but not
+    finished; its consumer scales its own sums (gemm / gemm_partial with scale_from)."""
+    M, K = a.shape
+    N = w.shape[0]
+    p_a = _need(a, "a", torch.bfloat16, (M, K))
+    p_w = _need(w, "w", torch.bfloat16, (N, K))
+    p_x = _need(x, "x", torch.float32, (M, N))
+    p_nw = _need(norm_w, "norm_w", torch.float32, (N,))
+    p_xn = _need(xn_out, "xn_out", torch.bfloat16, (M, N))
+    p_ss = _need(ss_out, "ss_out", torch.float32, (M, gemm_add_emit_parts(N)))
+    if workspace is None or workspace.numel() < M * N:
+        raise ValueError("gemm_add_emit needs a workspace of at least M * N floats")
+    p_ws = _need(workspace, "workspace", torch.float32, None)
+    library.check(library.lib().yalm_gemm_add_emit(p_a, p_w, p_x, p_ws, workspace.numel(), M, N, K, p_nw, p_xn, p_ss,
+                                                   _stream()), "gemm_add_emit")
+    return xn_out
+
+
 def can_gemm_partial(M, K, dtype):
     """True if gemm_partial takes the shape (more than 16 rows of bfloat16; more than 64: K a multiple of 64)."""
     return can_add_norm(M, K, dtype)
 
 
-def gemm_partial(a, w, workspace):
+def gemm_partial(a, w, workspace, scale_from=None):
     """The K slices of a[M,K] @ w[N,K]^T, more than 16 rows of bfloat16 (more than 64: K a multiple of
     64), left unadded in `workspace`
     ([slices][M][N] float32, flat; gemm_workspace_floats(M, N, K) elements let it split as it likes).
-    Returns the number of slices, for a consumer that adds them (rope_kv_write)."""
+    Returns the number of slices, for a consumer that adds them (rope_kv_write).  scale_from as in gemm
+    (every slice is scaled)."""
     M, K = a.shape
     N = w.shape[0]
     p_a = _need(a, "a", torch.bfloat16, (M, K))
@@ -286,6 +328,13 @@ def gemm_partial(a, w, workspace):
     if workspace.numel() < M * N:
         raise ValueError("workspace holds %d floats, at least %d are needed" % (workspace.numel(), M * N))
     slices = ctypes.c_int(0)
+    if scale_from is not None:
+        ss, eps = scale_from
+        p_ss = _need(ss, "ss", torch.float32, (M, None))
+        library.check(library.lib().yalm_gemm_partial_scaled(p_a, p_w, p_ws, workspace.numel(), M, N, K,
+                                                             ctypes.byref(slices), p_ss, ss.shape[1], float(eps),
+                                                             _stream()), "gemm_partial with a row scale")
+        return slices.value
     library.check(library.lib().yalm_gemm_partial(p_a, p_w, p_ws, workspace.numel(), M, N, K, ctypes.byref(slices),
                                                   _stream()), "gemm_partial")
     return slices.value

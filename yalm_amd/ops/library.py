@@ -43,11 +43,15 @@ _SIGNATURES = {
     "yalm_argmax": (_I, [_P, _P, _I, _I, _P]),
     "yalm_sample": (_I, [_P, _P, _F, _P, _I, _I, _P]),
     "yalm_token_prob": (_I, [_P, _P, _P, _I, _I, _P]),
+    "yalm_gemm_add_emit": (_I, [_P, _P, _P, _P, ctypes.c_long, _I, _I, _I, _P, _P, _P, _P]),
+    "yalm_gemm_add_emit_parts": (_I, [_I]),
+    "yalm_gemm_scaled": (_I, [_P, _P, _P, _P, ctypes.c_long, _I, _I, _I, _I, _I, _P, _I, _F, _P]),
+    "yalm_gemm_partial_scaled": (_I, [_P, _P, _P, ctypes.c_long, _I, _I, _I, _P, _P, _I, _F, _P]),
     "yalm_probe_read": (_I, [_P, ctypes.c_long, _P, _I, _P]),
     "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 
 class KernelError(RuntimeError):

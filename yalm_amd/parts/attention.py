@@ -159,7 +159,7 @@ class GQAttention(Part):
         k_pages, v_pages = group.line_pages(line)
         q = ctx.ws.get("attn.q", (T, self.q_dim), self.wo.dtype)
         src = ctx.normed.pop(id(norm), None)
-        if src is not None and src[1] is not None:
+        if src is not None and src[1] is not None and kernels.can_chain(T, self.dim, self.wo.dtype):
             xn, ss, eps = src
             kernels.gemm_chain_qkv_rope(xn, (ss, eps), self.wqkv, q, k_pages, v_pages, group.table, group.ring_pages,
                                         ctx.tok_pos, ctx.seq_slot, pos.table, self.n_heads, self.n_kv_heads,
@@ -169,8 +169,11 @@ class GQAttention(Part):
             kernels.gemm_norm_qkv_rope(x, nw, eps, self.wqkv, q, k_pages, v_pages, group.table, group.ring_pages,
                                        ctx.tok_pos, ctx.seq_slot, pos.table, self.n_heads, self.n_kv_heads,
                                        self.head_dim, pos.rotary_dim)
-        else:             # the norm's output is ready, or nothing is prepared and the rows are too many for one kernel
-            if src is not None:
+        else:             # the norm's output is ready or prepared, or the rows are too many for one kernel
+            scale = None
+            if src is not None and src[1] is not None:        # prepared: the product's sums are scaled row by row
+                h, scale = src[0], (src[1], src[2])
+            elif src is not None:
                 h = src[0]
             else:
                 h = ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
@@ -179,10 +182,10 @@ class GQAttention(Part):
             if kernels.can_gemm_partial(T, self.dim, h.dtype):
                 # the GEMM's K slices go to the rotation kernel as they are, which adds them: no kernel in between
                 qkv = ctx.ws.get("gemm.partial", (kernels.fused_workspace_floats(T, n_qkv, self.dim),), torch.float32)
-                slices = kernels.gemm_partial(h, self.wqkv, qkv)
+                slices = kernels.gemm_partial(h, self.wqkv, qkv, scale_from=scale)
             else:
                 qkv = ctx.ws.get("attn.qkv", (T, n_qkv), torch.float32)
-                self._gemm(ctx, h, self.wqkv, qkv, kernels.EPI_STORE_F32)
+                self._gemm(ctx, h, self.wqkv, qkv, kernels.EPI_STORE_F32, scale_from=scale)
                 slices = 1
             kernels.rope_kv_write(qkv, q, None, None, None, k_pages, v_pages, group.table, group.ring_pages,
                                   ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, ctx.seq_len, pos.table, self.n_heads,
@@ -190,10 +193,15 @@ class GQAttention(Part):
         o = ctx.ws.get("attn.o", (T, self.q_dim), self.wo.dtype)
         self._decode_attention(q, o, ctx, group, line, k_pages, v_pages, True)
         emit = self._emit_args(emit_for, ctx, T, self.dim)
-        ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.q_dim) if emit is None else None
+        prepared = self._add_emit_args(emit_for, ctx, T, self.dim, self.q_dim) if emit is None else None
+        ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.q_dim) if emit is None and prepared is None else None
         if emit is not None and kernels.can_chain(T, self.q_dim, o.dtype):
             nw2, xn2, ss2, eps2 = emit
             kernels.gemm_chain(o, self.wo, x, kernels.EPI_ADD_F32, emit=(nw2, xn2, ss2))
+            ctx.normed[id(emit_for)] = (xn2, ss2, eps2)
+        elif prepared is not None:                # 17..128 rows: the K slices are added and the next norm prepared at once
+            nw2, eps2, xn2, ss2, ws2 = prepared
+            kernels.gemm_add_emit(o, self.wo, x, nw2, xn2, ss2, ws2)
             ctx.normed[id(emit_for)] = (xn2, ss2, eps2)
         elif ready is not None and kernels.can_add_norm(T, self.q_dim, o.dtype):
             nw2, eps2, h2, ws2 = ready

@@ -21,9 +21,10 @@ A mixer, feed-forward or head may fold the norm in front of it into its first
 product: fuses_norm(norm, x, ctx) says so for a step, and forward_prenorm(x, norm,
 ..., emit_for=next_norm) then replaces norm.forward + forward.  With emit_for it may
 also leave, in ctx.normed[id(next_norm)], either (xn, ss, eps): the activations already
-multiplied by that norm's weights and the partial sums of squares (its residual-add GEMM
-writes them; up to 16 rows), or (h, None, None): the norm's finished output (more than 16 rows),
-which the next consumer takes instead of reading the residual stream.
+multiplied by that norm's weights and the partial sums of squares [rows, parts] (its residual-add GEMM,
+or the kernel that adds that GEMM's K slices, writes them: decode steps of up to 128 rows), or
+(h, None, None): the norm's finished output (more rows, and steps of whole prompts), which the next
+consumer takes instead of reading the residual stream.
 
 A part whose launches in a decode step depend on host values (it reads ctx.host_*, or sizes that
 change from step to step) says so with the class attribute `graph_safe = False`; the layers around
@@ -132,7 +133,7 @@ class Part:
         return type(self).__name__, False
 
     @staticmethod
-    def _gemm(ctx, a, w, out, epilogue, hidden=0):
+    def _gemm(ctx, a, w, out, epilogue, hidden=0, scale_from=None):
         """kernels.gemm with the scratch that lets small batches split K."""
         from ..ops import kernels
         import torch
@@ -140,7 +141,7 @@ class Part:
         n = kernels.gemm_workspace_floats(a.shape[0], w.shape[0], a.shape[1]) if a.dtype == torch.bfloat16 else 0
         if n and ctx is not None:
             ws = ctx.ws.get("gemm.partial", (n,), torch.float32)
-        return kernels.gemm(a, w, out, epilogue, hidden=hidden, workspace=ws)
+        return kernels.gemm(a, w, out, epilogue, hidden=hidden, workspace=ws, scale_from=scale_from)
 
     def _emit_args(self, emit_for, ctx, T, width):
         """Operands for a residual-add GEMM that also prepares the activations of the norm
@@ -169,6 +170,22 @@ class Part:
         h = ctx.ws.get("chain.h", (T, width), torch.bfloat16)          # read by the consumer before the next is written
         ws = ctx.ws.get("gemm.partial", (kernels.fused_workspace_floats(T, width, K),), torch.float32)
         return nw, eps, h, ws
+
+    def _add_emit_args(self, emit_for, ctx, T, width, K):
+        """Operands for a residual-add GEMM [T, K] x [width, K] of a decode step of 17..128 rows that prepares the
+        norm `emit_for` as the chain of the small batches does (activations times the norm's weights, partial sums of
+        squares; the consumer scales its sums), or None."""
+        from ..ops import kernels
+        if emit_for is None or not hasattr(emit_for, "fused") or ctx.mode != "decode":
+            return None
+        if not (kernels.can_add_emit(T, K, ctx.act_dtype) and kernels.can_add_emit(T, width, ctx.act_dtype)):
+            return None
+        import torch
+        nw, eps = emit_for.fused()
+        xn = ctx.ws.get("chain.h", (T, width), torch.bfloat16)
+        ss = ctx.ws.get("chain.ss", (T, kernels.gemm_add_emit_parts(width)), torch.float32)
+        ws = ctx.ws.get("gemm.partial", (kernels.fused_workspace_floats(T, width, K),), torch.float32)
+        return nw, eps, xn, ss, ws
 
     def fuses_norm(self, norm, x, ctx):
         """True if this part can take the float32 residual stream x and do `norm` itself

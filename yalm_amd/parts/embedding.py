@@ -65,7 +65,9 @@ class LMHead(Part):
             return self._gemm(ctx, src[0], self.weight, logits, kernels.EPI_STORE_F32)
         if src is not None:
             xn, ss, eps = src
-            return kernels.gemm_chain(xn, self.weight, logits, kernels.EPI_STORE_F32, scale_from=(ss, eps))
+            if kernels.can_chain(xn.shape[0], self.dim, self.weight.dtype):
+                return kernels.gemm_chain(xn, self.weight, logits, kernels.EPI_STORE_F32, scale_from=(ss, eps))
+            return self._gemm(ctx, xn, self.weight, logits, kernels.EPI_STORE_F32, scale_from=(ss, eps))
         nw, eps = norm.fused()
         return kernels.gemm_norm(x, nw, eps, self.weight, logits, kernels.EPI_STORE_F32)
 

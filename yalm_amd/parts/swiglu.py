@@ -64,9 +64,12 @@ class SwiGLU(Part):
         T = x.shape[0]
         mid = ctx.ws.get("ffn.hidden", (T, self.hidden), self.w_down.dtype)
         src = ctx.normed.pop(id(norm), None)
-        if src is not None and src[1] is not None:
+        if src is not None and src[1] is not None and kernels.can_chain(T, self.dim, self.w_down.dtype):
             xn, ss, eps = src
             kernels.gemm_chain(xn, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden, scale_from=(ss, eps))
+        elif src is not None and src[1] is not None:          # 17..128 rows: prepared by the kernel that added the K slices
+            xn, ss, eps = src
+            self._gemm(ctx, xn, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden, scale_from=(ss, eps))
         elif src is not None:                     # the norm's output is ready
             self._gemm(ctx, src[0], self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
         elif kernels.can_fuse_norm(T, self.dim, self.w_down.dtype):
@@ -77,10 +80,15 @@ class SwiGLU(Part):
             norm.forward(x, h, ctx)
             self._gemm(ctx, h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
         emit = self._emit_args(emit_for, ctx, T, self.dim)
-        ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.hidden) if emit is None else None
+        prepared = self._add_emit_args(emit_for, ctx, T, self.dim, self.hidden) if emit is None else None
+        ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.hidden) if emit is None and prepared is None else None
         if emit is not None and kernels.can_chain(T, self.hidden, mid.dtype):
             nw2, xn2, ss2, eps2 = emit
             kernels.gemm_chain(mid, self.w_down, x, kernels.EPI_ADD_F32, emit=(nw2, xn2, ss2))
+            ctx.normed[id(emit_for)] = (xn2, ss2, eps2)
+        elif prepared is not None:
+            nw2, eps2, xn2, ss2, ws2 = prepared
+            kernels.gemm_add_emit(mid, self.w_down, x, nw2, xn2, ss2, ws2)
             ctx.normed[id(emit_for)] = (xn2, ss2, eps2)
         elif ready is not None and kernels.can_add_norm(T, self.hidden, mid.dtype):
             nw2, eps2, h2, ws2 = ready
