@@ -220,6 +220,10 @@ def time_kernel_groups(calls, kv_tokens, torch, dtype, reps=5):
     return out
 
 
+def mean_of(values):
+    return int(sum(values) / len(values))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -441,11 +445,12 @@ def main():
         from yalm_amd.generate import GenerationStats, generate
         lens = torch.randint(RAGGED_LENS[0], RAGGED_LENS[1] + 1, (RAGGED_B,), generator=gen).tolist()
         prompts = [torch.randint(0, V, (n,), generator=gen).tolist() for n in lens]
-        engine.warmup([RAGGED_B], min_len=min(lens), max_len=max(lens) + args.ragged_new + 1)
+        engine.warmup([RAGGED_B], min_len=max(lens), max_len=max(lens) + args.ragged_new + 1, ragged=True)
+        engine.warmup([RAGGED_B], min_len=mean_of(lens), max_len=mean_of(lens) + args.ragged_new + 1)
         stats = GenerationStats()
         generate(engine, prompts, max_new_tokens=args.ragged_new, temperature=0.0, stop_ids=(), batch_size=RAGGED_B,
                  sampler=sampler, stats=stats)
-        mean_len = int(sum(lens) / len(lens))
+        mean_len = mean_of(lens)
         equal = decode(RAGGED_B, args.ragged_new - 8, 8, prompt_len=mean_len)
         line["ragged"] = {
             "requests": RAGGED_B, "prompt_min": min(lens), "prompt_max": max(lens), "prompt_mean": mean_len,

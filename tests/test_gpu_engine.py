@@ -365,3 +365,27 @@ def test_decode_batches_of_17_to_128_rows(tmp_path_factory, n, which, dtype):
     for rid, rows in got.items():
         want = helpers.plain_logits(folder, tuple(requests[rid]), dtype)
         helpers.check_logits(np.stack(rows), want, dtype, "%d rows (%s) %s request %s" % (n, which, dtype, rid))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_decode_batch_of_very_unequal_lengths(tmp_path_factory, dtype):
+    """Sequences of 30 to 900 tokens decode together: the step counts as ragged (its own captured graphs), the
+    attention cuts every sequence into splits of the longest one's split size, and the short ones end early."""
+    from yalm_amd.engine import Engine, Model
+    folder = helpers.make_folder(tmp_path_factory.mktemp("ragged"), "many_rows", MANY_ROWS, seed=10)
+    lengths = [900, 30, 410, 64, 65, 700, 129, 33, 512, 250, 31, 880]
+    requests = helpers.random_requests(MANY_ROWS, lengths, seed=41)
+    first = {rid: len(t) - 3 - (i % 5) for i, (rid, t) in enumerate(requests.items())}
+    steps = schedules.batches(requests, [list(requests)], first)
+    model = Model.from_folder(folder, dtype=helpers.torch_dtype(dtype), device="cuda:0")
+    engine = Engine(model, max_tokens=schedules.max_tokens_needed(steps), max_batch=len(lengths))
+    assert engine._is_ragged(lengths) and not engine._is_ragged([900, 880, 860]) and not engine._is_ragged([5])
+    out = schedules.replay_in_process(engine, steps)
+    assert any(key[2] for key in engine._graphs)                  # graphs of the ragged kind were captured and used
+    if dtype == "bfloat16":
+        mixer = model.blocks[0].mixer
+        assert mixer.decode_splits(64, 16, ragged=True) == 4 and mixer.decode_splits(64, 16) == 2
+    got = schedules.per_request(steps, out, requests)
+    for rid, toks in requests.items():
+        want = helpers.plain_logits(folder, tuple(toks), dtype)
+        helpers.check_logits(got[rid][first[rid] - 1:], want[first[rid] - 1:], dtype, "ragged batch %s request %s" % (dtype, rid))

@@ -671,6 +671,21 @@ def one_query_reference(q, keys, vals, window):
     (4, 2, 16, 0, [5, 64, 65, 1], 1), (3, 1, 32, 16, [2, 30, 200], 2), (6, 3, 48, 100, [130, 640, 99], 3),
     (8, 2, 128, 0, [1000, 3], 7), (2, 2, 80, 0, [129], 4), (32, 8, 128, 0, [300], 2), (5, 5, 64, 70, [700, 64], 16)])
 def test_attn_decode(n_heads, n_kv, hd, window, lens, splits, dtype, simple):
+    _attn_decode_case(n_heads, n_kv, hd, window, lens, splits, dtype, simple, None)
+
+
+@pytest.mark.parametrize("said", ["longest", 1, 100000])
+@pytest.mark.parametrize("n_heads,n_kv,hd,window,lens,splits", [
+    (8, 2, 128, 0, [1000, 3, 517, 64, 65], 4), (4, 1, 64, 0, [40, 900], 7), (5, 5, 64, 150, [700, 64, 164, 150, 128], 3),
+    (8, 2, 128, 100, [164, 150, 128, 100, 99], 2)])
+def test_attn_decode_with_the_length_of_the_longest_sequence(n_heads, n_kv, hd, window, lens, splits, said):
+    """Splits of the longest sequence's split size: the same results, whatever length the step says its longest
+    sequence has (the truth, too little, too much), also where a window makes a shorter sequence span more pages
+    than the longest does; and the workgroups take the rows in another order than the rows'."""
+    _attn_decode_case(n_heads, n_kv, hd, window, lens, splits, torch.bfloat16, False, max(lens) if said == "longest" else said)
+
+
+def _attn_decode_case(n_heads, n_kv, hd, window, lens, splits, dtype, simple, step_max_len):
     k = K()
     B = len(lens)
     kp, vp, bt, slots, ring, keys, vals = paged_case(lens, n_kv, hd, window, dtype, 20)
@@ -682,7 +697,8 @@ def test_attn_decode(n_heads, n_kv, hd, window, lens, splits, dtype, simple):
     k.FORCE_SIMPLE = simple
     try:
         k.attn_decode(qd, kp.to(DEV), vp.to(DEV), bt.to(DEV), ring, i32(slots + [-1]), i32(lens + [0]), out, partial,
-                      n_heads, n_kv, hd, window, splits)
+                      n_heads, n_kv, hd, window, splits, step_max_len=None if step_max_len is None else i32([step_max_len]),
+                      seq_order=None if step_max_len is None else i32(list(np.random.default_rng(5).permutation(B + 1))))
     finally:
         k.FORCE_SIMPLE = False
     for b, n in enumerate(lens):

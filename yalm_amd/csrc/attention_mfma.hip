@@ -53,12 +53,15 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out, float* __restrict__ lse,
-    int n_heads, int n_kv_heads, int window, int n_splits, int n_pages) {
+    int n_heads, int n_kv_heads, int window, int n_splits, int n_pages, const int* __restrict__ step_max_len,
+    const int* __restrict__ seq_order) {
   constexpr int KS = HD / 32, DT = HD / 16;
   __shared__ float sm_m[NW][16];
   __shared__ float sm_l[NW][16];
   __shared__ f32x4 sm_o[NW][DT][WAVE];
-  const int split = blockIdx.x, g = blockIdx.y, b = blockIdx.z;
+  // seq_order: the rows in the order of their cost (only which workgroup takes which row changes)
+  const int split = blockIdx.x, g = blockIdx.y;
+  const int b = seq_order != nullptr ? min(max(seq_order[blockIdx.z], 0), (int)gridDim.z - 1) : (int)blockIdx.z;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE, qd = lane / 16,
             j = lane % 16;
   const int G = n_heads / n_kv_heads;
@@ -74,7 +77,16 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
     const int lo = window > 0 ? max(0, L - window) : 0;
     const int first_page = lo / PAGE, last_page = (L - 1) / PAGE;
     const int total = last_page - first_page + 1;
-    const int per = (total + n_splits - 1) / n_splits;
+    int per = (total + n_splits - 1) / n_splits;
+    if (step_max_len != nullptr) {
+      // Sequences of unequal lengths: a split is as many pages as the longest sequence's split, so that every working
+      // workgroup has the same work and a short sequence uses fewer of its splits (the others find nothing to do),
+      // instead of every sequence cutting its own length into n_splits pieces of unequal cost.  Whatever the value
+      // says, the sequence's own pages are all covered.
+      const int Lm = max(step_max_len[0], 1);
+      const int total_m = (Lm - 1) / PAGE - (window > 0 ? max(0, Lm - window) / PAGE : 0) + 1;
+      per = max(per, (total_m + n_splits - 1) / n_splits);
+    }
     const int p_begin = first_page + split * per;
     const int p_end = min(last_page + 1, p_begin + per);
     // scores and the running maximum are kept in units of log2(e) / sqrt(head_dim): one multiply, and 2^x is one instruction
@@ -597,7 +609,7 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                                int n_splits, int n_pages, int page_layout, const SinkArgs& sinks,
-                               hipStream_t stream) {
+                               const int* step_max_len, const int* seq_order, hipStream_t stream) {
   // with sinks the merge kernel always runs: it takes them in, also where there is one split
   const bool merge = n_splits > 1 || sinks.n_sinks > 0;
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_heads / n_kv_heads > 16) return YALM_ERR_ARG;
@@ -605,7 +617,8 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
 #define YALM_DECODE(HD_, NW_, BLOCKS_)                                                                              \
   attn_decode_mfma_kernel<HD_, NW_, BLOCKS_><<<grid, NW_ * WAVE, 0, stream>>>(                                      \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot, \
-      seq_len, partial, merge ? nullptr : (bf16*)out, lse, n_heads, n_kv_heads, window, n_splits, n_pages)
+      seq_len, partial, merge ? nullptr : (bf16*)out, lse, n_heads, n_kv_heads, window, n_splits, n_pages, \
+      step_max_len, seq_order)
   // 4 waves a workgroup: 8 measured no faster with one split and slower with more (a CU draws about
   // 33 GB/s whatever its number of waves, so a small batch needs its workgroups spread over all CUs)
   if (page_layout == YALM_PAGE_BLOCKS) {

@@ -15,7 +15,8 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
-                               int n_splits, int n_pages, int page_layout, const SinkArgs& sinks, hipStream_t stream);
+                               int n_splits, int n_pages, int page_layout, const SinkArgs& sinks,
+                               const int* step_max_len, const int* seq_order, hipStream_t stream);
 
 namespace {
 constexpr int MAX_HD = 256;              // head sizes up to 256 (4 output elements per lane)
@@ -348,7 +349,8 @@ namespace {
 int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, const int* block_table, int table_stride,
                     int ring_pages, const int* seq_slot, const int* seq_len, void* out, float* lse, float* partial,
                     int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits, int n_pages,
-                    int page_layout, int dtype, int force_simple, const SinkArgs& sinks, hipStream_t stream) {
+                    int page_layout, int dtype, int force_simple, const SinkArgs& sinks, const int* step_max_len,
+                    const int* seq_order, hipStream_t stream) {
   if (B <= 0) return YALM_OK;
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0 ||
       !page_layout_ok(page_layout, head_dim))
@@ -366,7 +368,7 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
   if (!force_simple) {
     int rc = yalm_attn_decode_bf16_mfma(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len,
                                         out, lse, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits,
-                                        n_pages, page_layout, sinks, stream);
+                                        n_pages, page_layout, sinks, step_max_len, seq_order, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   attn_decode_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>(
@@ -382,11 +384,12 @@ extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const vo
                                     int table_stride, int ring_pages, const int* seq_slot, const int* seq_len,
                                     void* out, float* lse, float* partial, int B, int n_heads, int n_kv_heads,
                                     int head_dim, int window, int n_splits, int n_pages, int page_layout, int dtype,
-                                    int force_simple, hipStream_t stream) {
+                                    int force_simple, const int* step_max_len, const int* seq_order,
+                                    hipStream_t stream) {
   SinkArgs none = {};
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, lse,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, none, stream);
+                         force_simple, none, step_max_len, seq_order, stream);
 }
 
 extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -395,7 +398,7 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
                                 int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream) {
   return yalm_attn_decode_lse(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out,
                               nullptr, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages,
-                              YALM_PAGE_ROWS, dtype, force_simple, stream);
+                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, stream);
 }
 
 extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -404,7 +407,7 @@ extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const 
                                       const float* cos_sin, int n_positions, int n_slots, int rotary_dim, int n_sinks,
                                       int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits,
                                       int n_pages, int page_layout, int dtype, int force_simple,
-                                      hipStream_t stream) {
+                                      const int* step_max_len, const int* seq_order, hipStream_t stream) {
   if (n_sinks <= 0 || n_sinks > YALM_MAX_SINKS || window < n_sinks || n_slots <= 0 || sink_k == nullptr ||
       sink_v == nullptr || rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2 || head_dim % 2)
     return YALM_ERR_ARG;
@@ -431,7 +434,7 @@ extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const 
   sk.n_sinks = n_sinks;
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, nullptr,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, sk, stream);
+                         force_simple, sk, step_max_len, seq_order, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -155,7 +155,10 @@ long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits);
 
 // The two above, which also leave lse[token, head] (float32; may be null) = the natural logarithm of the
 // sum of exp(score) over the keys the query saw (-FLT_MAX for a padding row), so that further keys can be
-// mixed in afterwards (yalm_attn_sink_mix).
+// mixed in afterwards (yalm_attn_sink_mix).  step_max_len (device, one int, may be null): the length of the step's
+// longest sequence; the matrix-core decode kernel then cuts every sequence into splits of that sequence's split size,
+// so that sequences of unequal lengths give workgroups of equal work (no result depends on it).  seq_order (device,
+// B ints, a permutation of the rows; may be null): the order in which that kernel's workgroups take the rows.
 int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* lse,
                           const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                           const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads, int n_kv_heads,
@@ -164,7 +167,7 @@ int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages
                          int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                          float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                          int n_splits, int n_pages, int page_layout, int dtype, int force_simple,
-                         hipStream_t stream);
+                         const int* step_max_len, const int* seq_order, hipStream_t stream);
 
 // Attention sinks beside a window (src/infer.cpp:305-319, 486-488): the first n_sinks positions of a
 // sequence stay visible when the window has moved past them, and each then counts as lying
@@ -196,7 +199,8 @@ int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pag
                            float* partial, void* sink_k, void* sink_v, int store, const float* cos_sin,
                            int n_positions, int n_slots, int rotary_dim, int n_sinks, int B, int n_heads,
                            int n_kv_heads, int head_dim, int window, int n_splits, int n_pages, int page_layout,
-                           int dtype, int force_simple, hipStream_t stream);
+                           int dtype, int force_simple, const int* step_max_len, const int* seq_order,
+                           hipStream_t stream);
 
 // yalm_attn_decode without a workspace argument, for callers that cannot allocate device memory
 // (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no

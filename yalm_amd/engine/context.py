@@ -74,7 +74,11 @@ class StepContext:
     host_slots, host_n_tokens, host_start: the step's real sequences as host lists (a decode step's
     padding rows, seq_slot -1, are not in them), for parts whose launches depend on host values.
     pages_bucket: decode only; an upper bound (a power of two) of the pages of the step's
-    longest sequence, the only way launch shapes may depend on lengths."""
+    longest sequence; with `ragged` (decode only: the step's sequences differ much in length, so that work
+    cut per sequence would be uneven) the only way launch shapes may depend on lengths.
+    step_max_len: decode only; int32 [1] on the device, the length of the step's longest sequence.
+    seq_order: ragged decode steps only; int32 [B] on the device, the rows in the order in which a kernel whose
+    work grows with a row's length should take them (the longest first, the second half from the shortest up)."""
 
     def __init__(self, mode, cache, ws, act_dtype, shared_lines=()):
         self.mode = mode
@@ -87,6 +91,9 @@ class StepContext:
         self.x = None                     # the residual stream of the step, float32 [T, dim]
         self.normed = {}                  # id(norm part) -> (xn, ss, eps): activations a producer emitted for it
         self.pages_bucket = 1 << 30       # decode: no sequence of the step has more pages than this
+        self.ragged = False
+        self.step_max_len = None
+        self.seq_order = None
         self.max_position = 0
         self.host_slots = []
         self.host_n_tokens = []

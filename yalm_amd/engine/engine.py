@@ -37,7 +37,7 @@ class _BucketBuffers:
 
     def __init__(self, engine, bucket):
         self.bucket = bucket
-        n_meta = 6 * bucket + 1
+        n_meta = 7 * bucket + 2
         self.meta_host = [torch.empty(n_meta, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         self.copied = [None, None]    # the event after the last upload of each host copy
         self.turn = 0
@@ -61,13 +61,16 @@ class _DecodeGraph:
     """A decode step for one (batch bucket, pages bucket): the model's graph-safe runs of units as
     captured graphs, the others as (None, first, end) to be run kernel by kernel in between."""
 
-    def __init__(self, engine, bufs, pages_bucket):
+    def __init__(self, engine, bufs, pages_bucket, ragged):
         B = bufs.bucket
         self.bufs = bufs
         self.ctx = engine._context("decode", engine.graph_ws, bufs.meta, B, B, 0)
-        self.ctx.pages_bucket = pages_bucket
         self.eager_ctx = engine._context("decode", engine.ws, bufs.meta, B, B, 0)
-        self.eager_ctx.pages_bucket = pages_bucket
+        for ctx in (self.ctx, self.eager_ctx):
+            ctx.pages_bucket = pages_bucket
+            ctx.ragged = ragged
+            ctx.step_max_len = bufs.meta[6 * B + 1:6 * B + 2]
+            ctx.seq_order = bufs.meta[6 * B + 2:7 * B + 2] if ragged else None
         self.segments = []
         self.x = None
         self.logits = None
@@ -113,7 +116,7 @@ class Engine:
         self._any_graph = any(safe for safe, _, _ in self._segments)
         for text in model.describe()[1]:                # a slow fallback is said once, not hidden
             sys.stderr.write("[yalm_amd] %s\n" % text)
-        self._graphs = OrderedDict()                    # (batch bucket, pages bucket) -> _DecodeGraph, least recently used first
+        self._graphs = OrderedDict()                    # (batch bucket, pages bucket, ragged) -> _DecodeGraph, least recently used first
         self._buckets = {}
         self.graphs_captured = 0
 
@@ -335,9 +338,10 @@ class Engine:
         return B
 
     @staticmethod
-    def _fill_decode_meta(host, Bk, tokens, starts, slots, new_lens):
+    def _fill_decode_meta(host, Bk, tokens, starts, slots, new_lens, ragged=False):
         """The metadata of a decode step of len(slots) sequences in Bk rows; the rows behind
-        them are padding (token -1, slot -1, length 0)."""
+        them are padding (token -1, slot -1, length 0).  Behind the tensors of the context: the longest
+        sequence's length, and an order of the rows for kernels whose work grows with a row's length."""
         B = len(slots)
         host[0:Bk] = -1
         host[0:B] = tokens
@@ -349,6 +353,27 @@ class Engine:
         host[4 * Bk:5 * Bk] = 0
         host[4 * Bk:4 * Bk + B] = new_lens
         host[5 * Bk:6 * Bk + 1] = np.arange(Bk + 1, dtype=np.int32)
+        host[6 * Bk + 1] = max(new_lens) if len(new_lens) else 0
+        order = host[6 * Bk + 2:7 * Bk + 2]
+        order[:] = np.arange(Bk, dtype=np.int32)
+        if ragged and B > 1:
+            # The rows by length, the longest first, and the second half turned round: where a kernel's workgroups
+            # stand two to a compute unit, the one that follows the longest sequence's is the shortest one's.
+            ranks = np.argsort(-np.asarray(new_lens, dtype=np.int64), kind="stable").astype(np.int32)
+            half = (Bk + 1) // 2
+            rows = np.concatenate([ranks, np.arange(B, Bk, dtype=np.int32)])
+            order[:half] = rows[:half]
+            order[half:] = rows[half:][::-1]
+
+    @staticmethod
+    def _is_ragged(new_lens):
+        """True if the sequences of a decode step differ so much in length that cutting each into the same number
+        of pieces would leave workgroups of very unequal work (the longest is a fifth and two pages above the mean)."""
+        n = len(new_lens)
+        if n < 2:
+            return False
+        longest, mean = max(new_lens), sum(new_lens) / n
+        return longest - mean >= max(2 * PAGE, 0.2 * longest)
 
     @staticmethod
     def _pages_bucket(n_tokens):
@@ -365,22 +390,26 @@ class Engine:
         use_graph = self.use_graphs and self._any_graph
         Bk = self._bucket(B) if use_graph else B
         pages_bucket = self._pages_bucket(max(new_lens))
+        ragged = self._is_ragged(new_lens)
         if firsts is None:
             firsts = 0                                                # a place holder; fed below
         if not use_graph:
-            host = np.empty(6 * Bk + 1, dtype=np.int32)
-            self._fill_decode_meta(host, Bk, firsts, starts, slots, new_lens)
-            meta = self.ws.get("meta", (6 * Bk + 1,), torch.int32)
+            host = np.empty(7 * Bk + 2, dtype=np.int32)
+            self._fill_decode_meta(host, Bk, firsts, starts, slots, new_lens, ragged)
+            meta = self.ws.get("meta", (7 * Bk + 2,), torch.int32)
             meta.copy_(torch.from_numpy(host))
             self._feed(meta, B, source, source_rows)
             ctx = self._context("decode", self.ws, meta, Bk, Bk, max(starts))
             ctx.pages_bucket = pages_bucket
+            ctx.ragged = ragged
+            ctx.step_max_len = meta[6 * Bk + 1:6 * Bk + 2]
+            ctx.seq_order = meta[6 * Bk + 2:7 * Bk + 2] if ragged else None
             ctx.host_slots, ctx.host_n_tokens, ctx.host_start = list(slots), [1] * B, list(starts)
             logits = self.ws.get("logits", (Bk, self.model.vocab_size), torch.float32)
             self.model.forward(ctx, None, logits)                     # every row
         else:
-            g = self._graph(Bk, pages_bucket)
-            self._fill_decode_meta(g.bufs.host(), Bk, firsts, starts, slots, new_lens)
+            g = self._graph(Bk, pages_bucket, ragged)
+            self._fill_decode_meta(g.bufs.host(), Bk, firsts, starts, slots, new_lens, ragged)
             g.bufs.upload()
             self._feed(g.bufs.meta, B, source, source_rows)
             for graph, lo, hi in g.segments:
@@ -413,12 +442,13 @@ class Engine:
             torch.index_select(source, 0, index, out=meta[0:B])
 
     # ------------------------------------------------------------------ captured decode steps
-    def _graph(self, Bk, pages_bucket):
-        """The captured step for the bucket pair, made now if there is none (most recently used last)."""
+    def _graph(self, Bk, pages_bucket, ragged=False):
+        """The captured step for the bucket pair (and for sequences of much the same or of very unequal lengths),
+        made now if there is none (most recently used last)."""
         if self.model.tables_version != self._tables_version:       # a table the graphs point to was replaced
             self.drop_graphs()
             self._tables_version = self.model.tables_version
-        key = (Bk, pages_bucket)
+        key = (Bk, pages_bucket, bool(ragged))
         g = self._graphs.get(key)
         if g is None:
             if len(self._graphs) >= self.max_graphs or not self._graphs:
@@ -427,13 +457,13 @@ class Engine:
                 self._graphs.popitem(last=False)
             if not self._graphs:
                 self.graph_ws.drop_retired()
-            g = self._capture(Bk, pages_bucket)
+            g = self._capture(Bk, pages_bucket, bool(ragged))
             self._graphs[key] = g
         else:
             self._graphs.move_to_end(key)
         return g
 
-    def _capture(self, Bk, pages_bucket):
+    def _capture(self, Bk, pages_bucket, ragged=False):
         """Captures the decode step of a bucket pair on rows of padding only: nothing that a live
         sequence holds (cache pages, per-sequence state) is read or written, so capturing in the
         middle of a request changes nothing for it.  The step runs once kernel by kernel first
@@ -443,7 +473,7 @@ class Engine:
             bufs = self._buckets[Bk] = _BucketBuffers(self, Bk)
         self._fill_decode_meta(bufs.host(), Bk, [], [], [], [])
         bufs.upload()
-        g = _DecodeGraph(self, bufs, pages_bucket)
+        g = _DecodeGraph(self, bufs, pages_bucket, ragged)
         ws, ctx = self.graph_ws, g.ctx
         ctx.max_position = 0
         ctx.x = g.x = ws.get("x", (Bk, self.model.dim), torch.float32)
@@ -467,9 +497,10 @@ class Engine:
         self.graphs_captured += 1
         return g
 
-    def warmup(self, batch_sizes=(1,), max_len=None, min_len=1):
+    def warmup(self, batch_sizes=(1,), max_len=None, min_len=1, ragged=False):
         """Captures the decode graphs for batches of the given sizes and for sequences of min_len to
-        max_len tokens (default: the longest the engine holds) ahead of the first request, so that no
+        max_len tokens (default: the longest the engine holds; ragged: for batches whose sequences differ
+        much in length) ahead of the first request, so that no
         live step pays for a capture.  It runs on padding rows: no slot or page is taken and live
         sequences are left alone (the reference runs one forward before it measures,
         src/main.cpp:81-85, which overwrites a cache row).  Returns the number of graphs captured."""
@@ -490,7 +521,7 @@ class Engine:
             raise StepError("warmup asks for %d graphs, the engine keeps %d (max_graphs)" % (len(pairs), self.max_graphs))
         before = self.graphs_captured
         for Bk, pb in pairs:
-            self._graph(Bk, pb)
+            self._graph(Bk, pb, ragged)
         return self.graphs_captured - before
 
     def drop_graphs(self):

@@ -590,9 +590,12 @@ def attn_decode_workspace_floats(B, n_heads, head_dim, n_splits):
 
 
 def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len, out, partial, n_heads, n_kv_heads,
-                head_dim, window, n_splits, lse=None, sinks=None, layout=None):
+                head_dim, window, n_splits, lse=None, sinks=None, layout=None, step_max_len=None, seq_order=None):
     """One query per sequence over the cache pages (laid out as `layout` says, default page_layout(head_dim));
-    seq_len counts the new key.  lse as in attn_prefill.
+    seq_len counts the new key.  lse as in attn_prefill.  step_max_len (int32 [1] on the device, optional): the
+    length of the step's longest sequence, with which sequences of unequal lengths are cut into splits of equal
+    size; seq_order (int32 [B] on the device, a permutation of the rows, optional): the order in which the
+    workgroups take the rows (both change the division of the work and no result).
     sinks = (sink_k, sink_v [slots, n_kv_heads, n_sinks, head_dim], cos_sin or None, rotary_dim, store):
     the attention sinks that a query's window no longer covers are taken in where the splits are merged
     (their keys turned by max(0, position - window - n_sinks + 1) positions with the table cos_sin); with
@@ -616,11 +619,13 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
     if partial.numel() < need:
         raise ValueError("attn_decode workspace too small: %d floats, %d needed" % (partial.numel(), need))
     force = 1 if FORCE_SIMPLE else 0
+    p_max = _opt(step_max_len, "step_max_len", torch.int32, (1,))
+    p_ord = _opt(seq_order, "seq_order", torch.int32, (B,))
     if sinks is None:
         p_lse = None if lse is None else _need(lse, "lse", torch.float32, (B, n_heads))
         library.check(library.lib().yalm_attn_decode_lse(
             p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_lse, p_w, B, n_heads, n_kv_heads, head_dim,
-            int(window), int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, _stream()),
+            int(window), int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, p_max, p_ord, _stream()),
             "attn_decode")
         return out
     if lse is not None:
@@ -640,7 +645,8 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
         _need(sink_k, "sink_k", dt, (n_slots, n_kv_heads, n_sinks, head_dim)),
         _need(sink_v, "sink_v", dt, (n_slots, n_kv_heads, n_sinks, head_dim)), 1 if store else 0, p_cs, n_pos, n_slots,
         int(rotary_dim) if p_cs is not None else 0, n_sinks, B, n_heads, n_kv_heads, head_dim, int(window),
-        int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, _stream()), "attn_decode with sinks")
+        int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, p_max, p_ord, _stream()),
+        "attn_decode with sinks")
     return out
 
 

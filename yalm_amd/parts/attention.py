@@ -114,13 +114,20 @@ class GQAttention(Part):
         return what + ": float32-arithmetic kernels on bfloat16 storage (the matrix-core kernels take head sizes " \
                       "64 and 128 and up to 16 heads a group, not %s): correct, several times slower" % why, True
 
-    def decode_splits(self, B, max_pages):
+    def decode_splits(self, B, max_pages, ragged=False):
         mfma = self.head_dim in (64, 128) and self.n_heads // self.n_kv_heads <= 16 and not kernels.FORCE_SIMPLE
         if mfma:         # a workgroup of 4 waves per (split, KV head, sequence), a page per wave at a time
             per = max(1, B * self.n_kv_heads)
+            quarters = max(1, min((max_pages + 3) // 4, 4))
             if per > RESIDENT_WORKGROUPS:         # more than run at once: in quarters the last round is short
-                return max(1, min((max_pages + 3) // 4, 4))
-            return max(1, min((max_pages + 3) // 4, TARGET_WORKGROUPS // per))
+                return quarters
+            even = max(1, min((max_pages + 3) // 4, TARGET_WORKGROUPS // per))
+            # Sequences of very unequal lengths.  Where the workgroups stand two to a compute unit anyway, one split and
+            # the rows in the order that pairs a long sequence with a short one; else splits of the longest sequence's
+            # split size (the kernel cuts them so), enough of them that the long sequences' work spreads over the chip.
+            if ragged and per <= TARGET_WORKGROUPS:
+                return max(even, quarters)
+            return even
         return max(1, min(max_pages, TARGET_WORKGROUPS // max(1, B * self.n_heads)))
 
     def fuses_norm(self, norm, x, ctx):
@@ -212,7 +219,7 @@ class GQAttention(Part):
 
     def _decode_attention(self, q, o, ctx, group, line, k_pages, v_pages, writes_cache):
         T = q.shape[0]
-        n_splits = self.decode_splits(T, min(group.ring_pages, ctx.pages_bucket))
+        n_splits = self.decode_splits(T, min(group.ring_pages, ctx.pages_bucket), ctx.ragged)
         partial = ctx.ws.get("attn.partial",
                              (kernels.attn_decode_workspace_floats(T, self.n_heads, self.head_dim, n_splits),),
                              torch.float32)
@@ -221,7 +228,8 @@ class GQAttention(Part):
             sink_k, sink_v = group.line_sinks(line)        # has just written a sink, which is stored on the way
             sinks = (sink_k, sink_v, self.position.table, self.position.rotary_dim, writes_cache)
         kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o, partial,
-                            self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits, sinks=sinks)
+                            self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits, sinks=sinks,
+                            step_max_len=ctx.step_max_len, seq_order=ctx.seq_order)
 
     def forward(self, h, x, ctx, line, writes_cache=True, emit_for=None):
         T = h.shape[0]
