@@ -699,3 +699,31 @@ def test_a_library_built_from_other_sources_is_built_again(tmp_path, monkeypatch
     with pytest.raises(Reached):
         build.build(force=True)
     assert len(build.sources_digest()) == 64
+
+
+def test_decode_metadata_orders_a_ragged_batch_by_length():
+    """The step's metadata: tokens, rows, positions, slots, lengths, offsets, then the longest length and an order
+    of the rows, which is a permutation whatever the lengths are: the longest rows first, the second half from the
+    shortest up, padding rows in the middle."""
+    import numpy as np
+    from yalm_amd.engine.engine import Engine
+    Bk = 8
+    host = np.full(7 * Bk + 2, -7, dtype=np.int32)
+    lens = [900, 30, 410, 64, 700]
+    Engine._fill_decode_meta(host, Bk, [5, 6, 7, 8, 9], [n - 1 for n in lens], [3, 0, 4, 1, 2], lens, ragged=True)
+    assert list(host[0:Bk]) == [5, 6, 7, 8, 9, -1, -1, -1] and list(host[3 * Bk:4 * Bk]) == [3, 0, 4, 1, 2, -1, -1, -1]
+    assert list(host[4 * Bk:5 * Bk]) == lens + [0, 0, 0] and host[6 * Bk + 1] == 900
+    order = list(host[6 * Bk + 2:7 * Bk + 2])
+    assert sorted(order) == list(range(Bk))
+    assert order[:4] == [0, 4, 2, 3] and order[4:] == [7, 6, 5, 1]        # 900, 700, 410, 64 | padding ..., then 30
+    Engine._fill_decode_meta(host, Bk, [5, 6, 7, 8, 9], [n - 1 for n in lens], [3, 0, 4, 1, 2], lens)
+    assert list(host[6 * Bk + 2:7 * Bk + 2]) == list(range(Bk))
+    Engine._fill_decode_meta(host, Bk, [], [], [], [], ragged=True)        # a capture's rows of padding
+    assert host[6 * Bk + 1] == 0 and list(host[6 * Bk + 2:]) == list(range(Bk))
+    assert Engine._is_ragged(lens) and not Engine._is_ragged([900, 880]) and not Engine._is_ragged([100, 20, 60])
+    for trial in range(50):
+        rng = np.random.default_rng(trial)
+        B = int(rng.integers(1, Bk + 1))
+        ls = [int(x) for x in rng.integers(1, 5000, size=B)]
+        Engine._fill_decode_meta(host, Bk, [0] * B, [n - 1 for n in ls], list(range(B)), ls, ragged=True)
+        assert sorted(host[6 * Bk + 2:7 * Bk + 2]) == list(range(Bk))

@@ -553,14 +553,10 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
     const size_t lds = 4 * tile_bytes;
     auto k128 = &attn_prefill_mfma_kernel<128, 1, 2>;
     auto k64 = &attn_prefill_mfma_kernel<64, 1, 2>;
-    static bool allowed = false;                   // more than 64 KB of LDS has to be asked for once
-    if (!allowed) {
-      hipError_t e = hipFuncSetAttribute((const void*)k128, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-      if (e == hipSuccess)
-        e = hipFuncSetAttribute((const void*)k64, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-      if (e != hipSuccess) return (int)e;
-      allowed = true;
-    }
+    static LdsAllowance allowed128, allowed64;     // more than 64 KB of LDS has to be asked for once a device
+    int rc_lds = head_dim == 128 ? allow_dynamic_lds(allowed128, (const void*)k128, 150 * 1024)
+                                 : allow_dynamic_lds(allowed64, (const void*)k64, 150 * 1024);
+    if (rc_lds != YALM_OK) return rc_lds;
     dim3 all(n_heads, n_tiles);
     if (head_dim == 128)
       k128<<<all, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, nullptr, 0, B, n_heads,
@@ -575,14 +571,10 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
     const size_t lds = 4 * tile_bytes;
     auto k128 = &attn_prefill_mfma_kernel<128, 2, 2>;
     auto k64 = &attn_prefill_mfma_kernel<64, 2, 2>;
-    static bool allowed = false;                   // more than 64 KB of LDS has to be asked for once
-    if (!allowed) {
-      hipError_t e = hipFuncSetAttribute((const void*)k128, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-      if (e == hipSuccess)
-        e = hipFuncSetAttribute((const void*)k64, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-      if (e != hipSuccess) return (int)e;
-      allowed = true;
-    }
+    static LdsAllowance allowed128, allowed64;     // more than 64 KB of LDS has to be asked for once a device
+    int rc_lds = head_dim == 128 ? allow_dynamic_lds(allowed128, (const void*)k128, 150 * 1024)
+                                 : allow_dynamic_lds(allowed64, (const void*)k64, 150 * 1024);
+    if (rc_lds != YALM_OK) return rc_lds;
     if (head_dim == 128)
       k128<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
                                        n_kv_heads, window);

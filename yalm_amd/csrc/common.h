@@ -3,6 +3,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <mutex>
 
 #define YALM_OK 0
 #define YALM_ERR_ARG 1001          // an argument the kernel family refuses
@@ -90,6 +91,25 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 #pragma unroll
   for (int i = 1; i < NW; ++i) s = fmaxf(s, red[i]);
   return s;
+}
+
+// More than 64 KB of dynamic LDS has to be allowed for a kernel before its first launch, on every device it is
+// launched on.  One LdsAllowance (a static of the launcher) per kernel: a bit per device, set under a lock.
+struct LdsAllowance {
+  std::mutex lock;
+  unsigned long long devices = 0;
+};
+static inline int allow_dynamic_lds(LdsAllowance& a, const void* kernel, int bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= 64) return YALM_ERR_ARG;
+  std::lock_guard<std::mutex> hold(a.lock);
+  if ((a.devices >> dev) & 1ull) return YALM_OK;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return (int)e;
+  a.devices |= 1ull << dev;
+  return YALM_OK;
 }
 
 static inline int launch_status() {

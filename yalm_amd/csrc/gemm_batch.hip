@@ -369,12 +369,8 @@ int launch_kernel(dim3 grid, const bf16* X, const bf16* W, void* C, float* ws, i
     constexpr size_t lds = (size_t)NW * S * NTW * 2048 + (size_t)S * XG * 1024;
     static_assert(lds <= 128 * 1024, "the rings fit the LDS of a CU");
     auto kernel = &gemm_batch_dma_kernel<MT, NTW, EPI, S, NW>;
-    static bool allowed = false;                   // more than 64 KB of LDS has to be asked for once
-    if (!allowed) {
-      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (e != hipSuccess) return (int)e;
-      allowed = true;
-    }
+    static LdsAllowance allowed;                   // more than 64 KB of LDS has to be asked for once a device
+    if (int rc = allow_dynamic_lds(allowed, (const void*)kernel, (int)lds); rc != YALM_OK) return rc;
     kernel<<<grid, NW * WAVE, lds, stream>>>(X, W, C, ws, M, N, K, H, k_per_slice, always_partial, rs);
     return launch_status();
   }

@@ -204,13 +204,10 @@ int launch_shape(const bf16* A, const bf16* W, void* C, int M, int N, int K, int
   if (n_tiles < 0) n_tiles = ceil_div(N, TN) - n_tile0;     // column tiles n_tile0 ... of this launch
   const dim3 grid(n_tiles, ceil_div(M, TM), ceil_div(K / TK, tiles_per_slice));
   const size_t lds = (size_t)S * (TM + TN) * ROWB;
-  static bool allowed = false;                     // more than 64 KB of LDS has to be asked for once
-  if (!allowed) {
-    hipError_t e = hipFuncSetAttribute((const void*)&gemm_dma_kernel<EPI, TM, TN, S, NWM, NWN, MINW>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    allowed = true;
-  }
+  static LdsAllowance allowed;                     // more than 64 KB of LDS has to be asked for once a device
+  if (int rc = allow_dynamic_lds(allowed, (const void*)&gemm_dma_kernel<EPI, TM, TN, S, NWM, NWN, MINW>, (int)lds);
+      rc != YALM_OK)
+    return rc;
   gemm_dma_kernel<EPI, TM, TN, S, NWM, NWN, MINW><<<grid, NWM * NWN * WAVE, lds, stream>>>(A, W, C, M, N, K, H, partial,
                                                                                        tiles_per_slice, n_tile0);
   int rc = launch_status();
@@ -698,12 +695,8 @@ int launch_ring(const bf16* A, const bf16* W, void* C, int M, int N, int K, int 
   void (*kernel)(const bf16*, const bf16*, void*, int, int, int, int, int, int, float*, int);
   if constexpr (TN == 128) kernel = &gemm_ring_kernel<EPI, TN, MAP>;
   else kernel = &gemm_ring16_kernel<EPI, TN, MAP>;
-  static bool allowed = false;                     // more than 64 KB of LDS has to be asked for once
-  if (!allowed) {
-    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    allowed = true;
-  }
+  static LdsAllowance allowed;                     // more than 64 KB of LDS has to be asked for once a device
+  if (int rc = allow_dynamic_lds(allowed, (const void*)kernel, (int)lds); rc != YALM_OK) return rc;
   kernel<<<grid, 512, lds, stream>>>(A, W, C, M, N, K, H, n_tile0, n_tiles, partial, tiles_per_slice);
   return launch_status();
 }

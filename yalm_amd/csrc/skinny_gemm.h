@@ -418,12 +418,8 @@ int launch_dma(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H
   constexpr size_t lds = (size_t)NWAVES * S * (16 * TW + XR) * 128;
   static_assert(lds + NWAVES * TW * WAVE * 16 + 1024 <= 160 * 1024, "the ring and the partial sums fit the LDS of a CU");
   auto kernel = &gemm_skinny_kernel<1, NT, NWAVES, EPI, 1, false, TW, S, XR>;
-  static bool allowed = false;
-  if (!allowed) {
-    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return (int)e;
-    allowed = true;
-  }
+  static LdsAllowance allowed;                     // once a device
+  if (int rc = allow_dynamic_lds(allowed, (const void*)kernel, (int)lds); rc != YALM_OK) return rc;
   kernel<<<ceil_div(N, 16 * NT), NWAVES * WAVE, lds, stream>>>(X, W, C, M, N, K, H, ca);
   return launch_status();
 }
