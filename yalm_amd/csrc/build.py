@@ -137,6 +137,20 @@ def build(force=True, jobs=None):
     return lib
 
 
+def build_kernel_bench():
+    """Compiles kernel_bench.cpp (single kernels at 7B sizes, no Python) against the built library; returns the
+    program's path (beside the library)."""
+    lib = library_path()
+    out = os.path.join(os.path.dirname(lib), "kernel_bench")
+    cmd = [_hipcc(), "-O2", "-std=c++17", "-I" + HERE, os.path.join(HERE, "kernel_bench.cpp"), "-o", out,
+           "-L" + os.path.dirname(lib), "-lyalm_hip", "-Wl,-rpath,$ORIGIN"]
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("building kernel_bench failed:\n" + p.stderr)
+    _say("built " + out)
+    return out
+
+
 def library_path():
     """The built library; compiled now if none exists."""
     return build(force=False)
@@ -144,3 +158,5 @@ def library_path():
 
 if __name__ == "__main__":
     build(force=True)
+    if len(sys.argv) > 1 and sys.argv[1] == "kernel_bench":
+        build_kernel_bench()
