@@ -840,9 +840,15 @@ def test_attn_prefill_with_sinks(n_heads, n_kv, hd, rd, window, sinks, lens, dty
     k.FORCE_SIMPLE = simple
     try:
         k.sink_store(ksd, vsd, i32(tile0), i32(slots), i32(lens), sink_k, sink_v)
-        k.attn_prefill(qd, ksd, vsd, out, i32(cu), i32(tile0), i32(seq), i32(pos), n_heads, n_kv, hd, window, lse=lse)
+        # the unrounded result beside the rounded one: the row with the sinks mixed in is then rounded once
+        o32 = torch.full((T, n_heads * hd), float("nan"), device=DEV) if dtype == torch.bfloat16 else None
+        k.attn_prefill(qd, ksd, vsd, out, i32(cu), i32(tile0), i32(seq), i32(pos), n_heads, n_kv, hd, window, lse=lse,
+                       out_f32=o32)
         plain_window = out.clone()
-        k.attn_sink_mix(qd, out, lse, sink_k, sink_v, i32(seq), i32(pos), i32(slots), table, n_heads, rd, window)
+        if o32 is not None:
+            assert torch.equal(o32.to(dtype), out)
+        k.attn_sink_mix(qd, out, lse, sink_k, sink_v, i32(seq), i32(pos), i32(slots), table, n_heads, rd, window,
+                        src_f32=o32)
     finally:
         k.FORCE_SIMPLE = False
     inv = R.rope_inv_freq(hd, rd, 80.0)

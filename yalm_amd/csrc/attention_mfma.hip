@@ -266,7 +266,7 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 template <int HD, int NC, int KSPL>
 __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_stage, const bf16* __restrict__ v_stage,
-    bf16* __restrict__ out, float* __restrict__ lse, const int* __restrict__ cu_seqlens,
+    bf16* __restrict__ out, float* __restrict__ out_f32, float* __restrict__ lse, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_tile0, const int* __restrict__ tile_order, int fold_at, int B, int n_heads,
     int n_kv_heads, int window) {
   constexpr int KS = HD / 32, DT = HD / 16;
@@ -507,6 +507,13 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
       for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int r = 0; r < 4; ++r) orow[dt * 16 + 4 * qd + r] = static_cast<bf16>(o[c][dt][r] * inv_l);
+      if (out_f32 != nullptr) {                   // the unrounded row too, for whoever mixes further keys in
+        float* frow = out_f32 + ((size_t)(start + pos_q[c]) * n_heads + h) * HD;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) frow[dt * 16 + 4 * qd + r] = o[c][dt][r] * inv_l;
+      }
       if (lse != nullptr && qd == 0) lse[(size_t)(start + pos_q[c]) * n_heads + h] = m[c] * LN2 + logf(lt);
     }
   }
@@ -530,7 +537,8 @@ bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
 }
 }  // namespace
 
-int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out, float* lse,
+int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out, float* out_f32,
+                                float* lse,
                                 const int* cu_seqlens, const int* seq_tile0, const int* tile_order, int n_order,
                                 int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
                                 hipStream_t stream) {
@@ -559,10 +567,10 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
     if (rc_lds != YALM_OK) return rc_lds;
     dim3 all(n_heads, n_tiles);
     if (head_dim == 128)
-      k128<<<all, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, nullptr, 0, B, n_heads,
+      k128<<<all, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, nullptr, 0, B, n_heads,
                                       n_kv_heads, window);
     else
-      k64<<<all, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, nullptr, 0, B, n_heads,
+      k64<<<all, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, nullptr, 0, B, n_heads,
                                      n_kv_heads, window);
     return launch_status();
   }
@@ -576,10 +584,10 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
                                  : allow_dynamic_lds(allowed64, (const void*)k64, 150 * 1024);
     if (rc_lds != YALM_OK) return rc_lds;
     if (head_dim == 128)
-      k128<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
+      k128<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
                                        n_kv_heads, window);
     else
-      k64<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
+      k64<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
                                       n_kv_heads, window);
     return launch_status();
   }
@@ -589,10 +597,10 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
   const int fold_at = total > cus && total <= 2 * cus ? cus : (int)total;
   const size_t lds = 2 * tile_bytes;
   if (head_dim == 128)
-    attn_prefill_mfma_kernel<128, 2, 1><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, tile_order,
+    attn_prefill_mfma_kernel<128, 2, 1><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, tile_order,
                                                                    fold_at, B, n_heads, n_kv_heads, window);
   else
-    attn_prefill_mfma_kernel<64, 2, 1><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, lse, cu_seqlens, seq_tile0, tile_order,
+    attn_prefill_mfma_kernel<64, 2, 1><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, tile_order,
                                                                   fold_at, B, n_heads, n_kv_heads, window);
   return launch_status();
 }

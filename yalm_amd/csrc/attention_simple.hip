@@ -8,7 +8,8 @@
 #include "sinks.h"
 #include "yalm_hip.h"
 
-int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out, float* lse,
+int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* v_stage, void* out, float* out_f32,
+                                float* lse,
                                 const int* cu_seqlens, const int* seq_tile0, const int* tile_order, int n_order,
                                 int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
                                 hipStream_t stream);
@@ -29,8 +30,8 @@ constexpr int COMBINE_THREADS = 256;
 template <typename T>
 __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
     const T* __restrict__ q, const T* __restrict__ k_stage, const T* __restrict__ v_stage, T* __restrict__ out,
-    float* __restrict__ lse, const int* __restrict__ seq_tile0, const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_heads,
-    int n_kv_heads, int hd, int window) {
+    float* __restrict__ out_f32, float* __restrict__ lse, const int* __restrict__ seq_tile0,
+    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_heads, int n_kv_heads, int hd, int window) {
   __shared__ float qs[MAX_HD];
   __shared__ float ps[WAVE];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -85,7 +86,10 @@ __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
 #pragma unroll
   for (int a = 0; a < ACC; ++a) {
     int d = lane + a * WAVE;
-    if (d < hd) out[((size_t)t * n_heads + h) * hd + d] = from_f32<T>(acc[a] / l);
+    if (d < hd) {
+      out[((size_t)t * n_heads + h) * hd + d] = from_f32<T>(acc[a] / l);
+      if (out_f32 != nullptr) out_f32[((size_t)t * n_heads + h) * hd + d] = acc[a] / l;
+    }
   }
   // natural logarithm of the sum of exp(score) over the keys seen: for a later mix with further keys
   if (lse != nullptr && lane == 0) lse[(size_t)t * n_heads + h] = m + logf(l);
@@ -291,7 +295,8 @@ bool bad_heads(int n_heads, int n_kv_heads, int hd) {
 }
 }  // namespace
 
-extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* lse,
+extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* out_f32,
+                                     float* lse,
                                      const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                                  const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads,
                                  int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
@@ -301,19 +306,19 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32) {
     attn_prefill_simple_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)q, (const float*)k_stage,
-                                                                 (const float*)v_stage, (float*)out, lse, seq_tile0,
+                                                                 (const float*)v_stage, (float*)out, out_f32, lse, seq_tile0,
                                                                  tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
                                                                  window);
     return launch_status();
   }
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
   if (!force_simple) {
-    int rc = yalm_attn_prefill_bf16_mfma(q, k_stage, v_stage, out, lse, cu_seqlens, seq_tile0, tile_order, n_order, T, B,
+    int rc = yalm_attn_prefill_bf16_mfma(q, k_stage, v_stage, out, out_f32, lse, cu_seqlens, seq_tile0, tile_order, n_order, T, B,
                                          n_tiles, n_heads, n_kv_heads, head_dim, window, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   attn_prefill_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,
-                                                              (const bf16*)v_stage, (bf16*)out, lse, seq_tile0, tok_seq,
+                                                              (const bf16*)v_stage, (bf16*)out, out_f32, lse, seq_tile0, tok_seq,
                                                               tok_pos, n_heads, n_kv_heads, head_dim, window);
   return launch_status();
 }
@@ -323,7 +328,7 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
                                  const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads,
                                  int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
                                  hipStream_t stream) {
-  return yalm_attn_prefill_lse(q, k_stage, v_stage, out, nullptr, cu_seqlens, seq_tile0, tok_seq, tok_pos, tile_order,
+  return yalm_attn_prefill_lse(q, k_stage, v_stage, out, nullptr, nullptr, cu_seqlens, seq_tile0, tok_seq, tok_pos, tile_order,
                                n_order, T, B, n_tiles, n_heads, n_kv_heads, head_dim, window, dtype, force_simple,
                                stream);
 }

@@ -34,6 +34,7 @@ __global__ __launch_bounds__(WAVE) void sink_store_kernel(const T* __restrict__ 
 // grid (token, head); lanes over the head's elements, pairs (2p, 2p + 1) in one lane
 template <typename T>
 __global__ __launch_bounds__(WAVE) void attn_sink_mix_kernel(const T* __restrict__ q, T* __restrict__ out,
+                                                             const float* __restrict__ src_f32,
                                                              const float* __restrict__ lse,
                                                              const T* __restrict__ sink_k,
                                                              const T* __restrict__ sink_v,
@@ -71,7 +72,9 @@ __global__ __launch_bounds__(WAVE) void attn_sink_mix_kernel(const T* __restrict
   float denom = w0;
   for (int j = 0; j < n_out; ++j) denom += expf(w[j] - top);
   for (int i = lane; i < hd; i += WAVE) {
-    float acc = w0 * to_f32(orow[i]);
+    // the attention's result before it was rounded to the storage type, where the caller kept it: the mixed row is
+    // then rounded once, as a decode step's is
+    float acc = w0 * (src_f32 != nullptr ? src_f32[((size_t)t * n_heads + h) * hd + i] : to_f32(orow[i]));
     for (int j = 0; j < n_out; ++j)
       acc = fmaf(expf(w[j] - top), to_f32(sink_v[(((size_t)slot * n_kv_heads + g) * n_sinks + j) * hd + i]), acc);
     orow[i] = from_f32<T>(acc / denom);
@@ -102,7 +105,8 @@ extern "C" int yalm_sink_store(const void* k_stage, const void* v_stage, const i
   return launch_status();
 }
 
-extern "C" int yalm_attn_sink_mix(const void* q, void* out, const float* lse, const void* sink_k, const void* sink_v,
+extern "C" int yalm_attn_sink_mix(const void* q, void* out, const float* src_f32, const float* lse, const void* sink_k,
+                                  const void* sink_v,
                                   const int* tok_seq, const int* tok_pos, const int* seq_slot, const float* cos_sin,
                                   int n_positions, int T, int n_slots, int n_heads, int n_kv_heads, int head_dim,
                                   int rotary_dim, int window, int n_sinks, int dtype, hipStream_t stream) {
@@ -113,11 +117,11 @@ extern "C" int yalm_attn_sink_mix(const void* q, void* out, const float* lse, co
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32)
     attn_sink_mix_kernel<float><<<grid, WAVE, 0, stream>>>(
-        (const float*)q, (float*)out, lse, (const float*)sink_k, (const float*)sink_v, tok_seq, tok_pos, seq_slot,
+        (const float*)q, (float*)out, src_f32, lse, (const float*)sink_k, (const float*)sink_v, tok_seq, tok_pos, seq_slot,
         (const float2*)cos_sin, n_positions, n_slots, n_heads, n_kv_heads, head_dim, rotary_dim, window, n_sinks);
   else if (dtype == YALM_BF16)
     attn_sink_mix_kernel<bf16><<<grid, WAVE, 0, stream>>>(
-        (const bf16*)q, (bf16*)out, lse, (const bf16*)sink_k, (const bf16*)sink_v, tok_seq, tok_pos, seq_slot,
+        (const bf16*)q, (bf16*)out, src_f32, lse, (const bf16*)sink_k, (const bf16*)sink_v, tok_seq, tok_pos, seq_slot,
         (const float2*)cos_sin, n_positions, n_slots, n_heads, n_kv_heads, head_dim, rotary_dim, window, n_sinks);
   else
     return YALM_ERR_DTYPE;

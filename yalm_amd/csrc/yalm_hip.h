@@ -155,11 +155,12 @@ long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits);
 
 // The two above, which also leave lse[token, head] (float32; may be null) = the natural logarithm of the
 // sum of exp(score) over the keys the query saw (-FLT_MAX for a padding row), so that further keys can be
-// mixed in afterwards (yalm_attn_sink_mix).  step_max_len (device, one int, may be null): the length of the step's
+// mixed in afterwards (yalm_attn_sink_mix).  out_f32 (prefill only; float32 [T, n_heads, hd], may be null) receives
+// the result before its rounding to `dtype`, for the same purpose.  step_max_len (device, one int, may be null): the length of the step's
 // longest sequence; the matrix-core decode kernel then cuts every sequence into splits of that sequence's split size,
 // so that sequences of unequal lengths give workgroups of equal work (no result depends on it).  seq_order (device,
 // B ints, a permutation of the rows; may be null): the order in which that kernel's workgroups take the rows.
-int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* lse,
+int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* out_f32, float* lse,
                           const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                           const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads, int n_kv_heads,
                           int head_dim, int window, int dtype, int force_simple, hipStream_t stream);
@@ -182,7 +183,9 @@ int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages
 //   yalm_attn_sink_mix adds the sinks that the window no longer covers to a finished attention result:
 //   for token t at position p the sinks j < min(n_sinks, p - window + 1), keys turned by
 //   max(0, p - window - n_sinks + 1) positions with cos_sin (null or rotary_dim 0: not turned);
-//   out[t, h] = (e^lse out + sum_j e^s_j v_j) / (e^lse + sum_j e^s_j), s_j = q . k_j / sqrt(hd).
+//   out[t, h] = (e^lse out + sum_j e^s_j v_j) / (e^lse + sum_j e^s_j), s_j = q . k_j / sqrt(hd); with src_f32 (the
+//   out_f32 of yalm_attn_prefill_lse; may be null) the unrounded result is read from there, so that the mixed row
+//   is rounded once.
 // A decode step: yalm_attn_decode_sinks is yalm_attn_decode whose merge of the splits takes those sinks in
 //   as further splits of one key each (no rounding in between, no launch more; the merge runs with one
 //   split too); with store != 0 a token at a position < n_sinks first stores its own key and value from its
@@ -190,7 +193,8 @@ int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages
 int yalm_sink_store(const void* k_stage, const void* v_stage, const int* seq_tile0, const int* seq_slot,
                     const int* seq_len, void* sink_k, void* sink_v, int B, int n_tiles, int n_slots, int n_kv_heads,
                     int head_dim, int n_sinks, int dtype, hipStream_t stream);
-int yalm_attn_sink_mix(const void* q, void* out, const float* lse, const void* sink_k, const void* sink_v,
+int yalm_attn_sink_mix(const void* q, void* out, const float* src_f32, const float* lse, const void* sink_k,
+                       const void* sink_v,
                        const int* tok_seq, const int* tok_pos, const int* seq_slot, const float* cos_sin,
                        int n_positions, int T, int n_slots, int n_heads, int n_kv_heads, int head_dim, int rotary_dim,
                        int window, int n_sinks, int dtype, hipStream_t stream);

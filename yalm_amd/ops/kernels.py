@@ -555,11 +555,12 @@ def prefill_tile_order(n_tokens):
 
 
 def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
-                 window, tile_order=None, lse=None):
+                 window, tile_order=None, lse=None, out_f32=None):
     """Causal (and windowed) attention of packed sequences that start at position 0, over
     the keys and values that rope_kv_write staged for this step.  tile_order (device int32,
     from prefill_tile_order) only changes the order of the work.  lse (float32 [T, n_heads], optional)
-    receives the logarithm of every query's sum of exp(score), for attn_sink_mix."""
+    receives the logarithm of every query's sum of exp(score), for attn_sink_mix; out_f32 (float32 [T, n_heads *
+    head_dim], optional) the result before it is rounded to out's dtype, for the same."""
     _check_heads(n_heads, n_kv_heads, head_dim)
     T = q.shape[0]
     dt = q.dtype
@@ -578,7 +579,8 @@ def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_p
         n_order = tile_order.shape[0]
         p_or = _need(tile_order, "tile_order", torch.int32, (n_order,))
     p_lse = None if lse is None else _need(lse, "lse", torch.float32, (T, n_heads))
-    library.check(library.lib().yalm_attn_prefill_lse(p_q, p_k, p_v, p_o, p_lse, p_cu, p_t0, p_ts, p_tp, p_or, n_order,
+    p_o32 = _opt(out_f32, "out_f32", torch.float32, (T, n_heads * head_dim))
+    library.check(library.lib().yalm_attn_prefill_lse(p_q, p_k, p_v, p_o, p_o32, p_lse, p_cu, p_t0, p_ts, p_tp, p_or, n_order,
                                                       T, B, n_tiles, n_heads, n_kv_heads, head_dim, int(window),
                                                       dtype_code(dt), 1 if FORCE_SIMPLE else 0, _stream()),
                   "attn_prefill")
@@ -670,11 +672,13 @@ def sink_store(k_stage, v_stage, seq_tile0, seq_slot, seq_len, sink_k, sink_v):
         head_dim, n_sinks, dtype_code(dt), _stream()), "sink_store")
 
 
-def attn_sink_mix(q, out, lse, sink_k, sink_v, tok_seq, tok_pos, seq_slot, cos_sin, n_heads, rotary_dim, window):
+def attn_sink_mix(q, out, lse, sink_k, sink_v, tok_seq, tok_pos, seq_slot, cos_sin, n_heads, rotary_dim, window,
+                  src_f32=None):
     """A step of whole prompts: adds the attention sinks that the window no longer covers to the attention
     result `out` (in place): for the token at position p the sinks j < min(n_sinks, p - window + 1), their
     keys turned by max(0, p - window - n_sinks + 1) positions with the table cos_sin (None: not turned).
-    lse is what attn_prefill left for these queries."""
+    lse is what attn_prefill left for these queries; src_f32 (optional) its out_f32: the unrounded result is then read
+    from there and the mixed row rounded once."""
     n_slots, n_kv_heads, n_sinks, head_dim = sink_k.shape
     _check_heads(n_heads, n_kv_heads, head_dim)
     T = q.shape[0]
@@ -688,6 +692,7 @@ def attn_sink_mix(q, out, lse, sink_k, sink_v, tok_seq, tok_pos, seq_slot, cos_s
         p_cs = _need(cos_sin, "cos_sin", torch.float32, (n_pos, rotary_dim // 2, 2))
     library.check(library.lib().yalm_attn_sink_mix(
         _need(q, "q", dt, (T, n_heads * head_dim)), _need(out, "out", dt, (T, n_heads * head_dim)),
+        _opt(src_f32, "src_f32", torch.float32, (T, n_heads * head_dim)),
         _need(lse, "lse", torch.float32, (T, n_heads)), _need(sink_k, "sink_k", dt),
         _need(sink_v, "sink_v", dt, (n_slots, n_kv_heads, n_sinks, head_dim)),
         _need(tok_seq, "tok_seq", torch.int32, (T,)), _need(tok_pos, "tok_pos", torch.int32, (T,)),

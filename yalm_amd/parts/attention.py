@@ -278,16 +278,18 @@ class GQAttention(Part):
         o = ws.get("attn.o", (T, self.q_dim), act)
         if prefill:
             lse = ws.get("attn.lse", (T, self.n_heads), torch.float32) if self.sinks else None
+            # with sinks the result is kept unrounded too, so that the row with the sinks mixed in is rounded once
+            o32 = ws.get("attn.o32", (T, self.q_dim), torch.float32) if self.sinks and act != torch.float32 else None
             if self.sinks and writes_cache:
                 sink_k, sink_v = group.line_sinks(line)
                 kernels.sink_store(kst, vst, seq_tile0, ctx.seq_slot, ctx.seq_len, sink_k, sink_v)
             kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, seq_tile0, ctx.tok_seq, ctx.tok_pos,
                                  self.n_heads, self.n_kv_heads, self.head_dim, self.window, tiles.get("tile_order"),
-                                 lse=lse)
+                                 lse=lse, out_f32=o32)
             if self.sinks:
                 sink_k, sink_v = group.line_sinks(line)
                 kernels.attn_sink_mix(q, o, lse, sink_k, sink_v, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, pos.table,
-                                      self.n_heads, pos.rotary_dim, self.window)
+                                      self.n_heads, pos.rotary_dim, self.window, src_f32=o32)
         else:
             self._decode_attention(q, o, ctx, group, line, k_pages, v_pages, writes_cache)
         ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.q_dim) if prefill else None
