@@ -14,6 +14,7 @@
 // sums by rsqrt(mean(x^2) + eps) per row.  No norm kernel runs in between, and the sums
 // are added in a fixed order.
 #pragma once
+#include <type_traits>
 #include "common.h"
 
 namespace skinny {
@@ -84,7 +85,13 @@ struct ChainArgs {
 // the global address each lane asks for, so that the fragment reads of 8 rows fall on different
 // banks.  XR (8 or 16) rows of the activations are staged.  No wave waits for another before the
 // partial sums meet.
-template <int MT, int NT, int NWAVES, int EPI, int KS, bool PREFETCH = true, int TW = NT, int DMA_S = 0, int XR = 16>
+//
+// RW < 16 * NT (one tile a wave, DMA path): the workgroup owns RW weight rows, its last tile only the first 8 of its
+// 16 (the waves of that tile ask for one instruction of weights a stage instead of two, and the tile's other columns,
+// which hold whatever was in LDS, are never stored).  6,144 rows are 256 workgroups of 24, one for every compute unit,
+// where 192 of 32 left a quarter of the units idle.
+template <int MT, int NT, int NWAVES, int EPI, int KS, bool PREFETCH = true, int TW = NT, int DMA_S = 0, int XR = 16,
+          int RW = 16 * NT>
 __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* __restrict__ X,
                                                                      const bf16* __restrict__ W,
                                                                      void* __restrict__ Cv, int M, int N, int K,
@@ -93,11 +100,13 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
   constexpr int G = NT / TW;                     // groups of waves, each with TW tiles
   constexpr int KW = NWAVES / G;                 // waves of a group: they split K
   static_assert(NT % TW == 0 && NWAVES % G == 0, "tiles and waves divide evenly");
+  static_assert(RW == 16 * NT || (RW == 16 * NT - 8 && TW == 1 && DMA_S > 0 && EPI != EPI_GATED),
+                "a last tile of 8 rows: one tile a wave, the DMA path, no gated pairs");
   __shared__ f32x4 red[NWAVES][MT * TW][WAVE];
   __shared__ float sm_scale[MT * 16];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const int q = lane / 16, j = lane % 16;
-  const int n0 = blockIdx.x * 16 * NT;
+  const int n0 = blockIdx.x * RW;
 
   const int grp = wave % G, kw = wave / G;
   const bf16* wrow[TW];
@@ -171,14 +180,17 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
     static_assert(MT == 1 && (XR == 8 || XR == 16) && DMA_S >= 2 && DMA_S <= 4, "one batch tile; 8 or 16 staged rows; 2..4 stages");
     constexpr int KD = 64;                         // k a stage: one 128-byte line of every row
     constexpr int XI = XR / 8;                     // DMA instructions a stage: 8 rows each
-    constexpr int L = 2 * TW + XI;
     constexpr int STAGE_B = (16 * TW + XR) * 128;
     extern __shared__ __attribute__((aligned(1024))) unsigned char dma_ring[];   // [NWAVES][DMA_S][STAGE_B]
     unsigned char* ring = dma_ring + (size_t)wave * DMA_S * STAGE_B;
     const int r8 = lane / 8, chunk = (lane % 8) ^ r8;          // this lane's row of an instruction and the chunk it asks for
-    const bf16* gw[2 * TW];
+    // NWI: instructions of weights a stage (8 rows each): 2 * TW, or 1 for the waves of a last tile of 8 rows
+    auto run = [&](auto nwi_tag) {
+    constexpr int NWI = decltype(nwi_tag)::value;
+    constexpr int L = NWI + XI;
+    const bf16* gw[NWI];
 #pragma unroll
-    for (int i = 0; i < 2 * TW; ++i) {
+    for (int i = 0; i < NWI; ++i) {
       const int n = min(n0 + (grp * TW + i / 2) * 16 + (i % 2) * 8 + r8, N - 1);
       gw[i] = W + (size_t)n * K + chunk * 8;
     }
@@ -194,7 +206,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
       unsigned char* dst = ring + buf * STAGE_B;
 #if defined(__HIP_DEVICE_COMPILE__)   // the host pass drops a template that names this builtin, and its launch stub with it
 #pragma unroll
-      for (int u = 0; u < 2 * TW; ++u)
+      for (int u = 0; u < NWI; ++u)
         __builtin_amdgcn_global_load_lds(gw[u] + (size_t)c * KD, dst + u * 1024, 16, 0, YALM_READ_ONCE);
 #pragma unroll
       for (int u = 0; u < XI; ++u)
@@ -236,6 +248,15 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
         }
       }
       if (++buf == DMA_S) buf = 0;
+    }
+    };
+    if constexpr (RW < 16 * NT) {
+      if (grp == G - 1)
+        run(std::integral_constant<int, 1>{});
+      else
+        run(std::integral_constant<int, 2 * TW>{});
+    } else {
+      run(std::integral_constant<int, 2 * TW>{});
     }
   } else {
     bf16x8 wv[TW][KS], xv[MT][KS];
@@ -320,7 +341,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
     f32x4 v = tile_sum(mt, tp);
 #pragma unroll
     for (int r = 0; r < 4; ++r) v[r] *= scale[r];
-    const int n = n0 + tp * 16 + j;
+    const int n = (tp * 16 + j < RW) ? n0 + tp * 16 + j : N;        // a column beyond the workgroup's rows counts as beyond N
     if (EPI == EPI_F32 || EPI == EPI_STORE) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
@@ -412,15 +433,15 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
 // 512-wide chunks; the small projections 16 rows, 8 waves and prefetched 128-wide chunks.  More
 // batch rows (only when the split-K kernel refused the shape) keep 128-wide chunks for the registers.
 // the LDS-DMA variant: its ring of stages is dynamic LDS, which has to be allowed once beyond 64 KB
-template <int NT, int NWAVES, int EPI, int TW, int S, int XR>
+template <int NT, int NWAVES, int EPI, int TW, int S, int XR, int RW = 16 * NT>
 int launch_dma(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, const ChainArgs& ca,
                hipStream_t stream) {
   constexpr size_t lds = (size_t)NWAVES * S * (16 * TW + XR) * 128;
   static_assert(lds + NWAVES * TW * WAVE * 16 + 1024 <= 160 * 1024, "the ring and the partial sums fit the LDS of a CU");
-  auto kernel = &gemm_skinny_kernel<1, NT, NWAVES, EPI, 1, false, TW, S, XR>;
+  auto kernel = &gemm_skinny_kernel<1, NT, NWAVES, EPI, 1, false, TW, S, XR, RW>;
   static LdsAllowance allowed;                     // once a device
   if (int rc = allow_dynamic_lds(allowed, (const void*)kernel, (int)lds); rc != YALM_OK) return rc;
-  kernel<<<ceil_div(N, 16 * NT), NWAVES * WAVE, lds, stream>>>(X, W, C, M, N, K, H, ca);
+  kernel<<<ceil_div(N, RW), NWAVES * WAVE, lds, stream>>>(X, W, C, M, N, K, H, ca);
   return launch_status();
 }
 
@@ -439,6 +460,13 @@ int launch_mt(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H,
         if (N >= 200 * 64)                         // (9..16 rows: a wave with two row tiles stages the activations once
           return few ? launch_dma<4, 16, EPI, 1, 2, 8>(X, W, C, M, N, K, H, ca, stream)   // for both; gate/up at 16
                      : launch_dma<4, 8, EPI, 2, 2, 16>(X, W, C, M, N, K, H, ca, stream);  // rows 41.6 -> 37.8 us)
+        if constexpr (EPI != EPI_GATED) {
+          // workgroups of 24 rows where they are at most one a compute unit (6,144 rows: 256 workgroups instead of
+          // 192 of 32 rows, which leave a quarter of the chip idle)
+          if (ceil_div(N, 24) <= 256)
+            return few ? launch_dma<2, 16, EPI, 1, 2, 8, 24>(X, W, C, M, N, K, H, ca, stream)
+                       : launch_dma<2, 16, EPI, 1, 2, 16, 24>(X, W, C, M, N, K, H, ca, stream);
+        }
         return few ? launch_dma<2, 16, EPI, 1, 2, 8>(X, W, C, M, N, K, H, ca, stream)
                    : launch_dma<2, 16, EPI, 1, 2, 16>(X, W, C, M, N, K, H, ca, stream);
       }
