@@ -521,7 +521,8 @@ def stage(kk, v, lens, n_kv, hd, dtype, poison=True):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens", [
     (4, 2, 16, 0, [5, 17, 1]), (3, 1, 32, 16, [2, 30, 70]), (6, 3, 48, 100, [130, 64]), (8, 2, 128, 0, [200]),
-    (2, 2, 80, 7, [65, 3]), (5, 5, 64, 0, [129]), (4, 1, 64, 70, [300, 64, 1]), (8, 2, 128, 100, [17, 257])])
+    (2, 2, 80, 7, [65, 3]), (5, 5, 64, 0, [129]), (4, 1, 64, 70, [300, 64, 1]), (8, 2, 128, 100, [17, 257]),
+    (6, 2, 96, 50, [150, 64, 333]), (9, 3, 32, 0, [257, 1])])
 def test_attn_prefill(n_heads, n_kv, hd, window, lens, dtype, simple):
     k = K()
     T = sum(lens)
@@ -560,7 +561,8 @@ def masked_attention_float64(q, k, v, n_heads, n_kv, hd, window):
 
 
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens", [(40, 8, 64, 0, [1700]), (40, 8, 128, 300, [1500, 260]),
-                                                         (32, 8, 128, 0, [2048])])
+                                                         (32, 8, 128, 0, [2048]), (40, 8, 96, 0, [1500]),
+                                                         (40, 10, 32, 200, [2200, 70]), (12, 4, 96, 0, [1300])])
 def test_attn_prefill_with_many_and_with_few_workgroups(n_heads, n_kv, hd, window, lens):
     """The matrix-core prefill kernel has two forms: workgroups of eight waves that take a tile's keys in two
     halves (launches of at most two workgroups a compute unit, the third case) and of four waves (more, the
@@ -669,7 +671,8 @@ def one_query_reference(q, keys, vals, window):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens,splits", [
     (4, 2, 16, 0, [5, 64, 65, 1], 1), (3, 1, 32, 16, [2, 30, 200], 2), (6, 3, 48, 100, [130, 640, 99], 3),
-    (8, 2, 128, 0, [1000, 3], 7), (2, 2, 80, 0, [129], 4), (32, 8, 128, 0, [300], 2), (5, 5, 64, 70, [700, 64], 16)])
+    (8, 2, 128, 0, [1000, 3], 7), (2, 2, 80, 0, [129], 4), (32, 8, 128, 0, [300], 2), (5, 5, 64, 70, [700, 64], 16),
+    (6, 2, 96, 0, [900, 65, 2], 5), (12, 3, 96, 130, [400, 129], 2), (16, 1, 32, 0, [2000, 7], 9)])
 def test_attn_decode(n_heads, n_kv, hd, window, lens, splits, dtype, simple):
     _attn_decode_case(n_heads, n_kv, hd, window, lens, splits, dtype, simple, None)
 

@@ -532,8 +532,35 @@ int compute_units() {
   return n;
 }
 
+// head sizes the kernels are built for (any multiple of 32 would do: the products take 32 elements at a time)
 bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
-  return (head_dim == 64 || head_dim == 128) && n_kv_heads > 0 && n_heads % n_kv_heads == 0;
+  return (head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128) && n_kv_heads > 0 &&
+         n_heads % n_kv_heads == 0;
+}
+
+// launches attn_prefill_mfma_kernel<head_dim, NC, KSPL> (more than 64 KB of LDS is asked for once a device)
+template <int HD, int NC, int KSPL>
+int launch_prefill(dim3 grid, int threads, size_t lds, hipStream_t stream, const bf16* qp, const bf16* kp, const bf16* vp,
+                   bf16* out, float* out_f32, float* lse, const int* cu_seqlens, const int* seq_tile0,
+                   const int* tile_order, int fold_at, int B, int n_heads, int n_kv_heads, int window) {
+  auto kernel = &attn_prefill_mfma_kernel<HD, NC, KSPL>;
+  if (lds > 64 * 1024) {
+    static LdsAllowance allowed;
+    if (int rc = allow_dynamic_lds(allowed, (const void*)kernel, 150 * 1024); rc != YALM_OK) return rc;
+  }
+  kernel<<<grid, threads, lds, stream>>>(qp, kp, vp, out, out_f32, lse, cu_seqlens, seq_tile0, tile_order, fold_at, B,
+                                         n_heads, n_kv_heads, window);
+  return launch_status();
+}
+template <int NC, int KSPL, typename... Args>
+int launch_prefill_hd(int head_dim, Args... args) {
+  switch (head_dim) {
+    case 32: return launch_prefill<32, NC, KSPL>(args...);
+    case 64: return launch_prefill<64, NC, KSPL>(args...);
+    case 96: return launch_prefill<96, NC, KSPL>(args...);
+    case 128: return launch_prefill<128, NC, KSPL>(args...);
+  }
+  return YALM_ERR_ARG;
 }
 }  // namespace
 
@@ -558,51 +585,21 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
     // a short step: a workgroup of eight waves for every tile of 64 queries (not 128), so that twice as many
     // compute units work (512 tokens with 32 heads: 19.6 -> 15.9 us a layer); all of them run at once, so their order
     // does not matter
-    const size_t lds = 4 * tile_bytes;
-    auto k128 = &attn_prefill_mfma_kernel<128, 1, 2>;
-    auto k64 = &attn_prefill_mfma_kernel<64, 1, 2>;
-    static LdsAllowance allowed128, allowed64;     // more than 64 KB of LDS has to be asked for once a device
-    int rc_lds = head_dim == 128 ? allow_dynamic_lds(allowed128, (const void*)k128, 150 * 1024)
-                                 : allow_dynamic_lds(allowed64, (const void*)k64, 150 * 1024);
-    if (rc_lds != YALM_OK) return rc_lds;
-    dim3 all(n_heads, n_tiles);
-    if (head_dim == 128)
-      k128<<<all, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, nullptr, 0, B, n_heads,
-                                      n_kv_heads, window);
-    else
-      k64<<<all, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, nullptr, 0, B, n_heads,
-                                     n_kv_heads, window);
-    return launch_status();
+    return launch_prefill_hd<1, 2>(head_dim, dim3(n_heads, n_tiles), 512, 4 * tile_bytes, stream, qp, kp, vp, (bf16*)out,
+                                   out_f32, lse, cu_seqlens, seq_tile0, (const int*)nullptr, 0, B, n_heads, n_kv_heads,
+                                   window);
   }
   if (working <= 2L * compute_units()) {
     // a workgroup of eight waves a compute unit, the workgroups that see the most keys first
-    const size_t lds = 4 * tile_bytes;
-    auto k128 = &attn_prefill_mfma_kernel<128, 2, 2>;
-    auto k64 = &attn_prefill_mfma_kernel<64, 2, 2>;
-    static LdsAllowance allowed128, allowed64;     // more than 64 KB of LDS has to be asked for once a device
-    int rc_lds = head_dim == 128 ? allow_dynamic_lds(allowed128, (const void*)k128, 150 * 1024)
-                                 : allow_dynamic_lds(allowed64, (const void*)k64, 150 * 1024);
-    if (rc_lds != YALM_OK) return rc_lds;
-    if (head_dim == 128)
-      k128<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
-                                       n_kv_heads, window);
-    else
-      k64<<<grid, 512, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads,
-                                      n_kv_heads, window);
-    return launch_status();
+    return launch_prefill_hd<2, 2>(head_dim, grid, 512, 4 * tile_bytes, stream, qp, kp, vp, (bf16*)out, out_f32, lse,
+                                   cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads, n_kv_heads, window);
   }
   // two workgroups fit a compute unit: with more than one and at most two each, the second
   // half of the launch runs from the shortest workgroup up
   const int cus = compute_units();
   const int fold_at = total > cus && total <= 2 * cus ? cus : (int)total;
-  const size_t lds = 2 * tile_bytes;
-  if (head_dim == 128)
-    attn_prefill_mfma_kernel<128, 2, 1><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, tile_order,
-                                                                   fold_at, B, n_heads, n_kv_heads, window);
-  else
-    attn_prefill_mfma_kernel<64, 2, 1><<<grid, 256, lds, stream>>>(qp, kp, vp, (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, tile_order,
-                                                                  fold_at, B, n_heads, n_kv_heads, window);
-  return launch_status();
+  return launch_prefill_hd<2, 1>(head_dim, grid, 256, 2 * tile_bytes, stream, qp, kp, vp, (bf16*)out, out_f32, lse,
+                                 cu_seqlens, seq_tile0, tile_order, fold_at, B, n_heads, n_kv_heads, window);
 }
 
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -622,9 +619,19 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
   // 4 waves a workgroup: 8 measured no faster with one split and slower with more (a CU draws about
   // 33 GB/s whatever its number of waves, so a small batch needs its workgroups spread over all CUs)
   if (page_layout == YALM_PAGE_BLOCKS) {
-    if (head_dim == 128) YALM_DECODE(128, 4, true); else YALM_DECODE(64, 4, true);
+    switch (head_dim) {
+      case 32: YALM_DECODE(32, 4, true); break;
+      case 64: YALM_DECODE(64, 4, true); break;
+      case 96: YALM_DECODE(96, 4, true); break;
+      default: YALM_DECODE(128, 4, true); break;
+    }
   } else {
-    if (head_dim == 128) YALM_DECODE(128, 4, false); else YALM_DECODE(64, 4, false);
+    switch (head_dim) {
+      case 32: YALM_DECODE(32, 4, false); break;
+      case 64: YALM_DECODE(64, 4, false); break;
+      case 96: YALM_DECODE(96, 4, false); break;
+      default: YALM_DECODE(128, 4, false); break;
+    }
   }
 #undef YALM_DECODE
   int rc = launch_status();

@@ -108,14 +108,15 @@ class GQAttention(Part):
         if compute_dtype != torch.bfloat16:
             return what + ": float32-arithmetic kernels", False
         group = self.n_heads // self.n_kv_heads
-        if self.head_dim in (64, 128) and group <= 16:
+        if self.head_dim in kernels.MFMA_HEAD_DIMS and group <= 16:
             return what + ": matrix-core kernels", False
-        why = "head size %d" % self.head_dim if self.head_dim not in (64, 128) else "%d heads a group" % group
+        why = "head size %d" % self.head_dim if self.head_dim not in kernels.MFMA_HEAD_DIMS else "%d heads a group" % group
         return what + ": float32-arithmetic kernels on bfloat16 storage (the matrix-core kernels take head sizes " \
-                      "64 and 128 and up to 16 heads a group, not %s): correct, several times slower" % why, True
+                      "32, 64, 96 and 128 and up to 16 heads a group, not %s): correct, several times slower" % why, True
 
     def decode_splits(self, B, max_pages, ragged=False):
-        mfma = self.head_dim in (64, 128) and self.n_heads // self.n_kv_heads <= 16 and not kernels.FORCE_SIMPLE
+        mfma = self.head_dim in kernels.MFMA_HEAD_DIMS and self.n_heads // self.n_kv_heads <= 16 \
+            and not kernels.FORCE_SIMPLE
         if mfma:         # a workgroup of 4 waves per (split, KV head, sequence), a page per wave at a time
             per = max(1, B * self.n_kv_heads)
             quarters = max(1, min((max_pages + 3) // 4, 4))
