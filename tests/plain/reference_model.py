@@ -207,14 +207,19 @@ def silu(x):
     return x / (1.0 + torch.exp(-x))
 
 
-def swiglu_ffn(x, w_gate, w_down, w_up):
+def gelu(x):
+    """src/infer.cpp:189-191: the tanh form, with the reference's rounded constants."""
+    return 0.5 * x * (1.0 + torch.tanh(0.797885 * (x + 0.044715 * x * x * x)))
+
+
+def swiglu_ffn(x, w_gate, w_down, w_up, act="silu"):
     """src/infer.cpp:356-385 with one expert of weight 1:
-    down( silu(gate x) * (up x) ).  w1 = gate_proj, w3 = up_proj,
+    down( act(gate x) * (up x) ), act silu or gelu (src/infer.cpp:364-372).  w1 = gate_proj, w3 = up_proj,
     w2 = down_proj (convert.py:195-197)."""
     x = x.to(F64)
     g = x @ w_gate.to(F64).T
     u = x @ w_up.to(F64).T
-    return (silu(g) * u) @ w_down.to(F64).T
+    return ({"silu": silu, "gelu": gelu}[act](g) * u) @ w_down.to(F64).T
 
 
 def embedding(table, tokens):
@@ -245,7 +250,8 @@ def read_config(cfg):
     c["sinks"] = cfg.get("attention_sinks") or 0
     c["tied"] = cfg.get("tie_word_embeddings", None) is not False   # convert.py:200-204, 241
     c["rope_scaling"] = cfg.get("rope_scaling")
-    assert cfg.get("hidden_act", "silu") == "silu"
+    c["act"] = cfg.get("hidden_act", "silu")               # convert.py:51-52
+    assert c["act"] in ("gelu", "silu")
     return c
 
 
@@ -297,7 +303,7 @@ def forward(weights, cfg, tokens, window_override=None, position_offset=0, sinks
         x = x + a @ weights[p + "self_attn.o_proj.weight"].to(F64).T
         xb = rmsnorm(x, weights[p + "post_attention_layernorm.weight"], c["norm_eps"])
         x = x + swiglu_ffn(xb, weights[p + "mlp.gate_proj.weight"], weights[p + "mlp.down_proj.weight"],
-                           weights[p + "mlp.up_proj.weight"])
+                           weights[p + "mlp.up_proj.weight"], c["act"])
     x = rmsnorm(x, weights["model.norm.weight"], c["norm_eps"])
     wcls = weights["model.embed_tokens.weight"] if c["tied"] else weights["lm_head.weight"]
     return x @ wcls.to(F64).T

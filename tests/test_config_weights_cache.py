@@ -62,10 +62,18 @@ def test_a_context_is_two_sinks_and_a_window():
     assert (s.sliding_window, s.attention_sinks, s.rotary_dim) == (37, 3, 24)
 
 
+def test_the_activation_comes_from_the_configuration():
+    """hidden_act (silu or gelu, convert.py:51-52) reaches the feed-forward part as a parameter."""
+    for act in ("silu", "gelu"):
+        spec = config_from_dict(dict(tiny_configs.TINY_LLAMA, hidden_act=act)).to_spec()
+        assert all(layer.part("feed_forward").params["activation"] == act for layer in spec.layers)
+    assert config_from_dict(tiny_configs.TINY_WIDE_HEADS).hidden_act == "gelu"
+
+
 @pytest.mark.parametrize("change,text", [
     ({"architectures": ["GPT2LMHeadModel"]}, "not supported"),
     ({"num_key_value_heads": 3}, "multiple"),
-    ({"hidden_act": "gelu"}, "hidden_act"),
+    ({"hidden_act": "relu"}, "hidden_act"),
     ({"attention_bias": True}, "bias"),
     ({"head_dim": 15}, "even"),
     ({"rope_scaling": {"rope_type": "yarn", "factor": 2.0}}, "rope_scaling"),
@@ -103,7 +111,7 @@ def test_spec_is_data_layer_by_layer():
     assert len(spec.layers) == 3 and [e.layer for e in spec.schedule] == [0, 1, 2]
     m = spec.layers[1].mixer
     assert m.kind == "gqa_attention" and m.params["window"] == 16 and m.params["position"].kind == "rope"
-    assert spec.layers[2].feed_forward.params == {"hidden": 256}
+    assert spec.layers[2].feed_forward.params == {"hidden": 256, "activation": "silu"}
     # the order of the layers is data: a layer twice, a layer that reads another's cache
     s2 = ModelSpec(spec.architecture, spec.dim, spec.vocab_size, spec.max_positions, spec.embedding, spec.layers,
                    spec.final_norm, spec.head,

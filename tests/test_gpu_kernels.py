@@ -30,6 +30,15 @@ def tol(dtype):
     return 2e-5 if dtype == torch.float32 else 1.2e-2
 
 
+ACTS = ["silu", "gelu"]
+
+
+def gate(act):
+    """The plain activation and the epilogue code of a gated product."""
+    k = K()
+    return {"silu": (R.silu, k.EPI_GATED), "gelu": (R.gelu, k.EPI_GATED_GELU)}[act]
+
+
 def close(got, want, dtype, what, factor=1.0):
     got = got.detach().to("cpu", torch.float64)
     want = want.to(torch.float64)
@@ -188,7 +197,8 @@ def test_gemm_of_prompt_steps(M, N, Kd, epi, with_workspace):
         w = interleave_gate_up(wg, wu).to(DEV)
         rows = w.shape[0]
         ad = a.double()
-        want = (R.silu(ad @ wg.to(DEV).double().T) * (ad @ wu.to(DEV).double().T)).cpu()
+        act_fn, epi_code = gate("gelu" if M == 384 else "silu")
+        want = (act_fn(ad @ wg.to(DEV).double().T) * (ad @ wu.to(DEV).double().T)).cpu()
     else:
         w = rnd((N, Kd), 92, torch.bfloat16, scale=1 / math.sqrt(Kd)).to(DEV)
         rows = N
@@ -197,7 +207,7 @@ def test_gemm_of_prompt_steps(M, N, Kd, epi, with_workspace):
     ws = torch.full((floats,), float("nan"), device=DEV) if floats else None
     if epi == "gated":
         out = torch.empty((M, N), dtype=torch.bfloat16, device=DEV)
-        k.gemm(a, w, out, k.EPI_GATED, hidden=N, workspace=ws)
+        k.gemm(a, w, out, epi_code, hidden=N, workspace=ws)
         close(out, want, torch.bfloat16, "gated", factor=2.0)
     elif epi == "f32":
         out = torch.full((M, N), float("nan"), device=DEV)
@@ -287,7 +297,8 @@ def test_gemm_random_shapes(with_workspace):
                                    (70, 100, 128), (300, 10300, 64), (260, 1000, 256), (7, 100, 192), (13, 7000, 128),
                                    (16, 13000, 64), (9, 3300, 320), (24, 100, 192), (61, 1000, 128),
                                    (513, 12820, 64), (2048, 14336, 64)])   # whole rounds of 256x256 tiles + a launch of 256x128
-def test_gemm_gated(M, H, D, dtype, simple):
+@pytest.mark.parametrize("act", ACTS)
+def test_gemm_gated(M, H, D, dtype, simple, act):
     from yalm_amd.parts.swiglu import interleave_gate_up
     k = K()
     x = rnd((M, D), 7, dtype)
@@ -295,11 +306,12 @@ def test_gemm_gated(M, H, D, dtype, simple):
     wu = rnd((H, D), 9, dtype, scale=1 / math.sqrt(D))
     g = x.double() @ wg.double().T
     u = x.double() @ wu.double().T
-    want = R.silu(g) * u
+    act_fn, epi_code = gate(act)
+    want = act_fn(g) * u
     k.FORCE_SIMPLE = simple
     try:
         out = torch.empty((M, H), dtype=dtype, device=DEV)
-        k.gemm(x.to(DEV), interleave_gate_up(wg, wu).to(DEV), out, k.EPI_GATED, hidden=H)
+        k.gemm(x.to(DEV), interleave_gate_up(wg, wu).to(DEV), out, epi_code, hidden=H)
         close(out, want, dtype, "gated gemm")
     finally:
         k.FORCE_SIMPLE = False
@@ -1074,8 +1086,9 @@ def test_gemm_norm(M, N, Kd):
     close(out, want, torch.bfloat16, "gemm_norm")          # the activations are rounded to bfloat16 on the way
 
 
+@pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("M,H,D", [(1, 176, 64), (8, 1000, 264), (5, 14336, 128)])
-def test_gemm_norm_gated(M, H, D):
+def test_gemm_norm_gated(M, H, D, act):
     from yalm_amd.parts.swiglu import interleave_gate_up
     k = K()
     x = rnd((M, D), 53, scale=2.0)
@@ -1083,9 +1096,10 @@ def test_gemm_norm_gated(M, H, D):
     wg = rnd((H, D), 55, torch.bfloat16, scale=1 / math.sqrt(D))
     wu = rnd((H, D), 56, torch.bfloat16, scale=1 / math.sqrt(D))
     h = R.rmsnorm(x, nw, 1e-6)
-    want = R.silu(h @ wg.double().T) * (h @ wu.double().T)
+    act_fn, epi_code = gate(act)
+    want = act_fn(h @ wg.double().T) * (h @ wu.double().T)
     out = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
-    k.gemm_norm(x.to(DEV), nw.to(DEV), 1e-6, interleave_gate_up(wg, wu).to(DEV), out, k.EPI_GATED, hidden=H)
+    k.gemm_norm(x.to(DEV), nw.to(DEV), 1e-6, interleave_gate_up(wg, wu).to(DEV), out, epi_code, hidden=H)
     close(out, want, torch.bfloat16, "gemm_norm gated", factor=1.5)
 
 
@@ -1218,9 +1232,11 @@ def test_gemm_chain_producer_and_consumer(M, N, Kd):
     wg = rnd((H, N), 65, torch.bfloat16, scale=1 / math.sqrt(N))
     wu = rnd((H, N), 66, torch.bfloat16, scale=1 / math.sqrt(N))
     outg = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
-    k.gemm_chain(xn, interleave_gate_up(wg, wu).to(DEV), outg, k.EPI_GATED, hidden=H, scale_from=(ss, 1e-5))
     h = R.rmsnorm(x_want, nw, 1e-5)
-    close(outg, R.silu(h @ wg.double().T) * (h @ wu.double().T), torch.bfloat16, "chained gated", factor=2.0)
+    for act in ACTS:
+        act_fn, epi_code = gate(act)
+        k.gemm_chain(xn, interleave_gate_up(wg, wu).to(DEV), outg, epi_code, hidden=H, scale_from=(ss, 1e-5))
+        close(outg, act_fn(h @ wg.double().T) * (h @ wu.double().T), torch.bfloat16, "chained gated " + act, factor=2.0)
 
 
 @pytest.mark.parametrize("with_workspace", [True, False])
@@ -1245,18 +1261,20 @@ def test_gemm_batches_of_17_to_64_rows(M, N, Kd, with_workspace):
 
 
 @pytest.mark.parametrize("with_workspace", [True, False])
+@pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("M,H,D", [(64, 14336, 256), (20, 1000, 264), (40, 176, 4096)])
-def test_gemm_gated_batches_of_17_to_64_rows(M, H, D, with_workspace):
+def test_gemm_gated_batches_of_17_to_64_rows(M, H, D, with_workspace, act):
     from yalm_amd.parts.swiglu import interleave_gate_up
     k = K()
     x = rnd((M, D), 73, torch.bfloat16)
     wg = rnd((H, D), 74, torch.bfloat16, scale=1 / math.sqrt(D))
     wu = rnd((H, D), 75, torch.bfloat16, scale=1 / math.sqrt(D))
-    want = R.silu(x.double() @ wg.double().T) * (x.double() @ wu.double().T)
+    act_fn, epi_code = gate(act)
+    want = act_fn(x.double() @ wg.double().T) * (x.double() @ wu.double().T)
     w = interleave_gate_up(wg, wu).to(DEV)
     ws = torch.empty(k.gemm_workspace_floats(M, w.shape[0], D), device=DEV) if with_workspace else None
     out = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
-    k.gemm(x.to(DEV), w, out, k.EPI_GATED, hidden=H, workspace=ws)
+    k.gemm(x.to(DEV), w, out, epi_code, hidden=H, workspace=ws)
     close(out, want, torch.bfloat16, "gated")
 
 
@@ -1286,19 +1304,21 @@ def test_gemm_of_more_than_64_rows_splits_k(M, N, Kd):
     assert k.gemm_workspace_floats(8192, 4096, 4096) == 0       # enough tiles: no slices
 
 
+@pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("M,H,D", [(100, 1000, 4096), (128, 176, 2048), (65, 3000, 1024)])
-def test_gemm_gated_of_more_than_64_rows_splits_k(M, H, D):
+def test_gemm_gated_of_more_than_64_rows_splits_k(M, H, D, act):
     from yalm_amd.parts.swiglu import interleave_gate_up
     k = K()
     x = rnd((M, D), 79, torch.bfloat16)
     wg = rnd((H, D), 84, torch.bfloat16, scale=1 / math.sqrt(D))
     wu = rnd((H, D), 85, torch.bfloat16, scale=1 / math.sqrt(D))
-    want = R.silu(x.double() @ wg.double().T) * (x.double() @ wu.double().T)
+    act_fn, epi_code = gate(act)
+    want = act_fn(x.double() @ wg.double().T) * (x.double() @ wu.double().T)
     w = interleave_gate_up(wg, wu).to(DEV)
     floats = k.gemm_workspace_floats(M, w.shape[0], D)
     assert floats >= 2 * M * w.shape[0]
     out = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
-    k.gemm(x.to(DEV), w, out, k.EPI_GATED, hidden=H, workspace=torch.full((floats,), float("nan"), device=DEV))
+    k.gemm(x.to(DEV), w, out, epi_code, hidden=H, workspace=torch.full((floats,), float("nan"), device=DEV))
     close(out, want, torch.bfloat16, "gated")
 
 
@@ -1372,7 +1392,9 @@ def test_gemm_add_emit_and_its_consumers(M, N, Kd, N2, small_workspace):
     wgu = interleave_gate_up(wg, wu).to(DEV)
     mid = torch.empty((M, H), dtype=torch.bfloat16, device=DEV)
     ws4 = torch.full((k.gemm_workspace_floats(M, wgu.shape[0], N),), float("nan"), device=DEV)
-    k.gemm(xn, wgu, mid, k.EPI_GATED, hidden=H, workspace=ws4, scale_from=(ss, eps))
-    close(mid, R.silu(h @ wg.double().T) * (h @ wu.double().T), torch.bfloat16, "scaled gated product", factor=2)
+    for act in ACTS:
+        act_fn, epi_code = gate(act)
+        k.gemm(xn, wgu, mid, epi_code, hidden=H, workspace=ws4, scale_from=(ss, eps))
+        close(mid, act_fn(h @ wg.double().T) * (h @ wu.double().T), torch.bfloat16, "scaled gated product " + act, factor=2)
     with pytest.raises(Exception):                        # a row scale is for these batches only
         k.gemm(xn[:8].contiguous(), w2.to(DEV), out[:8].contiguous(), k.EPI_STORE_F32, scale_from=(ss[:8].contiguous(), eps))

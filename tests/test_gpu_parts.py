@@ -145,13 +145,15 @@ def test_attention_part_prefill_then_decode(n_heads, n_kv, hd, window, D, dtype)
         assert (got[i] - want[i][-1]).abs().max() <= lim * max(1, want[i].abs().max()), ("decode", i)
 
 
+@pytest.mark.parametrize("act", ["silu", "gelu", None])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_feed_forward_part(dtype):
+def test_feed_forward_part(dtype, act):
     from yalm_amd.config import PartSpec
     from yalm_amd.engine.context import StepContext, Workspace
     from yalm_amd.parts import build_part
     D, H = 72, 200
-    part = build_part("feed_forward", PartSpec("swiglu", {"hidden": H}, prefix="mlp."), D, "l.")
+    params = {"hidden": H} if act is None else {"hidden": H, "activation": act}      # silu unless said otherwise
+    part = build_part("feed_forward", PartSpec("swiglu", params, prefix="mlp."), D, "l.")
     w = {"l.mlp.gate_proj.weight": rnd((H, D), 1, D ** -0.5), "l.mlp.up_proj.weight": rnd((H, D), 2, D ** -0.5),
          "l.mlp.down_proj.weight": rnd((D, H), 3, H ** -0.5)}
     if dtype == torch.bfloat16:
@@ -163,7 +165,7 @@ def test_feed_forward_part(dtype):
     x = x0.to(DEV).clone()
     part.forward(h.to(DEV), x, StepContext("prefill", None, Workspace(DEV), dtype))
     want = x0.double() + R.swiglu_ffn(h.float(), w["l.mlp.gate_proj.weight"], w["l.mlp.down_proj.weight"],
-                                      w["l.mlp.up_proj.weight"])
+                                      w["l.mlp.up_proj.weight"], act or "silu")
     lim = 2e-5 if dtype == torch.float32 else 2e-2
     assert (x.cpu().double() - want).abs().max() <= lim * want.abs().max()
 

@@ -44,6 +44,7 @@ def random_config(seed):
     rotary = pick([1.0, 1.0, 0.5])
     if rotary != 1.0:
         cfg["partial_rotary_factor"] = rotary
+    cfg["hidden_act"] = pick(["silu", "gelu"])
     return cfg
 
 

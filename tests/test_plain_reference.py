@@ -229,6 +229,27 @@ def test_swiglu():
     assert not torch.allclose(R.swiglu_ffn(x, w3, w2, w1), lib)
 
 
+def test_gelu_gate():
+    """The reference's other activation (src/infer.cpp:189-191): the tanh form with constants rounded to six
+    figures, so the library's tanh form agrees to about 1e-6 and no closer; its ends (0 far left, the identity far
+    right), the place of its minimum, and a gated feed-forward that differs from the silu one."""
+    t = torch.linspace(-6, 6, 241, dtype=F64)
+    lib = torch.nn.functional.gelu(t, approximate="tanh")
+    assert (R.gelu(t) - lib).abs().max() < 3e-6
+    assert (R.gelu(t) - torch.nn.functional.gelu(t)).abs().max() < 1e-3          # and the erf form to three figures
+    ends = R.gelu(torch.tensor([0.0, 30.0, -30.0, 1.0], dtype=F64))
+    assert torch.allclose(ends, torch.tensor([0.0, 30.0, 0.0, 0.841192], dtype=F64), atol=1e-6)
+    assert abs(float(t[R.gelu(t).argmin()]) + 0.75) <= 0.05                       # silu's minimum lies at -1.28
+    g = torch.Generator().manual_seed(8)
+    D, H = 6, 10
+    x = torch.randn(4, D, generator=g, dtype=F64)
+    w1, w3, w2 = (torch.randn(H, D, generator=g, dtype=F64), torch.randn(H, D, generator=g, dtype=F64),
+                  torch.randn(D, H, generator=g, dtype=F64))
+    lib = (torch.nn.functional.gelu(x @ w1.T, approximate="tanh") * (x @ w3.T)) @ w2.T
+    assert torch.allclose(R.swiglu_ffn(x, w1, w2, w3, "gelu"), lib, atol=1e-4)
+    assert not torch.allclose(R.swiglu_ffn(x, w1, w2, w3, "gelu"), R.swiglu_ffn(x, w1, w2, w3), atol=1e-2)
+
+
 # ---------------------------------------------------------------- whole model
 
 @pytest.mark.parametrize("name", ["tiny_llama", "tiny_mistral", "tiny_llama3", "tiny_wide_heads"])

@@ -2,7 +2,8 @@
 
 TINY_LLAMA and TINY_MISTRAL differ in every size and option: head counts and
 groups, head size, width and hidden width that are no powers of two, number of
-layers, vocabulary, eps, theta, window, tied / untied head."""
+layers, vocabulary, eps, theta, window, tied / untied head; TINY_WIDE_HEADS and what is made from it
+have the reference's other activation (gelu)."""
 import copy
 
 TINY_LLAMA = {
@@ -70,6 +71,7 @@ TINY_WIDE_HEADS.update({
     "sliding_window": 100,
     "max_position_embeddings": 512,
     "rms_norm_eps": 3e-6,
+    "hidden_act": "gelu",
 })
 
 # a long context without a window: many pages of the cache, far keys

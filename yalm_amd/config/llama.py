@@ -122,8 +122,8 @@ class LlamaConfig:
         if self.num_attention_heads % self.num_key_value_heads != 0:
             raise ConfigError("num_attention_heads %d is no multiple of num_key_value_heads %d"
                               % (self.num_attention_heads, self.num_key_value_heads))
-        if self.hidden_act != "silu":
-            raise ConfigError("hidden_act %r is not supported (only 'silu')" % (self.hidden_act,))
+        if self.hidden_act not in ("silu", "gelu"):       # the two of the reference (convert.py:51-52)
+            raise ConfigError("hidden_act %r is not supported ('silu' or 'gelu')" % (self.hidden_act,))
         if self.head_dim % 2 != 0:
             raise ConfigError("head_dim %d must be even" % self.head_dim)
         if self.rotary_dim % 2 != 0 or not 0 <= self.rotary_dim <= self.head_dim:
@@ -205,7 +205,8 @@ class LlamaConfig:
                     "head_dim": self.head_dim, "window": self.sliding_window, "sinks": self.attention_sinks,
                     "position": pos,
                 }, prefix="self_attn."),
-                feed_forward=PartSpec("swiglu", {"hidden": self.intermediate_size}, prefix="mlp."),
+                feed_forward=PartSpec("swiglu", {"hidden": self.intermediate_size, "activation": self.hidden_act},
+                                      prefix="mlp."),
                 mixer_norm=PartSpec("rmsnorm", norm, prefix="input_layernorm."),
                 feed_forward_norm=PartSpec("rmsnorm", norm, prefix="post_attention_layernorm."),
                 prefix="model.layers.%d." % i))

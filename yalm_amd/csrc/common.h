@@ -56,6 +56,16 @@ template <typename T> __device__ __forceinline__ T from_f32(float v);
 template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ bf16 from_f32<bf16>(float v) { return static_cast<bf16>(v); }
 
+// Epilogue codes of the GEMMs (yalm_hip.h).  The two gated ones differ in the gate's activation
+// (src/infer.cpp:189-195): silu(z) = z / (1 + exp(-z)); gelu(z) = z/2 (1 + tanh(0.797885 (z + 0.044715 z^3))).
+constexpr int EPI_GATED_SILU = 3, EPI_GATED_GELU = 5;
+constexpr bool gated(int epilogue) { return epilogue == EPI_GATED_SILU || epilogue == EPI_GATED_GELU; }
+template <int EPI>
+__device__ __forceinline__ float gate_act(float z) {
+  if constexpr (EPI == EPI_GATED_GELU) return 0.5f * z * (1.0f + tanhf(0.797885f * (z + 0.044715f * z * z * z)));
+  return z / (1.0f + expf(-z));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);

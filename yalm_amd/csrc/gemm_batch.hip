@@ -68,14 +68,12 @@ constexpr int NWAVES = 8;
 constexpr int KC = 128;                          // k per chunk
 constexpr int XROW = KC + 8;                     // LDS row stride (elements): 16 bytes of padding
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
-
 __device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
   bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
   return ok ? *reinterpret_cast<const bf16x8*>(p) : z;
 }
 
-// epilogue codes as in yalm_gemm: 0 float32 store, 1 bfloat16 store, 2 float32 add, 3 gated
+// epilogue codes as in yalm_gemm: 0 float32 store, 1 bfloat16 store, 2 float32 add, 3 and 5 gated
 template <int EPI>
 __device__ __forceinline__ void store_tile(void* Cv, const f32x4& v, const f32x4& u, int m_base, int n, int hcol,
                                            int M, int N, int H) {
@@ -83,8 +81,8 @@ __device__ __forceinline__ void store_tile(void* Cv, const f32x4& v, const f32x4
   for (int r = 0; r < 4; ++r) {
     int m = m_base + r;
     if (m >= M) continue;
-    if (EPI == 3) {
-      if (hcol < H) ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(v[r]) * u[r]);
+    if (gated(EPI)) {
+      if (hcol < H) ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(gate_act<EPI>(v[r]) * u[r]);
     } else if (n < N) {
       size_t o = (size_t)m * N + n;
       if (EPI == 0) ((float*)Cv)[o] = v[r];
@@ -193,8 +191,8 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_batch_kernel(const bf16* _
   if (gridDim.y == 1 && !always_partial) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      if (EPI == 3) {
-        store_tile<3>(Cv, acc[mt][0], acc[mt][NTW - 1], mt * 16 + 4 * q, 0, n0 / 2 + j, M, N, H);
+      if (gated(EPI)) {
+        store_tile<EPI>(Cv, acc[mt][0], acc[mt][NTW - 1], mt * 16 + 4 * q, 0, n0 / 2 + j, M, N, H);
       } else {
 #pragma unroll
         for (int t = 0; t < NTW; ++t)
@@ -333,8 +331,8 @@ __global__ __launch_bounds__(NW * WAVE) void gemm_batch_dma_kernel(const bf16* _
   if (gridDim.y == 1 && !always_partial) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
-      if (EPI == 3) {
-        store_tile<3>(Cv, acc[mt][0], acc[mt][NTW - 1], mt * 16 + 4 * q, 0, n0 / 2 + j, M, N, H);
+      if (gated(EPI)) {
+        store_tile<EPI>(Cv, acc[mt][0], acc[mt][NTW - 1], mt * 16 + 4 * q, 0, n0 / 2 + j, M, N, H);
       } else {
 #pragma unroll
         for (int t = 0; t < NTW; ++t)
@@ -386,12 +384,12 @@ int launch_kernel(dim3 grid, const bf16* X, const bf16* W, void* C, float* ws, i
 template <int EPI>
 __global__ void splitk_reduce_kernel(const float* __restrict__ partial, void* __restrict__ Cv, int M, int N, int H,
                                      int slices) {
-  const int cols4 = (EPI == 3) ? (N / 2) / 4 : (N + 3) / 4;     // gated: N = 32 * blocks, a thread per 4 hidden columns
+  const int cols4 = (gated(EPI)) ? (N / 2) / 4 : (N + 3) / 4;     // gated: N = 32 * blocks, a thread per 4 hidden columns
   const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (long)M * cols4) return;
   const int m = (int)(idx / cols4), c4 = (int)(idx % cols4) * 4;
   const size_t plane = (size_t)M * N;
-  if (EPI == 3) {
+  if (gated(EPI)) {
     const int blk = c4 / 16, off = c4 % 16;      // hidden column c4 = blk * 16 + off; gate at blk*32+off, up 16 further
     const float* pg = partial + (size_t)m * N + blk * 32 + off;
     float4 g = make_float4(0.f, 0.f, 0.f, 0.f), u = g;
@@ -405,7 +403,7 @@ __global__ void splitk_reduce_kernel(const float* __restrict__ partial, void* __
     const float gv[4] = {g.x, g.y, g.z, g.w}, uv[4] = {u.x, u.y, u.z, u.w};
 #pragma unroll
     for (int e = 0; e < 4; ++e)
-      if (c4 + e < H) C[c4 + e] = static_cast<bf16>(silu_f(gv[e]) * uv[e]);
+      if (c4 + e < H) C[c4 + e] = static_cast<bf16>(gate_act<EPI>(gv[e]) * uv[e]);
   } else {
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     const float* p = partial + (size_t)m * N + c4;
@@ -451,8 +449,8 @@ void slice_k(int K, int wanted, int* k_per_slice, int* slices) {
 template <int MT, int EPI, int NW, int NTW_ = 0>
 int launch_nw(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, int M, int N, int K, int H,
               const RowScale& rs, hipStream_t stream) {
-  constexpr int NTW = NTW_ ? NTW_ : (EPI == 3 ? 2 : 1);
-  if constexpr (NTW_ == 0 && EPI != 3 && MT <= 4 && NW <= 4) {
+  constexpr int NTW = NTW_ ? NTW_ : (gated(EPI) ? 2 : 1);
+  if constexpr (NTW_ == 0 && !gated(EPI) && MT <= 4 && NW <= 4) {
     // a matrix with rows enough (the head): workgroups of 128 rows fill the chip by themselves, K unsplit
     if (K % 64 == 0 && ceil_div(N, NW * 32) >= 200)
       return launch_nw<MT, EPI, NW, 2>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
@@ -465,7 +463,7 @@ int launch_nw(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, 
   dim3 grid(n_blocks, slices);
   int rc = launch_kernel<MT, NTW, EPI, NW>(grid, X, W, C, ws, M, N, K, H, k_per_slice, 0, rs, stream);
   if (rc != YALM_OK || slices == 1) return rc;
-  const long items = (long)M * (EPI == 3 ? (N / 2) / 4 : (N + 3) / 4);
+  const long items = (long)M * (gated(EPI) ? (N / 2) / 4 : (N + 3) / 4);
   splitk_reduce_kernel<EPI><<<ceil_div(items, 256), 256, 0, stream>>>(ws, C, M, N, H, slices);
   return launch_status();
 }
@@ -476,7 +474,7 @@ int launch_mt(const bf16* X, const bf16* W, void* C, float* ws, long ws_floats, 
   // waves a workgroup of the DMA kernel (they share the activations' stage): measured at batch 64
   // 8 waves 8120, 4 waves 8580, 2 waves 8410 tokens a second; at batch 32 5490, 5740 and 5870; with more than 64
   // rows 8 waves where their rings fit (not the gated product's): batch 96 8,950 -> 9,060, batch 128 9,540 -> 9,590
-  constexpr int NW = MT <= 2 ? 2 : (MT > 4 && EPI != 3 ? 8 : 4);
+  constexpr int NW = MT <= 2 ? 2 : (MT > 4 && !gated(EPI) ? 8 : 4);
   if (K % 64 == 0) return launch_nw<MT, EPI, NW>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
   if constexpr (MT > 4) return YALM_ERR_ARG;
   else return launch_nw<MT, EPI, 8>(X, W, C, ws, ws_floats, M, N, K, H, rs, stream);
@@ -780,6 +778,7 @@ static int gemm_batch_scaled(const void* A, const void* W, void* C, float* works
     case 1: return dispatch<1>(a, w, C, workspace, workspace_floats, M, N, K, H, rs, stream);
     case 2: return dispatch<2>(a, w, C, workspace, workspace_floats, M, N, K, H, rs, stream);
     case 3: return dispatch<3>(a, w, C, workspace, workspace_floats, M, N, K, H, rs, stream);
+    case 5: return dispatch<5>(a, w, C, workspace, workspace_floats, M, N, K, H, rs, stream);
   }
   return YALM_ERR_ARG;
 }
@@ -795,7 +794,7 @@ extern "C" int yalm_gemm_scaled(const void* A, const void* W, void* C, float* wo
                                 int N, int K, int epilogue, int H, const float* ss, int n_parts, float eps,
                                 hipStream_t stream) {
   if (ss == nullptr) return YALM_ERR_ARG;
-  if (epilogue == 3 && (H <= 0 || N != 32 * ((H + 15) / 16))) return YALM_ERR_ARG;
+  if (gated(epilogue) && (H <= 0 || N != 32 * ((H + 15) / 16))) return YALM_ERR_ARG;
   return gemm_batch_scaled(A, W, C, workspace, workspace_floats, M, N, K, epilogue, H, ss, n_parts, eps, stream);
 }
 
@@ -883,13 +882,14 @@ extern "C" int yalm_gemm_add_emit_parts(int N) { return emit_parts(N); }
 // kernels that split K: this file's and the tiled one of gemm_dma.hip).
 int yalm_splitk_reduce(const float* partial, void* C, int M, int N, int H, int slices, int epilogue,
                        hipStream_t stream) {
-  const long items = (long)M * (epilogue == 3 ? (N / 2) / 4 : (N + 3) / 4);
+  const long items = (long)M * (gated(epilogue) ? (N / 2) / 4 : (N + 3) / 4);
   const int blocks = ceil_div(items, 256);
   switch (epilogue) {
     case 0: splitk_reduce_kernel<0><<<blocks, 256, 0, stream>>>(partial, C, M, N, H, slices); break;
     case 1: splitk_reduce_kernel<1><<<blocks, 256, 0, stream>>>(partial, C, M, N, H, slices); break;
     case 2: splitk_reduce_kernel<2><<<blocks, 256, 0, stream>>>(partial, C, M, N, H, slices); break;
     case 3: splitk_reduce_kernel<3><<<blocks, 256, 0, stream>>>(partial, C, M, N, H, slices); break;
+    case 5: splitk_reduce_kernel<5><<<blocks, 256, 0, stream>>>(partial, C, M, N, H, slices); break;
     default: return YALM_ERR_ARG;
   }
   return launch_status();

@@ -37,7 +37,6 @@ constexpr int ROWB = TK * 2;                     // bytes a row of a stage
 constexpr int CPR = ROWB / 16;                   // 16-byte chunks a row
 constexpr int RPI = WAVE / CPR;                  // rows one wave instruction brings
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 __device__ __forceinline__ int swizzle_of(int row) { return (row >> 1) & (CPR - 1); }
 
 template <int N_>
@@ -107,7 +106,7 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const 
   }
 #pragma unroll
   for (int b = 0; b < FB; ++b) {
-    const int r = (EPI == 3) ? wn * WN + (b / 2) * 64 + (li / 16) * 32 + (b % 2) * 16 + (li % 16) : wn * WN + b * 32 + li;
+    const int r = (gated(EPI)) ? wn * WN + (b / 2) * 64 + (li / 16) * 32 + (b % 2) * 16 + (li % 16) : wn * WN + b * 32 + li;
     const int row = TM + r;
     w_base[b] = row * ROWB;
     w_swz[b] = swizzle_of(row);
@@ -162,7 +161,7 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const 
         if (m >= M) continue;
 #pragma unroll
         for (int b = 0; b < FB; ++b) {
-          const int wr = (EPI == 3) ? wn * WN + (b / 2) * 64 + (li / 16) * 32 + (b % 2) * 16 + (li % 16) : wn * WN + b * 32 + li;
+          const int wr = (gated(EPI)) ? wn * WN + (b / 2) * 64 + (li / 16) * 32 + (b % 2) * 16 + (li % 16) : wn * WN + b * 32 + li;
           const int n = n0 + wr;
           if (n < N) plane[(size_t)m * N + n] = acc[a][b][r];
         }
@@ -175,12 +174,12 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_dma_kernel(const 
     for (int r = 0; r < 16; ++r) {
       const int m = m0 + wm * WM + a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
       if (m >= M) continue;
-      if (EPI == 3) {
+      if (gated(EPI)) {
 #pragma unroll
         for (int pp = 0; pp < FB / 2; ++pp) {
           const int hcol = (n0 + wn * WN + pp * 64) / 2 + li;
           if (hcol < H)
-            ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
+            ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(gate_act<EPI>(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
         }
       } else {
 #pragma unroll
@@ -253,7 +252,7 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   constexpr int NMF = FA * FB;                              // products a k step
   static_assert(TM % (8 * NW) == 0 && TN % (8 * NW) == 0 && DA % 2 == 0, "the rows of a slot must divide over the waves");
   static_assert(FA + FB <= NMF, "a fragment read follows a product");
-  static_assert(EPI != 3 || FB % 2 == 0, "the gated epilogue pairs column tiles");
+  static_assert(!gated(EPI) || FB % 2 == 0, "the gated epilogue pairs column tiles");
   extern __shared__ __attribute__((aligned(1024))) unsigned char stages[];
   const int tid = threadIdx.x, lane = tid % WAVE;
   const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
@@ -314,7 +313,7 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
   // are the gate rows and odd tiles the up rows of two 16-row blocks.  Address in a slot: row * 128 + ((2 ks + lh)
   // ^ swizzle) * 16; tiles 32 (16, 64) rows apart share the swizzle.
   const int a_row = wm * WM + li;
-  const int w_row = (EPI == 3) ? wn * WN + (li / 16) * 32 + (li % 16) : wn * WN + li;
+  const int w_row = (gated(EPI)) ? wn * WN + (li / 16) * 32 + (li % 16) : wn * WN + li;
   int a_at[KS], w_at[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
@@ -325,7 +324,7 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
     return *reinterpret_cast<const bf16x8*>(stages + slot * RING_SLOT + a_at[ks] + a * 32 * ROWB);
   };
   auto frag_w = [&](int slot, int ks, int b) {
-    const int rows = (EPI == 3) ? (b / 2) * 64 + (b % 2) * 16 : b * 32;
+    const int rows = (gated(EPI)) ? (b / 2) * 64 + (b % 2) * 16 : b * 32;
     return *reinterpret_cast<const bf16x8*>(stages + slot * RING_SLOT + w_at[ks] + rows * ROWB);
   };
 
@@ -422,7 +421,7 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
         if (m >= M) continue;
 #pragma unroll
         for (int b = 0; b < FB; ++b) {
-          const int wr = (EPI == 3) ? wn * WN + (b / 2) * 64 + (li / 16) * 32 + (b % 2) * 16 + (li % 16) : wn * WN + b * 32 + li;
+          const int wr = (gated(EPI)) ? wn * WN + (b / 2) * 64 + (li / 16) * 32 + (b % 2) * 16 + (li % 16) : wn * WN + b * 32 + li;
           if (n0 + wr < N) plane[(size_t)m * N + n0 + wr] = acc[a][b][r];
         }
       }
@@ -434,12 +433,12 @@ __global__ __launch_bounds__(512, 1) void gemm_ring_kernel(const bf16* __restric
     for (int r = 0; r < 16; ++r) {
       const int m = m0 + wm * WM + a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
       if (m >= M) continue;
-      if (EPI == 3) {
+      if (gated(EPI)) {
 #pragma unroll
         for (int pp = 0; pp < FB / 2; ++pp) {
           const int hcol = (n0 + wn * WN + pp * 64) / 2 + li;
           if (hcol < H)
-            ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
+            ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(gate_act<EPI>(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
         }
       } else {
 #pragma unroll
@@ -483,7 +482,7 @@ __global__ __launch_bounds__(512, 1) void gemm_ring16_kernel(const bf16* __restr
   constexpr int G3 = GB > 3 * QG ? GB : 3 * QG;             // the first group of the last quarter behind the barrier
   static_assert(FA == 4 && NG % RB == 0 && NG % 4 == 0, "64 rows a wave; the ring goes round whole times a tile");
   static_assert(2 * QG <= GB && NG - G3 >= 1, "W(kt + 2) is issued in front of the barrier, half of A(kt + 2) behind it");
-  static_assert(EPI != 3 || FB % 2 == 0, "the gated epilogue pairs column tiles");
+  static_assert(!gated(EPI) || FB % 2 == 0, "the gated epilogue pairs column tiles");
   extern __shared__ __attribute__((aligned(1024))) unsigned char stages[];
   const int tid = threadIdx.x, lane = tid % WAVE;
   const int wave = __builtin_amdgcn_readfirstlane(tid / WAVE);
@@ -658,12 +657,12 @@ __global__ __launch_bounds__(512, 1) void gemm_ring16_kernel(const bf16* __restr
     for (int r = 0; r < 4; ++r) {
       const int m = m0 + wm * WM + a * 16 + 4 * lq + r;
       if (m >= M) continue;
-      if (EPI == 3) {                              // weight rows: 16 gate rows, 16 up rows, ...: even tiles gate, odd tiles up
+      if (gated(EPI)) {                              // weight rows: 16 gate rows, 16 up rows, ...: even tiles gate, odd tiles up
 #pragma unroll
         for (int pp = 0; pp < FB / 2; ++pp) {
           const int hcol = (n0 + wn * WN) / 2 + pp * 16 + l16;
           if (hcol < H)
-            ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
+            ((bf16*)Cv)[(size_t)m * H + hcol] = static_cast<bf16>(gate_act<EPI>(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
         }
       } else {
 #pragma unroll
@@ -865,6 +864,7 @@ int yalm_gemm_bf16_dma(const void* A, const void* W, void* C, float* workspace, 
     case 1: return launch<1>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
     case 2: return launch<2>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
     case 3: return launch<3>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
+    case 5: return launch<5>(a, w, C, workspace, workspace_floats, M, N, K, H, stream);
   }
   return YALM_ERR_ARG;
 }

@@ -138,12 +138,12 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_norm_kernel(const float* _
   for (int t = 0; t < NT; ++t) red[wave][t][lane] = acc[t];
   __syncthreads();
 
-  constexpr int NTP = (EPI == EPI_GATED) ? NT / 2 : NT;
+  constexpr int NTP = (gated(EPI)) ? NT / 2 : NT;
   for (int tp = wave; tp < NTP; tp += NWAVES) {
     float scale[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) scale[r] = sm_scale[4 * q + r];
-    if (EPI == EPI_GATED) {
+    if (gated(EPI)) {
       f32x4 g = (f32x4){0.f, 0.f, 0.f, 0.f}, u = g;
 #pragma unroll
       for (int w = 0; w < NWAVES; ++w) {
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_norm_kernel(const float* _
       for (int r = 0; r < 4; ++r) {
         int m = 4 * q + r;
         if (m < M && hcol < H)
-          C[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(g[r] * scale[r]) * (u[r] * scale[r]));
+          C[(size_t)m * H + hcol] = static_cast<bf16>(gate_act<EPI>(g[r] * scale[r]) * (u[r] * scale[r]));
       }
     } else {
       f32x4 v = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -215,12 +215,12 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_norm_kernel(const float* _
 template <int EPI>
 int launch_norm(const float* X, const float* norm_w, float eps, const bf16* W, void* C, int M, int N, int K, int H,
            const RopeArgs& ra, hipStream_t stream) {
-  bool wide = EPI == EPI_GATED || N >= 16384;
+  bool wide = gated(EPI) || N >= 16384;
   size_t lds = (size_t)M * (K + 8) * sizeof(bf16);
   if (wide)
     gemm_norm_kernel<4, 4, EPI><<<ceil_div(N, 64), 4 * WAVE, lds, stream>>>(X, norm_w, eps, W, C, M, N, K, H, ra);
   else
-    gemm_norm_kernel<1, 8, (EPI == EPI_GATED ? EPI_F32 : EPI)><<<ceil_div(N, 16), 8 * WAVE, lds, stream>>>(
+    gemm_norm_kernel<1, 8, (gated(EPI) ? EPI_F32 : EPI)><<<ceil_div(N, 16), 8 * WAVE, lds, stream>>>(
         X, norm_w, eps, W, C, M, N, K, H, ra);
   return launch_status();
 }
@@ -236,8 +236,10 @@ extern "C" int yalm_gemm_norm(const float* x, const float* norm_w, float eps, co
   if (!shape_ok(x, norm_w, W, M, N, K)) return YALM_ERR_ARG;
   RopeArgs ra = {};
   if (epilogue == EPI_F32) return launch_norm<EPI_F32>(x, norm_w, eps, (const bf16*)W, C, M, N, K, H, ra, stream);
-  if (epilogue == EPI_GATED) {
+  if (gated(epilogue)) {
     if (H <= 0 || N != 32 * ((H + 15) / 16)) return YALM_ERR_ARG;
+    if (epilogue == EPI_GATED_GELU)
+      return launch_norm<EPI_GATED_GELU>(x, norm_w, eps, (const bf16*)W, C, M, N, K, H, ra, stream);
     return launch_norm<EPI_GATED>(x, norm_w, eps, (const bf16*)W, C, M, N, K, H, ra, stream);
   }
   return YALM_ERR_ARG;
@@ -300,8 +302,9 @@ extern "C" int yalm_gemm_chain(const void* X, const void* W, void* C, int M, int
   }
   if (emit_nw != nullptr) return YALM_ERR_ARG;
   if (epilogue == EPI_F32) return skinny::launch<EPI_F32>(x, w, C, M, N, K, H, ca, stream);
-  if (epilogue == EPI_GATED) {
+  if (gated(epilogue)) {
     if (H <= 0 || N != 32 * ((H + 15) / 16)) return YALM_ERR_ARG;
+    if (epilogue == EPI_GATED_GELU) return skinny::launch<EPI_GATED_GELU>(x, w, C, M, N, K, H, ca, stream);
     return skinny::launch<EPI_GATED>(x, w, C, M, N, K, H, ca, stream);
   }
   return YALM_ERR_ARG;

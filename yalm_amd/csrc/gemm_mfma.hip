@@ -21,7 +21,6 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
 __device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
   bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -93,7 +92,7 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_tiled_kernel(cons
   int wrow_lds[FB];
 #pragma unroll
   for (int b = 0; b < FB; ++b) {
-    if (EPI == 3)
+    if (gated(EPI))
       wrow_lds[b] = wn * WN + (b / 2) * 64 + (li / 16) * 32 + (b % 2) * 16 + (li % 16);
     else
       wrow_lds[b] = wn * WN + b * 32 + li;
@@ -146,13 +145,13 @@ __global__ __launch_bounds__(NWM * NWN * WAVE, MINW) void gemm_tiled_kernel(cons
     for (int r = 0; r < 16; ++r) {
       int m = m0 + wm * WM + a * 32 + 8 * (r / 4) + 4 * lh + (r % 4);
       if (m >= M) continue;
-      if (EPI == 3) {
+      if (gated(EPI)) {
 #pragma unroll
         for (int pp = 0; pp < FB / 2; ++pp) {
           int hcol = (n0 + wn * WN + pp * 64) / 2 + li;
           if (hcol < H)
             ((bf16*)Cv)[(size_t)m * H + hcol] =
-                static_cast<bf16>(silu_f(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
+                static_cast<bf16>(gate_act<EPI>(acc[a][2 * pp][r]) * acc[a][2 * pp + 1][r]);
         }
       } else {
 #pragma unroll
@@ -208,6 +207,7 @@ int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, float* workspace,
       case 1: return skinny_dispatch<1>(a, w, C, M, N, K, H, stream);
       case 2: return skinny_dispatch<2>(a, w, C, M, N, K, H, stream);
       case 3: return skinny_dispatch<3>(a, w, C, M, N, K, H, stream);
+      case 5: return skinny_dispatch<5>(a, w, C, M, N, K, H, stream);
     }
     return YALM_ERR_ARG;
   }
@@ -220,6 +220,7 @@ int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, float* workspace,
     case 1: return tiled_launch<1>(a, w, C, M, N, K, H, stream);
     case 2: return tiled_launch<2>(a, w, C, M, N, K, H, stream);
     case 3: return tiled_launch<3>(a, w, C, M, N, K, H, stream);
+    case 5: return tiled_launch<5>(a, w, C, M, N, K, H, stream);
   }
   return YALM_ERR_ARG;
 }

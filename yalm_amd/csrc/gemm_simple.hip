@@ -12,7 +12,6 @@ int yalm_gemm_bf16_mfma(const void* A, const void* W, void* C, float* workspace,
 namespace {
 constexpr int BM = 64, BN = 64, BK = 16;
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
 template <typename T, int EPI>
 __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ A, const T* __restrict__ W,
@@ -60,12 +59,12 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
   for (int i = 0; i < 4; ++i) {
     int m = m0 + ty * 4 + i;
     if (m >= M) continue;
-    if (EPI == 3) {
+    if (gated(EPI)) {
       T* C = (T*)Cv;
 #pragma unroll
       for (int jj = 0; jj < 2; ++jj) {
         int hcol = (n0 / 32 + jj) * 16 + tx;
-        if (hcol < H) C[(size_t)m * H + hcol] = from_f32<T>(silu_f(acc[i][2 * jj]) * acc[i][2 * jj + 1]);
+        if (hcol < H) C[(size_t)m * H + hcol] = from_f32<T>(gate_act<EPI>(acc[i][2 * jj]) * acc[i][2 * jj + 1]);
       }
     } else {
 #pragma unroll
@@ -93,11 +92,11 @@ __global__ __launch_bounds__(256) void gemm_simple_kernel(const T* __restrict__ 
 constexpr int RK = 256;                            // k a chunk: 64 lanes x 4
 
 template <int MB, int EPI>
-__global__ __launch_bounds__(EPI == 3 ? 512 : 256) void gemm_rows_f32_kernel(const float* __restrict__ A,
+__global__ __launch_bounds__(gated(EPI) ? 512 : 256) void gemm_rows_f32_kernel(const float* __restrict__ A,
                                                                              const float* __restrict__ W,
                                                                              void* __restrict__ Cv, int M, int N, int K,
                                                                              int H) {
-  constexpr int NWV = EPI == 3 ? 8 : 4;
+  constexpr int NWV = gated(EPI) ? 8 : 4;
   __shared__ __attribute__((aligned(16))) float xs[2][MB][RK];
   __shared__ float sums[NWV * 4][MB];
   const int tid = threadIdx.x, wave = tid / WAVE, lane = tid % WAVE;
@@ -167,12 +166,12 @@ __global__ __launch_bounds__(EPI == 3 ? 512 : 256) void gemm_rows_f32_kernel(con
       if (lane == 0) sums[wave * 4 + r][m] = t;
     }
   __syncthreads();
-  if (EPI == 3) {                                  // rows 0..15 of the workgroup are gate rows, 16..31 their up rows
+  if (gated(EPI)) {                                  // rows 0..15 of the workgroup are gate rows, 16..31 their up rows
     const int base = blockIdx.x * 16;
     for (int e = tid; e < 16 * MB; e += NWV * WAVE) {
       const int j = e % 16, m = e / 16, hcol = base + j;
       if (m < M && hcol < H)
-        ((float*)Cv)[(size_t)m * H + hcol] = silu_f(sums[j][m]) * sums[16 + j][m];
+        ((float*)Cv)[(size_t)m * H + hcol] = gate_act<EPI>(sums[j][m]) * sums[16 + j][m];
     }
   } else {
     const int nb = blockIdx.x * NWV * 4;
@@ -194,6 +193,7 @@ int launch_rows_f32(const float* A, const float* W, void* C, int M, int N, int K
     case 1: gemm_rows_f32_kernel<MB, 1><<<ceil_div(N, 16), 256, 0, stream>>>(A, W, C, M, N, K, H); break;
     case 2: gemm_rows_f32_kernel<MB, 2><<<ceil_div(N, 16), 256, 0, stream>>>(A, W, C, M, N, K, H); break;
     case 3: gemm_rows_f32_kernel<MB, 3><<<ceil_div(N, 32), 512, 0, stream>>>(A, W, C, M, N, K, H); break;
+    case 5: gemm_rows_f32_kernel<MB, 5><<<ceil_div(N, 32), 512, 0, stream>>>(A, W, C, M, N, K, H); break;
     default: return YALM_ERR_ARG;
   }
   return launch_status();
@@ -204,7 +204,7 @@ int launch_rows_f32(const float* A, const float* W, void* C, int M, int N, int K
 int gemm_rows_f32(const void* A, const void* W, void* C, int M, int N, int K, int epilogue, int H, hipStream_t stream) {
   if (M > 64 || K % 4 != 0 || ((uintptr_t)A & 15) || ((uintptr_t)W & 15)) return YALM_ERR_ARG;
   const float* w = (const float*)W;
-  const int out_cols = epilogue == 3 ? H : N;
+  const int out_cols = gated(epilogue) ? H : N;
   for (int m0 = 0; m0 < M; m0 += 16) {
     const float* a = (const float*)A + (size_t)m0 * K;
     float* c = (float*)C + (size_t)m0 * out_cols;
@@ -228,6 +228,7 @@ int gemm_simple(const void* A, const void* W, void* C, int M, int N, int K, int 
     case 1: gemm_simple_kernel<T, 1><<<grid, 256, 0, stream>>>(a, w, C, M, N, K, H); break;
     case 2: gemm_simple_kernel<T, 2><<<grid, 256, 0, stream>>>(a, w, C, M, N, K, H); break;
     case 3: gemm_simple_kernel<T, 3><<<grid, 256, 0, stream>>>(a, w, C, M, N, K, H); break;
+    case 5: gemm_simple_kernel<T, 5><<<grid, 256, 0, stream>>>(a, w, C, M, N, K, H); break;
     default: return YALM_ERR_ARG;
   }
   return launch_status();
@@ -237,8 +238,8 @@ int gemm_simple(const void* A, const void* W, void* C, int M, int N, int K, int 
 extern "C" int yalm_gemm(const void* A, const void* W, void* C, float* workspace, long workspace_floats, int M, int N,
                          int K, int dtype, int epilogue, int H, int force_simple, hipStream_t stream) {
   if (M <= 0) return YALM_OK;
-  if (N <= 0 || K <= 0 || epilogue < 0 || epilogue > 3) return YALM_ERR_ARG;
-  if (epilogue == 3 && (H <= 0 || N != 32 * ((H + 15) / 16))) return YALM_ERR_ARG;
+  if (N <= 0 || K <= 0 || epilogue < 0 || (epilogue > 3 && epilogue != EPI_GATED_GELU)) return YALM_ERR_ARG;
+  if (gated(epilogue) && (H <= 0 || N != 32 * ((H + 15) / 16))) return YALM_ERR_ARG;
   if (dtype == YALM_F32) {
     if (!force_simple) {
       int rc = gemm_rows_f32(A, W, C, M, N, K, epilogue, H, stream);

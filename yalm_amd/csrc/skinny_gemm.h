@@ -22,8 +22,6 @@ namespace skinny {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
-
 __device__ __forceinline__ bf16x8 load8(const bf16* p, bool ok) {
   bf16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
   return ok ? *reinterpret_cast<const bf16x8*>(p) : z;
@@ -42,7 +40,7 @@ __device__ __forceinline__ void skinny_wait_vmcnt() {   // vmcnt only: expcnt an
   __builtin_amdgcn_s_waitcnt((N_ & 0xF) | ((N_ >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
 
-constexpr int EPI_F32 = 0, EPI_STORE = 1, EPI_ADD = 2, EPI_GATED = 3, EPI_ROPE = 4;
+constexpr int EPI_F32 = 0, EPI_STORE = 1, EPI_ADD = 2, EPI_GATED = EPI_GATED_SILU, EPI_ROPE = 4;   // and EPI_GATED_GELU = 5
 
 struct RopeArgs {                                // epilogue of the fused q/k/v projection
   bf16* q_out;
@@ -100,7 +98,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
   constexpr int G = NT / TW;                     // groups of waves, each with TW tiles
   constexpr int KW = NWAVES / G;                 // waves of a group: they split K
   static_assert(NT % TW == 0 && NWAVES % G == 0, "tiles and waves divide evenly");
-  static_assert(RW == 16 * NT || (RW == 16 * NT - 8 && TW == 1 && DMA_S > 0 && EPI != EPI_GATED),
+  static_assert(RW == 16 * NT || (RW == 16 * NT - 8 && TW == 1 && DMA_S > 0 && !gated(EPI)),
                 "a last tile of 8 rows: one tile a wave, the DMA path, no gated pairs");
   __shared__ f32x4 red[NWAVES][MT * TW][WAVE];
   __shared__ float sm_scale[MT * 16];
@@ -320,13 +318,13 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
   };
 
   const bool scaled = ca.ss_in != nullptr;
-  constexpr int NTP = (EPI == EPI_GATED) ? NT / 2 : NT;  // gated: a gate tile and its up tile finish together
+  constexpr int NTP = (gated(EPI)) ? NT / 2 : NT;  // gated: a gate tile and its up tile finish together
   for (int idx = wave; idx < MT * NTP; idx += NWAVES) {
     const int mt = idx / NTP, tp = idx % NTP;
     float scale[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) scale[r] = scaled ? sm_scale[mt * 16 + 4 * q + r] : 1.0f;
-    if (EPI == EPI_GATED) {
+    if (gated(EPI)) {
       const f32x4 g = tile_sum(mt, 2 * tp), u = tile_sum(mt, 2 * tp + 1);
       int hcol = (n0 / 32 + tp) * 16 + j;
       bf16* C = (bf16*)Cv;
@@ -334,7 +332,7 @@ __global__ __launch_bounds__(NWAVES * WAVE) void gemm_skinny_kernel(const bf16* 
       for (int r = 0; r < 4; ++r) {
         int m = mt * 16 + 4 * q + r;
         if (m < M && hcol < H)
-          C[(size_t)m * H + hcol] = static_cast<bf16>(silu_f(g[r] * scale[r]) * (u[r] * scale[r]));
+          C[(size_t)m * H + hcol] = static_cast<bf16>(gate_act<EPI>(g[r] * scale[r]) * (u[r] * scale[r]));
       }
       continue;
     }
@@ -448,19 +446,19 @@ int launch_dma(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H
 template <int MT, int EPI>
 int launch_mt(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H, const ChainArgs& ca,
               hipStream_t stream) {
-  constexpr int E = EPI == EPI_GATED ? EPI_F32 : EPI;   // the gated epilogue needs pairs of tiles
+  constexpr int E = gated(EPI) ? EPI_F32 : EPI;   // the gated epilogue needs pairs of tiles
   const bool emit = ca.emit_nw != nullptr;
   if constexpr (MT == 1) {
     if (K % 64 == 0) {                            // through LDS; measured at 8 rows against the register path:
       const bool few = M <= 8;                     // gate/up 41.9 against 52.6 us, q/k/v 11.0 against 15.3,
-      if (EPI == EPI_GATED || (!emit && N > 4096 && K < 8192)) {   // down 21.3 against 25.2, o 7.0 against 8.3
+      if (gated(EPI) || (!emit && N > 4096 && K < 8192)) {   // down 21.3 against 25.2, o 7.0 against 8.3
         if (N >= 200 * 128)                        // workgroups of 128 weight rows while they still fill the chip
           return few ? launch_dma<8, 8, EPI, 2, 3, 8>(X, W, C, M, N, K, H, ca, stream)
                      : launch_dma<8, 8, EPI, 2, 2, 16>(X, W, C, M, N, K, H, ca, stream);
         if (N >= 200 * 64)                         // (9..16 rows: a wave with two row tiles stages the activations once
           return few ? launch_dma<4, 16, EPI, 1, 2, 8>(X, W, C, M, N, K, H, ca, stream)   // for both; gate/up at 16
                      : launch_dma<4, 8, EPI, 2, 2, 16>(X, W, C, M, N, K, H, ca, stream);  // rows 41.6 -> 37.8 us)
-        if constexpr (EPI != EPI_GATED) {
+        if constexpr (!gated(EPI)) {
           // workgroups of 24 rows where they are at most one a compute unit (6,144 rows: 256 workgroups instead of
           // 192 of 32 rows, which leave a quarter of the chip idle)
           if (ceil_div(N, 24) <= 256)
@@ -473,7 +471,7 @@ int launch_mt(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H,
       return few ? launch_dma<1, 8, E, 1, 3, 8>(X, W, C, M, N, K, H, ca, stream)
                  : launch_dma<1, 8, E, 1, 3, 16>(X, W, C, M, N, K, H, ca, stream);
     }
-    if (EPI == EPI_GATED)
+    if (gated(EPI))
       gemm_skinny_kernel<1, 2, 4, EPI, 8, false><<<ceil_div(N, 32), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
     else if (!emit && N > 4096 && K < 8192)
       gemm_skinny_kernel<1, 2, 16, EPI, 8, false, 1><<<ceil_div(N, 32), 16 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
@@ -482,7 +480,7 @@ int launch_mt(const bf16* X, const bf16* W, void* C, int M, int N, int K, int H,
     else
       gemm_skinny_kernel<1, 1, 8, E, 4><<<ceil_div(N, 16), 8 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
   } else {
-    const bool wide = EPI == EPI_GATED || (N >= 16384 && !emit);
+    const bool wide = gated(EPI) || (N >= 16384 && !emit);
     if (wide && MT <= 2)
       gemm_skinny_kernel<MT, 4, 4, EPI, 4><<<ceil_div(N, 64), 4 * WAVE, 0, stream>>>(X, W, C, M, N, K, H, ca);
     else if (wide)

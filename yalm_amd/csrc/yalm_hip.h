@@ -29,7 +29,9 @@ int yalm_rmsnorm(const float* x, const void* w, int w_dtype, void* out, int out_
 //          2: C float32 [M,N] += acc                      (residual add)
 //          3: gated: W holds gate and up rows interleaved in blocks of 16
 //             (16 gate rows, 16 up rows, ...), N = 32 * ceil(H/16);
-//             C `dtype` [M,H] = silu(gate) * up
+//             C `dtype` [M,H] = silu(gate) * up, silu(z) = z / (1 + exp(-z))
+//          5: as 3 with gelu(z) = z/2 (1 + tanh(0.797885 (z + 0.044715 z^3))) in silu's place
+//             (the reference's two activations, src/infer.cpp:189-195)
 // reference: matmul_wide, fused_matmul_add_residuals, fused_qkv_matmul_clip,
 // fused_ffn_w1_w3_glu_act (src/infer.cu:250-337, 610-634)
 // workspace: float32 scratch (may be null) for kernels that split K across workgroups; they
@@ -42,7 +44,7 @@ int yalm_gemm(const void* A, const void* W, void* C, float* workspace, long work
 long yalm_gemm_bf16_dma_workspace(int M, int N, int K);
 
 // Decode GEMMs from the float32 residual stream, M <= 8 rows (M * (K + 8) * 2 bytes <= 72 KB), bfloat16 weights:
-// C = epilogue(rmsnorm(x, norm_w, eps) * W^T); epilogue 0 (float32 store) or 3 (gated, as yalm_gemm).
+// C = epilogue(rmsnorm(x, norm_w, eps) * W^T); epilogue 0 (float32 store) or 3 or 5 (gated, as yalm_gemm).
 // norm_w is float32 [K].  Refuses (YALM_ERR_ARG) other shapes: use yalm_rmsnorm + yalm_gemm then.
 int yalm_gemm_norm(const float* x, const float* norm_w, float eps, const void* W, void* C, int M, int N, int K,
                    int epilogue, int H, hipStream_t stream);
@@ -85,7 +87,7 @@ int yalm_gemm_partial_scaled(const void* A, const void* W, float* workspace, lon
 // emit_xn[M,N] = bfloat16(C_new * emit_nw[n]) and emit_ss[M, parts] = sums of squares of
 // C_new over the columns of each workgroup (parts = yalm_gemm_chain_parts(N), N < 16384).
 // Consumer: X is such an emit_xn; with ss_in [M, n_parts_in] the float32 sums are scaled by
-// rsqrt(sum(ss_in[m, :]) / K + eps) per row before the epilogue (0: float32 store, 2, 3: gated).
+// rsqrt(sum(ss_in[m, :]) / K + eps) per row before the epilogue (0: float32 store, 2, 3 and 5: gated).
 int yalm_gemm_chain(const void* X, const void* W, void* C, int M, int N, int K, int epilogue, int H,
                     const float* ss_in, int n_parts_in, float eps, const float* emit_nw, void* emit_xn,
                     float* emit_ss, hipStream_t stream);

@@ -102,6 +102,8 @@ def rmsnorm(x, weight, out, eps, row_index=None):
 
 
 EPI_STORE_F32, EPI_STORE, EPI_ADD_F32, EPI_GATED = 0, 1, 2, 3
+EPI_GATED_GELU = 5          # as EPI_GATED with the reference's gelu (tanh form) in silu's place (src/infer.cpp:189-195)
+GATED = (EPI_GATED, EPI_GATED_GELU)
 
 
 GEMM_SPLIT_MAX = 16          # most K slices a GEMM uses, given the workspace
@@ -121,7 +123,7 @@ def gemm(a, w, out, epilogue, hidden=0, workspace=None, scale_from=None):
     """out = a[M,K] @ w[N,K]^T with float32 accumulation and one of four epilogues:
     EPI_STORE_F32 (float32 out), EPI_STORE (out in a's dtype), EPI_ADD_F32
     (float32 out += product), EPI_GATED (w = gate/up rows interleaved in blocks of
-    16; out[M, hidden] = silu(gate) * up in a's dtype).  workspace: float32 scratch of
+    16; out[M, hidden] = silu(gate) * up in a's dtype; EPI_GATED_GELU: gelu(gate) * up).  workspace: float32 scratch of
     gemm_workspace_floats(M, N, K) elements, with which small batches split K.
     scale_from = (ss float32 [M, parts], eps), 17..128 bfloat16 rows only (can_add_emit): a was emitted by
     gemm_add_emit, and the sums are scaled by rsqrt(sum(ss[m]) / K + eps) per row before the epilogue."""
@@ -130,7 +132,7 @@ def gemm(a, w, out, epilogue, hidden=0, workspace=None, scale_from=None):
     dt = a.dtype
     p_a = _need(a, "a", dt, (M, K))
     p_w = _need(w, "w", dt, (N, K))
-    if epilogue == EPI_GATED:
+    if epilogue in GATED:
         if hidden <= 0 or N != 32 * ((hidden + 15) // 16):
             raise ValueError("gated gemm: weight rows %d do not match hidden %d" % (N, hidden))
         p_o = _need(out, "out", dt, (M, hidden))
@@ -167,14 +169,14 @@ def can_fuse_norm(M, K, dtype):
 
 def gemm_norm(x, norm_w, eps, w, out, epilogue, hidden=0):
     """out = epilogue(rmsnorm(x, norm_w, eps) @ w^T) for at most 16 rows of the float32
-    residual stream x; w bfloat16 [N, K], norm_w float32 [K]; EPI_STORE_F32 or EPI_GATED.
+    residual stream x; w bfloat16 [N, K], norm_w float32 [K]; EPI_STORE_F32, EPI_GATED or EPI_GATED_GELU.
     (Shapes: see can_fuse_norm.)"""
     M, K = x.shape
     N = w.shape[0]
     p_x = _need(x, "x", torch.float32, (M, K))
     p_n = _need(norm_w, "norm_w", torch.float32, (K,))
     p_w = _need(w, "w", torch.bfloat16, (N, K))
-    if epilogue == EPI_GATED:
+    if epilogue in GATED:
         if hidden <= 0 or N != 32 * ((hidden + 15) // 16):
             raise ValueError("gated gemm: weight rows %d do not match hidden %d" % (N, hidden))
         p_o = _need(out, "out", torch.bfloat16, (M, hidden))
@@ -357,7 +359,7 @@ def gemm_chain(x, w, out, epilogue, hidden=0, scale_from=None, emit=None):
     N = w.shape[0]
     p_x = _need(x, "x", torch.bfloat16, (M, K))
     p_w = _need(w, "w", torch.bfloat16, (N, K))
-    if epilogue == EPI_GATED:
+    if epilogue in GATED:
         if hidden <= 0 or N != 32 * ((hidden + 15) // 16):
             raise ValueError("gated gemm: weight rows %d do not match hidden %d" % (N, hidden))
         p_o = _need(out, "out", torch.bfloat16, (M, hidden))

@@ -1,5 +1,7 @@
-"""SwiGLU feed-forward, dense: x += down( silu(gate h) * (up h) )
-(src/infer.cpp:356-385 with one expert of weight 1; silu(z) = z / (1 + exp(-z))).
+"""Gated feed-forward, dense: x += down( act(gate h) * (up h) )
+(src/infer.cpp:356-385 with one expert of weight 1).  act is silu(z) = z / (1 + exp(-z)) (SwiGLU) or, with the
+parameter `activation` = "gelu", gelu(z) = z/2 (1 + tanh(0.797885 (z + 0.044715 z^3))): the two the reference
+knows (src/infer.cpp:189-195, convert.py:51-52).
 Gate and up rows are interleaved in blocks of 16 at load so that one GEMM
 produces both and its epilogue multiplies them (the reference fuses the two
 products by pointer, src/infer.cu:610-634)."""
@@ -10,6 +12,7 @@ from ..weights.loader import ParamSpec, place
 from .base import Part, part
 
 GATE_BLOCK = 16
+ACTIVATIONS = {"silu": kernels.EPI_GATED, "gelu": kernels.EPI_GATED_GELU}
 
 
 def interleave_gate_up(gate, up):
@@ -32,6 +35,10 @@ class SwiGLU(Part):
     def __init__(self, spec, dim, prefix):
         super().__init__(spec, dim, prefix)
         self.hidden = int(spec.params["hidden"])
+        self.activation = str(spec.params.get("activation", "silu"))
+        if self.activation not in ACTIVATIONS:
+            raise ValueError("feed-forward activation %r is not offered (%s)" % (self.activation, ", ".join(ACTIVATIONS)))
+        self.gated = ACTIVATIONS[self.activation]          # the GEMM epilogue that applies it
         self.w_gate_up = None
         self.w_down = None
 
@@ -66,19 +73,19 @@ class SwiGLU(Part):
         src = ctx.normed.pop(id(norm), None)
         if src is not None and src[1] is not None and kernels.can_chain(T, self.dim, self.w_down.dtype):
             xn, ss, eps = src
-            kernels.gemm_chain(xn, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden, scale_from=(ss, eps))
+            kernels.gemm_chain(xn, self.w_gate_up, mid, self.gated, hidden=self.hidden, scale_from=(ss, eps))
         elif src is not None and src[1] is not None:          # 17..128 rows: prepared by the kernel that added the K slices
             xn, ss, eps = src
-            self._gemm(ctx, xn, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden, scale_from=(ss, eps))
+            self._gemm(ctx, xn, self.w_gate_up, mid, self.gated, hidden=self.hidden, scale_from=(ss, eps))
         elif src is not None:                     # the norm's output is ready
-            self._gemm(ctx, src[0], self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
+            self._gemm(ctx, src[0], self.w_gate_up, mid, self.gated, hidden=self.hidden)
         elif kernels.can_fuse_norm(T, self.dim, self.w_down.dtype):
             nw, eps = norm.fused()
-            kernels.gemm_norm(x, nw, eps, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
+            kernels.gemm_norm(x, nw, eps, self.w_gate_up, mid, self.gated, hidden=self.hidden)
         else:
             h = ctx.ws.get("block.h", (T, self.dim), ctx.act_dtype)
             norm.forward(x, h, ctx)
-            self._gemm(ctx, h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
+            self._gemm(ctx, h, self.w_gate_up, mid, self.gated, hidden=self.hidden)
         emit = self._emit_args(emit_for, ctx, T, self.dim)
         prepared = self._add_emit_args(emit_for, ctx, T, self.dim, self.hidden) if emit is None else None
         ready = self._add_norm_args(emit_for, ctx, T, self.dim, self.hidden) if emit is None and prepared is None else None
@@ -100,5 +107,5 @@ class SwiGLU(Part):
     def forward(self, h, x, ctx):
         T = h.shape[0]
         mid = ctx.ws.get("ffn.hidden", (T, self.hidden), h.dtype)
-        self._gemm(ctx, h, self.w_gate_up, mid, kernels.EPI_GATED, hidden=self.hidden)
+        self._gemm(ctx, h, self.w_gate_up, mid, self.gated, hidden=self.hidden)
         self._gemm(ctx, mid, self.w_down, x, kernels.EPI_ADD_F32)
