@@ -555,8 +555,9 @@ def test_attn_prefill(n_heads, n_kv, hd, window, lens, dtype, simple):
     close(out, packed_attention_reference(q, kk, v, lens, n_heads, n_kv, hd, window), dtype, "prefill attention")
 
 
-def masked_attention_float64(q, k, v, n_heads, n_kv, hd, window):
-    """softmax(q k^T / sqrt(hd) + mask) v for one sequence, all positions at once (float64)."""
+def masked_attention_float64(q, k, v, n_heads, n_kv, hd, window, bias=None):
+    """softmax(q k^T / sqrt(hd) + mask) v for one sequence, all positions at once (float64).  bias ([n_heads,
+    distances], optional): bias[h, min(i - j, distances - 1)] is added to the score of query i and key j."""
     n = q.shape[0]
     qh = q.double().reshape(n, n_heads, hd).transpose(0, 1)
     kh = k.double().reshape(n, n_kv, hd).transpose(0, 1).repeat_interleave(n_heads // n_kv, dim=0)
@@ -567,6 +568,8 @@ def masked_attention_float64(q, k, v, n_heads, n_kv, hd, window):
     out = torch.empty((n_heads, n, hd), dtype=torch.float64)
     for h in range(n_heads):                          # a head at a time: [n, n] scores
         s = (qh[h] @ kh[h].T) / math.sqrt(hd)
+        if bias is not None:
+            s = s + bias[h].double()[(i - j).clamp(0, bias.shape[1] - 1)]
         s = s.masked_fill(~visible, float("-inf"))
         out[h] = torch.softmax(s, dim=-1) @ vh[h]
     return out.transpose(0, 1).reshape(n, n_heads * hd)
@@ -720,6 +723,59 @@ def _attn_decode_case(n_heads, n_kv, hd, window, lens, splits, dtype, simple, st
         want = one_query_reference(q[b].double().reshape(n_heads, hd), keys[b], vals[b], window).reshape(-1)
         close(out[b], want, dtype, "decode attention row %d" % b)
     assert (out[B] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_heads,n_kv,hd,window,lens,n_bias", [
+    (4, 2, 16, 0, [5, 130, 64], 200), (6, 3, 64, 70, [300, 1], 40), (8, 2, 128, 0, [257], 300), (3, 1, 48, 20, [90, 65], 7)])
+def test_attn_with_a_score_bias(n_heads, n_kv, hd, window, lens, n_bias, dtype):
+    """A term added to every score by the distance of query and key (a table a head, the last entry for every
+    distance beyond it): prompt and decode kernels against a float64 softmax with the same term.  The table is steep
+    (a slope a head plus noise), so that dropping it, taking another head's row or counting the distance from the
+    wrong end changes the result by far more than rounding; the matrix-core kernels would ignore it, so the
+    float32-arithmetic ones run."""
+    k = K()
+    slopes = 2.0 ** -(torch.arange(n_heads, dtype=torch.float64) * 3.0 / n_heads)
+    bias = (-slopes[:, None] * torch.arange(n_bias, dtype=torch.float64)[None, :] + rnd((n_heads, n_bias), 77).double()).float()
+    T = sum(lens)
+    q = rnd((T, n_heads * hd), 13, dtype)
+    kk = rnd((T, n_kv * hd), 14, dtype)
+    v = rnd((T, n_kv * hd), 15, dtype)
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    seq = np.repeat(np.arange(len(lens)), lens)
+    pos = np.concatenate([np.arange(n) for n in lens])
+    ks, vs, tile0 = stage(kk, v, lens, n_kv, hd, dtype)
+    out = torch.empty((T, n_heads * hd), dtype=dtype, device=DEV)
+    k.attn_prefill(q.to(DEV), ks.to(DEV), vs.to(DEV), out, i32(cu), i32(tile0), i32(seq), i32(pos), n_heads, n_kv, hd,
+                   window, score_bias=bias.to(DEV))
+    want, plain, o = [], [], 0
+    for n in lens:
+        want.append(masked_attention_float64(q[o:o + n], kk[o:o + n], v[o:o + n], n_heads, n_kv, hd, window, bias))
+        plain.append(masked_attention_float64(q[o:o + n], kk[o:o + n], v[o:o + n], n_heads, n_kv, hd, window))
+        o += n
+    want, plain = torch.cat(want), torch.cat(plain)
+    assert (want - plain).abs().max() > 0.1                     # the bias matters here
+    close(out, want, dtype, "prefill attention with a score bias")
+    # decode: the last query of every sequence over the cache pages
+    B = len(lens)
+    kp, vp, bt, slots, ring, keys, vals = paged_case(lens, n_kv, hd, window, dtype, 20)
+    qd = rnd((B, n_heads * hd), 16, dtype)
+    outd = torch.empty((B, n_heads * hd), dtype=dtype, device=DEV)
+    partial = torch.empty(k.attn_decode_workspace_floats(B, n_heads, hd, 3), device=DEV)
+    k.attn_decode(qd.to(DEV), kp.to(DEV), vp.to(DEV), bt.to(DEV), ring, i32(slots), i32(lens), outd, partial,
+                  n_heads, n_kv, hd, window, 3, score_bias=bias.to(DEV))
+    for b, n in enumerate(lens):
+        lo = max(0, n - window) if window else 0
+        got_want = torch.zeros((n_heads, hd), dtype=torch.float64)
+        for h in range(n_heads):
+            g = h // (n_heads // n_kv)
+            sc = keys[b][lo:n, g].double() @ qd[b].double().reshape(n_heads, hd)[h] / math.sqrt(hd)
+            sc = sc + bias[h].double()[(n - 1 - torch.arange(lo, n)).clamp(0, n_bias - 1)]
+            got_want[h] = torch.softmax(sc, dim=0) @ vals[b][lo:n, g].double()
+        close(outd[b], got_want.reshape(-1), dtype, "decode attention with a score bias, row %d" % b)
+    with pytest.raises(Exception):                              # a table for another number of heads
+        k.attn_decode(qd.to(DEV), kp.to(DEV), vp.to(DEV), bt.to(DEV), ring, i32(slots), i32(lens), outd, partial,
+                      n_heads, n_kv, hd, window, 3, score_bias=bias[:-1].contiguous().to(DEV))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -547,6 +547,131 @@ def test_toy_routed_feed_forward_and_position_encoding_from_outside(tmp_path):
 
 
 # ---------------------------------------------------------------------------
+# a toy position encoding that is no rotation: a term added to the scores by the distance of query and key
+# ---------------------------------------------------------------------------
+
+def define_distance_slopes():
+    from yalm_amd.parts import Part, register_part
+
+    class DistanceSlopes(Part):
+        """No rotation.  Head h's score of a key `d` positions behind the query gets -slope * 2^(-h) * min(d, far)
+        added: the framework's attention asks its position part for `score_bias` and hands it to the kernels."""
+        rotary_dim = 0
+        table = None
+        n_positions = 0
+
+        def __init__(self, spec, dim, prefix):
+            super().__init__(spec, dim, prefix)
+            self.n_heads, self.far, self.slope = int(spec.params["n_heads"]), int(spec.params["far"]), float(spec.params["slope"])
+            self.score_bias = None
+
+        def prepare(self, n_positions, device):
+            if self.score_bias is None:                          # made once: captured graphs keep its address
+                self.score_bias = distance_slopes_table(self.n_heads, self.far, self.slope).float().to(device)
+
+        def arrange_projection_rows(self, w, n_heads):
+            return w
+
+    register_part("position", "toy_distance_slopes", DistanceSlopes, replace=True)
+
+
+def distance_slopes_table(n_heads, far, slope):
+    return -slope * (2.0 ** -torch.arange(n_heads, dtype=torch.float64))[:, None] * torch.arange(far + 1, dtype=torch.float64)[None, :]
+
+
+class SlopesToyConfig:
+    """Two layers of the framework's attention with the toy position part, the second with a window."""
+
+    def __init__(self, d):
+        self.d = d
+
+    @classmethod
+    def from_dict(cls, d):
+        return cls(d)
+
+    def to_dict(self):
+        return dict(self.d)
+
+    def to_spec(self):
+        from yalm_amd.config import LayerSpec, ModelSpec, PartSpec
+        d = self.d
+        norm = {"eps": d["eps"]}
+        pos = PartSpec("toy_distance_slopes", {"n_heads": d["heads"], "far": d["far"], "slope": d["slope"]})
+
+        def attn(window):
+            return PartSpec("gqa_attention", {"n_heads": d["heads"], "n_kv_heads": d["groups"], "head_dim": d["head"],
+                                              "window": window, "position": pos}, prefix="attn.")
+        layers = [LayerSpec("prenorm_residual", prefix="toy.%d." % i, mixer=attn(w),
+                            feed_forward=PartSpec("swiglu", {"hidden": d["hidden"], "activation": "gelu"}, prefix="ff."),
+                            mixer_norm=PartSpec("rmsnorm", norm, prefix="n1."),
+                            feed_forward_norm=PartSpec("rmsnorm", norm, prefix="n2."))
+                  for i, w in enumerate((0, d["window"]))]
+        return ModelSpec("SlopesToyForCausalLM", d["width"], d["vocab"], d["positions"],
+                         PartSpec("token_embedding", {"vocab_size": d["vocab"]}, prefix="toy.emb."), layers,
+                         PartSpec("rmsnorm", norm, prefix="toy.norm."),
+                         PartSpec("lm_head", {"vocab_size": d["vocab"], "tied": True}, prefix="toy.emb."))
+
+
+def slopes_toy_plain_forward(w, d, tokens):
+    T, H, G, hd = len(tokens), d["heads"], d["groups"], d["head"]
+    x = R.embedding(w["toy.emb.weight"], torch.tensor(tokens))
+    bias = distance_slopes_table(H, d["far"], d["slope"])
+    i, j = torch.arange(T)[:, None], torch.arange(T)[None, :]
+    for l, window in enumerate((0, d["window"])):
+        p = "toy.%d." % l
+        h = R.rmsnorm(x, w[p + "n1.weight"], d["eps"])
+        q = (h @ w[p + "attn.q_proj.weight"].double().T).reshape(T, H, hd)
+        k = (h @ w[p + "attn.k_proj.weight"].double().T).reshape(T, G, hd)
+        v = (h @ w[p + "attn.v_proj.weight"].double().T).reshape(T, G, hd)
+        visible = (j <= i) & ((i - j < window) if window else torch.ones((T, T), dtype=torch.bool))
+        a = torch.empty((T, H, hd), dtype=torch.float64)
+        for hh in range(H):
+            sc = q[:, hh] @ k[:, hh // (H // G)].T / hd ** 0.5 + bias[hh][(i - j).clamp(0, d["far"])]
+            a[:, hh] = torch.softmax(sc.masked_fill(~visible, float("-inf")), dim=-1) @ v[:, hh // (H // G)]
+        x = x + a.reshape(T, H * hd) @ w[p + "attn.o_proj.weight"].double().T
+        h = R.rmsnorm(x, w[p + "n2.weight"], d["eps"])
+        x = x + R.swiglu_ffn(h, w[p + "ff.gate_proj.weight"], w[p + "ff.down_proj.weight"], w[p + "ff.up_proj.weight"], "gelu")
+    return R.rmsnorm(x, w["toy.norm.weight"], d["eps"]) @ w["toy.emb.weight"].double().T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_position_encoding_that_is_no_rotation_from_outside(tmp_path, dtype):
+    """A position part without any rotation, which instead has a term for every score by the distance of query and
+    key, takes its place by configuration alone; prompts, single tokens and batches agree with the toy written out in
+    float64 (and differ from the same model without the term, so the term is not lost on the way)."""
+    from yalm_amd import Engine, Model, register_architecture, write_random_model
+    from yalm_amd.config import unregister_architecture
+    from yalm_amd.parts import unregister_part
+    define_distance_slopes()
+    register_architecture("SlopesToyForCausalLM", SlopesToyConfig, replace=True)
+    try:
+        d = {"architectures": ["SlopesToyForCausalLM"], "width": 72, "hidden": 104, "vocab": 91, "positions": 256,
+             "eps": 1e-5, "heads": 6, "groups": 2, "head": 64, "window": 40, "far": 50, "slope": 0.8}
+        folder = write_random_model(str(tmp_path / "slopes_toy"), d, seed=6)
+        model = Model.from_folder(folder, dtype=helpers.torch_dtype(dtype), device=DEV)
+        engine = Engine(model, max_tokens=2048)
+        assert bool(model.describe()[1]) == (dtype == "bfloat16")      # bfloat16: the slower kernels, and it says so
+        cfg, w = R.read_folder(folder)
+        if dtype == "bfloat16":
+            w = {n: (t.bfloat16().float() if t.dim() > 1 else t) for n, t in w.items()}
+        rng = np.random.default_rng(5)
+        requests = {rid: [int(t) for t in rng.integers(0, d["vocab"], size=n)]
+                    for rid, n in (("a", 30), ("b", 3), ("c", 150), ("d", 70))}
+        want = {rid: slopes_toy_plain_forward(w, d, toks).float().numpy() for rid, toks in requests.items()}
+        flat = slopes_toy_plain_forward(w, dict(d, slope=0.0), requests["c"]).float().numpy()
+        assert np.abs(flat - want["c"]).max() > 0.05 * np.abs(want["c"]).max()
+        for steps in (schedules.whole(requests), schedules.tail_one_by_one(requests, 32),
+                      schedules.batches(requests, [["a", "b"], ["c", "d"]], {"a": 11, "b": 1, "c": 64, "d": 2})):
+            out = schedules.replay_in_process(engine, steps)
+            got = schedules.per_request(steps, out, requests)
+            for rid in requests:
+                helpers.check_logits(got[rid], want[rid], dtype, "slopes toy %s" % rid)
+    finally:
+        unregister_architecture("SlopesToyForCausalLM")
+        unregister_part("position", "toy_distance_slopes")
+
+
+# ---------------------------------------------------------------------------
 # toy arrangements of a layer with other members than the reference's block has
 # ---------------------------------------------------------------------------
 

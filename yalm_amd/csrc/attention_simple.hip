@@ -20,6 +20,16 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
                                const int* step_max_len, const int* seq_order, hipStream_t stream);
 
 namespace {
+// A term added to every score by the distance between query and key: table[head][min(distance, n - 1)] (float32), or
+// nothing.  What a position encoding that is no rotation needs (a slope per head times the distance, a learned table).
+struct ScoreBias {
+  const float* table;
+  int n;
+  __device__ __forceinline__ float at(int head, int distance) const {
+    return table != nullptr ? table[(size_t)head * n + min(max(distance, 0), n - 1)] : 0.f;
+  }
+};
+
 constexpr int MAX_HD = 256;              // head sizes up to 256 (4 output elements per lane)
 constexpr int ACC = MAX_HD / WAVE;
 constexpr int COMBINE_THREADS = 256;
@@ -31,7 +41,8 @@ template <typename T>
 __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
     const T* __restrict__ q, const T* __restrict__ k_stage, const T* __restrict__ v_stage, T* __restrict__ out,
     float* __restrict__ out_f32, float* __restrict__ lse, const int* __restrict__ seq_tile0,
-    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_heads, int n_kv_heads, int hd, int window) {
+    const int* __restrict__ tok_seq, const int* __restrict__ tok_pos, int n_heads, int n_kv_heads, int hd, int window,
+    ScoreBias sb) {
   __shared__ float qs[MAX_HD];
   __shared__ float ps[WAVE];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -59,7 +70,7 @@ __global__ __launch_bounds__(WAVE) void attn_prefill_simple_kernel(
       const T* kr = kp + (size_t)lane * hd;
       float d = 0.f;
       for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kr[i]), d);
-      s = d / inv;
+      s = d / inv + sb.at(h, pos - j);
     }
     float m_new = fmaxf(m, wave_max(s));
     float p = valid ? expf(s - m_new) : 0.f;
@@ -104,7 +115,7 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
     const T* __restrict__ q, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_len, float* __restrict__ partial, int n_heads, int n_kv_heads, int hd, int window,
-    int n_splits, int n_pages, int page_layout) {
+    int n_splits, int n_pages, int page_layout, ScoreBias sb) {
   __shared__ float qs[MAX_HD];
   __shared__ float ps[WAVE];
   const int b = blockIdx.x, h = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
@@ -138,7 +149,7 @@ __global__ __launch_bounds__(WAVE) void attn_decode_simple_kernel(
       if (valid) {
         float d = 0.f;
         for (int i = 0; i < hd; ++i) d = fmaf(qs[i], to_f32(kp[page_k_offset(page_layout, lane, i, hd)]), d);
-        s = d / inv;
+        s = d / inv + sb.at(h, L - 1 - pos);
       }
       float m_new = fmaxf(m, wave_max(s));
       float p = valid ? expf(s - m_new) : 0.f;
@@ -300,15 +311,18 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
                                      const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                                  const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads,
                                  int n_kv_heads, int head_dim, int window, int dtype, int force_simple,
-                                 hipStream_t stream) {
+                                 const float* score_bias, int n_bias, hipStream_t stream) {
   if (T <= 0) return YALM_OK;
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_tiles <= 0) return YALM_ERR_ARG;
+  if (score_bias != nullptr && n_bias <= 0) return YALM_ERR_ARG;
+  const ScoreBias sb = {score_bias, n_bias};
+  if (score_bias != nullptr) force_simple = 1;     // the matrix-core kernels take no bias
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32) {
     attn_prefill_simple_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)q, (const float*)k_stage,
                                                                  (const float*)v_stage, (float*)out, out_f32, lse, seq_tile0,
                                                                  tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
-                                                                 window);
+                                                                 window, sb);
     return launch_status();
   }
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
@@ -319,7 +333,7 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
   }
   attn_prefill_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,
                                                               (const bf16*)v_stage, (bf16*)out, out_f32, lse, seq_tile0, tok_seq,
-                                                              tok_pos, n_heads, n_kv_heads, head_dim, window);
+                                                              tok_pos, n_heads, n_kv_heads, head_dim, window, sb);
   return launch_status();
 }
 
@@ -330,7 +344,7 @@ extern "C" int yalm_attn_prefill(const void* q, const void* k_stage, const void*
                                  hipStream_t stream) {
   return yalm_attn_prefill_lse(q, k_stage, v_stage, out, nullptr, nullptr, cu_seqlens, seq_tile0, tok_seq, tok_pos, tile_order,
                                n_order, T, B, n_tiles, n_heads, n_kv_heads, head_dim, window, dtype, force_simple,
-                               stream);
+                               nullptr, 0, stream);
 }
 
 // merges the partial results of the splits (also used by the MFMA kernel)
@@ -355,8 +369,11 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
                     int ring_pages, const int* seq_slot, const int* seq_len, void* out, float* lse, float* partial,
                     int B, int n_heads, int n_kv_heads, int head_dim, int window, int n_splits, int n_pages,
                     int page_layout, int dtype, int force_simple, const SinkArgs& sinks, const int* step_max_len,
-                    const int* seq_order, hipStream_t stream) {
+                    const int* seq_order, const float* score_bias, int n_bias, hipStream_t stream) {
   if (B <= 0) return YALM_OK;
+  if (score_bias != nullptr && (n_bias <= 0 || sinks.n_sinks > 0)) return YALM_ERR_ARG;   // sinks are scored without it
+  const ScoreBias sb = {score_bias, n_bias};
+  if (score_bias != nullptr) force_simple = 1;     // the matrix-core kernel takes no bias
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0 ||
       !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
@@ -364,7 +381,7 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
   if (dtype == YALM_F32) {
     attn_decode_simple_kernel<float><<<grid, WAVE, 0, stream>>>(
         (const float*)q, (const float*)k_pages, (const float*)v_pages, block_table, table_stride, ring_pages,
-        seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout);
+        seq_slot, seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
     attn_decode_combine_kernel<float><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (float*)out, lse, n_heads,
                                                                              head_dim, n_splits, sinks);
     return launch_status();
@@ -378,7 +395,7 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
   }
   attn_decode_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>(
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot,
-      seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout);
+      seq_len, partial, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, sb);
   attn_decode_combine_kernel<bf16><<<cgrid, COMBINE_THREADS, 0, stream>>>(partial, (bf16*)out, lse, n_heads, head_dim,
                                                                           n_splits, sinks);
   return launch_status();
@@ -390,11 +407,11 @@ extern "C" int yalm_attn_decode_lse(const void* q, const void* k_pages, const vo
                                     void* out, float* lse, float* partial, int B, int n_heads, int n_kv_heads,
                                     int head_dim, int window, int n_splits, int n_pages, int page_layout, int dtype,
                                     int force_simple, const int* step_max_len, const int* seq_order,
-                                    hipStream_t stream) {
+                                    const float* score_bias, int n_bias, hipStream_t stream) {
   SinkArgs none = {};
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, lse,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, none, step_max_len, seq_order, stream);
+                         force_simple, none, step_max_len, seq_order, score_bias, n_bias, stream);
 }
 
 extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -403,7 +420,7 @@ extern "C" int yalm_attn_decode(const void* q, const void* k_pages, const void* 
                                 int n_splits, int n_pages, int dtype, int force_simple, hipStream_t stream) {
   return yalm_attn_decode_lse(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out,
                               nullptr, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages,
-                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, stream);
+                              YALM_PAGE_ROWS, dtype, force_simple, nullptr, nullptr, nullptr, 0, stream);
 }
 
 extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
@@ -439,7 +456,7 @@ extern "C" int yalm_attn_decode_sinks(const void* q, const void* k_pages, const 
   sk.n_sinks = n_sinks;
   return attn_decode_any(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len, out, nullptr,
                          partial, B, n_heads, n_kv_heads, head_dim, window, n_splits, n_pages, page_layout, dtype,
-                         force_simple, sk, step_max_len, seq_order, stream);
+                         force_simple, sk, step_max_len, seq_order, nullptr, 0, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -12,4 +12,4 @@ extern "C" const char* yalm_error_string(int code) {
   }
 }
 
-extern "C" int yalm_abi_version(void) { return 23; }
+extern "C" int yalm_abi_version(void) { return 24; }

@@ -162,15 +162,20 @@ long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits);
 // longest sequence; the matrix-core decode kernel then cuts every sequence into splits of that sequence's split size,
 // so that sequences of unequal lengths give workgroups of equal work (no result depends on it).  seq_order (device,
 // B ints, a permutation of the rows; may be null): the order in which that kernel's workgroups take the rows.
+// score_bias (device, float32 [n_heads, n_bias]; may be null): a term added to every score (after the 1/sqrt(head_dim)
+// scaling) by the distance between query and key, score_bias[head, min(distance, n_bias - 1)]: what a position
+// encoding that is no rotation needs.  With it the float32-arithmetic kernels run, whatever the dtype.
 int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* out_f32, float* lse,
                           const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                           const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads, int n_kv_heads,
-                          int head_dim, int window, int dtype, int force_simple, hipStream_t stream);
+                          int head_dim, int window, int dtype, int force_simple, const float* score_bias, int n_bias,
+                          hipStream_t stream);
 int yalm_attn_decode_lse(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                          int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                          float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                          int n_splits, int n_pages, int page_layout, int dtype, int force_simple,
-                         const int* step_max_len, const int* seq_order, hipStream_t stream);
+                         const int* step_max_len, const int* seq_order, const float* score_bias, int n_bias,
+                         hipStream_t stream);
 
 // Attention sinks beside a window (src/infer.cpp:305-319, 486-488): the first n_sinks positions of a
 // sequence stay visible when the window has moved past them, and each then counts as lying

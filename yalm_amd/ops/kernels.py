@@ -557,13 +557,24 @@ def prefill_tile_order(n_tokens):
     return tiles
 
 
+def _bias(score_bias, n_heads):
+    """(address, distances) of a score bias: float32 [n_heads, n] on the device, added to every score (scaled by
+    1/sqrt(head_dim) already) as score_bias[head, min(query position - key position, n - 1)]; None: no bias.  What a
+    position encoding that is no rotation needs (a slope per head times the distance, a learned table).  With it the
+    float32-arithmetic attention kernels run, in both dtypes."""
+    if score_bias is None:
+        return None, 0
+    n = score_bias.shape[-1]
+    return _need(score_bias, "score_bias", torch.float32, (n_heads, n)), n
+
+
 def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_pos, n_heads, n_kv_heads, head_dim,
-                 window, tile_order=None, lse=None, out_f32=None):
+                 window, tile_order=None, lse=None, out_f32=None, score_bias=None):
     """Causal (and windowed) attention of packed sequences that start at position 0, over
     the keys and values that rope_kv_write staged for this step.  tile_order (device int32,
     from prefill_tile_order) only changes the order of the work.  lse (float32 [T, n_heads], optional)
     receives the logarithm of every query's sum of exp(score), for attn_sink_mix; out_f32 (float32 [T, n_heads *
-    head_dim], optional) the result before it is rounded to out's dtype, for the same."""
+    head_dim], optional) the result before it is rounded to out's dtype, for the same.  score_bias: see _bias."""
     _check_heads(n_heads, n_kv_heads, head_dim)
     T = q.shape[0]
     dt = q.dtype
@@ -585,7 +596,8 @@ def attn_prefill(q, k_stage, v_stage, out, cu_seqlens, seq_tile0, tok_seq, tok_p
     p_o32 = _opt(out_f32, "out_f32", torch.float32, (T, n_heads * head_dim))
     library.check(library.lib().yalm_attn_prefill_lse(p_q, p_k, p_v, p_o, p_o32, p_lse, p_cu, p_t0, p_ts, p_tp, p_or, n_order,
                                                       T, B, n_tiles, n_heads, n_kv_heads, head_dim, int(window),
-                                                      dtype_code(dt), 1 if FORCE_SIMPLE else 0, _stream()),
+                                                      dtype_code(dt), 1 if FORCE_SIMPLE else 0,
+                                                      *_bias(score_bias, n_heads), _stream()),
                   "attn_prefill")
     return out
 
@@ -595,12 +607,14 @@ def attn_decode_workspace_floats(B, n_heads, head_dim, n_splits):
 
 
 def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len, out, partial, n_heads, n_kv_heads,
-                head_dim, window, n_splits, lse=None, sinks=None, layout=None, step_max_len=None, seq_order=None):
+                head_dim, window, n_splits, lse=None, sinks=None, layout=None, step_max_len=None, seq_order=None,
+                score_bias=None):
     """One query per sequence over the cache pages (laid out as `layout` says, default page_layout(head_dim));
     seq_len counts the new key.  lse as in attn_prefill.  step_max_len (int32 [1] on the device, optional): the
     length of the step's longest sequence, with which sequences of unequal lengths are cut into splits of equal
     size; seq_order (int32 [B] on the device, a permutation of the rows, optional): the order in which the
-    workgroups take the rows (both change the division of the work and no result).
+    workgroups take the rows (both change the division of the work and no result).  score_bias: see _bias (not with
+    sinks).
     sinks = (sink_k, sink_v [slots, n_kv_heads, n_sinks, head_dim], cos_sin or None, rotary_dim, store):
     the attention sinks that a query's window no longer covers are taken in where the splits are merged
     (their keys turned by max(0, position - window - n_sinks + 1) positions with the table cos_sin); with
@@ -630,11 +644,13 @@ def attn_decode(q, k_pages, v_pages, block_table, ring_pages, seq_slot, seq_len,
         p_lse = None if lse is None else _need(lse, "lse", torch.float32, (B, n_heads))
         library.check(library.lib().yalm_attn_decode_lse(
             p_q, p_kp, p_vp, p_bt, stride, ring_pages, p_ss, p_sl, p_o, p_lse, p_w, B, n_heads, n_kv_heads, head_dim,
-            int(window), int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, p_max, p_ord, _stream()),
-            "attn_decode")
+            int(window), int(n_splits), n_pages, _layout(layout, head_dim), dtype_code(dt), force, p_max, p_ord,
+            *_bias(score_bias, n_heads), _stream()), "attn_decode")
         return out
     if lse is not None:
         raise ValueError("attn_decode leaves no lse when it takes the sinks in itself")
+    if score_bias is not None:
+        raise ValueError("attention sinks are scored without a score bias: the two do not go together")
     sink_k, sink_v, cos_sin, rotary_dim, store = sinks
     n_slots, _, n_sinks, _ = sink_k.shape
     if window < n_sinks:

@@ -34,8 +34,9 @@ _SIGNATURES = {
     "yalm_attn_decode": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_workspace": (ctypes.c_long, [_I, _I, _I, _I]),
     "yalm_attn_prefill_lse": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I,
-                                   _P]),
-    "yalm_attn_decode_lse": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P]),
+                                   _P, _I, _P]),
+    "yalm_attn_decode_lse": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P,
+                                  _P, _I, _P]),
     "yalm_sink_store": (_I, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_sink_mix": (_I, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]),
     "yalm_attn_decode_sinks": (_I, [_P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P]),
@@ -51,7 +52,7 @@ _SIGNATURES = {
     "yalm_probe_mfma": (_I, [_I, _I, _I, _P, _P, _P]),
 }
 
-ABI_VERSION = 23
+ABI_VERSION = 24
 
 
 class KernelError(RuntimeError):

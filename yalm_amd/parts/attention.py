@@ -77,6 +77,15 @@ class GQAttention(Part):
     def children(self):
         return [self.position]
 
+    @property
+    def score_bias(self):
+        """The position part's term for every score by the distance of query and key (float32 [n_heads, distances]
+        on the device), if it has one: a position encoding that is no rotation."""
+        bias = getattr(self.position, "score_bias", None)
+        if bias is not None and self.sinks:
+            raise ValueError("attention sinks are scored without a score bias: the two do not go together")
+        return bias
+
     def param_specs(self):
         D = self.dim
         return [ParamSpec(self.prefix + "q_proj.weight", (self.q_dim, D), fan_in=D),
@@ -108,6 +117,9 @@ class GQAttention(Part):
         if compute_dtype != torch.bfloat16:
             return what + ": float32-arithmetic kernels", False
         group = self.n_heads // self.n_kv_heads
+        if getattr(self.position, "score_bias", None) is not None:
+            return what + ": float32-arithmetic kernels on bfloat16 storage (the matrix-core kernels take no score " \
+                          "bias, which this position encoding has): correct, several times slower", True
         if self.head_dim in kernels.MFMA_HEAD_DIMS and group <= 16:
             return what + ": matrix-core kernels", False
         why = "head size %d" % self.head_dim if self.head_dim not in kernels.MFMA_HEAD_DIMS else "%d heads a group" % group
@@ -116,7 +128,7 @@ class GQAttention(Part):
 
     def decode_splits(self, B, max_pages, ragged=False):
         mfma = self.head_dim in kernels.MFMA_HEAD_DIMS and self.n_heads // self.n_kv_heads <= 16 \
-            and not kernels.FORCE_SIMPLE
+            and not kernels.FORCE_SIMPLE and getattr(self.position, "score_bias", None) is None
         if mfma:         # a workgroup of 4 waves per (split, KV head, sequence), a page per wave at a time
             per = max(1, B * self.n_kv_heads)
             quarters = max(1, min((max_pages + 3) // 4, 4))
@@ -230,7 +242,7 @@ class GQAttention(Part):
             sinks = (sink_k, sink_v, self.position.table, self.position.rotary_dim, writes_cache)
         kernels.attn_decode(q, k_pages, v_pages, group.table, group.ring_pages, ctx.seq_slot, ctx.seq_len, o, partial,
                             self.n_heads, self.n_kv_heads, self.head_dim, self.window, n_splits, sinks=sinks,
-                            step_max_len=ctx.step_max_len, seq_order=ctx.seq_order)
+                            step_max_len=ctx.step_max_len, seq_order=ctx.seq_order, score_bias=self.score_bias)
 
     def forward(self, h, x, ctx, line, writes_cache=True, emit_for=None):
         T = h.shape[0]
@@ -286,7 +298,7 @@ class GQAttention(Part):
                 kernels.sink_store(kst, vst, seq_tile0, ctx.seq_slot, ctx.seq_len, sink_k, sink_v)
             kernels.attn_prefill(q, kst, vst, o, ctx.cu_seqlens, seq_tile0, ctx.tok_seq, ctx.tok_pos,
                                  self.n_heads, self.n_kv_heads, self.head_dim, self.window, tiles.get("tile_order"),
-                                 lse=lse, out_f32=o32)
+                                 lse=lse, out_f32=o32, score_bias=self.score_bias)
             if self.sinks:
                 sink_k, sink_v = group.line_sinks(line)
                 kernels.attn_sink_mix(q, o, lse, sink_k, sink_v, ctx.tok_seq, ctx.tok_pos, ctx.seq_slot, pos.table,
