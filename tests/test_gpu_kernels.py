@@ -1143,6 +1143,35 @@ def test_gemm_norm(M, N, Kd):
 
 
 @pytest.mark.parametrize("act", ACTS)
+@pytest.mark.parametrize("M,H,D", [(8, 14336, 4096), (1, 14336, 192), (16, 14336, 1024), (11, 13003, 64), (4, 12810, 320),
+                                   (9, 20000, 128), (3, 28672, 256)])
+def test_gemm_gated_wide_at_up_to_16_rows(M, H, D, act):
+    """Up to 16 rows and a gated matrix wide enough for the workgroups of 128 weight rows: hidden widths that are no
+    multiples of 8 or of 64, one and many stages of K, with and without the row scale of the norm chain; every hidden
+    column is written, nothing beyond them."""
+    from yalm_amd.parts.swiglu import interleave_gate_up
+    k = K()
+    act_fn, epi_code = gate(act)
+    x = rnd((M, D), 53, torch.bfloat16, scale=2.0)
+    wg = rnd((H, D), 55, torch.bfloat16, scale=1 / math.sqrt(D))
+    wu = rnd((H, D), 56, torch.bfloat16, scale=1 / math.sqrt(D))
+    w = interleave_gate_up(wg, wu).to(DEV)
+    g, u = x.double() @ wg.double().T, x.double() @ wu.double().T
+    out = torch.full((M + 1, H), 7.0, dtype=torch.bfloat16, device=DEV)
+    k.gemm(x.to(DEV), w, out[:M], epi_code, hidden=H)
+    close(out[:M], act_fn(g) * u, torch.bfloat16, "gated product")
+    assert (out[M] == 7.0).all()
+    # the same behind the norm chain: the sums are scaled row by row before the activation
+    ss = (x.double() ** 2).sum(dim=1, keepdim=True).float() * torch.tensor([[0.25, 0.5, 0.25]])
+    eps = 1e-5
+    scale = 1.0 / torch.sqrt((x.double() ** 2).sum(dim=1, keepdim=True) / D + eps)
+    out2 = torch.full((M + 1, H), 7.0, dtype=torch.bfloat16, device=DEV)
+    k.gemm_chain(x.to(DEV), w, out2[:M], epi_code, hidden=H, scale_from=(ss.to(DEV).contiguous(), eps))
+    close(out2[:M], act_fn(g * scale) * (u * scale), torch.bfloat16, "gated product with a row scale", factor=2.0)
+    assert (out2[M] == 7.0).all()
+
+
+@pytest.mark.parametrize("act", ACTS)
 @pytest.mark.parametrize("M,H,D", [(1, 176, 64), (8, 1000, 264), (5, 14336, 128)])
 def test_gemm_norm_gated(M, H, D, act):
     from yalm_amd.parts.swiglu import interleave_gate_up
