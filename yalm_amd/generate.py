@@ -75,8 +75,10 @@ def generate(engine, prompts, max_new_tokens=256, temperature=0.0, seed=0, stop_
     each request, in the order of the prompts.  stop_ids None means the model's own
     (config eos); on_token(request index, token) is called for every new token.
     ahead: queue each step before the host has read the tokens of the step before
-    (default: if the engine has step_from and the sampler has draw); the tokens are
-    the same either way."""
+    (default: if the engine has step_from and the sampler has draw).  A request that has ended
+    leaves the batch a step later then, so a step may run with another number of rows and take other
+    kernels: in float32 the tokens are the same either way, in bfloat16 up to choices between logits
+    that lie within rounding of each other."""
     from .sampling import Sampler
     sampler = sampler or Sampler(seed)
     stats = stats if stats is not None else GenerationStats()
