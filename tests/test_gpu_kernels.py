@@ -725,16 +725,26 @@ def _attn_decode_case(n_heads, n_kv, hd, window, lens, splits, dtype, simple, st
     assert (out[B] == 0).all()
 
 
+@pytest.mark.parametrize("simple", [False, True])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens,n_bias", [
-    (4, 2, 16, 0, [5, 130, 64], 200), (6, 3, 64, 70, [300, 1], 40), (8, 2, 128, 0, [257], 300), (3, 1, 48, 20, [90, 65], 7)])
-def test_attn_with_a_score_bias(n_heads, n_kv, hd, window, lens, n_bias, dtype):
+    (4, 2, 16, 0, [5, 130, 64], 200), (6, 3, 64, 70, [300, 1], 40), (8, 2, 128, 0, [257], 300), (3, 1, 48, 20, [90, 65], 7),
+    (40, 8, 128, 0, [1500], 900), (40, 8, 96, 200, [1100, 1200], 64), (12, 4, 32, 0, [1300], 2000), (16, 1, 64, 0, [70, 2], 3)])
+def test_attn_with_a_score_bias(n_heads, n_kv, hd, window, lens, n_bias, dtype, simple):
     """A term added to every score by the distance of query and key (a table a head, the last entry for every
     distance beyond it): prompt and decode kernels against a float64 softmax with the same term.  The table is steep
     (a slope a head plus noise), so that dropping it, taking another head's row or counting the distance from the
-    wrong end changes the result by far more than rounding; the matrix-core kernels would ignore it, so the
-    float32-arithmetic ones run."""
+    wrong end changes the result by far more than rounding.  Both kinds of kernels take it; the long prompts reach
+    each launch shape of the matrix-core prompt kernel."""
     k = K()
+    k.FORCE_SIMPLE = simple
+    try:
+        _score_bias_case(k, n_heads, n_kv, hd, window, lens, n_bias, dtype)
+    finally:
+        k.FORCE_SIMPLE = False
+
+
+def _score_bias_case(k, n_heads, n_kv, hd, window, lens, n_bias, dtype):
     slopes = 2.0 ** -(torch.arange(n_heads, dtype=torch.float64) * 3.0 / n_heads)
     bias = (-slopes[:, None] * torch.arange(n_bias, dtype=torch.float64)[None, :] + rnd((n_heads, n_bias), 77).double()).float()
     T = sum(lens)

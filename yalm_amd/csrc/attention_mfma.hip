@@ -48,13 +48,14 @@ __device__ __forceinline__ int key_row(int t, int i) { return 32 * (t >> 1) + 8 
 // BLOCKS: the pages are laid out in blocks (YALM_PAGE_BLOCKS): every load instruction reads 1 KB of consecutive
 // bytes, and asks for them non-temporally (a step reads a page once; with pieces of lines the hint costs more
 // than it gains: the other half of a line would be fetched again).
-template <int HD, int NW, bool BLOCKS>
+// BIAS: a term is added to every score by the distance of query and key, bias[head][min(distance, n_bias - 1)].
+template <int HD, int NW, bool BLOCKS, bool BIAS>
 __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_kernel(   // 2 waves a SIMD: head size 128 needs their registers
     const bf16* __restrict__ q, const bf16* __restrict__ k_pages, const bf16* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_stride, int ring_pages, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out, float* __restrict__ lse,
     int n_heads, int n_kv_heads, int window, int n_splits, int n_pages, const int* __restrict__ step_max_len,
-    const int* __restrict__ seq_order) {
+    const int* __restrict__ seq_order, const float* __restrict__ bias, int n_bias) {
   constexpr int KS = HD / 32, DT = HD / 16;
   __shared__ float sm_m[NW][16];
   __shared__ float sm_l[NW][16];
@@ -102,6 +103,7 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
       for (int ks = 0; ks < KS; ++ks) qv[ks] = head_ok ? ld8(qrow + ks * 32 + qd * 8) : zero8();
     }
 
+    const float* bias_row = BIAS ? bias + (size_t)(g * G + min(j, G - 1)) * n_bias : nullptr;   // the column's head
     bf16x8 kreg[4][KS];
     auto page_of = [&](int a) { return min(max(table[a % ring_pages], 0), n_pages - 1); };
     auto load_keys = [&](int phys) {
@@ -153,6 +155,10 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           float v = sc[t][r] * score_scale;
+          if constexpr (BIAS) {                    // in the same units as the scores: exponents of 2
+            const int dist = L - 1 - (base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r);
+            v = fmaf(bias_row[min(max(dist, 0), n_bias - 1)], 1.4426950408889634f, v);
+          }
           if (edge) {
             int pos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
             if (pos < lo || pos >= L) v = -INFINITY;
@@ -263,12 +269,13 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 // compute unit alone and is done in half the time, so that the compute units are no longer held by
 // the few workgroups that see the most keys (with KSPL = 1 the launch lasts as long as its longest
 // workgroup, 32 key tiles at 2,048 tokens, while the mean is 17).
-template <int HD, int NC, int KSPL>
+// BIAS: a term is added to every score by the distance of query and key, bias[head][min(distance, n_bias - 1)].
+template <int HD, int NC, int KSPL, bool BIAS>
 __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mfma_kernel(
     const bf16* __restrict__ q, const bf16* __restrict__ k_stage, const bf16* __restrict__ v_stage,
     bf16* __restrict__ out, float* __restrict__ out_f32, float* __restrict__ lse, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_tile0, const int* __restrict__ tile_order, int fold_at, int B, int n_heads,
-    int n_kv_heads, int window) {
+    int n_kv_heads, int window, const float* __restrict__ bias, int n_bias) {
   constexpr int KS = HD / 32, DT = HD / 16;
   constexpr int KROW = HD + 8;                    // LDS row strides (elements): 16 bytes of padding
   constexpr int VROW = PAGE + 8;
@@ -306,6 +313,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
   const int start = cu_seqlens[b], len = cu_seqlens[b + 1] - start;
   const int g = h / (n_heads / n_kv_heads);
   const float score_scale = 1.4426950408889634f / sqrtf((float)HD);   // log2(e) / sqrt(head_dim)
+  const float* bias_row = BIAS ? bias + (size_t)h * n_bias : nullptr;
 
   const int blk0 = tq * PAGE;                     // first position of the workgroup
   const int pos0 = blk0 + wave * 16 * NC;         // first position of the wave
@@ -410,6 +418,11 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               float v = sc[c][t][r];
+              if constexpr (BIAS) {               // scaled here, with the distance's term in the same units (exponents of 2)
+                const int dist = pos_q[c] - (base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r);
+                v = fmaf(v, score_scale, bias_row[min(max(dist, 0), n_bias - 1)] * 1.4426950408889634f);
+                sc[c][t][r] = v;
+              }
               if (decltype(masked)::value) {
                 int kpos = base + 32 * (t >> 1) + 8 * qd + 4 * (t & 1) + r;
                 bool vis = kpos <= pos_q[c] && (window == 0 || pos_q[c] - kpos < window) && q_ok[c];
@@ -420,14 +433,15 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
             }
           mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
           mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-          const float m_new = fmaxf(m[c], mx * score_scale);
+          const float m_new = fmaxf(m[c], BIAS ? mx : mx * score_scale);
           corr[c] = __builtin_amdgcn_exp2f(m[c] - m_new);
           float psum = 0.f;
 #pragma unroll
           for (int s2 = 0; s2 < 2; ++s2)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-              float p = __builtin_amdgcn_exp2f(fmaf(sc[c][2 * s2 + (e >> 2)][e & 3], score_scale, -m_new));
+              const float sv = sc[c][2 * s2 + (e >> 2)][e & 3];
+              float p = __builtin_amdgcn_exp2f(BIAS ? sv - m_new : fmaf(sv, score_scale, -m_new));
               psum += p;
               pb[c][s2][e] = static_cast<bf16>(p);
             }
@@ -539,26 +553,36 @@ bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
 }
 
 // launches attn_prefill_mfma_kernel<head_dim, NC, KSPL> (more than 64 KB of LDS is asked for once a device)
-template <int HD, int NC, int KSPL>
+template <int HD, int NC, int KSPL, bool BIAS>
 int launch_prefill(dim3 grid, int threads, size_t lds, hipStream_t stream, const bf16* qp, const bf16* kp, const bf16* vp,
                    bf16* out, float* out_f32, float* lse, const int* cu_seqlens, const int* seq_tile0,
-                   const int* tile_order, int fold_at, int B, int n_heads, int n_kv_heads, int window) {
-  auto kernel = &attn_prefill_mfma_kernel<HD, NC, KSPL>;
+                   const int* tile_order, int fold_at, int B, int n_heads, int n_kv_heads, int window,
+                   const float* bias, int n_bias) {
+  auto kernel = &attn_prefill_mfma_kernel<HD, NC, KSPL, BIAS>;
   if (lds > 64 * 1024) {
     static LdsAllowance allowed;
     if (int rc = allow_dynamic_lds(allowed, (const void*)kernel, 150 * 1024); rc != YALM_OK) return rc;
   }
   kernel<<<grid, threads, lds, stream>>>(qp, kp, vp, out, out_f32, lse, cu_seqlens, seq_tile0, tile_order, fold_at, B,
-                                         n_heads, n_kv_heads, window);
+                                         n_heads, n_kv_heads, window, bias, n_bias);
   return launch_status();
 }
 template <int NC, int KSPL, typename... Args>
-int launch_prefill_hd(int head_dim, Args... args) {
+int launch_prefill_hd(int head_dim, bool biased, Args... args) {
+  if (biased) {
+    switch (head_dim) {
+      case 32: return launch_prefill<32, NC, KSPL, true>(args...);
+      case 64: return launch_prefill<64, NC, KSPL, true>(args...);
+      case 96: return launch_prefill<96, NC, KSPL, true>(args...);
+      case 128: return launch_prefill<128, NC, KSPL, true>(args...);
+    }
+    return YALM_ERR_ARG;
+  }
   switch (head_dim) {
-    case 32: return launch_prefill<32, NC, KSPL>(args...);
-    case 64: return launch_prefill<64, NC, KSPL>(args...);
-    case 96: return launch_prefill<96, NC, KSPL>(args...);
-    case 128: return launch_prefill<128, NC, KSPL>(args...);
+    case 32: return launch_prefill<32, NC, KSPL, false>(args...);
+    case 64: return launch_prefill<64, NC, KSPL, false>(args...);
+    case 96: return launch_prefill<96, NC, KSPL, false>(args...);
+    case 128: return launch_prefill<128, NC, KSPL, false>(args...);
   }
   return YALM_ERR_ARG;
 }
@@ -568,8 +592,10 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
                                 float* lse,
                                 const int* cu_seqlens, const int* seq_tile0, const int* tile_order, int n_order,
                                 int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
-                                hipStream_t stream) {
+                                const float* bias, int n_bias, hipStream_t stream) {
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_tiles > 65535) return YALM_ERR_ARG;
+  if (bias != nullptr && n_bias <= 0) return YALM_ERR_ARG;
+  const bool biased = bias != nullptr;
   if (tile_order && (n_order <= 0 || n_order > n_tiles)) return YALM_ERR_ARG;
   dim3 grid(n_heads, tile_order ? n_order : n_tiles);
   const long total = (long)grid.x * grid.y;
@@ -585,52 +611,64 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
     // a short step: a workgroup of eight waves for every tile of 64 queries (not 128), so that twice as many
     // compute units work (512 tokens with 32 heads: 19.6 -> 15.9 us a layer); all of them run at once, so their order
     // does not matter
-    return launch_prefill_hd<1, 2>(head_dim, dim3(n_heads, n_tiles), 512, 4 * tile_bytes, stream, qp, kp, vp, (bf16*)out,
-                                   out_f32, lse, cu_seqlens, seq_tile0, (const int*)nullptr, 0, B, n_heads, n_kv_heads,
-                                   window);
+    return launch_prefill_hd<1, 2>(head_dim, biased, dim3(n_heads, n_tiles), 512, 4 * tile_bytes, stream, qp, kp, vp,
+                                   (bf16*)out, out_f32, lse, cu_seqlens, seq_tile0, (const int*)nullptr, 0, B, n_heads,
+                                   n_kv_heads, window, bias, n_bias);
   }
   if (working <= 2L * compute_units()) {
     // a workgroup of eight waves a compute unit, the workgroups that see the most keys first
-    return launch_prefill_hd<2, 2>(head_dim, grid, 512, 4 * tile_bytes, stream, qp, kp, vp, (bf16*)out, out_f32, lse,
-                                   cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads, n_kv_heads, window);
+    return launch_prefill_hd<2, 2>(head_dim, biased, grid, 512, 4 * tile_bytes, stream, qp, kp, vp, (bf16*)out, out_f32,
+                                   lse, cu_seqlens, seq_tile0, tile_order, (int)total, B, n_heads, n_kv_heads, window,
+                                   bias, n_bias);
   }
   // two workgroups fit a compute unit: with more than one and at most two each, the second
   // half of the launch runs from the shortest workgroup up
   const int cus = compute_units();
   const int fold_at = total > cus && total <= 2 * cus ? cus : (int)total;
-  return launch_prefill_hd<2, 1>(head_dim, grid, 256, 2 * tile_bytes, stream, qp, kp, vp, (bf16*)out, out_f32, lse,
-                                 cu_seqlens, seq_tile0, tile_order, fold_at, B, n_heads, n_kv_heads, window);
+  return launch_prefill_hd<2, 1>(head_dim, biased, grid, 256, 2 * tile_bytes, stream, qp, kp, vp, (bf16*)out, out_f32,
+                                 lse, cu_seqlens, seq_tile0, tile_order, fold_at, B, n_heads, n_kv_heads, window, bias,
+                                 n_bias);
 }
 
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                                int n_splits, int n_pages, int page_layout, const SinkArgs& sinks,
-                               const int* step_max_len, const int* seq_order, hipStream_t stream) {
+                               const int* step_max_len, const int* seq_order, const float* bias, int n_bias,
+                               hipStream_t stream) {
   // with sinks the merge kernel always runs: it takes them in, also where there is one split
   const bool merge = n_splits > 1 || sinks.n_sinks > 0;
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_heads / n_kv_heads > 16) return YALM_ERR_ARG;
+  // a score bias: the pages in blocks only (the engine's layout), and no sinks (they are scored without it)
+  if (bias != nullptr && (n_bias <= 0 || page_layout != YALM_PAGE_BLOCKS || sinks.n_sinks > 0)) return YALM_ERR_ARG;
   dim3 grid(n_splits, n_kv_heads, B);
-#define YALM_DECODE(HD_, NW_, BLOCKS_)                                                                              \
-  attn_decode_mfma_kernel<HD_, NW_, BLOCKS_><<<grid, NW_ * WAVE, 0, stream>>>(                                      \
+#define YALM_DECODE(HD_, NW_, BLOCKS_, BIAS_)                                                                       \
+  attn_decode_mfma_kernel<HD_, NW_, BLOCKS_, BIAS_><<<grid, NW_ * WAVE, 0, stream>>>(                               \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot, \
       seq_len, partial, merge ? nullptr : (bf16*)out, lse, n_heads, n_kv_heads, window, n_splits, n_pages, \
-      step_max_len, seq_order)
+      step_max_len, seq_order, bias, n_bias)
   // 4 waves a workgroup: 8 measured no faster with one split and slower with more (a CU draws about
   // 33 GB/s whatever its number of waves, so a small batch needs its workgroups spread over all CUs)
-  if (page_layout == YALM_PAGE_BLOCKS) {
+  if (bias != nullptr) {
     switch (head_dim) {
-      case 32: YALM_DECODE(32, 4, true); break;
-      case 64: YALM_DECODE(64, 4, true); break;
-      case 96: YALM_DECODE(96, 4, true); break;
-      default: YALM_DECODE(128, 4, true); break;
+      case 32: YALM_DECODE(32, 4, true, true); break;
+      case 64: YALM_DECODE(64, 4, true, true); break;
+      case 96: YALM_DECODE(96, 4, true, true); break;
+      default: YALM_DECODE(128, 4, true, true); break;
+    }
+  } else if (page_layout == YALM_PAGE_BLOCKS) {
+    switch (head_dim) {
+      case 32: YALM_DECODE(32, 4, true, false); break;
+      case 64: YALM_DECODE(64, 4, true, false); break;
+      case 96: YALM_DECODE(96, 4, true, false); break;
+      default: YALM_DECODE(128, 4, true, false); break;
     }
   } else {
     switch (head_dim) {
-      case 32: YALM_DECODE(32, 4, false); break;
-      case 64: YALM_DECODE(64, 4, false); break;
-      case 96: YALM_DECODE(96, 4, false); break;
-      default: YALM_DECODE(128, 4, false); break;
+      case 32: YALM_DECODE(32, 4, false, false); break;
+      case 64: YALM_DECODE(64, 4, false, false); break;
+      case 96: YALM_DECODE(96, 4, false, false); break;
+      default: YALM_DECODE(128, 4, false, false); break;
     }
   }
 #undef YALM_DECODE

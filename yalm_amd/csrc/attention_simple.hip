@@ -12,12 +12,13 @@ int yalm_attn_prefill_bf16_mfma(const void* q, const void* k_stage, const void* 
                                 float* lse,
                                 const int* cu_seqlens, const int* seq_tile0, const int* tile_order, int n_order,
                                 int T, int B, int n_tiles, int n_heads, int n_kv_heads, int head_dim, int window,
-                                hipStream_t stream);
+                                const float* bias, int n_bias, hipStream_t stream);
 int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v_pages, const int* block_table,
                                int table_stride, int ring_pages, const int* seq_slot, const int* seq_len, void* out,
                                float* lse, float* partial, int B, int n_heads, int n_kv_heads, int head_dim, int window,
                                int n_splits, int n_pages, int page_layout, const SinkArgs& sinks,
-                               const int* step_max_len, const int* seq_order, hipStream_t stream);
+                               const int* step_max_len, const int* seq_order, const float* bias, int n_bias,
+                               hipStream_t stream);
 
 namespace {
 // A term added to every score by the distance between query and key: table[head][min(distance, n - 1)] (float32), or
@@ -316,7 +317,6 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_tiles <= 0) return YALM_ERR_ARG;
   if (score_bias != nullptr && n_bias <= 0) return YALM_ERR_ARG;
   const ScoreBias sb = {score_bias, n_bias};
-  if (score_bias != nullptr) force_simple = 1;     // the matrix-core kernels take no bias
   dim3 grid(T, n_heads);
   if (dtype == YALM_F32) {
     attn_prefill_simple_kernel<float><<<grid, WAVE, 0, stream>>>((const float*)q, (const float*)k_stage,
@@ -328,7 +328,7 @@ extern "C" int yalm_attn_prefill_lse(const void* q, const void* k_stage, const v
   if (dtype != YALM_BF16) return YALM_ERR_DTYPE;
   if (!force_simple) {
     int rc = yalm_attn_prefill_bf16_mfma(q, k_stage, v_stage, out, out_f32, lse, cu_seqlens, seq_tile0, tile_order, n_order, T, B,
-                                         n_tiles, n_heads, n_kv_heads, head_dim, window, stream);
+                                         n_tiles, n_heads, n_kv_heads, head_dim, window, score_bias, n_bias, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   attn_prefill_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>((const bf16*)q, (const bf16*)k_stage,
@@ -373,7 +373,6 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
   if (B <= 0) return YALM_OK;
   if (score_bias != nullptr && (n_bias <= 0 || sinks.n_sinks > 0)) return YALM_ERR_ARG;   // sinks are scored without it
   const ScoreBias sb = {score_bias, n_bias};
-  if (score_bias != nullptr) force_simple = 1;     // the matrix-core kernel takes no bias
   if (bad_heads(n_heads, n_kv_heads, head_dim) || window < 0 || n_splits <= 0 || ring_pages <= 0 ||
       !page_layout_ok(page_layout, head_dim))
     return YALM_ERR_ARG;
@@ -390,7 +389,7 @@ int attn_decode_any(const void* q, const void* k_pages, const void* v_pages, con
   if (!force_simple) {
     int rc = yalm_attn_decode_bf16_mfma(q, k_pages, v_pages, block_table, table_stride, ring_pages, seq_slot, seq_len,
                                         out, lse, partial, B, n_heads, n_kv_heads, head_dim, window, n_splits,
-                                        n_pages, page_layout, sinks, step_max_len, seq_order, stream);
+                                        n_pages, page_layout, sinks, step_max_len, seq_order, score_bias, n_bias, stream);
     if (rc != YALM_ERR_ARG) return rc;
   }
   attn_decode_simple_kernel<bf16><<<grid, WAVE, 0, stream>>>(

@@ -164,7 +164,7 @@ long yalm_attn_decode_workspace(int B, int n_heads, int head_dim, int n_splits);
 // B ints, a permutation of the rows; may be null): the order in which that kernel's workgroups take the rows.
 // score_bias (device, float32 [n_heads, n_bias]; may be null): a term added to every score (after the 1/sqrt(head_dim)
 // scaling) by the distance between query and key, score_bias[head, min(distance, n_bias - 1)]: what a position
-// encoding that is no rotation needs.  With it the float32-arithmetic kernels run, whatever the dtype.
+// encoding that is no rotation needs (not together with attention sinks).
 int yalm_attn_prefill_lse(const void* q, const void* k_stage, const void* v_stage, void* out, float* out_f32, float* lse,
                           const int* cu_seqlens, const int* seq_tile0, const int* tok_seq, const int* tok_pos,
                           const int* tile_order, int n_order, int T, int B, int n_tiles, int n_heads, int n_kv_heads,

@@ -560,8 +560,7 @@ def prefill_tile_order(n_tokens):
 def _bias(score_bias, n_heads):
     """(address, distances) of a score bias: float32 [n_heads, n] on the device, added to every score (scaled by
     1/sqrt(head_dim) already) as score_bias[head, min(query position - key position, n - 1)]; None: no bias.  What a
-    position encoding that is no rotation needs (a slope per head times the distance, a learned table).  With it the
-    float32-arithmetic attention kernels run, in both dtypes."""
+    position encoding that is no rotation needs (a slope per head times the distance, a learned table)."""
     if score_bias is None:
         return None, 0
     n = score_bias.shape[-1]

@@ -117,9 +117,6 @@ class GQAttention(Part):
         if compute_dtype != torch.bfloat16:
             return what + ": float32-arithmetic kernels", False
         group = self.n_heads // self.n_kv_heads
-        if getattr(self.position, "score_bias", None) is not None:
-            return what + ": float32-arithmetic kernels on bfloat16 storage (the matrix-core kernels take no score " \
-                          "bias, which this position encoding has): correct, several times slower", True
         if self.head_dim in kernels.MFMA_HEAD_DIMS and group <= 16:
             return what + ": matrix-core kernels", False
         why = "head size %d" % self.head_dim if self.head_dim not in kernels.MFMA_HEAD_DIMS else "%d heads a group" % group
@@ -128,7 +125,7 @@ class GQAttention(Part):
 
     def decode_splits(self, B, max_pages, ragged=False):
         mfma = self.head_dim in kernels.MFMA_HEAD_DIMS and self.n_heads // self.n_kv_heads <= 16 \
-            and not kernels.FORCE_SIMPLE and getattr(self.position, "score_bias", None) is None
+            and not kernels.FORCE_SIMPLE
         if mfma:         # a workgroup of 4 waves per (split, KV head, sequence), a page per wave at a time
             per = max(1, B * self.n_kv_heads)
             quarters = max(1, min((max_pages + 3) // 4, 4))
