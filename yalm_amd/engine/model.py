@@ -130,13 +130,16 @@ class Model:
         """Lets position encodings build their tables for positions < n_positions.  A table that
         already reaches that far stays as it is (engines that share the model keep using it);
         `tables_version` counts the times a table was replaced, for whoever holds its address."""
+        def held(p):          # addresses of what a captured graph may point to: the rotation table, a score bias
+            return tuple(t.data_ptr() for t in (getattr(p, "table", None), getattr(p, "score_bias", None)) if t is not None)
         for p in self.all_parts():
             if hasattr(p, "prepare"):
                 before = getattr(p, "table", None)
                 if before is not None and getattr(p, "n_positions", 0) >= n_positions:
                     continue
+                was = held(p)
                 p.prepare(n_positions, self.device)
-                if before is not None:
+                if was and held(p) != was:
                     self.tables_version += 1
 
     # ------------------------------------------------------------------ the step as a row of units
