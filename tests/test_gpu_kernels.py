@@ -534,7 +534,7 @@ def stage(kk, v, lens, n_kv, hd, dtype, poison=True):
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens", [
     (4, 2, 16, 0, [5, 17, 1]), (3, 1, 32, 16, [2, 30, 70]), (6, 3, 48, 100, [130, 64]), (8, 2, 128, 0, [200]),
     (2, 2, 80, 7, [65, 3]), (5, 5, 64, 0, [129]), (4, 1, 64, 70, [300, 64, 1]), (8, 2, 128, 100, [17, 257]),
-    (6, 2, 96, 50, [150, 64, 333]), (9, 3, 32, 0, [257, 1])])
+    (6, 2, 96, 50, [150, 64, 333]), (9, 3, 32, 0, [257, 1]), (4, 2, 112, 30, [200, 64]), (5, 1, 16, 0, [131, 7])])
 def test_attn_prefill(n_heads, n_kv, hd, window, lens, dtype, simple):
     k = K()
     T = sum(lens)
@@ -577,7 +577,9 @@ def masked_attention_float64(q, k, v, n_heads, n_kv, hd, window, bias=None):
 
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens", [(40, 8, 64, 0, [1700]), (40, 8, 128, 300, [1500, 260]),
                                                          (32, 8, 128, 0, [2048]), (40, 8, 96, 0, [1500]),
-                                                         (40, 10, 32, 200, [2200, 70]), (12, 4, 96, 0, [1300])])
+                                                         (40, 10, 32, 200, [2200, 70]), (12, 4, 96, 0, [1300]),
+                                                         (40, 8, 80, 0, [1500]), (24, 8, 48, 100, [2300, 65]),
+                                                         (12, 4, 16, 0, [1300]), (40, 8, 112, 0, [1700])])
 def test_attn_prefill_with_many_and_with_few_workgroups(n_heads, n_kv, hd, window, lens):
     """The matrix-core prefill kernel has two forms: workgroups of eight waves that take a tile's keys in two
     halves (launches of at most two workgroups a compute unit, the third case) and of four waves (more, the
@@ -687,7 +689,8 @@ def one_query_reference(q, keys, vals, window):
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens,splits", [
     (4, 2, 16, 0, [5, 64, 65, 1], 1), (3, 1, 32, 16, [2, 30, 200], 2), (6, 3, 48, 100, [130, 640, 99], 3),
     (8, 2, 128, 0, [1000, 3], 7), (2, 2, 80, 0, [129], 4), (32, 8, 128, 0, [300], 2), (5, 5, 64, 70, [700, 64], 16),
-    (6, 2, 96, 0, [900, 65, 2], 5), (12, 3, 96, 130, [400, 129], 2), (16, 1, 32, 0, [2000, 7], 9)])
+    (6, 2, 96, 0, [900, 65, 2], 5), (12, 3, 96, 130, [400, 129], 2), (16, 1, 32, 0, [2000, 7], 9),
+    (10, 2, 112, 0, [777, 3], 4), (9, 3, 80, 64, [500, 64], 3), (4, 4, 16, 0, [129, 1000], 5)])
 def test_attn_decode(n_heads, n_kv, hd, window, lens, splits, dtype, simple):
     _attn_decode_case(n_heads, n_kv, hd, window, lens, splits, dtype, simple, None)
 
@@ -729,7 +732,8 @@ def _attn_decode_case(n_heads, n_kv, hd, window, lens, splits, dtype, simple, st
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens,n_bias", [
     (4, 2, 16, 0, [5, 130, 64], 200), (6, 3, 64, 70, [300, 1], 40), (8, 2, 128, 0, [257], 300), (3, 1, 48, 20, [90, 65], 7),
-    (40, 8, 128, 0, [1500], 900), (40, 8, 96, 200, [1100, 1200], 64), (12, 4, 32, 0, [1300], 2000), (16, 1, 64, 0, [70, 2], 3)])
+    (40, 8, 128, 0, [1500], 900), (40, 8, 96, 200, [1100, 1200], 64), (12, 4, 32, 0, [1300], 2000), (16, 1, 64, 0, [70, 2], 3),
+    (6, 2, 80, 0, [300, 65], 100), (10, 5, 112, 40, [200], 50)])
 def test_attn_with_a_score_bias(n_heads, n_kv, hd, window, lens, n_bias, dtype, simple):
     """A term added to every score by the distance of query and key (a table a head, the last entry for every
     distance beyond it): prompt and decode kernels against a float64 softmax with the same term.  The table is steep
@@ -806,7 +810,7 @@ def test_attn_decode_finds_a_far_key(dtype):
 
 @pytest.mark.parametrize("simple", [False, True])
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("hd,window,n", [(64, 70, 300), (128, 64, 200), (128, 100, 513), (32, 16, 90)])
+@pytest.mark.parametrize("hd,window,n", [(64, 70, 300), (128, 64, 200), (128, 100, 513), (32, 16, 90), (48, 33, 200), (112, 64, 150), (16, 8, 70)])
 def test_attn_window_edge_decides(hd, window, n, dtype, simple):
     """The key just outside the window has by far the largest score and a value of 1000; the key
     just inside has the next largest and a value of 7.  A window off by one, in either kernel,

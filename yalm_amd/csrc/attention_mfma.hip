@@ -56,7 +56,11 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
     const int* __restrict__ seq_len, float* __restrict__ partial, bf16* __restrict__ out, float* __restrict__ lse,
     int n_heads, int n_kv_heads, int window, int n_splits, int n_pages, const int* __restrict__ step_max_len,
     const int* __restrict__ seq_order, const float* __restrict__ bias, int n_bias) {
-  constexpr int KS = HD / 32, DT = HD / 16;
+  // A head size that is no multiple of 32 (pages in rows then): the last step of the scores' product is half empty.
+  // The query's lanes of that half hold zeros; the keys' lanes read the row's last 8 elements again (an address
+  // inside the row, finite values for every row that counts).
+  constexpr int KS = (HD + 31) / 32, DT = HD / 16;
+  static_assert(HD % 16 == 0 && (!BLOCKS || HD % 32 == 0), "head sizes in steps of 16; pages in blocks in steps of 32");
   __shared__ float sm_m[NW][16];
   __shared__ float sm_l[NW][16];
   __shared__ f32x4 sm_o[NW][DT][WAVE];
@@ -100,7 +104,8 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
       const bool head_ok = j < G;
       const bf16* qrow = q + ((size_t)b * n_heads + g * G + (head_ok ? j : 0)) * HD;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) qv[ks] = head_ok ? ld8(qrow + ks * 32 + qd * 8) : zero8();
+      for (int ks = 0; ks < KS; ++ks)
+        qv[ks] = head_ok && ks * 32 + qd * 8 < HD ? ld8(qrow + ks * 32 + qd * 8) : zero8();
     }
 
     const float* bias_row = BIAS ? bias + (size_t)(g * G + min(j, G - 1)) * n_bias : nullptr;   // the column's head
@@ -113,7 +118,7 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
           kreg[t][ks] = BLOCKS ? ld8_once(kp + ((ks * PAGE + t * 16 + j) * 32 + qd * 8))
-                               : ld8(kp + key_row(t, j) * HD + ks * 32 + qd * 8);
+                               : ld8(kp + key_row(t, j) * HD + min(ks * 32 + qd * 8, HD - 8));
     };
     int ap = p_begin + wave;
     int phys = ap < p_end ? page_of(ap) : 0;
@@ -276,11 +281,15 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
     bf16* __restrict__ out, float* __restrict__ out_f32, float* __restrict__ lse, const int* __restrict__ cu_seqlens,
     const int* __restrict__ seq_tile0, const int* __restrict__ tile_order, int fold_at, int B, int n_heads,
     int n_kv_heads, int window, const float* __restrict__ bias, int n_bias) {
-  constexpr int KS = HD / 32, DT = HD / 16;
+  // A head size that is no multiple of 32: the last step of the scores' product is half empty (zeros in the query's
+  // lanes, the row's last 8 elements once more in the keys'), and the tile's chunks do not divide evenly over the threads.
+  constexpr int KS = (HD + 31) / 32, DT = HD / 16;
+  static_assert(HD % 16 == 0, "head sizes in steps of 16");
   constexpr int KROW = HD + 8;                    // LDS row strides (elements): 16 bytes of padding
   constexpr int VROW = PAGE + 8;
   constexpr int KTILE = PAGE * KROW, VTILE = HD * VROW;
-  constexpr int NLOAD = HD / 32;                  // 16-byte chunks per thread and tile
+  constexpr int CHUNKS = PAGE * HD / 8;           // 16-byte chunks of a tile
+  constexpr int NLOAD = (CHUNKS + 255) / 256;     // chunks per thread and tile
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16* smem = reinterpret_cast<bf16*>(smem_raw);   // [2][KSPL][KTILE + VTILE]
 
@@ -327,7 +336,8 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
     q_ok[c] = pos_q[c] < len;
     const bf16* qrow = q + ((size_t)(start + (q_ok[c] ? pos_q[c] : 0)) * n_heads + h) * HD;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qv[c][ks] = q_ok[c] ? ld8(qrow + ks * 32 + qd * 8) : zero8();
+    for (int ks = 0; ks < KS; ++ks)
+      qv[c][ks] = q_ok[c] && ks * 32 + qd * 8 < HD ? ld8(qrow + ks * 32 + qd * 8) : zero8();
   }
   float m[NC], l[NC];
   f32x4 o[NC][DT];
@@ -354,7 +364,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
     const bf16* vp = v_stage + (tile0 + kt) * tile_elems + (size_t)g * PAGE * HD;
 #pragma unroll
     for (int p = 0; p < NLOAD; ++p) {
-      int c = tid + p * 256;
+      int c = min(tid + p * 256, CHUNKS - 1);       // a thread beyond the tile reads its last chunk and stores nothing
       rk[p] = ld8(kp + (size_t)c * 8);
       rv[p] = ld8(vp + (size_t)c * 8);
     }
@@ -365,6 +375,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
 #pragma unroll
     for (int p = 0; p < NLOAD; ++p) {
       int c = tid + p * 256;
+      if (CHUNKS % 256 != 0 && c >= CHUNKS) break;
       int row = c / (HD / 8), col = (c % (HD / 8)) * 8;              // key tile: [row][element]
       int t = 2 * (row >> 5) + ((row >> 2) & 1), i = 4 * ((row >> 3) & 3) + (row & 3);
       *reinterpret_cast<bf16x8*>(ks_l + (t * 16 + i) * KROW + col) = rk[p];
@@ -398,7 +409,7 @@ __global__ __launch_bounds__(256 * KSPL, KSPL == 1 ? 2 : 1) void attn_prefill_mf
       for (int t = 0; t < 4; ++t)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks_l + (t * 16 + j) * KROW + ks * 32 + qd * 8);
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(ks_l + (t * 16 + j) * KROW + min(ks * 32 + qd * 8, HD - 8));
 #pragma unroll
           for (int c = 0; c < NC; ++c)
             sc[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qv[c][ks], sc[c][t], 0, 0, 0);
@@ -546,10 +557,9 @@ int compute_units() {
   return n;
 }
 
-// head sizes the kernels are built for (any multiple of 32 would do: the products take 32 elements at a time)
+// head sizes the kernels are built for: 16 to 128 in steps of 16
 bool mfma_shape_ok(int n_heads, int n_kv_heads, int head_dim) {
-  return (head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128) && n_kv_heads > 0 &&
-         n_heads % n_kv_heads == 0;
+  return head_dim >= 16 && head_dim <= 128 && head_dim % 16 == 0 && n_kv_heads > 0 && n_heads % n_kv_heads == 0;
 }
 
 // launches attn_prefill_mfma_kernel<head_dim, NC, KSPL> (more than 64 KB of LDS is asked for once a device)
@@ -569,21 +579,20 @@ int launch_prefill(dim3 grid, int threads, size_t lds, hipStream_t stream, const
 }
 template <int NC, int KSPL, typename... Args>
 int launch_prefill_hd(int head_dim, bool biased, Args... args) {
-  if (biased) {
-    switch (head_dim) {
-      case 32: return launch_prefill<32, NC, KSPL, true>(args...);
-      case 64: return launch_prefill<64, NC, KSPL, true>(args...);
-      case 96: return launch_prefill<96, NC, KSPL, true>(args...);
-      case 128: return launch_prefill<128, NC, KSPL, true>(args...);
-    }
-    return YALM_ERR_ARG;
-  }
+#define YALM_PREFILL_HD(HD_)                                                        \
+  case HD_:                                                                         \
+    return biased ? launch_prefill<HD_, NC, KSPL, true>(args...) : launch_prefill<HD_, NC, KSPL, false>(args...)
   switch (head_dim) {
-    case 32: return launch_prefill<32, NC, KSPL, false>(args...);
-    case 64: return launch_prefill<64, NC, KSPL, false>(args...);
-    case 96: return launch_prefill<96, NC, KSPL, false>(args...);
-    case 128: return launch_prefill<128, NC, KSPL, false>(args...);
+    YALM_PREFILL_HD(16);
+    YALM_PREFILL_HD(32);
+    YALM_PREFILL_HD(48);
+    YALM_PREFILL_HD(64);
+    YALM_PREFILL_HD(80);
+    YALM_PREFILL_HD(96);
+    YALM_PREFILL_HD(112);
+    YALM_PREFILL_HD(128);
   }
+#undef YALM_PREFILL_HD
   return YALM_ERR_ARG;
 }
 }  // namespace
@@ -639,8 +648,10 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
   // with sinks the merge kernel always runs: it takes them in, also where there is one split
   const bool merge = n_splits > 1 || sinks.n_sinks > 0;
   if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_heads / n_kv_heads > 16) return YALM_ERR_ARG;
-  // a score bias: the pages in blocks only (the engine's layout), and no sinks (they are scored without it)
-  if (bias != nullptr && (n_bias <= 0 || page_layout != YALM_PAGE_BLOCKS || sinks.n_sinks > 0)) return YALM_ERR_ARG;
+  // a score bias: the engine's layout of the pages only (blocks where the head size allows), and no sinks (they are
+  // scored without it)
+  if (bias != nullptr && (n_bias <= 0 || (page_layout != YALM_PAGE_BLOCKS && head_dim % 32 == 0) || sinks.n_sinks > 0))
+    return YALM_ERR_ARG;
   dim3 grid(n_splits, n_kv_heads, B);
 #define YALM_DECODE(HD_, NW_, BLOCKS_, BIAS_)                                                                       \
   attn_decode_mfma_kernel<HD_, NW_, BLOCKS_, BIAS_><<<grid, NW_ * WAVE, 0, stream>>>(                               \
@@ -649,28 +660,32 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
       step_max_len, seq_order, bias, n_bias)
   // 4 waves a workgroup: 8 measured no faster with one split and slower with more (a CU draws about
   // 33 GB/s whatever its number of waves, so a small batch needs its workgroups spread over all CUs)
-  if (bias != nullptr) {
-    switch (head_dim) {
-      case 32: YALM_DECODE(32, 4, true, true); break;
-      case 64: YALM_DECODE(64, 4, true, true); break;
-      case 96: YALM_DECODE(96, 4, true, true); break;
-      default: YALM_DECODE(128, 4, true, true); break;
-    }
-  } else if (page_layout == YALM_PAGE_BLOCKS) {
-    switch (head_dim) {
-      case 32: YALM_DECODE(32, 4, true, false); break;
-      case 64: YALM_DECODE(64, 4, true, false); break;
-      case 96: YALM_DECODE(96, 4, true, false); break;
-      default: YALM_DECODE(128, 4, true, false); break;
-    }
-  } else {
-    switch (head_dim) {
-      case 32: YALM_DECODE(32, 4, false, false); break;
-      case 64: YALM_DECODE(64, 4, false, false); break;
-      case 96: YALM_DECODE(96, 4, false, false); break;
-      default: YALM_DECODE(128, 4, false, false); break;
-    }
+  // pages in blocks for the head sizes that are multiples of 32, in rows for the others (and for yalm_attn_decode)
+  const bool blocks = page_layout == YALM_PAGE_BLOCKS;
+  if (blocks && head_dim % 32 != 0) return YALM_ERR_ARG;
+#define YALM_DECODE_HD32(HD_)                                                       \
+  case HD_:                                                                         \
+    if (bias != nullptr) YALM_DECODE(HD_, 4, true, true);                           \
+    else if (blocks) YALM_DECODE(HD_, 4, true, false);                              \
+    else YALM_DECODE(HD_, 4, false, false);                                         \
+    break
+#define YALM_DECODE_HD16(HD_)                                                       \
+  case HD_:                                                                         \
+    if (bias != nullptr) YALM_DECODE(HD_, 4, false, true);                          \
+    else YALM_DECODE(HD_, 4, false, false);                                         \
+    break
+  switch (head_dim) {
+    YALM_DECODE_HD16(16);
+    YALM_DECODE_HD32(32);
+    YALM_DECODE_HD16(48);
+    YALM_DECODE_HD32(64);
+    YALM_DECODE_HD16(80);
+    YALM_DECODE_HD32(96);
+    YALM_DECODE_HD16(112);
+    YALM_DECODE_HD32(128);
   }
+#undef YALM_DECODE_HD32
+#undef YALM_DECODE_HD16
 #undef YALM_DECODE
   int rc = launch_status();
   if (rc != YALM_OK || !merge) return rc;          // one split writes the result itself

@@ -14,7 +14,7 @@ from . import library
 PAGE = 64                       # tokens per cache page (csrc/common.h)
 PREFILL_MIXED_TILES = 64        # prefill_tile_order mixes the sequences of a step up to this many tiles
 MAX_HEAD_DIM = 256
-MFMA_HEAD_DIMS = (32, 64, 96, 128)   # head sizes of the matrix-core attention kernels (others: float32 arithmetic)
+MFMA_HEAD_DIMS = tuple(range(16, 129, 16))   # head sizes of the matrix-core attention kernels (others: float32 arithmetic)
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
 

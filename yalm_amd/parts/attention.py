@@ -121,7 +121,7 @@ class GQAttention(Part):
             return what + ": matrix-core kernels", False
         why = "head size %d" % self.head_dim if self.head_dim not in kernels.MFMA_HEAD_DIMS else "%d heads a group" % group
         return what + ": float32-arithmetic kernels on bfloat16 storage (the matrix-core kernels take head sizes " \
-                      "32, 64, 96 and 128 and up to 16 heads a group, not %s): correct, several times slower" % why, True
+                      "of 16 to 128 in steps of 16 and up to 16 heads a group, not %s): correct, several times slower" % why, True
 
     def decode_splits(self, B, max_pages, ragged=False):
         mfma = self.head_dim in kernels.MFMA_HEAD_DIMS and self.n_heads // self.n_kv_heads <= 16 \
