@@ -690,7 +690,8 @@ def one_query_reference(q, keys, vals, window):
     (4, 2, 16, 0, [5, 64, 65, 1], 1), (3, 1, 32, 16, [2, 30, 200], 2), (6, 3, 48, 100, [130, 640, 99], 3),
     (8, 2, 128, 0, [1000, 3], 7), (2, 2, 80, 0, [129], 4), (32, 8, 128, 0, [300], 2), (5, 5, 64, 70, [700, 64], 16),
     (6, 2, 96, 0, [900, 65, 2], 5), (12, 3, 96, 130, [400, 129], 2), (16, 1, 32, 0, [2000, 7], 9),
-    (10, 2, 112, 0, [777, 3], 4), (9, 3, 80, 64, [500, 64], 3), (4, 4, 16, 0, [129, 1000], 5)])
+    (10, 2, 112, 0, [777, 3], 4), (9, 3, 80, 64, [500, 64], 3), (4, 4, 16, 0, [129, 1000], 5),
+    (34, 2, 64, 0, [300, 65], 3), (40, 1, 128, 100, [700], 4), (51, 3, 32, 0, [129, 2], 2)])   # more than 16 heads a group
 def test_attn_decode(n_heads, n_kv, hd, window, lens, splits, dtype, simple):
     _attn_decode_case(n_heads, n_kv, hd, window, lens, splits, dtype, simple, None)
 
@@ -733,7 +734,7 @@ def _attn_decode_case(n_heads, n_kv, hd, window, lens, splits, dtype, simple, st
 @pytest.mark.parametrize("n_heads,n_kv,hd,window,lens,n_bias", [
     (4, 2, 16, 0, [5, 130, 64], 200), (6, 3, 64, 70, [300, 1], 40), (8, 2, 128, 0, [257], 300), (3, 1, 48, 20, [90, 65], 7),
     (40, 8, 128, 0, [1500], 900), (40, 8, 96, 200, [1100, 1200], 64), (12, 4, 32, 0, [1300], 2000), (16, 1, 64, 0, [70, 2], 3),
-    (6, 2, 80, 0, [300, 65], 100), (10, 5, 112, 40, [200], 50)])
+    (6, 2, 80, 0, [300, 65], 100), (10, 5, 112, 40, [200], 50), (36, 2, 64, 0, [150, 70], 90)])
 def test_attn_with_a_score_bias(n_heads, n_kv, hd, window, lens, n_bias, dtype, simple):
     """A term added to every score by the distance of query and key (a table a head, the last entry for every
     distance beyond it): prompt and decode kernels against a float64 softmax with the same term.  The table is steep

@@ -65,11 +65,13 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
   __shared__ float sm_l[NW][16];
   __shared__ f32x4 sm_o[NW][DT][WAVE];
   // seq_order: the rows in the order of their cost (only which workgroup takes which row changes)
-  const int split = blockIdx.x, g = blockIdx.y;
+  // a group of more than 16 query heads is taken 16 heads (a tile's columns) a workgroup: blockIdx.y = (KV head, part)
+  const int Gall = n_heads / n_kv_heads, parts_g = (Gall + 15) / 16;
+  const int split = blockIdx.x, g = (int)blockIdx.y / parts_g, h0 = g * Gall + ((int)blockIdx.y % parts_g) * 16;
   const int b = seq_order != nullptr ? min(max(seq_order[blockIdx.z], 0), (int)gridDim.z - 1) : (int)blockIdx.z;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE), lane = threadIdx.x % WAVE, qd = lane / 16,
             j = lane % 16;
-  const int G = n_heads / n_kv_heads;
+  const int G = min(16, (g + 1) * Gall - h0);      // heads of this workgroup, the first being head h0
   const int slot = seq_slot[b];
   const int L = slot >= 0 ? seq_len[b] : 0;
 
@@ -102,13 +104,13 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
     bf16x8 qv[KS];
     {
       const bool head_ok = j < G;
-      const bf16* qrow = q + ((size_t)b * n_heads + g * G + (head_ok ? j : 0)) * HD;
+      const bf16* qrow = q + ((size_t)b * n_heads + h0 + (head_ok ? j : 0)) * HD;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
         qv[ks] = head_ok && ks * 32 + qd * 8 < HD ? ld8(qrow + ks * 32 + qd * 8) : zero8();
     }
 
-    const float* bias_row = BIAS ? bias + (size_t)(g * G + min(j, G - 1)) * n_bias : nullptr;   // the column's head
+    const float* bias_row = BIAS ? bias + (size_t)(h0 + min(j, G - 1)) * n_bias : nullptr;   // the column's head
     bf16x8 kreg[4][KS];
     auto page_of = [&](int a) { return min(max(table[a % ring_pages], 0), n_pages - 1); };
     auto load_keys = [&](int phys) {
@@ -227,7 +229,7 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
 #pragma unroll
     for (int w = 1; w < NW; ++w) lt += sm_l[w][j];
     if (n_splits == 1 && out != nullptr) {        // nothing to merge with: this is the result
-      bf16* orow = out + ((size_t)b * n_heads + g * G + j) * HD;
+      bf16* orow = out + ((size_t)b * n_heads + h0 + j) * HD;
       const float inv_l = lt > 0.f ? 1.0f / lt : 0.f;
       for (int dt = wave; dt < DT; dt += NW) {
         f32x4 v = sm_o[0][dt][lane];
@@ -237,9 +239,9 @@ __global__ __launch_bounds__(NW * WAVE, NW == 4 ? 2 : 1) void attn_decode_mfma_k
         for (int r = 0; r < 4; ++r) orow[dt * 16 + 4 * qd + r] = static_cast<bf16>(v[r] * inv_l);
       }
       if (lse != nullptr && wave == 0 && qd == 0)  // natural logarithm of the sum of exp(score): for a later mix with further keys
-        lse[(size_t)b * n_heads + g * G + j] = lt > 0.f ? m_all * LN2 + logf(lt) : -FLT_MAX;
+        lse[(size_t)b * n_heads + h0 + j] = lt > 0.f ? m_all * LN2 + logf(lt) : -FLT_MAX;
     } else {
-      float* part = partial + (((size_t)b * n_heads + g * G + j) * n_splits + split) * (HD + 2);
+      float* part = partial + (((size_t)b * n_heads + h0 + j) * n_splits + split) * (HD + 2);
       for (int dt = wave; dt < DT; dt += NW) {
         f32x4 v = sm_o[0][dt][lane];
 #pragma unroll
@@ -647,12 +649,14 @@ int yalm_attn_decode_bf16_mfma(const void* q, const void* k_pages, const void* v
                                hipStream_t stream) {
   // with sinks the merge kernel always runs: it takes them in, also where there is one split
   const bool merge = n_splits > 1 || sinks.n_sinks > 0;
-  if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim) || n_heads / n_kv_heads > 16) return YALM_ERR_ARG;
+  if (!mfma_shape_ok(n_heads, n_kv_heads, head_dim)) return YALM_ERR_ARG;
   // a score bias: the engine's layout of the pages only (blocks where the head size allows), and no sinks (they are
   // scored without it)
   if (bias != nullptr && (n_bias <= 0 || (page_layout != YALM_PAGE_BLOCKS && head_dim % 32 == 0) || sinks.n_sinks > 0))
     return YALM_ERR_ARG;
-  dim3 grid(n_splits, n_kv_heads, B);
+  const int parts_g = (n_heads / n_kv_heads + 15) / 16;      // workgroups a KV head: 16 query heads each
+  if ((long)n_kv_heads * parts_g > 65535) return YALM_ERR_ARG;
+  dim3 grid(n_splits, n_kv_heads * parts_g, B);
 #define YALM_DECODE(HD_, NW_, BLOCKS_, BIAS_)                                                                       \
   attn_decode_mfma_kernel<HD_, NW_, BLOCKS_, BIAS_><<<grid, NW_ * WAVE, 0, stream>>>(                               \
       (const bf16*)q, (const bf16*)k_pages, (const bf16*)v_pages, block_table, table_stride, ring_pages, seq_slot, \

@@ -116,18 +116,15 @@ class GQAttention(Part):
             (", window %d" % self.window if self.window else "") + (" + %d sinks" % self.sinks if self.sinks else ""))
         if compute_dtype != torch.bfloat16:
             return what + ": float32-arithmetic kernels", False
-        group = self.n_heads // self.n_kv_heads
-        if self.head_dim in kernels.MFMA_HEAD_DIMS and group <= 16:
+        if self.head_dim in kernels.MFMA_HEAD_DIMS:
             return what + ": matrix-core kernels", False
-        why = "head size %d" % self.head_dim if self.head_dim not in kernels.MFMA_HEAD_DIMS else "%d heads a group" % group
         return what + ": float32-arithmetic kernels on bfloat16 storage (the matrix-core kernels take head sizes " \
-                      "of 16 to 128 in steps of 16 and up to 16 heads a group, not %s): correct, several times slower" % why, True
+                      "of 16 to 128 in steps of 16, not %d): correct, several times slower" % self.head_dim, True
 
     def decode_splits(self, B, max_pages, ragged=False):
-        mfma = self.head_dim in kernels.MFMA_HEAD_DIMS and self.n_heads // self.n_kv_heads <= 16 \
-            and not kernels.FORCE_SIMPLE
-        if mfma:         # a workgroup of 4 waves per (split, KV head, sequence), a page per wave at a time
-            per = max(1, B * self.n_kv_heads)
+        mfma = self.head_dim in kernels.MFMA_HEAD_DIMS and not kernels.FORCE_SIMPLE
+        if mfma:         # a workgroup of 4 waves per (split, KV head and up to 16 of its query heads, sequence), a page per wave at a time
+            per = max(1, B * self.n_kv_heads * ((self.n_heads // self.n_kv_heads + 15) // 16))
             quarters = max(1, min((max_pages + 3) // 4, 4))
             if per > RESIDENT_WORKGROUPS:         # more than run at once: in quarters the last round is short
                 return quarters
