@@ -108,13 +108,13 @@ def build(force=True, jobs=None):
     objs = []
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
         futs = []
-        for s in srcs:
+        for s in sorted(srcs, key=lambda f: -os.path.getsize(os.path.join(HERE, f))):     # the longest compilations first
             obj = os.path.join(obj_dir, s[:-4] + ".o")
             objs.append(obj)
             futs.append(pool.submit(_compile_one, hipcc, s, obj))
         pending = set(futs)
         while pending:
-            done, pending = concurrent.futures.wait(pending, timeout=10)
+            done, pending = concurrent.futures.wait(pending, timeout=10, return_when=concurrent.futures.FIRST_COMPLETED)
             for f in done:
                 src, rc, err = f.result()
                 if rc != 0:
